@@ -1,0 +1,205 @@
+// Shared host-side declarations of the engine: error plumbing, the state
+// object, type-erased storage/tensor structs and the dispatch entry points
+// that the C ABI files call.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <exception>
+#include <string>
+
+#include "../../include/THC.h"
+#include "layout.hpp"
+
+namespace thc {
+
+// ---------------------------------------------------------------- errors --
+// Inside the library an error is a C++ exception, so temporaries unwind
+// cleanly; every extern "C" entry catches it and hands the message to the
+// installed TH handler (lib/THC uses THError/THArgCheck -> TH's handler,
+// e.g. THCGeneral.c:714-726, generic/THCTensorMathPointwise.cu:268-270).
+struct Error : std::exception {
+  std::string msg;
+  int arg;  // 0 = general error, >0 = argument number
+  Error(std::string m, int a) : msg(std::move(m)), arg(a) {}
+  const char* what() const noexcept override { return msg.c_str(); }
+};
+
+[[noreturn]] void raise_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+[[noreturn]] void raise_arg_error(int arg, const char* fmt, ...)
+    __attribute__((format(printf, 2, 3)));
+void deliver_error(const Error& e) noexcept;  // calls the handler or aborts
+void hip_check(hipError_t err, const char* file, int line);
+
+#define THC_CHECK(expr) ::thc::hip_check((expr), __FILE__, __LINE__)
+#define THC_ARG_CHECK(cond, arg, ...)                          \
+  do {                                                         \
+    if (!(cond)) ::thc::raise_arg_error((arg), __VA_ARGS__);   \
+  } while (0)
+
+// Body of a void entry point / of one that returns a value.
+#define THC_GUARD_VOID(...)                 \
+  try {                                     \
+    __VA_ARGS__;                            \
+  } catch (const ::thc::Error& e_) {        \
+    ::thc::deliver_error(e_);               \
+  }
+#define THC_GUARD_RET(fallback, ...)        \
+  try {                                     \
+    __VA_ARGS__;                            \
+  } catch (const ::thc::Error& e_) {        \
+    ::thc::deliver_error(e_);               \
+  }                                         \
+  return fallback;
+
+constexpr const char* kDimWarning =
+    "tensor too large or too many (>25) dimensions";  // THCTensorInfo.cuh:14-16
+
+// ------------------------------------------------------------ data types --
+enum class DType : int { F32 = 0, F16 = 1, I64 = 2 };
+inline size_t dtype_size(DType t) {
+  return t == DType::F32 ? 4 : (t == DType::F16 ? 2 : 8);
+}
+
+// Type-erased views of THCuda*Storage / THCuda*Tensor (all element types
+// share one field layout, generic/THCStorage.h:9-19, generic/THCTensor.h:7-19).
+struct AnyStorage {
+  void* data;
+  ptrdiff_t size;
+  int refcount;
+  char flag;
+  THCDeviceAllocator* allocator;
+  void* allocatorContext;
+  AnyStorage* view;
+  int device;
+};
+struct AnyTensor {
+  long* size;
+  long* stride;
+  int nDimension;
+  AnyStorage* storage;
+  ptrdiff_t storageOffset;
+  int refcount;
+  char flag;
+};
+
+inline void* tensor_data(const AnyTensor* t, DType dt) {
+  if (!t->storage || !t->storage->data) return nullptr;
+  return static_cast<char*>(t->storage->data) + t->storageOffset * (ptrdiff_t)dtype_size(dt);
+}
+inline ptrdiff_t tensor_numel(const AnyTensor* t) {
+  if (t->nDimension == 0) return 0;
+  ptrdiff_t n = 1;
+  for (int d = 0; d < t->nDimension; ++d) n *= t->size[d];
+  return n;
+}
+inline Layout tensor_layout(const AnyTensor* t) {
+  if (t->nDimension > kMaxDims) raise_arg_error(2, "%s", kDimWarning);
+  return make_layout(t->nDimension, t->size, t->stride);
+}
+
+// ----------------------------------------------------------------- state --
+hipStream_t current_stream(THCState* state);
+THCDeviceAllocator* state_allocator(THCState* state);  // THCGeneral.h.in:98-100
+int state_device(THCState* state);
+int num_compute_units(THCState* state);
+// Per-stream device scratch for partial results (THCGeneral.c:677-712).
+void* scratch_space(THCState* state, size_t* bytes);
+void check_same_gpu(THCState* state, int n, const AnyTensor* const* ts);
+void note_kernel(const char* name);  // for THCAmd_lastKernel
+long tuning(const char* key, long fallback);
+bool force_64bit_index();
+
+// --------------------------------------------------------- storage/tensor --
+AnyStorage* storage_new(THCState* s, DType dt, ptrdiff_t size);
+void storage_retain(AnyStorage* st);
+void storage_free(THCState* s, AnyStorage* st);
+void storage_resize(THCState* s, AnyStorage* st, ptrdiff_t size, DType dt);
+
+AnyTensor* tensor_new(THCState* s);
+AnyTensor* tensor_new_with_tensor(THCState* s, AnyTensor* src, DType dt);
+AnyTensor* tensor_new_with_size(THCState* s, int nd, const long* size, DType dt);
+void tensor_retain(AnyTensor* t);
+void tensor_free(THCState* s, AnyTensor* t);
+void tensor_set(THCState* s, AnyTensor* self, AnyTensor* src, DType dt);
+void tensor_set_storage_nd(THCState* s, AnyTensor* self, AnyStorage* st, ptrdiff_t off, int nd,
+                           const long* size, const long* stride, DType dt);
+void tensor_resize_nd(THCState* s, AnyTensor* self, int nd, const long* size, const long* stride,
+                      DType dt);
+void tensor_resize_as(THCState* s, AnyTensor* self, AnyTensor* src, DType dt);
+void tensor_narrow(THCState* s, AnyTensor* self, AnyTensor* src, int dim, long first, long size,
+                   DType dt);
+void tensor_select(THCState* s, AnyTensor* self, AnyTensor* src, int dim, long idx, DType dt);
+void tensor_transpose(THCState* s, AnyTensor* self, AnyTensor* src, int d1, int d2, DType dt);
+void tensor_squeeze(THCState* s, AnyTensor* self, AnyTensor* src, DType dt);
+void tensor_squeeze1d(THCState* s, AnyTensor* self, AnyTensor* src, int dim, DType dt);
+void tensor_unsqueeze1d(THCState* s, AnyTensor* self, AnyTensor* src, int dim, DType dt);
+int tensor_is_contiguous(const AnyTensor* t);
+AnyTensor* tensor_new_contiguous(THCState* s, AnyTensor* t, DType dt);
+AnyTensor* tensor_new_clone(THCState* s, AnyTensor* t, DType dt);
+void tensor_free_copy_to(THCState* s, AnyTensor* self, AnyTensor* dst, DType dt);
+
+// RAII holder for temporaries created inside an entry point.
+struct TensorRef {
+  THCState* s;
+  AnyTensor* t;
+  TensorRef(THCState* s_, AnyTensor* t_) : s(s_), t(t_) {}
+  TensorRef(const TensorRef&) = delete;
+  TensorRef& operator=(const TensorRef&) = delete;
+  ~TensorRef() {
+    if (t) tensor_free(s, t);
+  }
+  AnyTensor* release() {
+    AnyTensor* r = t;
+    t = nullptr;
+    return r;
+  }
+};
+
+// ---------------------------------------------------------- apply engine --
+// out[i] = f(in0[i], in1[i], in2[i]) at every logical index i. In-place forms
+// pass the same tensor as `out` and as an input. (THC_pointwiseApply1/2/3,
+// lib/THC/THCApply.cuh:124-640.)
+enum class PointOp : int {
+  Copy,     // out = in0
+  AddC,     // out = in0 + v
+  SubC,     // out = in0 - v
+  MulC,     // out = in0 * v
+  DivC,     // out = in0 / v
+  Add,      // out = in0 + in1
+  Sub,      // out = in0 - in1
+  Mul,      // out = in0 * in1
+  Div,      // out = in0 / in1
+  CAdd,     // out = in0 + v * in1
+  AddCMul,  // out = in0 + v * (in1 * in2)
+  AddCDiv,  // out = in0 + v * (in1 / in2)
+  Fill,     // out = v (no input)
+  Pow,      // out = powf(in0, v)
+};
+int point_op_inputs(PointOp op);
+
+// Returns false for the conditions on which the reference's engine returns
+// false (element-count mismatch, too many dims).
+bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* out,
+                     AnyTensor* in0, AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap = false);
+void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ignoreOverlap);
+void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src);
+
+// --------------------------------------------------------- reduce engine --
+enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP };
+enum class Epilogue : int { None, Sqrt, PowInv, DivN };
+
+// out[..., 0, ...] = reduce over dim (THC_reduceDim, lib/THC/THCReduce.cuh:263-453)
+bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* out,
+                AnyTensor* in, int dim, int keepdim);
+// (value, 1-based index) of the max/min along dim, lowest index on ties
+// (THC_reduceDimIndex, lib/THC/THCTensorMathReduce.cuh:619-661)
+void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyTensor* indices,
+                      AnyTensor* in, int dim, int keepdim);
+// Whole-tensor reduction returned on the host; blocks on a 4-byte D2H copy
+// (THC_reduceAll, lib/THC/THCReduceAll.cuh:239-342)
+bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result);
+
+}  // namespace thc

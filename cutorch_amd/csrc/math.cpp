@@ -1,0 +1,227 @@
+// C entry points of the pointwise and reduction math: argument checks,
+// in-place vs out-of-place selection, output resizing, functor choice.
+// One definition per reference entry point:
+//   generic/THCTensorMathPairwise.cu:5-81     add sub mul div (tensor, scalar)
+//   generic/THCTensorMathPointwise.cu:264-414 cadd csub cmul cdiv
+//   generic/THCTensorMathPointwise.cu:582-630 addcmul addcdiv
+//   generic/THCTensorMath.cu:5-36             fill zero
+//   generic/THCTensorMathReduce.cu:5-43       sum prod mean
+//   generic/THCTensorMathReduce.cu:160-232    norm normall
+//   generic/THCTensorMathReduce.cu:261-333    sumall prodall meanall minall maxall
+//   generic/THCTensorMathReduce.cu:400-436    max min
+#include <cfloat>
+#include <cmath>
+
+#include "common.hpp"
+
+using namespace thc;
+
+namespace {
+
+inline float to_float(float v) { return v; }
+inline float to_float(THHalf v) { return THC_half2float(v); }
+template <typename R>
+R from_float(float v);
+template <>
+inline float from_float<float>(float v) { return v; }
+template <>
+inline THHalf from_float<THHalf>(float v) { return THC_float2half(v); }
+
+#define TN(x) ((AnyTensor*)(x))
+
+void same_gpu(THCState* s, std::initializer_list<const void*> ts) {
+  const AnyTensor* arr[8];
+  int n = 0;
+  for (const void* t : ts) arr[n++] = (const AnyTensor*)t;
+  check_same_gpu(s, n, arr);
+}
+
+void apply_or_throw(THCState* s, DType dt, PointOp op, float v, AnyTensor* out, AnyTensor* a,
+                    AnyTensor* b = nullptr, AnyTensor* c = nullptr) {
+  if (!pointwise_apply(s, dt, op, v, out, a, b, c)) raise_arg_error(2, "%s", kDimWarning);
+}
+
+// tensor (op) scalar
+void scalar_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, AnyTensor* src) {
+  same_gpu(s, {self, src});
+  if (self != src) tensor_resize_as(s, self, src, dt);
+  apply_or_throw(s, dt, op, v, self, src);
+}
+
+// tensor (op) tensor; `self == src1` is the in-place form
+void binary_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, AnyTensor* src1,
+               AnyTensor* src2) {
+  same_gpu(s, {self, src1, src2});
+  THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), 3, "sizes do not match");
+  if (self != src1) tensor_resize_as(s, self, src1, dt);
+  apply_or_throw(s, dt, op, v, self, src1, src2);
+}
+
+// self = t + v * (src1 (op) src2). The reference copies t into self and then
+// runs an in-place apply3 (generic/THCTensorMathPointwise.cu:586-590); here
+// t is read directly as a fourth operand, which saves a full pass.
+void ternary_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, AnyTensor* t,
+                AnyTensor* src1, AnyTensor* src2) {
+  same_gpu(s, {self, t, src1, src2});
+  if (self != t)
+    tensor_resize_as(s, self, t, dt);
+  else
+    THC_ARG_CHECK(tensor_numel(self) == tensor_numel(src1), 1, "sizes do not match");
+  THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), 3, "sizes do not match");
+  apply_or_throw(s, dt, op, v, self, t, src1, src2);
+}
+
+void reduce_or_throw(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* self,
+                     AnyTensor* src, long dim, int keepdim) {
+  same_gpu(s, {self, src});
+  if (!reduce_dim(s, dt, op, ep, p, self, src, (int)dim, keepdim))
+    raise_arg_error(2, "%s", kDimWarning);
+}
+
+void norm_dim(THCState* s, DType dt, float p, AnyTensor* self, AnyTensor* src, long dim,
+              int keepdim) {
+  if (p == 0.f)
+    reduce_or_throw(s, dt, ReduceOp::Norm0, Epilogue::None, p, self, src, dim, keepdim);
+  else if (p == 1.f)
+    reduce_or_throw(s, dt, ReduceOp::Norm1, Epilogue::None, p, self, src, dim, keepdim);
+  else if (p == 2.f)
+    reduce_or_throw(s, dt, ReduceOp::Norm2, Epilogue::Sqrt, p, self, src, dim, keepdim);
+  else
+    reduce_or_throw(s, dt, ReduceOp::NormP, Epilogue::PowInv, p, self, src, dim, keepdim);
+}
+
+float all_or_throw(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* self) {
+  same_gpu(s, {self});
+  float r = 0.f;
+  if (!reduce_all(s, dt, op, p, self, &r)) raise_arg_error(1, "%s", kDimWarning);
+  return r;
+}
+
+float norm_all(THCState* s, DType dt, float p, AnyTensor* self) {
+  if (p == 0.f) return all_or_throw(s, dt, ReduceOp::Norm0, p, self);
+  if (p == 1.f) return all_or_throw(s, dt, ReduceOp::Norm1, p, self);
+  if (p == 2.f) return sqrtf(all_or_throw(s, dt, ReduceOp::Norm2, p, self));
+  return powf(all_or_throw(s, dt, ReduceOp::NormP, p, self), 1.0f / p);
+}
+
+void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
+  same_gpu(s, {self});
+  if (!pointwise_apply(s, dt, PointOp::Fill, v, self, nullptr, nullptr, nullptr))
+    raise_arg_error(1, "%s", kDimWarning);
+}
+
+}  // namespace
+
+#define THC_AMD_DEFINE_MATH_API(Tensor, real, DT, REAL_MAX)                                        \
+  THC_API void Tensor##_add(THCState* s, Tensor* self, Tensor* src, real v) {                      \
+    THC_GUARD_VOID(scalar_op(s, DT, PointOp::AddC, to_float(v), TN(self), TN(src)))                \
+  }                                                                                                \
+  THC_API void Tensor##_sub(THCState* s, Tensor* self, Tensor* src, real v) {                      \
+    THC_GUARD_VOID(scalar_op(s, DT, PointOp::SubC, to_float(v), TN(self), TN(src)))                \
+  }                                                                                                \
+  THC_API void Tensor##_mul(THCState* s, Tensor* self, Tensor* src, real v) {                      \
+    THC_GUARD_VOID(scalar_op(s, DT, PointOp::MulC, to_float(v), TN(self), TN(src)))                \
+  }                                                                                                \
+  THC_API void Tensor##_div(THCState* s, Tensor* self, Tensor* src, real v) {                      \
+    THC_GUARD_VOID({                                                                               \
+      THC_ARG_CHECK(to_float(v) != 0.f, 3, "divide by zero");                                      \
+      scalar_op(s, DT, PointOp::DivC, to_float(v), TN(self), TN(src));                             \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_cadd(THCState* s, Tensor* self, Tensor* src1, real v, Tensor* src2) {      \
+    THC_GUARD_VOID({                                                                               \
+      const float f = to_float(v);                                                                 \
+      binary_op(s, DT, f == 1.f ? PointOp::Add : PointOp::CAdd, f, TN(self), TN(src1), TN(src2));  \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_csub(THCState* s, Tensor* self, Tensor* src1, real v, Tensor* src2) {      \
+    THC_GUARD_VOID({                                                                               \
+      const float f = to_float(v);                                                                 \
+      if (f == 1.f)                                                                                \
+        binary_op(s, DT, PointOp::Sub, f, TN(self), TN(src1), TN(src2));                           \
+      else                                                                                         \
+        binary_op(s, DT, PointOp::CAdd, -f, TN(self), TN(src1), TN(src2));                         \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_cmul(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {              \
+    THC_GUARD_VOID(binary_op(s, DT, PointOp::Mul, 0.f, TN(self), TN(src1), TN(src2)))              \
+  }                                                                                                \
+  THC_API void Tensor##_cdiv(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {              \
+    THC_GUARD_VOID(binary_op(s, DT, PointOp::Div, 0.f, TN(self), TN(src1), TN(src2)))              \
+  }                                                                                                \
+  THC_API void Tensor##_addcmul(THCState* s, Tensor* self, Tensor* t, real v, Tensor* src1,        \
+                                Tensor* src2) {                                                    \
+    THC_GUARD_VOID(ternary_op(s, DT, PointOp::AddCMul, to_float(v), TN(self), TN(t), TN(src1),     \
+                              TN(src2)))                                                           \
+  }                                                                                                \
+  THC_API void Tensor##_addcdiv(THCState* s, Tensor* self, Tensor* t, real v, Tensor* src1,        \
+                                Tensor* src2) {                                                    \
+    THC_GUARD_VOID(ternary_op(s, DT, PointOp::AddCDiv, to_float(v), TN(self), TN(t), TN(src1),     \
+                              TN(src2)))                                                           \
+  }                                                                                                \
+  THC_API void Tensor##_fill(THCState* s, Tensor* self, real v) {                                  \
+    THC_GUARD_VOID(fill_tensor(s, DT, TN(self), to_float(v)))                                      \
+  }                                                                                                \
+  THC_API void Tensor##_zero(THCState* s, Tensor* self) {                                          \
+    THC_GUARD_VOID(fill_tensor(s, DT, TN(self), 0.f))                                              \
+  }                                                                                                \
+  THC_API void Tensor##_sum(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {       \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Sum, Epilogue::None, 0.f, TN(self), TN(src),   \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_prod(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {      \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Prod, Epilogue::None, 0.f, TN(self), TN(src),  \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_mean(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {      \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Sum, Epilogue::DivN, 0.f, TN(self), TN(src),   \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_norm(THCState* s, Tensor* self, Tensor* src, real p, long dim,             \
+                             int keepdim) {                                                        \
+    THC_GUARD_VOID(norm_dim(s, DT, to_float(p), TN(self), TN(src), dim, keepdim))                  \
+  }                                                                                                \
+  THC_API void Tensor##_max(THCState* s, Tensor* values, THCudaLongTensor* indices, Tensor* src,   \
+                            long dim, int keepdim) {                                               \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {values, indices, src});                                                         \
+      reduce_dim_index(s, DT, true, TN(values), TN(indices), TN(src), (int)dim, keepdim);          \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_min(THCState* s, Tensor* values, THCudaLongTensor* indices, Tensor* src,   \
+                            long dim, int keepdim) {                                               \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {values, indices, src});                                                         \
+      reduce_dim_index(s, DT, false, TN(values), TN(indices), TN(src), (int)dim, keepdim);         \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API float Tensor##_sumall(THCState* s, Tensor* self) {                                       \
+    THC_GUARD_RET(0.f, return all_or_throw(s, DT, ReduceOp::Sum, 0.f, TN(self)))                   \
+  }                                                                                                \
+  THC_API float Tensor##_prodall(THCState* s, Tensor* self) {                                      \
+    THC_GUARD_RET(0.f, return all_or_throw(s, DT, ReduceOp::Prod, 0.f, TN(self)))                  \
+  }                                                                                                \
+  THC_API float Tensor##_meanall(THCState* s, Tensor* self) {                                      \
+    THC_GUARD_RET(0.f, {                                                                           \
+      THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");                                      \
+      return all_or_throw(s, DT, ReduceOp::Sum, 0.f, TN(self)) / (float)tensor_numel(TN(self));    \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API float Tensor##_normall(THCState* s, Tensor* self, real p) {                              \
+    THC_GUARD_RET(0.f, return norm_all(s, DT, to_float(p), TN(self)))                              \
+  }                                                                                                \
+  THC_API real Tensor##_minall(THCState* s, Tensor* self) {                                        \
+    THC_GUARD_RET(from_float<real>(0.f), {                                                         \
+      if (self->nDimension == 0) return from_float<real>(REAL_MAX);                                \
+      return from_float<real>(all_or_throw(s, DT, ReduceOp::Min, 0.f, TN(self)));                  \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API real Tensor##_maxall(THCState* s, Tensor* self) {                                        \
+    THC_GUARD_RET(from_float<real>(0.f), {                                                         \
+      if (self->nDimension == 0) return from_float<real>(-REAL_MAX);                               \
+      return from_float<real>(all_or_throw(s, DT, ReduceOp::Max, 0.f, TN(self)));                  \
+    })                                                                                             \
+  }
+
+THC_AMD_DEFINE_MATH_API(THCudaTensor, float, DType::F32, FLT_MAX)
+THC_AMD_DEFINE_MATH_API(THCudaHalfTensor, THHalf, DType::F16, 65504.f)

@@ -1,0 +1,1057 @@
+// Dimension and whole-tensor reductions for gfx950 (wave64).
+//
+// Role of THC_reduceDim / THC_reduceAll / THC_reduceDimIndex and their kernels
+// (lib/THC/THCReduce.cuh:35-453, THCReduceAll.cuh:28-342,
+// THCTensorMathReduce.cuh:453-661). Redesigned around three access shapes:
+//
+//   rows   the reduced dim has stride 1. A group of G lanes (G = 1..64, a power
+//          of two chosen from the row length) owns one row, streams it with
+//          16-byte loads and finishes with an xor-butterfly inside the wave.
+//          Long rows with few siblings are cut into chunks ("virtual rows");
+//          the per-chunk partials land in scratch and a second launch of the
+//          same kernel folds them. reduceAll is the one-row case of this.
+//   cols   the reduced dim is strided and another dim has stride 1 (reducing
+//          a non-innermost dim of a dense tensor). Lanes run along the
+//          unit-stride dim with 16-byte loads, thread rows and, if the output
+//          is too small to fill 256 CUs, extra workgroups split the reduced
+//          dim; LDS folds the thread rows, a tiny second kernel folds the
+//          workgroup partials in a fixed order (bit-reproducible).
+//   generic  anything else: one thread per output walks the reduced dim.
+//
+// Accumulation is fp32 for float and half input (accreal = float,
+// THCGenerateFloatType.h:5-8, THCGenerateHalfType.h:9-10); results are rounded
+// once on store. max/min carry (value, index) pairs whose combine step prefers
+// the lower index on equal values at every level, so the first occurrence wins
+// as in a sequential scan; the first NaN wins over everything.
+#include <hip/hip_fp16.h>
+
+#include <cmath>
+#include <limits>
+
+#include "common.hpp"
+
+namespace thc {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack {
+  T v[N];
+};
+
+template <typename T>
+struct Cvt {
+  static __device__ __forceinline__ float up(T x) { return (float)x; }
+  static __device__ __forceinline__ T down(float x) { return (T)x; }
+};
+template <>
+struct Cvt<__half> {
+  static __device__ __forceinline__ float up(__half x) { return __half2float(x); }
+  static __device__ __forceinline__ __half down(float x) { return __float2half_rn(x); }
+};
+
+template <typename I>
+struct Divisor;
+template <>
+struct Divisor<uint32_t> {
+  uint32_t d, m, s;
+  __host__ void set(uint64_t div) {
+    d = (uint32_t)div;
+    for (s = 0; s < 32; ++s)
+      if ((uint64_t(1) << s) >= div) break;
+    m = (uint32_t)(((uint64_t(1) << 32) * ((uint64_t(1) << s) - div)) / div + 1);
+  }
+  __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+    q = (__umulhi(n, m) + n) >> s;
+    r = n - q * d;
+  }
+};
+template <>
+struct Divisor<uint64_t> {
+  uint64_t d;
+  __host__ void set(uint64_t div) { d = div; }
+  __device__ __forceinline__ void divmod(uint64_t n, uint64_t& q, uint64_t& r) const {
+    q = n / d;
+    r = n - q * d;
+  }
+};
+
+// --------------------------------------------------------------- functors --
+struct Epi {
+  int kind;   // Epilogue
+  float arg;  // 1/p for PowInv, n for DivN
+  template <typename T>
+  __device__ __forceinline__ T finish(float acc) const {
+    switch (kind) {
+      case (int)Epilogue::Sqrt: return Cvt<T>::down(sqrtf(acc));
+      case (int)Epilogue::PowInv: return Cvt<T>::down(powf(acc, arg));
+      case (int)Epilogue::DivN: return Cvt<T>::down(Cvt<T>::up(Cvt<T>::down(acc)) / arg);
+      default: return Cvt<T>::down(acc);
+    }
+  }
+};
+
+__device__ __forceinline__ float nan_max(float a, float b) {
+  return (a != a) ? a : ((b != b) ? b : fmaxf(a, b));
+}
+__device__ __forceinline__ float nan_min(float a, float b) {
+  return (a != a) ? a : ((b != b) ? b : fminf(a, b));
+}
+
+#define THC_REDUCE_FUNCTOR(Name, INIT, MODIFY, COMBINE)                              \
+  struct Name {                                                                      \
+    float p;                                                                         \
+    __host__ __device__ __forceinline__ float init() const { return INIT; }          \
+    __device__ __forceinline__ float modify(float x) const { return MODIFY; }        \
+    __device__ __forceinline__ float combine(float a, float b) const { return COMBINE; } \
+  };
+THC_REDUCE_FUNCTOR(FSum, 0.f, x, a + b)
+THC_REDUCE_FUNCTOR(FProd, 1.f, x, a * b)
+THC_REDUCE_FUNCTOR(FMax, -INFINITY, x, nan_max(a, b))
+THC_REDUCE_FUNCTOR(FMin, INFINITY, x, nan_min(a, b))
+THC_REDUCE_FUNCTOR(FNorm0, 0.f, (x != 0.f ? 1.f : 0.f), a + b)
+THC_REDUCE_FUNCTOR(FNorm1, 0.f, fabsf(x), a + b)
+THC_REDUCE_FUNCTOR(FNorm2, 0.f, x * x, a + b)
+THC_REDUCE_FUNCTOR(FNormP, 0.f, powf(fabsf(x), p), a + b)
+#undef THC_REDUCE_FUNCTOR
+
+// (value, index) pairs. `better(a, b)`: a must replace b.
+template <bool IS_MAX>
+struct PairOrder {
+  static __device__ __forceinline__ float worst() { return IS_MAX ? -INFINITY : INFINITY; }
+  template <typename X>
+  static __device__ __forceinline__ bool better(float av, X ai, float bv, X bi) {
+    const bool an = av != av, bn = bv != bv;
+    if (an || bn) return an && (!bn || ai < bi);
+    return (IS_MAX ? av > bv : av < bv) || (av == bv && ai < bi);
+  }
+};
+
+// Coordinates of an output element / a row in the joint (input, output)
+// space of the non-reduced dims.
+template <typename I>
+struct OuterArgs {
+  int dims;
+  Divisor<I> size[kMaxDims];
+  I inStride[kMaxDims];
+  I outStride[kMaxDims];
+  __device__ __forceinline__ void offsets(I lin, I& inOff, I& outOff) const {
+    inOff = 0;
+    outOff = 0;
+    for (int d = dims - 1; d > 0; --d) {
+      I r;
+      size[d].divmod(lin, lin, r);
+      inOff += r * inStride[d];
+      outOff += r * outStride[d];
+    }
+    inOff += lin * inStride[0];
+    outOff += lin * outStride[0];
+  }
+};
+
+// ------------------------------------------------------------------ rows --
+// Virtual row vr = row * S + s covers [s*chunk, min(R, (s+1)*chunk)) of `row`.
+// S == 1: the result goes to out at the row's output offset (with epilogue).
+// S  > 1: the fp32 partial goes to partial[vr].
+template <typename TIn, typename TOut, typename F, typename I, int VEC, bool FIRST>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restrict__ in,
+                                                             TOut* __restrict__ out,
+                                                             float* __restrict__ partial,
+                                                             OuterArgs<I> oa, I numRows, I R,
+                                                             Divisor<I> S, I chunk, uint32_t G,
+                                                             Epi epi, F f) {
+  using P = Pack<TIn, VEC>;
+  const uint32_t groups = kBlock / G;
+  const uint32_t lane = threadIdx.x % G;
+  const uint32_t grp = threadIdx.x / G;
+  const I total = numRows * S.d;
+  for (I vr0 = (I)blockIdx.x * groups; vr0 < total; vr0 += (I)gridDim.x * groups) {
+    const I vr = vr0 + grp;
+    const bool active = vr < total;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+    I outOff = 0;
+    if (active) {
+      I row, s, inOff;
+      S.divmod(vr, row, s);
+      oa.offsets(row, inOff, outOff);
+      const I begin = s * chunk;
+      const I end = min(R, begin + chunk);
+      const TIn* src = in + inOff;
+#pragma unroll 4
+      for (I i = begin + lane * VEC; i < end; i += (I)G * VEC) {
+        const P v = *reinterpret_cast<const P*>(src + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = Cvt<TIn>::up(v.v[e]);
+          acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+        }
+      }
+    }
+    float r = acc[0];
+#pragma unroll
+    for (int e = 1; e < VEC; ++e) r = f.combine(r, acc[e]);
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) r = f.combine(r, __shfl_xor(r, o, 64));
+    if (active && lane == 0) {
+      if (S.d > 1)
+        partial[vr] = r;
+      else
+        out[outOff] = epi.template finish<TOut>(r);
+    }
+  }
+}
+
+// max/min with index along a unit-stride dim: one group of G lanes per row.
+template <typename T, typename I, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __restrict__ in,
+                                                                   T* __restrict__ outV,
+                                                                   long* __restrict__ outI,
+                                                                   OuterArgs<I> oa,
+                                                                   OuterArgs<I> oaIdx, I numRows,
+                                                                   I R, uint32_t G) {
+  using P = Pack<T, VEC>;
+  using O = PairOrder<IS_MAX>;
+  const uint32_t groups = kBlock / G;
+  const uint32_t lane = threadIdx.x % G;
+  const uint32_t grp = threadIdx.x / G;
+  for (I r0 = (I)blockIdx.x * groups; r0 < numRows; r0 += (I)gridDim.x * groups) {
+    const I row = r0 + grp;
+    const bool active = row < numRows;
+    float bv = O::worst();
+    I bi = ~(I)0;
+    I outOff = 0, idxOff = 0;
+    if (active) {
+      I inOff, unused;
+      oa.offsets(row, inOff, outOff);
+      oaIdx.offsets(row, unused, idxOff);
+      const T* src = in + inOff;
+#pragma unroll 4
+      for (I i = lane * VEC; i < R; i += (I)G * VEC) {
+        const P v = *reinterpret_cast<const P*>(src + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = Cvt<T>::up(v.v[e]);
+          if (O::better(x, i + e, bv, bi)) {
+            bv = x;
+            bi = i + e;
+          }
+        }
+      }
+    }
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      I oi;
+      if (sizeof(I) == 8) {
+        const uint32_t lo = __shfl_xor((uint32_t)bi, o, 64);
+        const uint32_t hi = __shfl_xor((uint32_t)((uint64_t)bi >> 32), o, 64);
+        oi = (I)(((uint64_t)hi << 32) | lo);
+      } else {
+        oi = (I)__shfl_xor((uint32_t)bi, o, 64);
+      }
+      if (O::better(ov, oi, bv, bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (active && lane == 0) {
+      outV[outOff] = Cvt<T>::down(bv);
+      outI[idxOff] = (long)bi + 1;  // 1-based (TH_INDEX_BASE)
+    }
+  }
+}
+
+// ------------------------------------------------------------------ cols --
+template <typename I>
+struct ColsArgs {
+  OuterArgs<I> oa;      // dims other than the reduced one and the unit-stride one
+  I C;                  // length of the unit-stride dim
+  I R, sR;              // reduced dim: length, input stride
+  I outInner;           // output stride along the unit-stride dim
+  I chunkR;             // rows of the reduced dim per workgroup
+  Divisor<I> S;         // workgroups along the reduced dim
+  Divisor<I> colTiles;  // workgroups along the unit-stride dim
+  I outElems;           // number of outputs (stride between partial planes)
+  uint32_t TX;          // lanes along the unit-stride dim (power of two <= 256)
+};
+
+template <typename TIn, typename TOut, typename F, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restrict__ in,
+                                                             TOut* __restrict__ out,
+                                                             float* __restrict__ partial,
+                                                             ColsArgs<I> a, I totalBlocks, Epi epi,
+                                                             F f) {
+  using P = Pack<TIn, VEC>;
+  __shared__ float smem[kBlock * VEC];
+  const uint32_t TX = a.TX, TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I rest, s, ct;
+    a.S.divmod(b, rest, s);
+    a.colTiles.divmod(rest, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+    if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const TIn* src = in + inOff + col;
+#pragma unroll 4
+      for (I r = begin + ty; r < end; r += TY) {
+        const P v = *reinterpret_cast<const P*>(src + r * a.sR);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e])));
+      }
+    }
+    // fold the TY thread rows (fixed tree)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) smem[(ty * TX + tx) * VEC + e] = acc[e];
+    __syncthreads();
+    for (uint32_t h = TY >> 1; h > 0; h >>= 1) {
+      if (ty < h) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const uint32_t i = (ty * TX + tx) * VEC + e;
+          smem[i] = f.combine(smem[i], smem[i + h * TX * VEC]);
+        }
+      }
+      __syncthreads();
+    }
+    if (ty == 0 && col < a.C) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float r = smem[tx * VEC + e];
+        if (a.S.d > 1)
+          partial[s * a.outElems + rest * a.C + col + e] = r;
+        else
+          out[outOff + (col + e) * a.outInner] = epi.template finish<TOut>(r);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Fold S partial planes [S][outElems] in plane order and store.
+template <typename TOut, typename F, typename I>
+__global__ __launch_bounds__(kBlock) void reduce_partials_kernel(const float* __restrict__ partial,
+                                                                 TOut* __restrict__ out,
+                                                                 ColsArgs<I> a, Epi epi, F f) {
+  const I step = (I)gridDim.x * kBlock;
+  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < a.outElems; o += step) {
+    float r = f.init();
+    for (I s = 0; s < a.S.d; ++s) r = f.combine(r, partial[s * a.outElems + o]);
+    const I outer = o / a.C, col = o - outer * a.C;
+    I inOff, outOff;
+    a.oa.offsets(outer, inOff, outOff);
+    out[outOff + col * a.outInner] = epi.template finish<TOut>(r);
+  }
+}
+
+template <typename T, typename I, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
+    float* __restrict__ partV, I* __restrict__ partI, ColsArgs<I> a, OuterArgs<I> oaIdx,
+    I idxInner, I totalBlocks) {
+  using P = Pack<T, VEC>;
+  using O = PairOrder<IS_MAX>;
+  __shared__ float sv[kBlock * VEC];
+  __shared__ I si[kBlock * VEC];
+  const uint32_t TX = a.TX, TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I rest, s, ct;
+    a.S.divmod(b, rest, s);
+    a.colTiles.divmod(rest, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    float bv[VEC];
+    I bi[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      bv[e] = O::worst();
+      bi[e] = ~(I)0;
+    }
+    if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const T* src = in + inOff + col;
+#pragma unroll 4
+      for (I r = begin + ty; r < end; r += TY) {
+        const P v = *reinterpret_cast<const P*>(src + r * a.sR);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = Cvt<T>::up(v.v[e]);
+          if (O::better(x, r, bv[e], bi[e])) {
+            bv[e] = x;
+            bi[e] = r;
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      sv[(ty * TX + tx) * VEC + e] = bv[e];
+      si[(ty * TX + tx) * VEC + e] = bi[e];
+    }
+    __syncthreads();
+    for (uint32_t h = TY >> 1; h > 0; h >>= 1) {
+      if (ty < h) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const uint32_t i = (ty * TX + tx) * VEC + e, j = i + h * TX * VEC;
+          if (O::better(sv[j], si[j], sv[i], si[i])) {
+            sv[i] = sv[j];
+            si[i] = si[j];
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (ty == 0 && col < a.C) {
+      I unused, idxOff;
+      oaIdx.offsets(rest, unused, idxOff);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float v = sv[tx * VEC + e];
+        const I ix = si[tx * VEC + e];
+        if (a.S.d > 1) {
+          partV[s * a.outElems + rest * a.C + col + e] = v;
+          partI[s * a.outElems + rest * a.C + col + e] = ix;
+        } else {
+          outV[outOff + (col + e) * a.outInner] = Cvt<T>::down(v);
+          outI[idxOff + (col + e) * idxInner] = (long)ix + 1;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_partials_index_kernel(
+    const float* __restrict__ partV, const I* __restrict__ partI, T* __restrict__ outV,
+    long* __restrict__ outI, ColsArgs<I> a, OuterArgs<I> oaIdx, I idxInner) {
+  using O = PairOrder<IS_MAX>;
+  const I step = (I)gridDim.x * kBlock;
+  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < a.outElems; o += step) {
+    float bv = O::worst();
+    I bi = ~(I)0;
+    for (I s = 0; s < a.S.d; ++s) {
+      const float v = partV[s * a.outElems + o];
+      const I ix = partI[s * a.outElems + o];
+      if (O::better(v, ix, bv, bi)) {
+        bv = v;
+        bi = ix;
+      }
+    }
+    const I outer = o / a.C, col = o - outer * a.C;
+    I inOff, outOff, unused, idxOff;
+    a.oa.offsets(outer, inOff, outOff);
+    oaIdx.offsets(outer, unused, idxOff);
+    outV[outOff + col * a.outInner] = Cvt<T>::down(bv);
+    outI[idxOff + col * idxInner] = (long)bi + 1;
+  }
+}
+
+// --------------------------------------------------------------- generic --
+template <typename TIn, typename TOut, typename F, typename I>
+__global__ __launch_bounds__(kBlock) void reduce_generic_kernel(const TIn* __restrict__ in,
+                                                                TOut* __restrict__ out,
+                                                                OuterArgs<I> oa, I outElems, I R,
+                                                                I sR, Epi epi, F f) {
+  const I step = (I)gridDim.x * kBlock;
+  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < outElems; o += step) {
+    I inOff, outOff;
+    oa.offsets(o, inOff, outOff);
+    float r = f.init();
+    for (I i = 0; i < R; ++i) r = f.combine(r, f.modify(Cvt<TIn>::up(in[inOff + i * sR])));
+    out[outOff] = epi.template finish<TOut>(r);
+  }
+}
+
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_generic_index_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI, OuterArgs<I> oa,
+    OuterArgs<I> oaIdx, I outElems, I R, I sR) {
+  using O = PairOrder<IS_MAX>;
+  const I step = (I)gridDim.x * kBlock;
+  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < outElems; o += step) {
+    I inOff, outOff, unused, idxOff;
+    oa.offsets(o, inOff, outOff);
+    oaIdx.offsets(o, unused, idxOff);
+    float bv = O::worst();
+    I bi = ~(I)0;
+    for (I i = 0; i < R; ++i) {
+      const float x = Cvt<T>::up(in[inOff + i * sR]);
+      if (O::better(x, i, bv, bi)) {
+        bv = x;
+        bi = i;
+      }
+    }
+    outV[outOff] = Cvt<T>::down(bv);
+    outI[idxOff] = (long)bi + 1;
+  }
+}
+
+// ------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+uint32_t pow2_ceil(uint64_t x) {
+  uint32_t p = 1;
+  while (p < x && p < (1u << 30)) p <<= 1;
+  return p;
+}
+
+// What a reduction looks like after the non-reduced dims of input and output
+// were brought into one joint space (input = operand 0 decides the order).
+struct ReduceGeom {
+  Layout in, out;     // non-reduced dims, jointly collapsed (same sizes)
+  Layout idx;         // optional second output with the same joint sizes
+  int64_t R, sR;      // reduced dim
+  int64_t outElems;
+  bool wide;
+};
+
+template <typename I>
+OuterArgs<I> make_outer(const Layout& in, const Layout& out, int dims) {
+  OuterArgs<I> oa{};
+  oa.dims = dims < 1 ? 1 : dims;
+  if (dims < 1) {
+    oa.size[0].set(1);
+    oa.inStride[0] = 0;
+    oa.outStride[0] = 0;
+    return oa;
+  }
+  for (int d = 0; d < dims; ++d) {
+    oa.size[d].set((uint64_t)in.size[d]);
+    oa.inStride[d] = (I)in.stride[d];
+    oa.outStride[d] = (I)out.stride[d];
+  }
+  return oa;
+}
+
+int capped_grid(THCState* s, int64_t blocks, const char* key, int defaultPerCu) {
+  const int64_t cap = (int64_t)num_compute_units(s) * tuning(key, defaultPerCu);
+  return (int)std::max<int64_t>(1, std::min(blocks, cap));
+}
+
+// Build the joint geometry. `idxT` may be null.
+ReduceGeom make_geom(AnyTensor* in, AnyTensor* out, AnyTensor* idxT, int dim) {
+  ReduceGeom g{};
+  Layout li = tensor_layout(in), lo = tensor_layout(out), lx = idxT ? tensor_layout(idxT) : lo;
+  g.R = li.size[dim];
+  g.sR = li.stride[dim];
+  g.wide = force_64bit_index() || !fits_32bit(li) || !fits_32bit(lo) || !fits_32bit(lx);
+  for (int d = 0; d < li.dims; ++d) g.wide = g.wide || li.stride[d] < 0;
+  for (int d = 0; d < lo.dims; ++d) g.wide = g.wide || lo.stride[d] < 0 || lx.stride[d] < 0;
+  li.size[dim] = 1;  // the reduced dim drops out of the joint space
+  Layout ops[3] = {li, lo, lx};
+  // out (and idx) have size 1 at `dim` already
+  if (!joint_collapse(3, ops, /*reorder=*/true)) raise_error("reduce: output shape mismatch");
+  g.in = ops[0];
+  g.out = ops[1];
+  g.idx = ops[2];
+  g.outElems = g.in.numel();
+  if (g.R == 1) g.sR = 1;
+  return g;
+}
+
+template <typename TIn, typename TOut, typename F, typename I, bool FIRST>
+void launch_rows_pass(THCState* s, const TIn* in, TOut* out, float* partial, const OuterArgs<I>& oa,
+                      int64_t numRows, int64_t R, int64_t S, int64_t chunk, bool vec, Epi epi,
+                      F f) {
+  constexpr int VEC = 16 / sizeof(TIn);
+  const int pack = vec ? VEC : 1;
+  const int64_t span = std::min(R, chunk);
+  const int64_t perLane = tuning("reduce.rows.packs_per_lane", 4);
+  uint32_t G = pow2_ceil((uint64_t)((span + pack * perLane - 1) / (pack * perLane)));
+  G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+  const int64_t groups = kBlock / G;
+  const int64_t blocks = (numRows * S + groups - 1) / groups;
+  const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+  Divisor<I> Sd;
+  Sd.set((uint64_t)S);
+  hipStream_t st = current_stream(s);
+  if (vec)
+    hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, VEC, FIRST>), dim3(grid), dim3(kBlock),
+                       0, st, in, out, partial, oa, (I)numRows, (I)R, Sd, (I)chunk, G, epi, f);
+  else
+    hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, 1, FIRST>), dim3(grid), dim3(kBlock), 0,
+                       st, in, out, partial, oa, (I)numRows, (I)R, Sd, (I)chunk, G, epi, f);
+}
+
+// rows: reduced dim has unit stride.
+template <typename T, typename F, typename I>
+void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
+  constexpr int VEC = 16 / sizeof(T);
+  const int64_t rows = g.outElems;
+  bool vec = aligned16(in) && g.R % VEC == 0;
+  for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+  OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
+
+  // Few long rows: cut them so that about `target` waves have work.
+  const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+  const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
+  size_t scratchBytes = 0;
+  int64_t S = 1, chunk = g.R;
+  if (rows < target && g.R >= 2 * minChunk) {
+    S = std::min<int64_t>((target + rows - 1) / rows, g.R / minChunk);
+    float* scratch = (float*)scratch_space(s, &scratchBytes);
+    (void)scratch;
+    S = std::min<int64_t>(S, (int64_t)(scratchBytes / sizeof(float)) / std::max<int64_t>(rows, 1));
+    if (S < 2) S = 1;
+    chunk = (g.R + S - 1) / S;
+    chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
+    S = (g.R + chunk - 1) / chunk;
+  }
+  if (S == 1) {
+    launch_rows_pass<T, T, F, I, true>(s, in, out, nullptr, oa, rows, g.R, 1, g.R, vec, epi, f);
+    note_kernel(vec ? "rows" : "rows-scalar");
+    return;
+  }
+  float* scratch = (float*)scratch_space(s, &scratchBytes);
+  launch_rows_pass<T, T, F, I, true>(s, in, (T*)nullptr, scratch, oa, rows, g.R, S, chunk, vec,
+                                     Epi{(int)Epilogue::None, 0.f}, f);
+  // pass 2: partial[row*S + s] is a dense rows x S matrix
+  Layout pin = g.in;
+  int64_t run = S;
+  for (int d = pin.dims - 1; d >= 0; --d) {
+    pin.stride[d] = run;
+    run *= pin.size[d];
+  }
+  OuterArgs<I> oa2 = make_outer<I>(pin, g.out, pin.dims);
+  launch_rows_pass<float, T, F, I, false>(s, scratch, out, nullptr, oa2, rows, S, 1, S,
+                                          S % 4 == 0, epi, f);
+  note_kernel(vec ? "rows-split" : "rows-split-scalar");
+}
+
+template <typename I>
+struct ColsPlan {
+  ColsArgs<I> a;
+  int64_t totalBlocks;
+  bool vec;
+};
+
+// cols: reduced dim strided, innermost joint dim has unit input stride.
+template <typename T, typename I>
+ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t partialElemBytes) {
+  constexpr int VEC = 16 / sizeof(T);
+  ColsPlan<I> p{};
+  const int nd = g.in.dims;
+  const int64_t C = g.in.size[nd - 1];
+  bool vec = aligned16(in) && C % VEC == 0 && g.sR % VEC == 0;
+  for (int d = 0; d < nd - 1 && vec; ++d) vec = g.in.stride[d] % VEC == 0;
+  const int pack = vec ? VEC : 1;
+  const uint32_t TX = std::min<uint32_t>(64, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
+  const uint32_t TY = kBlock / TX;
+  const int64_t colTiles = (C + (int64_t)TX * pack - 1) / ((int64_t)TX * pack);
+  const int64_t outer = g.outElems / C;
+  const int64_t base = outer * colTiles;
+  const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 8);
+  const int64_t minRows = (int64_t)TY * tuning("reduce.cols.min_rows_per_thread", 8);
+  int64_t S = 1;
+  if (base < target && g.R >= 2 * minRows) {
+    S = std::min<int64_t>((target + base - 1) / base, g.R / minRows);
+    size_t scratchBytes = 0;
+    scratch_space(s, &scratchBytes);
+    S = std::min<int64_t>(S, (int64_t)(scratchBytes / partialElemBytes) / std::max<int64_t>(g.outElems, 1));
+    if (S < 2) S = 1;
+  }
+  const int64_t forced = tuning("reduce.cols.force_split", 0);
+  if (forced > 0) S = std::min<int64_t>(forced, g.R);
+  int64_t chunk = (g.R + S - 1) / S;
+  S = (g.R + chunk - 1) / chunk;
+  p.vec = vec;
+  p.a.oa = make_outer<I>(g.in, g.out, nd - 1);
+  p.a.C = (I)C;
+  p.a.R = (I)g.R;
+  p.a.sR = (I)g.sR;
+  p.a.outInner = (I)g.out.stride[nd - 1];
+  p.a.chunkR = (I)chunk;
+  p.a.S.set((uint64_t)S);
+  p.a.colTiles.set((uint64_t)colTiles);
+  p.a.outElems = (I)g.outElems;
+  p.a.TX = TX;
+  p.totalBlocks = base * S;
+  return p;
+}
+
+template <typename T, typename F, typename I>
+void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
+  constexpr int VEC = 16 / sizeof(T);
+  ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(float));
+  const bool split = p.a.S.d > 1;
+  float* scratch = split ? (float*)scratch_space(s, nullptr) : nullptr;
+  const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+  hipStream_t st = current_stream(s);
+  if (p.vec)
+    hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, VEC>), dim3(grid), dim3(kBlock), 0, st, in,
+                       out, scratch, p.a, (I)p.totalBlocks, epi, f);
+  else
+    hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, 1>), dim3(grid), dim3(kBlock), 0, st, in, out,
+                       scratch, p.a, (I)p.totalBlocks, epi, f);
+  if (split) {
+    const int g2 = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.partials.blocks_per_cu", 8);
+    hipLaunchKernelGGL((reduce_partials_kernel<T, F, I>), dim3(g2), dim3(kBlock), 0, st, scratch, out,
+                       p.a, epi, f);
+  }
+  note_kernel(split ? (p.vec ? "cols-split" : "cols-split-scalar") : (p.vec ? "cols" : "cols-scalar"));
+}
+
+template <typename T, typename F, typename I>
+void run_generic(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
+  OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
+  const int grid = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.generic.blocks_per_cu", 32);
+  hipLaunchKernelGGL((reduce_generic_kernel<T, T, F, I>), dim3(grid), dim3(kBlock), 0,
+                     current_stream(s), in, out, oa, (I)g.outElems, (I)g.R, (I)g.sR, epi, f);
+  note_kernel("reduce-generic");
+}
+
+template <typename T, typename F, typename I>
+void run_dim_typed(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
+  if (g.sR == 1)
+    run_rows<T, F, I>(s, g, in, out, epi, f);
+  else if (g.in.stride[g.in.dims - 1] == 1 && g.in.size[g.in.dims - 1] > 1)
+    run_cols<T, F, I>(s, g, in, out, epi, f);
+  else
+    run_generic<T, F, I>(s, g, in, out, epi, f);
+}
+
+template <typename T, typename F>
+void run_dim(THCState* s, const ReduceGeom& g, const void* in, void* out, Epi epi, F f) {
+  if (g.wide)
+    run_dim_typed<T, F, uint64_t>(s, g, (const T*)in, (T*)out, epi, f);
+  else
+    run_dim_typed<T, F, uint32_t>(s, g, (const T*)in, (T*)out, epi, f);
+}
+
+template <typename T>
+void dispatch_reduce(THCState* s, const ReduceGeom& g, const void* in, void* out, ReduceOp op,
+                     Epi epi, float p) {
+  switch (op) {
+    case ReduceOp::Sum: run_dim<T>(s, g, in, out, epi, FSum{p}); break;
+    case ReduceOp::Prod: run_dim<T>(s, g, in, out, epi, FProd{p}); break;
+    case ReduceOp::Min: run_dim<T>(s, g, in, out, epi, FMin{p}); break;
+    case ReduceOp::Max: run_dim<T>(s, g, in, out, epi, FMax{p}); break;
+    case ReduceOp::Norm0: run_dim<T>(s, g, in, out, epi, FNorm0{p}); break;
+    case ReduceOp::Norm1: run_dim<T>(s, g, in, out, epi, FNorm1{p}); break;
+    case ReduceOp::Norm2: run_dim<T>(s, g, in, out, epi, FNorm2{p}); break;
+    case ReduceOp::NormP: run_dim<T>(s, g, in, out, epi, FNormP{p}); break;
+  }
+}
+
+// ---------------------------------------------------------------- index --
+template <typename T, typename I, bool IS_MAX>
+void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, long* outI) {
+  constexpr int VEC = 16 / sizeof(T);
+  hipStream_t st = current_stream(s);
+  const int nd = g.in.dims;
+  if (g.sR == 1) {
+    bool vec = aligned16(in) && g.R % VEC == 0;
+    for (int d = 0; d < nd && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+    const int pack = vec ? VEC : 1;
+    OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
+    OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
+    const int64_t perLane = tuning("reduce.rows.packs_per_lane", 4);
+    uint32_t G = pow2_ceil((uint64_t)((g.R + pack * perLane - 1) / (pack * perLane)));
+    G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+    const int64_t groups = kBlock / G;
+    const int grid = capped_grid(s, (g.outElems + groups - 1) / groups, "reduce.rows.blocks_per_cu", 64);
+    if (vec)
+      hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, VEC, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, G);
+    else
+      hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, 1, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, G);
+    note_kernel(vec ? "rows-index" : "rows-index-scalar");
+    return;
+  }
+  if (g.in.stride[nd - 1] == 1 && g.in.size[nd - 1] > 1) {
+    ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(float) + sizeof(I));
+    OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
+    const I idxInner = (I)g.idx.stride[nd - 1];
+    const bool split = p.a.S.d > 1;
+    float* partV = nullptr;
+    I* partI = nullptr;
+    if (split) {
+      char* scratch = (char*)scratch_space(s, nullptr);
+      partI = (I*)scratch;  // 8-byte aligned part first
+      partV = (float*)(scratch + sizeof(I) * (size_t)p.a.S.d * (size_t)g.outElems);
+    }
+    const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+    if (p.vec)
+      hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, VEC, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, (I)p.totalBlocks);
+    else
+      hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, 1, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, (I)p.totalBlocks);
+    if (split) {
+      const int g2 = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.partials.blocks_per_cu", 8);
+      hipLaunchKernelGGL((reduce_partials_index_kernel<T, I, IS_MAX>), dim3(g2), dim3(kBlock), 0, st,
+                         partV, partI, outV, outI, p.a, oaIdx, idxInner);
+    }
+    note_kernel(split ? "cols-index-split" : "cols-index");
+    return;
+  }
+  OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
+  OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
+  const int grid = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.generic.blocks_per_cu", 32);
+  hipLaunchKernelGGL((reduce_generic_index_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock), 0, st, in,
+                     outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, (I)g.sR);
+  note_kernel("generic-index");
+}
+
+template <typename T>
+void run_index(THCState* s, const ReduceGeom& g, bool isMax, const void* in, void* outV,
+               long* outI) {
+  if (g.wide) {
+    if (isMax) run_index_typed<T, uint64_t, true>(s, g, (const T*)in, (T*)outV, outI);
+    else run_index_typed<T, uint64_t, false>(s, g, (const T*)in, (T*)outV, outI);
+  } else {
+    if (isMax) run_index_typed<T, uint32_t, true>(s, g, (const T*)in, (T*)outV, outI);
+    else run_index_typed<T, uint32_t, false>(s, g, (const T*)in, (T*)outV, outI);
+  }
+}
+
+void resize_reduced(THCState* s, AnyTensor* out, AnyTensor* in, int dim, DType dt) {
+  long sizes[kMaxDims];
+  for (int d = 0; d < in->nDimension; ++d) sizes[d] = in->size[d];
+  sizes[dim] = 1;
+  tensor_resize_nd(s, out, in->nDimension, sizes, nullptr, dt);  // THCReduce.cuh:328-332
+}
+
+}  // namespace
+
+bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* out,
+                AnyTensor* in, int dim, int keepdim) {
+  if (out->nDimension > kMaxDims || in->nDimension > kMaxDims) return false;  // THCReduce.cuh:278-281
+  if (in->nDimension == 0) return true;                                        // :283-286
+  THC_ARG_CHECK(dim >= 0 && dim < in->nDimension, 3, "dimension out of range");
+  TensorRef hold(s, nullptr);
+  if (out == in) {  // the output is resized before the input is read
+    hold.t = tensor_new_with_tensor(s, in, dt);
+    in = hold.t;
+  }
+  resize_reduced(s, out, in, dim, dt);
+  ReduceGeom g = make_geom(in, out, nullptr, dim);
+  Epi epi{(int)ep, 0.f};
+  if (ep == Epilogue::PowInv) epi.arg = 1.0f / p;
+  if (ep == Epilogue::DivN) epi.arg = (float)g.R;
+  const void* ip = tensor_data(in, dt);
+  void* opn = tensor_data(out, dt);
+  if (dt == DType::F32)
+    dispatch_reduce<float>(s, g, ip, opn, op, epi, p);
+  else if (dt == DType::F16)
+    dispatch_reduce<__half>(s, g, ip, opn, op, epi, p);
+  else
+    raise_error("reduction not available for this element type");
+  THC_CHECK(hipGetLastError());
+  if (!keepdim) tensor_squeeze1d(s, out, nullptr, dim, dt);  // :449-451
+  return true;
+}
+
+void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyTensor* indices,
+                      AnyTensor* in, int dim, int keepdim) {
+  THC_ARG_CHECK(dim >= 0 && dim < in->nDimension, 3, "dimension out of range");
+  if (in->nDimension > kMaxDims) raise_arg_error(2, "%s", kDimWarning);
+  TensorRef hold(s, nullptr);
+  if (values == in) {
+    hold.t = tensor_new_with_tensor(s, in, dt);
+    in = hold.t;
+  }
+  resize_reduced(s, values, in, dim, dt);
+  resize_reduced(s, indices, in, dim, DType::I64);
+  ReduceGeom g = make_geom(in, values, indices, dim);
+  const void* ip = tensor_data(in, dt);
+  void* vp = tensor_data(values, dt);
+  long* xp = (long*)tensor_data(indices, DType::I64);
+  if (dt == DType::F32)
+    run_index<float>(s, g, isMax, ip, vp, xp);
+  else if (dt == DType::F16)
+    run_index<__half>(s, g, isMax, ip, vp, xp);
+  else
+    raise_error("reduction not available for this element type");
+  THC_CHECK(hipGetLastError());
+  if (!keepdim) {
+    tensor_squeeze1d(s, values, nullptr, dim, dt);
+    tensor_squeeze1d(s, indices, nullptr, dim, DType::I64);
+  }
+}
+
+namespace {
+template <typename F>
+float identity_of(F f) { return f.init(); }
+}  // namespace
+
+bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result) {
+  if (in->nDimension > kMaxDims) return false;  // THCReduceAll.cuh:249-251
+  float init = 0.f;
+  switch (op) {
+    case ReduceOp::Prod: init = 1.f; break;
+    case ReduceOp::Min: init = std::numeric_limits<float>::infinity(); break;
+    case ReduceOp::Max: init = -std::numeric_limits<float>::infinity(); break;
+    default: break;
+  }
+  if (in->nDimension == 0) {  // :253-257
+    *result = init;
+    return true;
+  }
+  // View the tensor as rows of its innermost collapsed dim; a tensor whose
+  // innermost dim is strided is densified first.
+  Layout l = tensor_layout(in);
+  collapse(l);
+  TensorRef dense(s, nullptr);
+  if (l.stride[l.dims - 1] != 1) {
+    dense.t = tensor_new_clone(s, in, dt);
+    in = dense.t;
+    l = tensor_layout(in);
+    collapse(l);
+  }
+  ReduceGeom g{};
+  g.wide = force_64bit_index() || !fits_32bit(l);
+  for (int d = 0; d < l.dims; ++d) g.wide = g.wide || l.stride[d] < 0;
+  g.R = l.size[l.dims - 1];
+  g.sR = 1;
+  g.in.dims = l.dims - 1;
+  for (int d = 0; d < l.dims - 1; ++d) {
+    g.in.size[d] = l.size[d];
+    g.in.stride[d] = l.stride[d];
+  }
+  if (g.in.dims == 0) {
+    g.in.dims = 1;
+    g.in.size[0] = 1;
+    g.in.stride[0] = 0;
+  }
+  g.outElems = g.in.numel();
+  const int64_t rows = g.outElems;
+
+  // Stage 1 (only if there are several rows): one fp32 partial per row, held
+  // in a temporary; stage 2: fold the dense vector of partials (or the single
+  // row) to one value in scratch-backed two-pass form.
+  size_t scratchBytes = 0;
+  char* scratch = (char*)scratch_space(s, &scratchBytes);
+  float* devOut = (float*)(scratch + scratchBytes - 256);  // last 256 bytes hold the result
+  TensorRef rowPartials(s, nullptr);
+  const void* src = tensor_data(in, dt);
+  DType srcT = dt;
+  ReduceOp op2 = op;
+  if (rows > 1) {
+    long n1 = rows;
+    rowPartials.t = tensor_new_with_size(s, 1, &n1, DType::F32);
+    g.out = g.in;  // dense row-major output
+    int64_t run = 1;
+    for (int d = g.out.dims - 1; d >= 0; --d) {
+      g.out.stride[d] = run;
+      run *= g.out.size[d];
+    }
+    float* rp = (float*)tensor_data(rowPartials.t, DType::F32);
+    Epi none{(int)Epilogue::None, 0.f};
+    // partial results are fp32 whatever the input type: reduce into a float
+    // buffer through the TIn != TOut instantiation
+    auto stage1 = [&](auto f) {
+      using F = decltype(f);
+      auto go = [&](auto idxTag) {
+        using I = decltype(idxTag);
+        OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
+        if (dt == DType::F32) {
+          bool vec = aligned16(src) && g.R % 4 == 0;
+          for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % 4 == 0 || g.in.size[d] == 1;
+          launch_rows_pass<float, float, F, I, true>(s, (const float*)src, rp, nullptr, oa, rows, g.R,
+                                                     1, g.R, vec, none, f);
+        } else {
+          bool vec = aligned16(src) && g.R % 8 == 0;
+          for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % 8 == 0 || g.in.size[d] == 1;
+          launch_rows_pass<__half, float, F, I, true>(s, (const __half*)src, rp, nullptr, oa, rows,
+                                                      g.R, 1, g.R, vec, none, f);
+        }
+      };
+      if (g.wide) go(uint64_t{}); else go(uint32_t{});
+    };
+    switch (op) {
+      case ReduceOp::Sum: stage1(FSum{p}); break;
+      case ReduceOp::Prod: stage1(FProd{p}); break;
+      case ReduceOp::Min: stage1(FMin{p}); break;
+      case ReduceOp::Max: stage1(FMax{p}); break;
+      case ReduceOp::Norm0: stage1(FNorm0{p}); op2 = ReduceOp::Sum; break;
+      case ReduceOp::Norm1: stage1(FNorm1{p}); op2 = ReduceOp::Sum; break;
+      case ReduceOp::Norm2: stage1(FNorm2{p}); op2 = ReduceOp::Sum; break;
+      case ReduceOp::NormP: stage1(FNormP{p}); op2 = ReduceOp::Sum; break;
+    }
+    src = rp;
+    srcT = DType::F32;
+    g.R = rows;
+    g.in.dims = 1;
+    g.in.size[0] = 1;
+    g.in.stride[0] = 0;
+    g.outElems = 1;
+    g.wide = force_64bit_index() || rows >= kIndex32Limit;
+  }
+  g.out = g.in;
+  g.out.stride[0] = 0;
+
+  auto stage2 = [&](auto f) {
+    using F = decltype(f);
+    Epi none{(int)Epilogue::None, 0.f};
+    auto go = [&](auto idxTag) {
+      using I = decltype(idxTag);
+      // float output regardless of the input type
+      const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+      const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
+      int64_t S = 1, chunk = g.R;
+      if (g.R >= 2 * minChunk) {
+        S = std::min<int64_t>(target, g.R / minChunk);
+        S = std::min<int64_t>(S, (int64_t)((scratchBytes - 256) / sizeof(float)));
+        chunk = (g.R + S - 1) / S;
+        chunk = (chunk + 63) / 64 * 64;
+        S = (g.R + chunk - 1) / chunk;
+      }
+      OuterArgs<I> oa = make_outer<I>(g.in, g.out, 1);
+      float* part = (float*)scratch;
+      auto pass1 = [&](float* outp, float* partp, int64_t S_, int64_t chunk_) {
+        if (srcT == DType::F32) {
+          const bool vec = aligned16(src) && g.R % 4 == 0;
+          launch_rows_pass<float, float, F, I, true>(s, (const float*)src, outp, partp, oa, 1, g.R,
+                                                     S_, chunk_, vec, none, f);
+        } else {
+          const bool vec = aligned16(src) && g.R % 8 == 0;
+          launch_rows_pass<__half, float, F, I, true>(s, (const __half*)src, outp, partp, oa, 1, g.R,
+                                                      S_, chunk_, vec, none, f);
+        }
+      };
+      if (S <= 1) {
+        pass1(devOut, nullptr, 1, g.R);
+      } else {
+        pass1(nullptr, part, S, chunk);
+        launch_rows_pass<float, float, F, I, false>(s, part, devOut, nullptr, oa, 1, S, 1, S,
+                                                    S % 4 == 0, none, f);
+      }
+    };
+    if (g.wide) go(uint64_t{}); else go(uint32_t{});
+  };
+  switch (op2) {
+    case ReduceOp::Sum: stage2(FSum{p}); break;
+    case ReduceOp::Prod: stage2(FProd{p}); break;
+    case ReduceOp::Min: stage2(FMin{p}); break;
+    case ReduceOp::Max: stage2(FMax{p}); break;
+    case ReduceOp::Norm0: stage2(FNorm0{p}); break;
+    case ReduceOp::Norm1: stage2(FNorm1{p}); break;
+    case ReduceOp::Norm2: stage2(FNorm2{p}); break;
+    case ReduceOp::NormP: stage2(FNormP{p}); break;
+  }
+  note_kernel(rows > 1 ? "all-rows" : "all");
+  THC_CHECK(hipGetLastError());
+  // The one place the caller blocks on the device (THCReduceAll.cuh:333-335).
+  THC_CHECK(hipMemcpyAsync(result, devOut, sizeof(float), hipMemcpyDeviceToHost, current_stream(s)));
+  THC_CHECK(hipStreamSynchronize(current_stream(s)));
+  return true;
+}
+
+}  // namespace thc

@@ -1,0 +1,286 @@
+/*
+ * THC.h -- C ABI of the MI355X-native pointwise-apply / reduction engine.
+ *
+ * The entry points keep the names, argument order and argument meaning of the
+ * cutorch THC C API so that a binding written against lib/THC (the
+ * cwrap-generated TensorMath.c, TensorOperator.c, a LuaJIT FFI cdef) links
+ * against this library unchanged for the functions declared here.
+ * Each block cites the reference declaration it replaces (paths relative to
+ * the cutorch source tree).
+ *
+ * Conventions shared with the reference:
+ *   - `long` is 64 bit (LP64); sizes, strides and storage offsets count
+ *     elements, not bytes.
+ *   - `dim` arguments of the reductions are 0-based (the Lua binding converts).
+ *   - indices written by max/min are 1-based int64 (Lua convention).
+ *   - outputs may be resized in place; arguments are never consumed.
+ *   - errors are reported through the TH error handler (THSetErrorHandler /
+ *     THSetArgErrorHandler); the default handler prints and aborts.
+ */
+#ifndef THC_AMD_THC_H
+#define THC_AMD_THC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+#define THC_API extern "C" __attribute__((visibility("default")))
+#else
+#define THC_API extern
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* TH error hooks (replaces THGeneral.h of torch7's TH, which cutorch takes   */
+/* from outside its own tree: lib/THC/THCGeneral.h.in:4-5).                   */
+/* ------------------------------------------------------------------------ */
+typedef void (*THErrorHandlerFunction)(const char *msg, void *data);
+typedef void (*THArgErrorHandlerFunction)(int argNumber, const char *msg, void *data);
+
+/* Install a handler (NULL restores print-and-abort). A handler may longjmp
+ * (Lua) or return; when it returns, the failing entry point returns to its
+ * caller without having launched anything and THCAmd_lastError() holds the
+ * message until THCAmd_clearLastError(). */
+THC_API void THSetErrorHandler(THErrorHandlerFunction handler, void *data);
+THC_API void THSetArgErrorHandler(THArgErrorHandlerFunction handler, void *data);
+THC_API const char *THCAmd_lastError(void);
+THC_API void THCAmd_clearLastError(void);
+
+/* ------------------------------------------------------------------------ */
+/* State, stream, raw device memory. lib/THC/THCGeneral.h.in:76-214           */
+/* ------------------------------------------------------------------------ */
+typedef struct THCState THCState;
+typedef struct ihipStream_t *hipStream_t_;   /* same pointee as hipStream_t */
+
+THC_API THCState *THCState_alloc(void);                       /* THCGeneral.h.in:125 */
+THC_API void THCState_free(THCState *state);                  /* :126 */
+THC_API void THCudaInit(THCState *state);                     /* :128 */
+THC_API void THCudaShutdown(THCState *state);                 /* :129 */
+THC_API int THCState_getNumDevices(THCState *state);          /* :161 */
+THC_API hipStream_t_ THCState_getCurrentStream(THCState *state);       /* :167 */
+/* The engine launches on `stream` (NULL = the device's default stream).
+ * Replaces THCState_setStream (:169) for a caller that owns a HIP stream. */
+THC_API void THCState_setCurrentStream(THCState *state, hipStream_t_ stream);
+THC_API void *THCState_getCurrentDeviceScratchSpace(THCState *state);  /* :197 */
+THC_API size_t THCState_getCurrentDeviceScratchSpaceSize(THCState *state); /* :199 */
+THC_API int THCudaMalloc(THCState *state, void **ptr, size_t size);    /* :213 */
+THC_API int THCudaFree(THCState *state, void *ptr);                    /* :214 */
+THC_API void __THCudaCheck(int err, const char *file, const int line); /* :208 */
+
+/* Diagnostics with no counterpart in the reference. */
+THC_API int THCAmd_getNumComputeUnits(THCState *state);
+/* Force the 64-bit index kernels even when 32 bits would do (tests). */
+THC_API void THCAmd_setForce64BitIndex(int enable);
+/* Kernel family chosen by the last apply / reduce call on this thread
+ * ("contig", "strided", "tiled", "generic", "rows", "cols", ...). */
+THC_API const char *THCAmd_lastKernel(void);
+/* Launch-shape tuning knobs, by name; returns 0 if the key is unknown. */
+THC_API int THCAmd_setTuning(const char *key, long value);
+THC_API long THCAmd_getTuning(const char *key);
+
+/* Layout core exposed for host-side tests (no GPU needed).
+ * collapse: lib/THC/THCTensorInfo.cuh:76-224; overlap and 32-bit rule:
+ * lib/THC/THCTensorTypeUtils.cu:164-245; offset: THCTensorInfo.cuh:229-278. */
+THC_API int THCAmd_collapseDims(int nDim, const long *size, const long *stride,
+                                int excludeDim, long *outSize, long *outStride,
+                                int *outDims);
+THC_API int THCAmd_overlappingIndices(int nDim, const long *size, const long *stride);
+THC_API int THCAmd_canUse32BitIndexMath(int nDim, const long *size, const long *stride);
+THC_API long THCAmd_indexToOffset(int nDim, const long *size, const long *stride, long linearId);
+/* Joint collapse of n same-shaped operands (strides laid out operand-major,
+ * n*nDim entries). Returns the collapsed rank, or -1 if the shapes cannot be
+ * walked jointly. */
+THC_API int THCAmd_jointCollapse(int nOperands, int nDim, const long *size,
+                                 const long *strides, long *outSize, long *outStrides);
+/* fp16 <-> fp32 conversion used for host staging (round-to-nearest-even);
+ * THC_float2half / THC_half2float, lib/THC/THCHalf.h and THCGeneral.c:960-972 */
+typedef struct { unsigned short x; } THHalf;
+THC_API THHalf THC_float2half(float a);
+THC_API float THC_half2float(THHalf a);
+
+/* ------------------------------------------------------------------------ */
+/* Storage / tensor structs. Field order and types follow                     */
+/* lib/THC/generic/THCStorage.h:9-19 and lib/THC/generic/THCTensor.h:7-19     */
+/* (mirrored a second time in FFI.lua:57-81).                                 */
+/* ------------------------------------------------------------------------ */
+#define TH_STORAGE_REFCOUNTED 1
+#define TH_STORAGE_RESIZABLE  2
+#define TH_STORAGE_FREEMEM    4
+#define TH_TENSOR_REFCOUNTED  1
+
+typedef struct _THCDeviceAllocator {          /* THCGeneral.h.in:48-55 */
+  int (*malloc)(void *, void **, size_t, hipStream_t_);
+  int (*realloc)(void *, void **, size_t, size_t, hipStream_t_);
+  int (*free)(void *, void *);
+  int (*emptyCache)(void *);
+  int (*cacheInfo)(void *, int, size_t *, size_t *);
+  void *state;
+} THCDeviceAllocator;
+
+#define THC_AMD_DECLARE_STRUCTS(Storage, Tensor, real)                        \
+  typedef struct Storage {                                                    \
+    real *data;                                                               \
+    ptrdiff_t size;                                                           \
+    int refcount;                                                             \
+    char flag;                                                                \
+    THCDeviceAllocator *allocator;                                            \
+    void *allocatorContext;                                                   \
+    struct Storage *view;                                                     \
+    int device;                                                               \
+  } Storage;                                                                  \
+  typedef struct Tensor {                                                     \
+    long *size;                                                               \
+    long *stride;                                                             \
+    int nDimension;                                                           \
+    Storage *storage;                                                         \
+    ptrdiff_t storageOffset;                                                  \
+    int refcount;                                                             \
+    char flag;                                                                \
+  } Tensor;
+
+THC_AMD_DECLARE_STRUCTS(THCudaStorage, THCudaTensor, float)
+THC_AMD_DECLARE_STRUCTS(THCudaHalfStorage, THCudaHalfTensor, THHalf)
+THC_AMD_DECLARE_STRUCTS(THCudaLongStorage, THCudaLongTensor, long)
+
+/* ------------------------------------------------------------------------ */
+/* Storage and tensor management. generic/THCStorage.h:22-61,                 */
+/* generic/THCTensor.h:22-139, generic/THCTensorCopy.h:5-6.                   */
+/* The *FromHost / *ToHost calls take raw host pointers and stand in for      */
+/* copyFloat / THFloatTensor_copyCuda (generic/THCTensorCopy.c:7-164), whose  */
+/* THFloatTensor argument type lives in torch7's TH.                          */
+/* ------------------------------------------------------------------------ */
+#define THC_AMD_DECLARE_TENSOR_API(Storage, Tensor, real)                      \
+  THC_API real *Storage##_data(THCState *, const Storage *);                   \
+  THC_API ptrdiff_t Storage##_size(THCState *, const Storage *);               \
+  THC_API int Storage##_elementSize(THCState *);                               \
+  THC_API void Storage##_set(THCState *, Storage *, ptrdiff_t, real);          \
+  THC_API real Storage##_get(THCState *, const Storage *, ptrdiff_t);          \
+  THC_API Storage *Storage##_new(THCState *);                                  \
+  THC_API Storage *Storage##_newWithSize(THCState *, ptrdiff_t size);          \
+  THC_API void Storage##_retain(THCState *, Storage *);                        \
+  THC_API void Storage##_free(THCState *, Storage *);                          \
+  THC_API void Storage##_resize(THCState *, Storage *, ptrdiff_t size);        \
+  THC_API int Storage##_getDevice(THCState *, const Storage *);                \
+  THC_API void Storage##_copyFromHost(THCState *, Storage *, const real *src,  \
+                                      ptrdiff_t n);                            \
+  THC_API void Storage##_copyToHost(THCState *, real *dst, const Storage *,    \
+                                    ptrdiff_t n);                              \
+  THC_API Storage *Tensor##_storage(THCState *, const Tensor *);               \
+  THC_API ptrdiff_t Tensor##_storageOffset(THCState *, const Tensor *);        \
+  THC_API int Tensor##_nDimension(THCState *, const Tensor *);                 \
+  THC_API long Tensor##_size(THCState *, const Tensor *, int dim);             \
+  THC_API long Tensor##_stride(THCState *, const Tensor *, int dim);           \
+  THC_API real *Tensor##_data(THCState *, const Tensor *);                     \
+  THC_API Tensor *Tensor##_new(THCState *);                                    \
+  THC_API Tensor *Tensor##_newWithTensor(THCState *, Tensor *);                \
+  THC_API Tensor *Tensor##_newWithStorage1d(THCState *, Storage *, ptrdiff_t,  \
+                                            long, long);                       \
+  THC_API Tensor *Tensor##_newWithStorage2d(THCState *, Storage *, ptrdiff_t,  \
+                                            long, long, long, long);           \
+  THC_API Tensor *Tensor##_newWithStorage3d(THCState *, Storage *, ptrdiff_t,  \
+                                            long, long, long, long, long,      \
+                                            long);                             \
+  THC_API Tensor *Tensor##_newWithStorage4d(THCState *, Storage *, ptrdiff_t,  \
+                                            long, long, long, long, long,      \
+                                            long, long, long);                 \
+  THC_API Tensor *Tensor##_newWithSize1d(THCState *, long);                    \
+  THC_API Tensor *Tensor##_newWithSize2d(THCState *, long, long);              \
+  THC_API Tensor *Tensor##_newWithSize3d(THCState *, long, long, long);        \
+  THC_API Tensor *Tensor##_newWithSize4d(THCState *, long, long, long, long);  \
+  THC_API Tensor *Tensor##_newClone(THCState *, Tensor *);                     \
+  THC_API Tensor *Tensor##_newContiguous(THCState *, Tensor *);                \
+  THC_API Tensor *Tensor##_newSelect(THCState *, Tensor *, int, long);         \
+  THC_API Tensor *Tensor##_newNarrow(THCState *, Tensor *, int, long, long);   \
+  THC_API Tensor *Tensor##_newTranspose(THCState *, Tensor *, int, int);       \
+  THC_API void Tensor##_resizeAs(THCState *, Tensor *, Tensor *src);           \
+  THC_API void Tensor##_resize1d(THCState *, Tensor *, long);                  \
+  THC_API void Tensor##_resize2d(THCState *, Tensor *, long, long);            \
+  THC_API void Tensor##_resize3d(THCState *, Tensor *, long, long, long);      \
+  THC_API void Tensor##_resize4d(THCState *, Tensor *, long, long, long,       \
+                                 long);                                        \
+  THC_API void Tensor##_resizeNd(THCState *, Tensor *, int nDimension,         \
+                                 long *size, long *stride);                    \
+  THC_API void Tensor##_set(THCState *, Tensor *, Tensor *src);                \
+  THC_API void Tensor##_setStorageNd(THCState *, Tensor *, Storage *,          \
+                                     ptrdiff_t, int, long *, long *);          \
+  THC_API void Tensor##_narrow(THCState *, Tensor *, Tensor *src, int, long,   \
+                               long);                                          \
+  THC_API void Tensor##_select(THCState *, Tensor *, Tensor *src, int, long);  \
+  THC_API void Tensor##_transpose(THCState *, Tensor *, Tensor *src, int,      \
+                                  int);                                        \
+  THC_API void Tensor##_squeeze(THCState *, Tensor *, Tensor *src);            \
+  THC_API void Tensor##_squeeze1d(THCState *, Tensor *, Tensor *src, int);     \
+  THC_API void Tensor##_unsqueeze1d(THCState *, Tensor *, Tensor *src, int);   \
+  THC_API int Tensor##_isContiguous(THCState *, const Tensor *);               \
+  THC_API int Tensor##_isSameSizeAs(THCState *, const Tensor *,                \
+                                    const Tensor *);                           \
+  THC_API int Tensor##_isSetTo(THCState *, const Tensor *, const Tensor *);    \
+  THC_API ptrdiff_t Tensor##_nElement(THCState *, const Tensor *);             \
+  THC_API void Tensor##_retain(THCState *, Tensor *);                          \
+  THC_API void Tensor##_free(THCState *, Tensor *);                            \
+  THC_API void Tensor##_freeCopyTo(THCState *, Tensor *, Tensor *dst);         \
+  THC_API int Tensor##_getDevice(THCState *, const Tensor *);                  \
+  THC_API void Tensor##_copy(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_copyIgnoringOverlaps(THCState *, Tensor *self,         \
+                                             Tensor *src);                     \
+  THC_API void Tensor##_copyFromHost(THCState *, Tensor *self,                 \
+                                     const real *src);                         \
+  THC_API void Tensor##_copyToHost(THCState *, real *dst, Tensor *src);
+
+THC_AMD_DECLARE_TENSOR_API(THCudaStorage, THCudaTensor, float)
+THC_AMD_DECLARE_TENSOR_API(THCudaHalfStorage, THCudaHalfTensor, THHalf)
+THC_AMD_DECLARE_TENSOR_API(THCudaLongStorage, THCudaLongTensor, long)
+
+/* Type-converting device copies. generic/THCTensorCopy.h:14-24 */
+THC_API void THCudaTensor_copyCudaHalf(THCState *, THCudaTensor *self, THCudaHalfTensor *src);
+THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCudaTensor *src);
+
+/* ------------------------------------------------------------------------ */
+/* Pointwise math on the apply engine.                                        */
+/*   tensor (op) scalar : generic/THCTensorMathPairwise.h:5-8                 */
+/*   tensor (op) tensor : generic/THCTensorMathPointwise.h:49-53,66-67        */
+/* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
+/* ------------------------------------------------------------------------ */
+#define THC_AMD_DECLARE_MATH_API(Tensor, real, accreal)                        \
+  THC_API void Tensor##_add(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_sub(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_mul(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_div(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_cadd(THCState *, Tensor *self, Tensor *src1, real v,   \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_csub(THCState *, Tensor *self, Tensor *src1, real v,   \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cmul(THCState *, Tensor *self, Tensor *src1,           \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cdiv(THCState *, Tensor *self, Tensor *src1,           \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_addcmul(THCState *, Tensor *self, Tensor *t, real v,   \
+                                Tensor *src1, Tensor *src2);                   \
+  THC_API void Tensor##_addcdiv(THCState *, Tensor *self, Tensor *t, real v,   \
+                                Tensor *src1, Tensor *src2);                   \
+  THC_API void Tensor##_fill(THCState *, Tensor *self, real v);                \
+  THC_API void Tensor##_zero(THCState *, Tensor *self);                        \
+  THC_API void Tensor##_sum(THCState *, Tensor *self, Tensor *src, long dim,   \
+                            int keepdim);                                      \
+  THC_API void Tensor##_prod(THCState *, Tensor *self, Tensor *src, long dim,  \
+                             int keepdim);                                     \
+  THC_API void Tensor##_mean(THCState *, Tensor *self, Tensor *src, long dim,  \
+                             int keepdim);                                     \
+  THC_API void Tensor##_norm(THCState *, Tensor *self, Tensor *src, real p,    \
+                             long dim, int keepdim);                           \
+  THC_API void Tensor##_max(THCState *, Tensor *values,                        \
+                            THCudaLongTensor *indices, Tensor *src, long dim,  \
+                            int keepdim);                                      \
+  THC_API void Tensor##_min(THCState *, Tensor *values,                        \
+                            THCudaLongTensor *indices, Tensor *src, long dim,  \
+                            int keepdim);                                      \
+  THC_API accreal Tensor##_sumall(THCState *, Tensor *self);                   \
+  THC_API accreal Tensor##_prodall(THCState *, Tensor *self);                  \
+  THC_API accreal Tensor##_meanall(THCState *, Tensor *self);                  \
+  THC_API accreal Tensor##_normall(THCState *, Tensor *self, real p);          \
+  THC_API real Tensor##_minall(THCState *, Tensor *self);                      \
+  THC_API real Tensor##_maxall(THCState *, Tensor *self);
+
+THC_AMD_DECLARE_MATH_API(THCudaTensor, float, float)
+THC_AMD_DECLARE_MATH_API(THCudaHalfTensor, THHalf, float)
+
+#endif /* THC_AMD_THC_H */

@@ -1,0 +1,155 @@
+"""ctypes loader for the CPU oracle (oracle/libth_oracle.so).
+
+TEST INFRASTRUCTURE: only tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py may import this module. Build the library with
+`make -C oracle`.
+
+A tensor is described the way a TH view is: a host storage array, a storage
+offset, sizes and strides in elements. `View` keeps that description; results
+are written into the storage array in place, so holes can be checked too.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libth_oracle.so")
+
+OPS = {"copy": 0, "addc": 1, "subc": 2, "mulc": 3, "divc": 4, "add": 5, "sub": 6, "mul": 7,
+       "div": 8, "cadd": 9, "addcmul": 10, "addcdiv": 11, "fill": 12, "pow": 13}
+KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "norm": 4, "mean": 5}
+
+
+class _CView(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("nd", C.c_int), ("size", C.POINTER(C.c_long)),
+                ("stride", C.POINTER(C.c_long))]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("%s is missing: run `make -C oracle`" % LIB_PATH)
+        l = C.CDLL(LIB_PATH)
+        VP = C.POINTER(_CView)
+        for suffix in ("float", "half"):
+            f = getattr(l, "th_pointwise_" + suffix)
+            f.argtypes = [C.c_int, C.c_float, VP, VP, VP, VP]
+            f.restype = C.c_int
+            f = getattr(l, "th_reduce_dim_" + suffix)
+            f.argtypes = [C.c_int, C.c_double, VP, VP, C.c_int]
+            f.restype = C.c_int
+            for mm in ("max", "min"):
+                f = getattr(l, "th_%s_dim_%s" % (mm, suffix))
+                f.argtypes = [VP, VP, VP, C.c_int]
+                f.restype = C.c_int
+            f = getattr(l, "th_reduce_all_" + suffix)
+            f.argtypes = [C.c_int, C.c_double, VP]
+            f.restype = C.c_double
+        l.th_half2float.argtypes = [C.c_uint16]
+        l.th_half2float.restype = C.c_float
+        l.th_float2half.argtypes = [C.c_float]
+        l.th_float2half.restype = C.c_uint16
+        l.th_half2float_array.argtypes = [C.c_void_p, C.c_void_p, C.c_long]
+        l.th_float2half_array.argtypes = [C.c_void_p, C.c_void_p, C.c_long]
+        l.th_set_num_threads.argtypes = [C.c_int]
+        _lib = l
+    return _lib
+
+
+class View(object):
+    """A strided view on a host storage array (float32, float16 or int64)."""
+
+    def __init__(self, storage, offset=0, size=None, stride=None):
+        assert storage.flags["C_CONTIGUOUS"] and storage.ndim == 1
+        self.storage = storage
+        self.offset = int(offset)
+        if size is None:
+            size = (storage.size,) if storage.size else ()
+        self.size = tuple(int(s) for s in size)
+        if stride is None:
+            stride, run = [], 1
+            for s in reversed(self.size):
+                stride.append(run)
+                run *= s
+            stride = tuple(reversed(stride))
+        self.stride = tuple(int(s) for s in stride)
+        n = max(1, len(self.size))
+        self._size = (C.c_long * n)(*self.size)
+        self._stride = (C.c_long * n)(*self.stride)
+        self.c = _CView(storage.ctypes.data + self.offset * storage.itemsize, len(self.size),
+                        self._size, self._stride)
+
+    @classmethod
+    def of(cls, arr):
+        """Contiguous view holding a copy of `arr`."""
+        arr = np.ascontiguousarray(arr)
+        return cls(arr.reshape(-1).copy(), 0, arr.shape)
+
+    @classmethod
+    def empty(cls, shape, dtype=np.float32):
+        n = int(np.prod(shape)) if len(shape) else 0
+        return cls(np.zeros(n, dtype=dtype), 0, shape)
+
+    @property
+    def is_half(self):
+        return self.storage.dtype == np.float16
+
+    def numpy(self):
+        """Logical contents, gathered through numpy's own stride machinery."""
+        if not self.size:
+            return np.empty((0,), dtype=self.storage.dtype)
+        item = self.storage.itemsize
+        return np.lib.stride_tricks.as_strided(
+            self.storage[self.offset:], shape=self.size,
+            strides=tuple(s * item for s in self.stride)).copy()
+
+
+def _ptr(v):
+    return C.byref(v.c) if v is not None else None
+
+
+def pointwise(op, out, a=None, b=None, c=None, value=0.0):
+    f = lib().th_pointwise_half if out.is_half else lib().th_pointwise_float
+    rc = f(OPS[op], value, _ptr(out), _ptr(a), _ptr(b), _ptr(c))
+    if rc:
+        raise ValueError("sizes do not match")
+    return out
+
+
+def reduced_shape(shape, dim):
+    return tuple(1 if d == dim else s for d, s in enumerate(shape))
+
+
+def reduce_dim(kind, src, dim, p=0.0, out=None):
+    if out is None:
+        out = View.empty(reduced_shape(src.size, dim), src.storage.dtype)
+    f = lib().th_reduce_dim_half if src.is_half else lib().th_reduce_dim_float
+    if f(KINDS[kind], p, _ptr(out), _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return out
+
+
+def minmax_dim(which, src, dim, values=None, indices=None):
+    shape = reduced_shape(src.size, dim)
+    if values is None:
+        values = View.empty(shape, src.storage.dtype)
+    if indices is None:
+        indices = View.empty(shape, np.int64)
+    f = getattr(lib(), "th_%s_dim_%s" % (which, "half" if src.is_half else "float"))
+    if f(_ptr(values), _ptr(indices), _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return values, indices
+
+
+def reduce_all(kind, src, p=0.0):
+    f = lib().th_reduce_all_half if src.is_half else lib().th_reduce_all_float
+    return f(KINDS[kind], p, _ptr(src))
+
+
+def set_num_threads(n):
+    lib().th_set_num_threads(int(n))
