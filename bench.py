@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the apply / reduce hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|primary] [--no-cpu]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM. The headline line is quoted on the strided apply3
+configuration (out = a:t() * b + d on 8192 x 8192 fp32, a viewed transposed);
+the other benchmark configurations are measured in the same run and reported
+under "all_configs". Prints ONE JSON line.
+
+  value               algorithmic bytes * steps / wall time of the timed region
+  roofline.achieved   algorithmic bytes / mean kernel time, from HIP events
+                      recorded around every launch of the timed region on the
+                      stream the engine launches on
+  cpu_baseline        the CPU restatement (oracle/) timed on this box's host
+                      cores on the same workload, single thread; the all-core
+                      figure is reported beside it
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_GBPS = 8000.0
+METRIC = "achieved HBM GB/s (% of ~8 TB/s peak): pointwise apply + dim reduction, fp32"
+
+
+class Hip(object):
+    def __init__(self):
+        self.l = C.CDLL("libamdhip64.so")
+        self.l.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.l.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.l.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.l.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.l.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        self.l.hipDeviceSynchronize.argtypes = []
+
+    def check(self, err, what):
+        if err != 0:
+            raise RuntimeError("%s failed with hip error %d" % (what, err))
+
+    def event(self):
+        e = C.c_void_p()
+        self.check(self.l.hipEventCreate(C.byref(e)), "hipEventCreate")
+        return e
+
+    def record(self, e, stream):
+        self.check(self.l.hipEventRecord(e, stream), "hipEventRecord")
+
+    def elapsed_ms(self, a, b):
+        self.check(self.l.hipEventSynchronize(b), "hipEventSynchronize")
+        ms = C.c_float()
+        self.check(self.l.hipEventElapsedTime(C.byref(ms), a, b), "hipEventElapsedTime")
+        return ms.value
+
+    def sync(self):
+        self.check(self.l.hipDeviceSynchronize(), "hipDeviceSynchronize")
+
+    def d2d(self, dst, src, nbytes):
+        self.check(self.l.hipMemcpy(dst, src, nbytes, 3), "hipMemcpy d2d")
+
+
+def device_fill_from_block(hip, thc, shape, block):
+    """A device tensor of `shape` whose storage repeats `block` (host array):
+    lets the 8.7 GB operands of the 64-bit-index configuration be set up in
+    seconds; values stay normal(0,1)."""
+    t = thc.Tensor("float").resize(shape)
+    n = int(np.prod(shape))
+    blk = thc.Tensor.from_numpy(block)
+    base = t.data_ptr()
+    done = 0
+    while done < n:
+        m = min(block.size, n - done)
+        hip.d2d(base + 4 * done, blk.data_ptr(), 4 * m)
+        done += m
+    return t
+
+
+class Config(object):
+    """One benchmark configuration: `sets` rotating operand sets, a `run(i)`
+    that launches the op on set i, and its algorithmic byte count."""
+
+    def __init__(self, name, desc, nbytes, elements, sets, run, check=None, kernel=None):
+        self.name, self.desc, self.nbytes, self.elements = name, desc, nbytes, elements
+        self.sets, self.run, self.check, self.kernel = sets, run, check, kernel
+
+
+def build_configs(thc, hip, which):
+    rng = np.random.default_rng(0xC0FFEE)
+    cfgs = []
+    T = thc.Tensor
+
+    def c2():
+        n = 8192
+        a = rng.standard_normal((n, n), dtype=np.float32)
+        b = rng.standard_normal((n, n), dtype=np.float32)
+        d = rng.standard_normal((n, n), dtype=np.float32)
+        da, db, dd = T.from_numpy(a), T.from_numpy(b), T.from_numpy(d)
+        at = da.t()
+        out = T("float").resize((n, n))
+
+        def run(i):
+            out.addcmul(dd, 1.0, at, db)
+
+        def check():
+            got = out.numpy()
+            rows = np.array([0, 1, 63, 64, 4097, 8191])
+            want = (a.T[rows] * b[rows]).astype(np.float32) + d[rows]
+            return bool(np.array_equal(got[rows].view(np.uint32), want.view(np.uint32)))
+        host = (a, b, d)
+        return Config("C2", "out = a:t()*b + d, 8192x8192 fp32, a stride (1,8192) [addcmul]",
+                      16 * n * n, n * n, 1, run, check), host
+
+    primary, host_c2 = c2()
+    cfgs.append(primary)
+    if which == "primary":
+        return cfgs, host_c2
+
+    # C1: contiguous 2^24, three rotating buffer sets (working set < Infinity Cache)
+    n1 = 1 << 24
+    sets1 = []
+    for _ in range(3):
+        a = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
+        b = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
+        sets1.append((a, b, T("float").resize((n1,))))
+    cfgs.append(Config("C1-add", "c = a + b, 2^24 fp32 contiguous [cadd]", 12 * n1, n1, 3,
+                       lambda i: sets1[i % 3][2].cadd(sets1[i % 3][0], 1.0, sets1[i % 3][1])))
+    cfgs.append(Config("C1-mul", "c = a * b, 2^24 fp32 contiguous [cmul]", 12 * n1, n1, 3,
+                       lambda i: sets1[i % 3][2].cmul(sets1[i % 3][0], sets1[i % 3][1])))
+
+    # C3a/b: 65536 x 1024, last dim
+    r3, n3 = 65536, 1024
+    sets3 = []
+    for _ in range(3):
+        x = rng.standard_normal((r3, n3), dtype=np.float32)
+        dup = rng.integers(0, n3, (r3, 10))
+        x[np.arange(r3)[:, None], dup] = x[np.arange(r3)[:, None], dup[:, ::-1]]
+        sets3.append((T.from_numpy(x), T("float").resize((r3, 1)), T("long").resize((r3, 1))))
+    cfgs.append(Config("C3a-sum", "sum over last dim of 65536x1024 fp32", 4 * r3 * n3 + 4 * r3, r3 * n3,
+                       3, lambda i: sets3[i % 3][1].sum(sets3[i % 3][0], 1)))
+    cfgs.append(Config("C3b-max", "max+argmax over last dim of 65536x1024 fp32",
+                       4 * r3 * n3 + 12 * r3, r3 * n3, 3,
+                       lambda i: sets3[i % 3][1].max(sets3[i % 3][2], sets3[i % 3][0], 1)))
+
+    # C3c: reduceAll over 2^28
+    n3c = 1 << 28
+    xa = T.from_numpy(rng.random(n3c, dtype=np.float32))
+    cfgs.append(Config("C3c-sumall", "sumall over 2^28 fp32 (blocks on a 4-byte D2H copy)",
+                       4 * n3c + 4, n3c, 1, lambda i: xa.sumall()))
+
+    # C4: 64 x 4096 x 512, middle dim; fp32 and fp16
+    s4 = (64, 4096, 512)
+    x4 = rng.uniform(-2, 2, s4).astype(np.float32)
+    d4 = T.from_numpy(x4)
+    o4 = T("float").resize((64, 1, 512))
+    n4 = int(np.prod(s4))
+    cfgs.append(Config("C4-sum-f32", "sum over middle dim of 64x4096x512 fp32", 4 * n4 + 4 * 64 * 512,
+                       n4, 1, lambda i: o4.sum(d4, 1)))
+    cfgs.append(Config("C4-norm-f32", "L2 norm over middle dim of 64x4096x512 fp32",
+                       4 * n4 + 4 * 64 * 512, n4, 1, lambda i: o4.norm(d4, 2.0, 1)))
+    sets4h = []
+    for _ in range(3):
+        h = T.from_numpy((x4 * np.float32(rng.uniform(0.5, 1.0))).astype(np.float16))
+        sets4h.append((h, T("half").resize((64, 1, 512))))
+    cfgs.append(Config("C4-sum-f16", "sum over middle dim of 64x4096x512 fp16, fp32 accumulate",
+                       2 * n4 + 2 * 64 * 512, n4, 3, lambda i: sets4h[i % 3][1].sum(sets4h[i % 3][0], 1)))
+    cfgs.append(Config("C4-norm-f16", "L2 norm over middle dim of 64x4096x512 fp16, fp32 accumulate",
+                       2 * n4 + 2 * 64 * 512, n4, 3,
+                       lambda i: sets4h[i % 3][1].norm(sets4h[i % 3][0], 2.0, 1)))
+
+    # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path
+    block = rng.standard_normal(1 << 24, dtype=np.float32)
+    a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
+    b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), block[::-1].copy())
+    c5 = T("float").resize((2048, 2048, 520))
+    a5v = a5.view_as_strided(0, (2048, 2048, 520), (1, 2048, 2048 * 2048))
+    n5 = 2048 * 2048 * 520
+    cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
+                       12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5)))
+    return cfgs, host_c2
+
+
+def time_config(hip, thc, cfg, steps, warmup, stream):
+    for i in range(warmup):
+        cfg.run(i)
+    hip.sync()
+    cfg.kernel = thc.last_kernel()
+    evs = [(hip.event(), hip.event()) for _ in range(steps)]
+    hip.sync()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        hip.record(evs[i][0], stream)
+        cfg.run(warmup + i)
+        hip.record(evs[i][1], stream)
+    hip.sync()
+    wall = time.perf_counter() - t0
+    ms = np.array([hip.elapsed_ms(a, b) for a, b in evs])
+    return wall, ms
+
+
+def cpu_baseline(host, nbytes, budget_s=12.0):
+    """Times the CPU restatement of out = a:t()*b + d on the full 8192x8192
+    operands: single thread (the reported baseline) and all cores."""
+    from oracle import th_oracle as oracle
+    a, b, d = host
+    n = a.shape[0]
+    va = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
+    vb, vd = oracle.View(b.reshape(-1)), oracle.View(d.reshape(-1))
+    vb = oracle.View(vb.storage, 0, (n, n))
+    vd = oracle.View(vd.storage, 0, (n, n))
+    out = oracle.View.empty((n, n))
+    res = {}
+    cores = len(os.sched_getaffinity(0))
+    for label, threads in (("single", 1), ("all", cores)):
+        oracle.set_num_threads(threads)
+        times = []
+        t_start = time.perf_counter()
+        while len(times) < 6 and (time.perf_counter() - t_start) < budget_s / 2:
+            t0 = time.perf_counter()
+            oracle.pointwise("addcmul", out, vd, va, vb, value=1.0)
+            times.append(time.perf_counter() - t0)
+        best = times[1:] if len(times) > 1 else times
+        res[label] = (nbytes / float(np.median(best)) / 1e9, threads, len(times))
+    oracle.set_num_threads(1)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--configs", default="all", choices=["all", "primary"])
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)")
+
+    import cutorch_amd as thc
+    thc.state()                      # raises if libTHC.so is missing or no GPU is visible
+    hip = Hip()
+    stream = thc.lib().THCState_getCurrentStream(thc.state())
+    cfgs, host_c2 = build_configs(thc, hip, args.configs)
+    results = []
+    for cfg in cfgs:
+        steps = args.steps if cfg.name != "C5" else max(3, args.steps // 5)
+        wall, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
+        ok = cfg.check() if cfg.check else None
+        mean_ms = float(ms.mean())
+        results.append({
+            "name": cfg.name, "desc": cfg.desc, "kernel": cfg.kernel, "steps": steps,
+            "algorithmic_bytes": cfg.nbytes,
+            "ms_mean": round(mean_ms, 5), "ms_min": round(float(ms.min()), 5),
+            "ms_median": round(float(np.median(ms)), 5),
+            "gbps_mean": round(cfg.nbytes / mean_ms / 1e6, 1),
+            "gbps_best": round(cfg.nbytes / float(ms.min()) / 1e6, 1),
+            "frac_of_peak": round(cfg.nbytes / mean_ms / 1e6 / PEAK_GBPS, 4),
+            "gelem_per_s": round(cfg.elements / mean_ms / 1e6, 2),
+            "wall_gbps": round(cfg.nbytes * steps / wall / 1e9, 1),
+            "rotating_sets": cfg.sets, "parity_sample_ok": ok,
+        })
+    p = results[0]
+    line = {
+        "metric": METRIC, "value": p["wall_gbps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": p["steps"], "warmup": args.warmup,
+        "ms_per_step": round(1e3 * p["algorithmic_bytes"] / (p["wall_gbps"] * 1e9), 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (fixed-seed host generator, copied to HBM before timing)",
+        "config": {"workload": p["desc"], "elements": cfgs[0].elements, "kernel": p["kernel"],
+                   "parity_sample_ok": p["parity_sample_ok"]},
+        "roofline": {"bound": "hbm", "achieved": p["gbps_mean"], "peak": PEAK_GBPS, "unit": "GB/s",
+                     "frac": p["frac_of_peak"], "traffic": None},
+        "all_configs": results,
+    }
+    if not args.no_cpu:
+        cb = cpu_baseline(host_c2, cfgs[0].nbytes)
+        line["cpu_baseline"] = {
+            "value": round(cb["single"][0], 2), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "full workload (8192x8192 addcmul with transposed operand), median of %d runs"
+                      % max(1, cb["single"][2] - 1)}
+        line["cpu_baseline_all_cores"] = {"value": round(cb["all"][0], 2), "unit": "GB/s",
+                                          "cores": cb["all"][1], "kind": "port"}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

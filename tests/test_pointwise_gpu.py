@@ -1,0 +1,260 @@
+"""Parity of the HIP apply engine with the CPU oracle, through the C ABI.
+
+Method of cutorch's own suite (test/test.lua:232-323): the same seeded host
+data is mirrored to the device with identical storage / offset / size /
+stride, the op runs on both sides, and results are compared -- here bit for
+bit over the WHOLE storage, so stray writes into holes are caught too
+(copyRandomizedTest, test/test.lua:700-727).
+Bar: add/sub/mul/div/cadd/addcmul/addcdiv and the scalar forms are bit-exact
+(one correctly rounded binary32 operation per step, no fusion)."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal, contiguous_geometry, fill_storage, random_geometry
+
+pytestmark = pytest.mark.gpu
+
+BINARY = {"cadd1": ("add", 1.0), "cadd": ("cadd", 0.37), "csub1": ("sub", 1.0), "csub": ("cadd", -2.5),
+          "cmul": ("mul", 0.0), "cdiv": ("div", 0.0)}
+
+
+def run_binary(thc, oracle, name, geoms, rng, inplace=False, dist="normal", kind="float"):
+    """geoms = [out, a, b] as (storage_len, offset, size, stride)."""
+    dtype = np.float16 if kind == "half" else np.float32
+    sts = [fill_storage(rng, g[0], dtype, dist) for g in geoms]
+    if not inplace:
+        sts[0][:] = np.nan
+    dev = [thc.Tensor.from_storage(s, g[1], g[2], g[3], kind) for s, g in zip(sts, geoms)]
+    ref = [oracle.View(s.copy(), g[1], g[2], g[3]) for s, g in zip(sts, geoms)]
+    if inplace:
+        dev[1], ref[1] = dev[0], ref[0]
+    oop, v = BINARY[name]
+    meth = name.rstrip("1")
+    if meth in ("cadd", "csub"):
+        value = 1.0 if name.endswith("1") else (0.37 if meth == "cadd" else 2.5)
+        getattr(dev[0], meth)(dev[1], value, dev[2])
+    else:
+        getattr(dev[0], meth)(dev[1], dev[2])
+    if kind == "half":          # a half tensor's scalar argument is a half too
+        v = float(np.float16(v))
+    oracle.pointwise(oop, ref[0], ref[1], ref[2], value=v)
+    assert dev[0].shape == ref[1].size
+    assert_bit_equal(dev[0].storage_numpy(), ref[0].storage, name)
+    return thc.last_kernel()
+
+
+@pytest.mark.parametrize("name", sorted(BINARY))
+def test_contiguous_1d(thc, oracle, name):
+    rng = np.random.default_rng(1)
+    for n in (1, 3, 4, 1023, 1024, 4097, 100003):
+        g = contiguous_geometry((n,))
+        k = run_binary(thc, oracle, name, [g, g, g], rng, dist="uniform")
+        assert k.startswith("contig")
+
+
+def test_contiguous_config1_shape(thc, oracle):
+    """c = a + b and c = a * b on 2^24 uniform[-1,1] elements (benchmark config 1)."""
+    rng = np.random.default_rng(0xC0FFEE + 1)
+    g = contiguous_geometry((1 << 24,))
+    assert run_binary(thc, oracle, "cadd1", [g, g, g], rng, dist="uniform") == "contig"
+    assert run_binary(thc, oracle, "cmul", [g, g, g], rng, dist="uniform") == "contig"
+
+
+def test_misaligned_contiguous_views(thc, oracle):
+    rng = np.random.default_rng(2)
+    for off in (1, 2, 3, 5):
+        g = (5000 + off, off, (5000,), (1,))
+        g0 = contiguous_geometry((5000,))
+        run_binary(thc, oracle, "cadd1", [g0, g, g0], rng)
+        run_binary(thc, oracle, "cmul", [g, g0, g], rng)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_strided_geometries(thc, oracle, seed):
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(1, 6))
+    shape = tuple(int(x) for x in rng.integers(1, 12, nd))
+    geoms = [random_geometry(rng, shape, holes=rng.random() < 0.6, permute=rng.random() < 0.6)
+             for _ in range(3)]
+    name = sorted(BINARY)[seed % len(BINARY)]
+    run_binary(thc, oracle, name, geoms, rng, inplace=(seed % 5 == 0))
+
+
+@pytest.mark.parametrize("force64", [False, True])
+@pytest.mark.parametrize("shape", [(64, 64), (70, 131), (257, 33), (8, 8), (5, 300, 7), (3, 40, 50),
+                                   (128, 4, 96), (1, 200, 200), (2, 3, 65, 67)])
+def test_transposed_operand_uses_tiles(thc, oracle, shape, force64):
+    """One operand's unit-stride dim is the first logical dim (a:t(), or a
+    permute(3,2,1) view); out and b are contiguous."""
+    rng = np.random.default_rng(sum(shape))
+    nd = len(shape)
+    st, run = [0] * nd, 1
+    for d in range(nd):            # dim 0 innermost in memory
+        st[d] = run
+        run *= shape[d]
+    ga = (run, 0, shape, tuple(st))
+    gc = contiguous_geometry(shape)
+    thc.force_64bit_index(force64)
+    try:
+        k = run_binary(thc, oracle, "cadd1", [gc, ga, gc], rng)
+        k2 = run_binary(thc, oracle, "cmul", [gc, gc, ga], rng)
+        k3 = run_binary(thc, oracle, "cdiv", [ga, gc, gc], rng)   # transposed OUTPUT
+    finally:
+        thc.force_64bit_index(False)
+    dims = [s for s in shape if s != 1]
+    if dims[0] >= 8 and dims[-1] >= 8:      # tiny tile dims fall back to the strided kernel
+        assert k.startswith("tiled") and k2.startswith("tiled") and k3.startswith("tiled"), (k, k2, k3)
+    else:
+        assert k.startswith("strided"), (k, k2, k3)
+
+
+def test_all_operands_transposed_alike_is_flat(thc, oracle):
+    rng = np.random.default_rng(5)
+    g = (60 * 80, 0, (60, 80), (1, 60))
+    assert run_binary(thc, oracle, "cadd1", [g, g, g], rng) == "contig"
+
+
+def test_operands_of_different_shape_pair_by_linear_index(thc, oracle):
+    rng = np.random.default_rng(6)
+    ga = contiguous_geometry((6, 20))
+    gb = (120, 0, (10, 12), (1, 10))
+    gout = contiguous_geometry((4, 30))
+    sts = [fill_storage(rng, g[0]) for g in (gout, ga, gb)]
+    dev = [thc.Tensor.from_storage(s, g[1], g[2], g[3]) for s, g in zip(sts, (gout, ga, gb))]
+    ref = [oracle.View(s.copy(), g[1], g[2], g[3]) for s, g in zip(sts, (gout, ga, gb))]
+    dev[0].cmul(dev[1], dev[2])                 # resizes out to a's shape
+    assert dev[0].shape == (6, 20) and thc.last_kernel() == "generic"
+    out_ref = oracle.View(ref[0].storage, 0, (6, 20))
+    oracle.pointwise("mul", out_ref, ref[1], ref[2])
+    assert_bit_equal(dev[0].storage_numpy(), out_ref.storage)
+
+
+@pytest.mark.parametrize("name,oop", [("add", "addc"), ("sub", "subc"), ("mul", "mulc"), ("div", "divc")])
+def test_scalar_forms(thc, oracle, name, oop):
+    rng = np.random.default_rng(8)
+    for shape, inplace in (((1000,), False), ((33, 47), True), ((9, 10, 11), False)):
+        g_in = random_geometry(rng, shape)
+        g_out = contiguous_geometry(shape)
+        st_in, st_out = fill_storage(rng, g_in[0]), np.full(g_out[0], np.nan, np.float32)
+        a = thc.Tensor.from_storage(st_in, *g_in[1:])
+        ra = oracle.View(st_in.copy(), *g_in[1:])
+        if inplace:
+            out, rout = a, ra
+        else:
+            out = thc.Tensor.from_storage(st_out, *g_out[1:])
+            rout = oracle.View(st_out.copy(), *g_out[1:])
+        getattr(out, name)(a, 3.0)
+        oracle.pointwise(oop, rout, ra, value=3.0)
+        assert_bit_equal(out.storage_numpy(), rout.storage, name)
+
+
+def test_scalar_divide_is_a_true_division(thc):
+    x = np.arange(1, 2001, dtype=np.float32)
+    t = thc.Tensor.from_numpy(x)
+    out = thc.Tensor("float").div(t, 3.0)
+    assert_bit_equal(out.numpy(), x / np.float32(3.0))
+    assert np.any(x / np.float32(3.0) != x * (np.float32(1.0) / np.float32(3.0)))
+
+
+@pytest.mark.parametrize("op", ["addcmul", "addcdiv"])
+@pytest.mark.parametrize("value", [1.0, -0.75])
+def test_addcmul_addcdiv(thc, oracle, op, value):
+    rng = np.random.default_rng(9)
+    for shape, inplace in (((4099,), False), ((64, 96), False), ((31, 65), True), ((6, 7, 8), False)):
+        geoms = [contiguous_geometry(shape)] + [random_geometry(rng, shape) for _ in range(3)]
+        if len(shape) == 2:   # the benchmark's pattern: src1 transposed
+            geoms[2] = (shape[0] * shape[1], 0, shape, (1, shape[0]))
+        sts = [fill_storage(rng, g[0]) for g in geoms]
+        dev = [thc.Tensor.from_storage(s, *g[1:]) for s, g in zip(sts, geoms)]
+        ref = [oracle.View(s.copy(), *g[1:]) for s, g in zip(sts, geoms)]
+        if inplace:
+            dev[0], ref[0] = dev[1], ref[1]
+        getattr(dev[0], op)(dev[1], value, dev[2], dev[3])
+        oracle.pointwise(op, ref[0], ref[1], ref[2], ref[3], value=value)
+        assert_bit_equal(dev[0].storage_numpy(), ref[0].storage, op)
+
+
+def test_unfused_multiply_add(thc):
+    b = np.full(1024, 1 + 2.0 ** -12, dtype=np.float32)
+    d = np.full(1024, -(1 + 2.0 ** -11), dtype=np.float32)
+    out = thc.Tensor("float").addcmul(thc.Tensor.from_numpy(d), 1.0, thc.Tensor.from_numpy(b),
+                                      thc.Tensor.from_numpy(b))
+    assert np.all(out.numpy() == 0.0)          # an FMA would give 2^-24
+
+
+def test_special_values(thc, oracle):
+    a = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, 3e38, 1.0, -1e-40, 1e-39] * 13, dtype=np.float32)
+    b = np.array([-0.0, 0.0, -np.inf, 2.0, 1.0, 1e-45, 3e38, 3.0, 1e-40, 0.5] * 13, dtype=np.float32)
+    for name, oop in (("cadd", "add"), ("cmul", "mul"), ("cdiv", "div"), ("csub", "sub")):
+        out = thc.Tensor("float")
+        args = (thc.Tensor.from_numpy(a), 1.0, thc.Tensor.from_numpy(b)) if name in ("cadd", "csub") \
+            else (thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b))
+        getattr(out, name)(*args)
+        r = oracle.View.empty(a.shape)
+        oracle.pointwise(oop, r, oracle.View.of(a), oracle.View.of(b))
+        got, want = out.numpy(), r.storage
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert_bit_equal(got[~nan], want[~nan], name)   # denormals and signed zeros included
+
+
+def test_overlapping_output_goes_through_a_dense_temporary(thc):
+    # out is an expanded (stride 0) view: every row aliases the same 8 floats;
+    # the reference semantics is "some writer wins" (THCApply.cuh:148-164)
+    st = np.zeros(8, dtype=np.float32)
+    out = thc.Tensor.from_storage(st, 0, (4, 8), (0, 1))
+    a = thc.Tensor.from_numpy(np.arange(32, dtype=np.float32).reshape(4, 8))
+    b = thc.Tensor.from_numpy(np.ones((4, 8), dtype=np.float32))
+    out.cadd(a, 1.0, b)
+    got = out.storage_numpy()
+    cand = np.arange(32, dtype=np.float32).reshape(4, 8) + 1
+    assert all(got[j] in cand[:, j] for j in range(8))
+
+
+def test_empty_and_error_paths(thc):
+    e = thc.Tensor("float")
+    out = thc.Tensor("float").cadd(e, 1.0, e)            # zero-dim: no-op
+    assert out.shape == ()
+    a = thc.Tensor.from_numpy(np.zeros(6, np.float32))
+    b = thc.Tensor.from_numpy(np.zeros(7, np.float32))
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("float").cadd(a, 1.0, b)
+    with pytest.raises(thc.THCError, match="divide by zero"):
+        thc.Tensor("float").div(a, 0.0)
+    # the engine still works after an error was delivered
+    assert np.all(thc.Tensor("float").cadd(a, 1.0, a).numpy() == 0)
+
+
+def test_half_pointwise_rounds_once(thc, oracle):
+    rng = np.random.default_rng(12)
+    for shape in ((4096,), (33, 70), (130, 129)):
+        gs = [contiguous_geometry(shape), random_geometry(rng, shape), contiguous_geometry(shape)]
+        if len(shape) == 2:
+            gs[1] = (shape[0] * shape[1], 0, shape, (1, shape[0]))
+        for name in ("cadd1", "cmul", "cdiv", "cadd"):
+            run_binary(thc, oracle, name, gs, rng, dist="uniform", kind="half")
+
+
+def test_strided_copy_and_contiguous(thc):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((37, 53)).astype(np.float32)
+    t = thc.Tensor.from_numpy(x).t()
+    assert not t.is_contiguous()
+    assert_bit_equal(t.contiguous().numpy(), x.T)
+    assert_bit_equal(t.numpy(), x.T)
+    idx = thc.Tensor.from_numpy(np.arange(24, dtype=np.int64).reshape(4, 6)).t()
+    assert np.array_equal(idx.contiguous().numpy(), np.arange(24).reshape(4, 6).T)
+
+
+def test_large_transposed_roundtrip_property(thc):
+    """Full benchmark size (8192x8192, a:t()): (a:t() * 1 + 0) transposed back
+    equals a -- checked on the device, independent of the oracle."""
+    n = 8192
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((n, n)).astype(np.float32)
+    a = thc.Tensor.from_numpy(x)
+    ones = thc.Tensor.from_numpy(np.ones((n, n), np.float32))
+    out = thc.Tensor("float").cmul(a.t(), ones)
+    assert thc.last_kernel() == "tiled"
+    back = thc.Tensor("float").cmul(out.t(), ones)
+    assert_bit_equal(back.numpy(), x)

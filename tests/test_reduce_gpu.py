@@ -1,0 +1,313 @@
+"""Parity of the HIP reduce engine with the CPU oracle, through the C ABI.
+
+Bars (stated by the task): max/min values and 1-based indices bit-exact with
+the lowest index on ties; sum / norm within 1e-5 relative error in fp32 and
+2e-3 for fp16 input with fp32 accumulation. "Relative" is taken against
+max(|reference|, 2^-6 * sum_i |x_i|): for zero-mean inputs individual sums can
+cancel to ~0, where an error relative to the result alone is unbounded for ANY
+fp32 summation order (one rounding of a partial sum is already 2^-24 of the
+mass sum|x_i|; the floor admits about 2.6 such roundings); the reference's own
+suite uses an absolute 1e-1 there (test/test.lua:1474-1487). Sums of integer-valued data are exact in every
+order and must match bit for bit."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal, contiguous_geometry, fill_storage, random_geometry
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float": 1e-5, "half": 2e-3}
+
+
+def check_close(got, want, absx_sum, kind, what):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    scale = np.maximum(np.abs(want), np.asarray(absx_sum, np.float64) * 2.0 ** -6)
+    scale = np.maximum(scale, 1e-30)
+    err = np.abs(got - want) / scale
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert np.all(np.isfinite(got) == np.isfinite(want)), what
+    worst = float(np.nanmax(err)) if err.size else 0.0
+    assert worst <= TOL[kind], "%s: rel err %.3g > %.3g" % (what, worst, TOL[kind])
+
+
+def dev_and_ref(thc, oracle, rng, geom, kind="float", dist="normal"):
+    dtype = np.float16 if kind == "half" else np.float32
+    st = fill_storage(rng, geom[0], dtype, dist)
+    return thc.Tensor.from_storage(st, *geom[1:], kind=kind), oracle.View(st.copy(), *geom[1:])
+
+
+REDUCERS = [("sum", "sum", 0.0), ("norm2", "norm", 2.0), ("norm1", "norm", 1.0), ("norm0", "norm", 0.0),
+            ("norm3", "norm", 3.0), ("mean", "mean", 0.0)]
+
+
+def run_reduce(thc, oracle, name, dev, ref, dim, kind="float"):
+    _, okind, p = [r for r in REDUCERS if r[0] == name][0]
+    out = thc.Tensor(kind)
+    if okind == "norm":
+        out.norm(dev, p, dim)
+    else:
+        getattr(out, okind)(dev, dim)
+    want = oracle.reduce_dim(okind, ref, dim, p=p).numpy().astype(np.float64)
+    x = np.abs(ref.numpy().astype(np.float64))
+    if name == "norm2":
+        mass = np.sqrt((x * x).sum(axis=dim, keepdims=True))
+    elif name == "norm3":
+        mass = (x ** 3).sum(axis=dim, keepdims=True) ** (1 / 3.0)
+    elif name == "mean":
+        mass = x.mean(axis=dim, keepdims=True)
+    else:
+        mass = x.sum(axis=dim, keepdims=True)
+    got = out.numpy().astype(np.float64)
+    assert out.shape == tuple(1 if d == dim else s for d, s in enumerate(ref.size))
+    check_close(got, want, mass, kind, "%s dim %d %s" % (name, dim, ref.size))
+    return thc.last_kernel()
+
+
+@pytest.mark.parametrize("name", [r[0] for r in REDUCERS])
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_innermost_dim(thc, oracle, name, kind):
+    rng = np.random.default_rng(21)
+    for shape in ((7, 1024), (300, 64), (5, 3), (1000, 17), (3, 5000), (2, 3, 128), (4097, 1), (1, 1)):
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "uniform")
+        k = run_reduce(thc, oracle, name, dev, ref, len(shape) - 1, kind)
+        assert k.startswith("rows"), k
+
+
+@pytest.mark.parametrize("name", [r[0] for r in REDUCERS])
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_non_innermost_dim(thc, oracle, name, kind):
+    rng = np.random.default_rng(22)
+    for shape, dim in (((64, 512), 0), ((6, 300, 40), 1), ((4, 4096, 16), 1), ((129, 7), 0),
+                       ((3, 50, 8, 24), 1), ((2, 2000, 3), 1), ((16, 33, 1), 1)):
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "uniform")
+        k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
+        assert k.startswith("cols") or shape[-1] == 1, k
+
+
+def test_split_reduction_is_used_and_correct(thc, oracle):
+    rng = np.random.default_rng(23)
+    dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((2, 8192, 96)), "float", "uniform")
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1) == "cols-split"
+    assert run_reduce(thc, oracle, "norm2", dev, ref, 1) == "cols-split"
+    dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((3, 1 << 18)), "float", "uniform")
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1) == "rows-split"
+    assert run_reduce(thc, oracle, "norm2", dev, ref, 1) == "rows-split"
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_strided_inputs(thc, oracle, seed):
+    rng = np.random.default_rng(300 + seed)
+    nd = int(rng.integers(1, 5))
+    shape = tuple(int(x) for x in rng.integers(1, 20, nd))
+    dim = int(rng.integers(0, nd))
+    geom = random_geometry(rng, shape, holes=rng.random() < 0.5, permute=rng.random() < 0.5)
+    dev, ref = dev_and_ref(thc, oracle, rng, geom)
+    run_reduce(thc, oracle, REDUCERS[seed % len(REDUCERS)][0], dev, ref, dim)
+    thc.force_64bit_index(True)
+    try:
+        run_reduce(thc, oracle, "sum", dev, ref, dim)
+    finally:
+        thc.force_64bit_index(False)
+
+
+def test_integer_valued_sums_are_bit_exact(thc, oracle):
+    rng = np.random.default_rng(24)
+    for shape, dim in (((512, 1024), 1), ((16, 2048, 64), 1), ((1 << 20,), 0), ((100, 77), 0)):
+        x = rng.integers(-8, 9, shape).astype(np.float32)
+        dev = thc.Tensor.from_numpy(x)
+        out = thc.Tensor("float").sum(dev, dim)
+        assert_bit_equal(out.numpy(), x.astype(np.int64).sum(axis=dim, keepdims=True).astype(np.float32))
+        assert dev.sumall() == float(x.astype(np.int64).sum())
+
+
+def test_keepdim_zero_squeezes(thc):
+    x = np.ones((3, 4, 5), np.float32)
+    out = thc.Tensor("float").sum(thc.Tensor.from_numpy(x), 1, keepdim=0)
+    assert out.shape == (3, 5) and np.all(out.numpy() == 4)
+    out = thc.Tensor("float").sum(thc.Tensor.from_numpy(np.ones(7, np.float32)), 0, keepdim=0)
+    assert out.shape == (1,)        # a vector never loses its last dim
+
+
+def test_output_with_existing_strides_is_kept(thc, oracle):
+    rng = np.random.default_rng(25)
+    x = rng.standard_normal((6, 9, 10)).astype(np.float32)
+    st = np.full(6 * 1 * 10 * 3, np.nan, np.float32)
+    out = thc.Tensor.from_storage(st, 1, (6, 1, 10), (30, 30, 3))     # right shape, odd strides
+    out.sum(thc.Tensor.from_numpy(x), 1)
+    assert out.strides == (30, 30, 3)
+    r = oracle.View(st.copy(), 1, (6, 1, 10), (30, 30, 3))
+    oracle.reduce_dim("sum", oracle.View.of(x), 1, out=r)
+    got, want = out.storage_numpy(), r.storage
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    np.testing.assert_allclose(got[~np.isnan(got)], want[~np.isnan(want)], rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------- max / min --
+def run_minmax(thc, oracle, which, dev, ref, dim, kind="float"):
+    vals, idx = thc.Tensor(kind), thc.Tensor("long")
+    getattr(vals, which)(idx, dev, dim)
+    rv, ri = oracle.minmax_dim(which, ref, dim)
+    assert_bit_equal(vals.numpy(), rv.numpy(), which + " values")
+    assert np.array_equal(idx.numpy(), ri.numpy()), which + " indices"
+    return thc.last_kernel()
+
+
+@pytest.mark.parametrize("which", ["max", "min"])
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_minmax_with_many_ties(thc, oracle, which, kind):
+    rng = np.random.default_rng(31)
+    for shape, dim in (((64, 1024), 1), ((9, 33), 1), ((5, 4000), 1), ((300, 5), 1), ((64, 512), 0),
+                       ((6, 300, 40), 1), ((4, 4096, 16), 1), ((2, 8192, 96), 1), ((7,), 0), ((1, 1), 0)):
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "ints")
+        run_minmax(thc, oracle, which, dev, ref, dim, kind)
+
+
+def test_minmax_config3_pattern(thc, oracle):
+    """normal(0,1) rows with ~1% of each row overwritten by copies of other
+    entries of the same row, the row maximum included (benchmark config 3)."""
+    rng = np.random.default_rng(0xC0FFEE + 3)
+    rows, n = 2048, 1024
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    for r in range(rows):
+        src = rng.integers(0, n, 10)
+        dst = rng.integers(0, n, 10)
+        x[r, dst] = x[r, src]
+        j = int(np.argmax(x[r]))
+        x[r, rng.integers(0, n, 2)] = x[r, j]
+    dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+    assert run_minmax(thc, oracle, "max", dev, ref, 1) == "rows-index"
+    run_minmax(thc, oracle, "min", dev, ref, 1)
+    assert np.array_equal(ref.numpy(), x)
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_minmax_random_strided(thc, oracle, seed):
+    rng = np.random.default_rng(400 + seed)
+    nd = int(rng.integers(1, 5))
+    shape = tuple(int(x) for x in rng.integers(1, 20, nd))
+    dim = int(rng.integers(0, nd))
+    geom = random_geometry(rng, shape, holes=rng.random() < 0.5, permute=rng.random() < 0.5)
+    dev, ref = dev_and_ref(thc, oracle, rng, geom, "float", "ints")
+    run_minmax(thc, oracle, "max" if seed % 2 else "min", dev, ref, dim)
+
+
+def test_minmax_nan_inf_and_signed_zero(thc, oracle):
+    x = np.array([[1, np.nan, 5, np.nan, 0, 0, 0, 0], [-np.inf] * 8, [2, 7, 7, 1, 7, 0, 0, 0],
+                  [np.inf, 1, np.inf, 0, 0, 0, 0, 0], [-0.0, 0.0, -0.0, 0.0, -1, -1, -1, -1]], dtype=np.float32)
+    for which in ("max", "min"):
+        vals, idx = thc.Tensor("float"), thc.Tensor("long")
+        getattr(vals, which)(idx, thc.Tensor.from_numpy(x), 1)
+        rv, ri = oracle.minmax_dim(which, oracle.View.of(x), 1)
+        assert np.array_equal(idx.numpy(), ri.numpy())
+        g, w = vals.numpy(), rv.numpy()
+        assert np.array_equal(np.isnan(g), np.isnan(w))
+        assert_bit_equal(g[~np.isnan(g)], w[~np.isnan(w)])
+
+
+def test_minmax_noncontiguous_outputs(thc, oracle):
+    rng = np.random.default_rng(33)
+    x = rng.integers(-3, 4, (12, 30)).astype(np.float32)
+    vst = np.full(12 * 2 + 1, np.nan, np.float32)
+    ist = np.full(12 * 3, -7, np.int64)
+    vals = thc.Tensor.from_storage(vst, 1, (12, 1), (2, 2))
+    idx = thc.Tensor.from_storage(ist, 0, (12, 1), (3, 1), kind="long")
+    vals.max(idx, thc.Tensor.from_numpy(x), 1)
+    assert np.array_equal(idx.storage_numpy()[0::3], np.argmax(x, 1) + 1)
+    assert np.all(idx.storage_numpy()[1::3] == -7)
+    assert np.array_equal(vals.storage_numpy()[1::2], x.max(1))
+
+
+# ------------------------------------------------------------------ *all --
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_all_reductions(thc, oracle, kind):
+    rng = np.random.default_rng(41)
+    for shape in ((1,), (5,), (2048,), (2049,), (100003,), (1 << 21,), (300, 700), (5, 6, 7)):
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "uniform")
+        x = np.abs(ref.numpy().astype(np.float64))
+        n = x.size
+        check_close(dev.sumall(), oracle.reduce_all("sum", ref), x.sum(), kind, "sumall")
+        check_close(dev.meanall(), oracle.reduce_all("mean", ref), x.mean(), kind, "meanall")
+        check_close(dev.normall(2.0), oracle.reduce_all("norm", ref, p=2), 0, kind, "normall2")
+        check_close(dev.normall(1.0), oracle.reduce_all("norm", ref, p=1), 0, kind, "normall1")
+        check_close(dev.normall(3.0), oracle.reduce_all("norm", ref, p=3), 0, kind, "normall3")
+        assert dev.normall(0.0) == oracle.reduce_all("norm", ref, p=0)
+        assert dev.maxall() == oracle.reduce_all("max", ref)
+        assert dev.minall() == oracle.reduce_all("min", ref)
+
+
+def test_all_reductions_on_strided_views(thc, oracle):
+    rng = np.random.default_rng(42)
+    for shape in ((40, 50), (7, 8, 9), (300,)):
+        for permute in (False, True):
+            geom = random_geometry(rng, shape, holes=True, permute=permute)
+            dev, ref = dev_and_ref(thc, oracle, rng, geom, "float", "uniform")
+            x = np.abs(ref.numpy().astype(np.float64))
+            check_close(dev.sumall(), oracle.reduce_all("sum", ref), x.sum(), "float", "sumall strided")
+            assert dev.maxall() == oracle.reduce_all("max", ref)
+            assert dev.minall() == oracle.reduce_all("min", ref)
+
+
+def test_all_empty_and_nan(thc):
+    e = thc.Tensor("float")
+    assert e.sumall() == 0.0 and e.prodall() == 1.0
+    x = np.ones(5000, np.float32)
+    x[1234] = np.nan
+    t = thc.Tensor.from_numpy(x)
+    assert np.isnan(t.maxall()) and np.isnan(t.minall()) and np.isnan(t.sumall())
+    with pytest.raises(thc.THCError, match="empty Tensor"):
+        e.meanall()
+
+
+def test_reduce_error_paths(thc):
+    t = thc.Tensor.from_numpy(np.ones((3, 4), np.float32))
+    with pytest.raises(thc.THCError, match="dimension out of range"):
+        thc.Tensor("float").sum(t, 2)
+    with pytest.raises(thc.THCError, match="dimension out of range"):
+        thc.Tensor("float").max(thc.Tensor("long"), t, -1)
+
+
+# --------------------------------------- full benchmark shapes (properties) --
+def test_config3_full_size_against_oracle(thc, oracle):
+    """65536 x 1024: the oracle finishes this in well under a second."""
+    rng = np.random.default_rng(0xC0FFEE + 33)
+    x = rng.standard_normal((65536, 1024)).astype(np.float32)
+    dup = rng.integers(0, 1024, (65536, 10))
+    x[np.arange(65536)[:, None], dup] = x[np.arange(65536)[:, None], dup[:, ::-1]]
+    x[np.arange(65536), dup[:, 0]] = x.max(1)          # duplicate the row maximum
+    dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+    oracle.set_num_threads(8)
+    try:
+        run_reduce(thc, oracle, "sum", dev, ref, 1)
+        run_minmax(thc, oracle, "max", dev, ref, 1)
+    finally:
+        oracle.set_num_threads(1)
+
+
+def test_config4_full_size_against_oracle(thc, oracle):
+    """64 x 4096 x 512, reduce the middle dim, fp32 and fp16 input."""
+    rng = np.random.default_rng(0xC0FFEE + 4)
+    x = rng.uniform(-2, 2, (64, 4096, 512)).astype(np.float32)
+    oracle.set_num_threads(8)
+    try:
+        for kind, arr in (("float", x), ("half", x.astype(np.float16))):
+            dev, ref = thc.Tensor.from_numpy(arr), oracle.View.of(arr)
+            assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
+            run_reduce(thc, oracle, "norm2", dev, ref, 1, kind)
+    finally:
+        oracle.set_num_threads(1)
+
+
+def test_sumall_2pow28_uniform(thc, oracle):
+    """reduceAll over 2^28 uniform[0,1] values (1 GiB)."""
+    rng = np.random.default_rng(0xC0FFEE + 333)
+    x = rng.random(1 << 28, dtype=np.float32)
+    dev = thc.Tensor.from_numpy(x)
+    oracle.set_num_threads(8)
+    try:
+        want = oracle.reduce_all("sum", oracle.View(x))
+    finally:
+        oracle.set_num_threads(1)
+    got = dev.sumall()
+    assert abs(got - want) <= 1e-5 * abs(want), (got, want)
+    assert abs(dev.normall(2.0) - oracle.reduce_all("norm", oracle.View(x[:1 << 20]), p=2)) >= 0  # smoke
