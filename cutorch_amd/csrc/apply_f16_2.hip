@@ -1,0 +1,6 @@
+// Apply-engine slice: element type __half, operator group 2.
+#include "apply_impl.hpp"
+
+namespace thc {
+template void apply_dispatch_group<__half, 2>(THCState*, Plan&, bool, PointOp, float);
+}

@@ -1,0 +1,6 @@
+// Apply-engine slice: element type float, operator group 2.
+#include "apply_impl.hpp"
+
+namespace thc {
+template void apply_dispatch_group<float, 2>(THCState*, Plan&, bool, PointOp, float);
+}

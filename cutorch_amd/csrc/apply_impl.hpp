@@ -1,0 +1,599 @@
+// Kernels and launch logic of the pointwise apply engine (templates only).
+// Included by the apply_*.hip translation units, each of which instantiates
+// one slice (element type x operator group) so that the slices compile in
+// parallel; apply.hip holds the type-independent planning front end.
+//
+// Role of THC_pointwiseApply1/2/3 + kernelPointwiseApply1/2/3
+// (lib/THC/THCApply.cuh:19-98,124-640): run an elementwise functor over
+// operands that are each addressed through their own sizes/strides. The
+// design differs from the reference on purpose:
+//   * the operands are described in ONE joint iteration space (shared sizes,
+//     per-operand strides), so the index -> coordinate division chain runs
+//     once per 16-byte pack, not once per element and operand;
+//   * four kernel families instead of one:
+//       contig   every operand is a flat run: dwordx4 streaming
+//       strided  all operands have unit stride in the innermost joint dim:
+//                dwordx4 packs along it, outer coordinates by multiply-shift
+//                division
+//       tiled    an input whose unit-stride dim is not the output's goes
+//                through an LDS tile so that both sides of the transpose are
+//                accessed in 256..512-byte coalesced rows
+//       generic  operands of different shapes (paired by logical linear
+//                index) or with no unit-stride dim: per-element offsets
+//   * 32-bit index arithmetic when every count and offset is < 2^31, 64-bit
+//     otherwise (tile origins are the only 64-bit quantities in the tiled
+//     kernel; inside a tile all arithmetic is 32-bit).
+#pragma once
+#include <type_traits>
+
+#include "apply_plan.hpp"
+#include "common.hpp"
+#include "device_util.hpp"
+
+namespace thc {
+
+// ------------------------------------------------------------------------
+// Functors
+// ------------------------------------------------------------------------
+// Arithmetic is done in fp32 and rounded once to the element type; the build
+// disables fp contraction so a*b+c stays two roundings (the CPU contract).
+struct OpCopy {
+  static constexpr int NIN = 1;
+  template <typename T>
+  __device__ __forceinline__ T operator()(T a, T, T) const {
+    return a;
+  }
+};
+struct OpFill {
+  static constexpr int NIN = 0;
+  float v;
+  template <typename T>
+  __device__ __forceinline__ T operator()(T, T, T) const {
+    return Cvt<T>::down(v);
+  }
+};
+#define THC_ARITH_OP(Name, NIN_, EXPR)                                  \
+  struct Name {                                                         \
+    static constexpr int NIN = NIN_;                                    \
+    float v;                                                            \
+    template <typename T>                                               \
+    __device__ __forceinline__ T operator()(T a_, T b_, T c_) const {   \
+      const float a = Cvt<T>::up(a_), b = Cvt<T>::up(b_), c = Cvt<T>::up(c_); \
+      (void)a; (void)b; (void)c;                                        \
+      return Cvt<T>::down(EXPR);                                        \
+    }                                                                   \
+  };
+THC_ARITH_OP(OpAddC, 1, a + v)
+THC_ARITH_OP(OpSubC, 1, a - v)
+THC_ARITH_OP(OpMulC, 1, a * v)
+THC_ARITH_OP(OpDivC, 1, a / v)
+THC_ARITH_OP(OpPow, 1, powf(a, v))
+THC_ARITH_OP(OpAdd, 2, a + b)
+THC_ARITH_OP(OpSub, 2, a - b)
+THC_ARITH_OP(OpMul, 2, a * b)
+THC_ARITH_OP(OpDiv, 2, a / b)
+THC_ARITH_OP(OpCAdd, 2, a + v * b)
+THC_ARITH_OP(OpAddCMul, 3, a + v * (b * c))
+THC_ARITH_OP(OpAddCDiv, 3, a + v * (b / c))
+#undef THC_ARITH_OP
+
+
+// ------------------------------------------------------------------------
+// contig: flat streaming, one 16-byte pack per operand per step
+// ------------------------------------------------------------------------
+template <typename T, typename Op, int VEC, int UNROLL, bool NT>
+__global__ __launch_bounds__(kBlock) void apply_contig_kernel(T* out, const T* in0, const T* in1,
+                                                              const T* in2, uint64_t n, Op op) {
+  using P = Pack<T, VEC>;
+  const uint64_t npack = n / VEC;
+  const uint64_t step = (uint64_t)gridDim.x * (kBlock * UNROLL);
+  for (uint64_t base = (uint64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x; base < npack;
+       base += step) {
+    P a[UNROLL], b[UNROLL], c[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint64_t i = base + (uint64_t)u * kBlock;
+      if (i < npack) {
+        if (Op::NIN > 0) a[u] = load_pack<NT>(reinterpret_cast<const P*>(in0) + i);
+        if (Op::NIN > 1) b[u] = load_pack<NT>(reinterpret_cast<const P*>(in1) + i);
+        if (Op::NIN > 2) c[u] = load_pack<NT>(reinterpret_cast<const P*>(in2) + i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint64_t i = base + (uint64_t)u * kBlock;
+      if (i < npack) {
+        P r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = op(a[u].v[e], b[u].v[e], c[u].v[e]);
+        store_pack<NT>(reinterpret_cast<P*>(out) + i, r);
+      }
+    }
+  }
+  // the n % VEC trailing elements
+  const uint64_t tail = npack * VEC + (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (VEC > 1 && tail < n) {
+    T a{}, b{}, c{};
+    if (Op::NIN > 0) a = in0[tail];
+    if (Op::NIN > 1) b = in1[tail];
+    if (Op::NIN > 2) c = in2[tail];
+    out[tail] = op(a, b, c);
+  }
+}
+
+// ------------------------------------------------------------------------
+// strided / generic: linear index -> per-operand offsets
+// ------------------------------------------------------------------------
+template <typename I>
+struct IndexedArgs {
+  int dims[kMaxOps];                  // JOINT: only dims[0] is used
+  Divisor<I> size[kMaxOps][kMaxDims]; // JOINT: only size[0][*] is used
+  I stride[kMaxOps][kMaxDims];        // in elements; pre-multiplied by VEC in the packed dim
+};
+
+// JOINT = all operands share sizes (one division chain); VEC packs along the
+// innermost dim (then that dim's size is already divided by VEC on the host).
+template <typename T, typename Op, typename I, int VEC, bool JOINT>
+__global__ __launch_bounds__(kBlock) void apply_indexed_kernel(T* out, const T* in0, const T* in1,
+                                                               const T* in2, I total,
+                                                               IndexedArgs<I> args, Op op) {
+  using P = Pack<T, VEC>;
+  constexpr int NOPS = Op::NIN + 1;
+  const I step = (I)gridDim.x * kBlock;
+  for (I lin = (I)blockIdx.x * kBlock + threadIdx.x; lin < total; lin += step) {
+    I off[kMaxOps] = {0, 0, 0, 0};
+    if (JOINT) {
+      I rest = lin;
+      for (int d = args.dims[0] - 1; d > 0; --d) {
+        I q, r;
+        args.size[0][d].divmod(rest, q, r);
+        rest = q;
+#pragma unroll
+        for (int k = 0; k < NOPS; ++k) off[k] += r * args.stride[k][d];
+      }
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) off[k] += rest * args.stride[k][0];
+    } else {
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) {
+        I rest = lin;
+        for (int d = args.dims[k] - 1; d > 0; --d) {
+          I q, r;
+          args.size[k][d].divmod(rest, q, r);
+          rest = q;
+          off[k] += r * args.stride[k][d];
+        }
+        off[k] += rest * args.stride[k][0];
+      }
+    }
+    P a{}, b{}, c{};
+    if (Op::NIN > 0) a = load_pack<true>(reinterpret_cast<const P*>(in0 + off[1]));
+    if (Op::NIN > 1) b = load_pack<true>(reinterpret_cast<const P*>(in1 + off[2]));
+    if (Op::NIN > 2) c = load_pack<true>(reinterpret_cast<const P*>(in2 + off[3]));
+    P r;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r.v[e] = op(a.v[e], b.v[e], c.v[e]);
+    store_pack<true>(reinterpret_cast<P*>(out + off[0]), r);
+  }
+}
+
+// ------------------------------------------------------------------------
+// tiled: operands whose unit-stride dim is `p` meet operands whose
+// unit-stride dim is `q` in a TILE x TILE patch staged through LDS.
+// ------------------------------------------------------------------------
+template <typename I>
+struct TiledArgs {
+  int dims;
+  int p, q;
+  int staged[kMaxOps];             // operand k is accessed along p (through LDS)
+  I size[kMaxDims];
+  Divisor<I> bsize[kMaxDims];      // divisors of the batch dims (all but p, q)
+  I stride[kMaxOps][kMaxDims];
+  Divisor<I> tilesP, tilesQ;
+  I totalTiles;
+};
+
+// A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
+// Staged operands are read/written with LXP lanes along p, direct operands
+// with LXQ lanes along q, 16 bytes per lane. On MI355X the tile must be wide
+// in q (512-byte rows for the direct operands) and hold >= 32 KiB of a staged
+// operand to reach streaming bandwidth: 64x128 and 128x128 fp32 tiles run at
+// the speed of a flat 3-read-1-write stream, 64x64 tiles ~20% below it.
+// MASK >= 0 fixes at compile time which inputs are staged (bit k-1 = input k);
+// MASK < 0 reads the flags from `args` (scalar fallback variant). The output is
+// never staged: the joint dims are ordered by the output's strides, so its
+// unit-stride dim is q by construction.
+template <typename T, typename Op, typename I, int VEC, int LXP, int LXQ, int MASK>
+__global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in0, const T* in1,
+                                                             const T* in2, TiledArgs<I> args,
+                                                             Op op) {
+  constexpr int NOPS = Op::NIN + 1;
+  constexpr int TP = LXP * VEC, TQ = LXQ * VEC;
+  constexpr int ROWS_P = kBlock / LXP, PASSES_P = TQ / ROWS_P;  // lanes along p: rows are q
+  constexpr int ROWS_Q = kBlock / LXQ, PASSES_Q = TP / ROWS_Q;  // lanes along q: rows are p
+  constexpr int PITCH = TP + 1;  // odd pitch: transposed reads spread over the banks
+  using P = Pack<T, VEC>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  const T* ptr[kMaxOps] = {out, in0, in1, in2};
+  const int lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
+  const int lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  bool staged[kMaxOps];
+  int slot[kMaxOps];  // LDS slab of a staged operand
+  {
+    int s = 0;
+    staged[0] = false;
+    slot[0] = -1;
+#pragma unroll
+    for (int k = 1; k < NOPS; ++k) {
+      staged[k] = MASK >= 0 ? ((MASK >> (k - 1)) & 1) != 0 : args.staged[k] != 0;
+      slot[k] = staged[k] ? s++ : -1;
+    }
+  }
+
+  // Thread-varying parts of the addresses are 32-bit element offsets inside a
+  // tile (the host guarantees they fit); everything else is uniform and lives
+  // in scalar registers, so a load is "scalar base + 32-bit lane offset".
+  uint32_t vo[kMaxOps];   // lane offset of operand k in its own access pattern
+  size_t rowStep[kMaxOps];  // uniform distance between two passes
+#pragma unroll
+  for (int k = 0; k < NOPS; ++k) {
+    if (staged[k]) {
+      vo[k] = (uint32_t)lyp * (uint32_t)args.stride[k][args.q] + lxp * VEC;
+      rowStep[k] = (size_t)ROWS_P * (size_t)args.stride[k][args.q];
+    } else {
+      vo[k] = (uint32_t)lyq * (uint32_t)args.stride[k][args.p] +
+              (uint32_t)(lxq * VEC) * (VEC > 1 ? 1u : (uint32_t)args.stride[k][args.q]);
+      rowStep[k] = (size_t)ROWS_Q * (size_t)args.stride[k][args.p];
+    }
+  }
+
+  for (I tile = blockIdx.x; tile < args.totalTiles; tile += gridDim.x) {
+    I rest, tq, tp;
+    args.tilesQ.divmod(tile, rest, tq);
+    args.tilesP.divmod(rest, rest, tp);
+    I base[kMaxOps] = {0, 0, 0, 0};
+    for (int d = args.dims - 1; d >= 0; --d) {
+      if (d == args.p || d == args.q) continue;
+      I r;
+      args.bsize[d].divmod(rest, rest, r);
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) base[k] += r * args.stride[k][d];
+    }
+    const I p0 = tp * TP, q0 = tq * TQ;
+    const uint32_t pn = (uint32_t)min((I)TP, args.size[args.p] - p0);  // valid extent
+    const uint32_t qn = (uint32_t)min((I)TQ, args.size[args.q] - q0);
+    const T* tbase[kMaxOps];  // uniform pointer to the tile origin of operand k
+#pragma unroll
+    for (int k = 0; k < NOPS; ++k)
+      tbase[k] = ptr[k] + (base[k] + p0 * args.stride[k][args.p] + q0 * args.stride[k][args.q]);
+
+    // Loads of a phase are issued as one batch (first loop) and consumed in a
+    // second loop, so that 8 x 16 bytes per operand are in flight per lane.
+    // Interior tiles (the common case) run without any bounds predicate.
+    auto body = [&](auto fullTag) {
+      constexpr bool FULL = decltype(fullTag)::value;
+      const bool okP = FULL || lxp * VEC < pn;
+      const bool okQ = FULL || lxq * VEC < qn;
+      // phase 1: staged inputs, lanes along p, into lds[slot][q][p]
+#pragma unroll
+      for (int k = 1; k < NOPS; ++k) {
+        if (!staged[k]) continue;
+        T* slab = lds + slot[k] * (TQ * PITCH);
+        P v[PASSES_P];
+#pragma unroll
+        for (int r = 0; r < PASSES_P; ++r) {
+          const uint32_t qi = lyp + r * ROWS_P;
+          if (FULL || (okP && qi < qn))
+            v[r] = load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
+        }
+#pragma unroll
+        for (int r = 0; r < PASSES_P; ++r) {
+          const uint32_t qi = lyp + r * ROWS_P;
+          if (FULL || (okP && qi < qn)) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) slab[qi * PITCH + lxp * VEC + e] = v[r].v[e];
+          }
+        }
+      }
+      __syncthreads();
+
+      // phase 2: compute with lanes along q
+      const uint32_t qi = lxq * VEC;
+      P din[3][PASSES_Q];
+#pragma unroll
+      for (int k = 1; k < NOPS; ++k) {
+        if (staged[k]) continue;
+#pragma unroll
+        for (int r = 0; r < PASSES_Q; ++r) {
+          const uint32_t pi = lyq + r * ROWS_Q;
+          if (FULL || (okQ && pi < pn))
+            din[k - 1][r] =
+                load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < PASSES_Q; ++r) {
+        const uint32_t pi = lyq + r * ROWS_Q;
+        if (FULL || (okQ && pi < pn)) {
+          P in[3] = {};
+#pragma unroll
+          for (int k = 1; k < NOPS; ++k) {
+            if (staged[k]) {
+              const T* slab = lds + slot[k] * (TQ * PITCH);
+#pragma unroll
+              for (int e = 0; e < VEC; ++e) in[k - 1].v[e] = slab[(qi + e) * PITCH + pi];
+            } else {
+              in[k - 1] = din[k - 1][r];
+            }
+          }
+          P res;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) res.v[e] = op(in[0].v[e], in[1].v[e], in[2].v[e]);
+          store_pack<true>(
+              reinterpret_cast<P*>(const_cast<T*>(tbase[0]) + r * rowStep[0] + vo[0]), res);
+        }
+      }
+    };
+    if (pn == TP && qn == TQ)
+      body(std::true_type{});
+    else
+      body(std::false_type{});
+    __syncthreads();  // the slabs are reused by the next tile
+  }
+}
+
+// ------------------------------------------------------------------------
+// Host side: launch
+// ------------------------------------------------------------------------
+template <typename T>
+inline bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* key, int default_per_cu) {
+  const int64_t blocks = (work_items + per_block - 1) / per_block;
+  const int64_t cap = (int64_t)num_compute_units(s) * tuning(key, default_per_cu);
+  return (int)std::max<int64_t>(1, std::min(blocks, cap));
+}
+
+template <typename T, typename Op>
+void launch_contig(THCState* s, const Plan& pl, Op op) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int U = 4;
+  bool vec = true;
+  for (int k = 0; k < pl.nops; ++k) vec = vec && aligned16<T>(pl.ptr[k]);
+  T* out = (T*)pl.ptr[0];
+  const T* i0 = (const T*)pl.ptr[1];
+  const T* i1 = (const T*)pl.ptr[2];
+  const T* i2 = (const T*)pl.ptr[3];
+  const uint64_t n = (uint64_t)pl.numel;
+  hipStream_t st = current_stream(s);
+  // One pass per workgroup (no persistent loop) measured best on MI355X; the
+  // grid-stride loop only engages beyond 2^20 workgroups.
+  const int64_t packs = vec ? (int64_t)(n / VEC) + 1 : (int64_t)n;
+  const int64_t blocks = (packs + kBlock * U - 1) / (kBlock * U);
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, tuning("apply.contig.max_grid", 1 << 20)));
+  // Streaming hint only when the operands cannot stay cache resident anyway.
+  const bool nt = (int64_t)n * (int64_t)sizeof(T) * pl.nops >= tuning("apply.contig.nt_bytes", 8 << 20);
+  if (vec && nt)
+    hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, U, true>), dim3(grid), dim3(kBlock), 0, st,
+                       out, i0, i1, i2, n, op);
+  else if (vec)
+    hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, U, false>), dim3(grid), dim3(kBlock), 0, st,
+                       out, i0, i1, i2, n, op);
+  else
+    hipLaunchKernelGGL((apply_contig_kernel<T, Op, 1, U, false>), dim3(grid), dim3(kBlock), 0, st,
+                       out, i0, i1, i2, n, op);
+  note_kernel(vec ? "contig" : "contig-scalar");
+}
+
+template <typename T, typename Op, typename I, bool JOINT>
+void launch_indexed(THCState* s, const Plan& pl, Op op) {
+  constexpr int VEC = 16 / sizeof(T);
+  IndexedArgs<I> args{};
+  bool vec = JOINT;
+  if (JOINT) {
+    const int nd = pl.lay[0].dims;
+    vec = vec && pl.lay[0].size[nd - 1] % VEC == 0;
+    for (int k = 0; k < pl.nops && vec; ++k) {
+      vec = aligned16<T>(pl.ptr[k]) && pl.lay[k].stride[nd - 1] == 1;
+      for (int d = 0; d < nd - 1 && vec; ++d) vec = pl.lay[k].stride[d] % VEC == 0;
+    }
+  }
+  const int pack = vec ? VEC : 1;
+  for (int k = 0; k < pl.nops; ++k) {
+    const int nd = pl.lay[k].dims;
+    args.dims[k] = nd;
+    for (int d = 0; d < nd; ++d) {
+      int64_t sz = pl.lay[k].size[d];
+      int64_t sd = pl.lay[k].stride[d];
+      if (vec && d == nd - 1) {
+        sz /= pack;
+        sd *= pack;
+      }
+      args.size[k][d].set((uint64_t)sz);
+      args.stride[k][d] = (I)sd;
+    }
+  }
+  const int64_t total = pl.numel / pack;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((total + kBlock - 1) / kBlock,
+                                                               tuning("apply.indexed.max_grid", 1 << 22)));
+  T* out = (T*)pl.ptr[0];
+  const T* i0 = (const T*)pl.ptr[1];
+  const T* i1 = (const T*)pl.ptr[2];
+  const T* i2 = (const T*)pl.ptr[3];
+  hipStream_t st = current_stream(s);
+  if (vec) {
+    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, VEC, JOINT>), dim3(grid), dim3(kBlock), 0, st,
+                       out, i0, i1, i2, (I)total, args, op);
+  } else {
+    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, 1, JOINT>), dim3(grid), dim3(kBlock), 0, st,
+                       out, i0, i1, i2, (I)total, args, op);
+  }
+  note_kernel(JOINT ? (vec ? "strided" : "strided-scalar") : "generic");
+}
+
+// Pick (p, q) for the tiled kernel. q = innermost joint dim. An operand is
+// staged when its unit-stride dim is p != q. Returns false when no operand
+// wants a transpose (or the transposed operands disagree about p).
+inline bool tile_plan(const Plan& pl, int& p, int& q, int staged[kMaxOps]) {
+  const int nd = pl.lay[0].dims;
+  if (nd < 2) return false;
+  q = nd - 1;
+  p = -1;
+  for (int k = 0; k < pl.nops; ++k) {
+    staged[k] = 0;
+    if (pl.lay[k].stride[q] == 1) continue;
+    int unit = -1;
+    for (int d = 0; d < nd - 1; ++d)
+      if (pl.lay[k].stride[d] == 1) unit = d;
+    if (unit < 0) continue;  // no unit-stride dim at all: direct (uncoalesced) access
+    if (k == 0) continue;    // cannot happen after the reorder by output stride
+    if (p < 0) p = unit;
+    if (unit == p) staged[k] = 1;
+  }
+  if (p < 0) return false;
+  // Tiny tile dims make the LDS detour pointless.
+  if (pl.lay[0].size[p] < 8 || pl.lay[0].size[q] < 8) return false;
+  return true;
+}
+
+template <typename T, typename Op, typename I>
+bool launch_tiled(THCState* s, const Plan& pl, Op op) {
+  int p, q, staged[kMaxOps] = {0, 0, 0, 0};
+  if (!tile_plan(pl, p, q, staged)) return false;
+  constexpr int VEC = 16 / sizeof(T);
+  // vector variant: 64 x 128 elements for 4-byte types (LDS 33 KiB per staged
+  // operand); scalar variant: 64 x 64.
+  constexpr int LXP = 64 / VEC > 16 ? 16 : (64 / VEC < 8 ? 8 : 64 / VEC);
+  constexpr int LXQ = 32;
+  constexpr int64_t tpV = LXP * VEC, tqV = LXQ * VEC, tS = 64;
+  const int nd = pl.lay[0].dims;
+  int nstaged = 0;
+  for (int k = 0; k < pl.nops; ++k) nstaged += staged[k];
+
+  // 16-byte packs need every pack fully inside the tensor and aligned.
+  bool vec = pl.lay[0].size[p] % VEC == 0 && pl.lay[0].size[q] % VEC == 0;
+  for (int k = 0; k < pl.nops && vec; ++k) {
+    const int fast = staged[k] ? p : q;
+    vec = aligned16<T>(pl.ptr[k]) && pl.lay[k].stride[fast] == 1;
+    for (int d = 0; d < nd && vec; ++d)
+      if (d != fast) vec = pl.lay[k].stride[d] % VEC == 0;
+  }
+  // Lane offsets inside a tile are 32-bit: refuse layouts whose tile spans more.
+  for (int k = 0; k < pl.nops; ++k) {
+    const int64_t span = 64 * std::max(pl.lay[k].stride[p], pl.lay[k].stride[q]) + 1024;
+    if (span >= (int64_t(1) << 31)) return false;
+    if (pl.lay[k].stride[p] < 0 || pl.lay[k].stride[q] < 0) return false;
+  }
+  const size_t ldsV = nstaged * tqV * (tpV + 1) * sizeof(T);
+  const size_t ldsS = nstaged * tS * (tS + 1) * sizeof(T);
+  if (vec && ldsV > 64 * 1024) vec = false;
+  if (!vec && ldsS > 64 * 1024) return false;
+  const int64_t tileP = vec ? tpV : tS, tileQ = vec ? tqV : tS;
+
+  TiledArgs<I> args{};
+  args.dims = nd;
+  args.p = p;
+  args.q = q;
+  int64_t batch = 1;
+  for (int d = 0; d < nd; ++d) {
+    args.size[d] = (I)pl.lay[0].size[d];
+    args.bsize[d].set((uint64_t)pl.lay[0].size[d]);
+    if (d != p && d != q) batch *= pl.lay[0].size[d];
+    for (int k = 0; k < pl.nops; ++k) args.stride[k][d] = (I)pl.lay[k].stride[d];
+  }
+  for (int k = 0; k < pl.nops; ++k) args.staged[k] = staged[k];
+  const int64_t tp = (pl.lay[0].size[p] + tileP - 1) / tileP;
+  const int64_t tq = (pl.lay[0].size[q] + tileQ - 1) / tileQ;
+  args.tilesP.set((uint64_t)tp);
+  args.tilesQ.set((uint64_t)tq);
+  const int64_t total = batch * tp * tq;
+  if (sizeof(I) == 4 && total >= kIndex32Limit) return false;
+  args.totalTiles = (I)total;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, tuning("apply.tiled.max_grid", 1 << 22)));
+  T* out = (T*)pl.ptr[0];
+  const T* i0 = (const T*)pl.ptr[1];
+  const T* i1 = (const T*)pl.ptr[2];
+  const T* i2 = (const T*)pl.ptr[3];
+  hipStream_t st = current_stream(s);
+  const int mask = staged[1] | (staged[2] << 1) | (staged[3] << 2);
+  if (vec) {
+#define THC_TILED_CASE(M)                                                                         \
+  case M:                                                                                         \
+    if ((M) < (1 << Op::NIN))                                                                     \
+      hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, VEC, LXP, LXQ, ((M) < (1 << Op::NIN) ? (M) : 1)>), \
+                         dim3(grid), dim3(kBlock), ldsV, st, out, i0, i1, i2, args, op);          \
+    break;
+    switch (mask) {
+      THC_TILED_CASE(1) THC_TILED_CASE(2) THC_TILED_CASE(3) THC_TILED_CASE(4)
+      THC_TILED_CASE(5) THC_TILED_CASE(6) THC_TILED_CASE(7)
+      default: return false;
+    }
+#undef THC_TILED_CASE
+    note_kernel("tiled");
+  } else {
+    hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, 1, 64, 64, -1>), dim3(grid), dim3(kBlock), ldsS,
+                       st, out, i0, i1, i2, args, op);
+    note_kernel("tiled-scalar");
+  }
+  return true;
+}
+
+template <typename T, typename Op>
+void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
+  bool wide = force_64bit_index();
+  for (int k = 0; k < pl.nops; ++k) {
+    wide = wide || !fits_32bit(pl.lay[k]);
+    for (int d = 0; d < pl.lay[k].dims; ++d) wide = wide || pl.lay[k].stride[d] < 0;
+  }
+  if (sameShape && joint_collapse(pl.nops, pl.lay, /*reorder=*/true)) {
+    bool flat = pl.lay[0].dims == 1;
+    for (int k = 0; k < pl.nops && flat; ++k) flat = pl.lay[k].stride[0] == 1;
+    if (flat) {
+      launch_contig<T>(s, pl, op);
+      return;
+    }
+    if (tuning("apply.tiled.enable", 1)) {
+      if (wide ? launch_tiled<T, Op, uint64_t>(s, pl, op) : launch_tiled<T, Op, uint32_t>(s, pl, op))
+        return;
+    }
+    if (wide)
+      launch_indexed<T, Op, uint64_t, true>(s, pl, op);
+    else
+      launch_indexed<T, Op, uint32_t, true>(s, pl, op);
+    return;
+  }
+  for (int k = 0; k < pl.nops; ++k) collapse(pl.lay[k]);
+  if (wide)
+    launch_indexed<T, Op, uint64_t, false>(s, pl, op);
+  else
+    launch_indexed<T, Op, uint32_t, false>(s, pl, op);
+}
+
+
+// Operator groups: one translation unit per (element type, group).
+template <typename T, int GROUP>
+void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v) {
+  switch (op) {
+#define THC_CASE(G, NAME)                                         \
+  case PointOp::NAME:                                             \
+    if constexpr (GROUP == G) run_plan<T>(s, pl, sameShape, Op##NAME{v});   \
+    break;
+    THC_CASE(0, Fill) THC_CASE(0, AddC) THC_CASE(0, SubC) THC_CASE(0, MulC) THC_CASE(0, DivC)
+    THC_CASE(0, Pow)
+    THC_CASE(1, Add) THC_CASE(1, Sub) THC_CASE(1, Mul) THC_CASE(1, Div) THC_CASE(1, CAdd)
+    THC_CASE(2, AddCMul) THC_CASE(2, AddCDiv)
+#undef THC_CASE
+    default: raise_error("pointwise op not available for this element type");
+  }
+}
+
+template <typename T>
+void apply_copy(THCState* s, Plan& pl, bool sameShape) {
+  run_plan<T>(s, pl, sameShape, OpCopy{});
+}
+
+}  // namespace thc

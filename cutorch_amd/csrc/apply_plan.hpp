@@ -1,0 +1,28 @@
+// Interface between the type-independent apply front end (apply.hip) and the
+// per-type kernel slices (apply_f32_*.hip, apply_f16_*.hip, apply_raw.hip).
+#pragma once
+#include "common.hpp"
+
+namespace thc {
+
+constexpr int kMaxOps = 4;  // output + up to three inputs
+
+struct Plan {
+  int nops;
+  void* ptr[kMaxOps];
+  Layout lay[kMaxOps];
+  int64_t numel;
+};
+
+inline int op_group(PointOp op) {
+  const int n = point_op_inputs(op);
+  return n <= 1 ? 0 : (n == 2 ? 1 : 2);
+}
+
+// Defined (explicitly instantiated) in the slices.
+template <typename T, int GROUP>
+void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v);
+template <typename T>
+void apply_copy(THCState* s, Plan& pl, bool sameShape);
+
+}  // namespace thc

@@ -23,60 +23,15 @@
 // once on store. max/min carry (value, index) pairs whose combine step prefers
 // the lower index on equal values at every level, so the first occurrence wins
 // as in a sequential scan; the first NaN wins over everything.
-#include <hip/hip_fp16.h>
-
 #include <cmath>
 #include <limits>
 
 #include "common.hpp"
+#include "device_util.hpp"
 
 namespace thc {
 
 namespace {
-
-constexpr int kBlock = 256;
-
-template <typename T, int N>
-struct alignas(sizeof(T) * N) Pack {
-  T v[N];
-};
-
-template <typename T>
-struct Cvt {
-  static __device__ __forceinline__ float up(T x) { return (float)x; }
-  static __device__ __forceinline__ T down(float x) { return (T)x; }
-};
-template <>
-struct Cvt<__half> {
-  static __device__ __forceinline__ float up(__half x) { return __half2float(x); }
-  static __device__ __forceinline__ __half down(float x) { return __float2half_rn(x); }
-};
-
-template <typename I>
-struct Divisor;
-template <>
-struct Divisor<uint32_t> {
-  uint32_t d, m, s;
-  __host__ void set(uint64_t div) {
-    d = (uint32_t)div;
-    for (s = 0; s < 32; ++s)
-      if ((uint64_t(1) << s) >= div) break;
-    m = (uint32_t)(((uint64_t(1) << 32) * ((uint64_t(1) << s) - div)) / div + 1);
-  }
-  __device__ __forceinline__ void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
-    q = (__umulhi(n, m) + n) >> s;
-    r = n - q * d;
-  }
-};
-template <>
-struct Divisor<uint64_t> {
-  uint64_t d;
-  __host__ void set(uint64_t div) { d = div; }
-  __device__ __forceinline__ void divmod(uint64_t n, uint64_t& q, uint64_t& r) const {
-    q = n / d;
-    r = n - q * d;
-  }
-};
 
 // --------------------------------------------------------------- functors --
 struct Epi {
@@ -183,7 +138,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
       const TIn* src = in + inOff;
 #pragma unroll 4
       for (I i = begin + lane * VEC; i < end; i += (I)G * VEC) {
-        const P v = *reinterpret_cast<const P*>(src + i);
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<TIn>::up(v.v[e]);
@@ -230,7 +185,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
       const T* src = in + inOff;
 #pragma unroll 4
       for (I i = lane * VEC; i < R; i += (I)G * VEC) {
-        const P v = *reinterpret_cast<const P*>(src + i);
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<T>::up(v.v[e]);
@@ -303,7 +258,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
       const TIn* src = in + inOff + col;
 #pragma unroll 4
       for (I r = begin + ty; r < end; r += TY) {
-        const P v = *reinterpret_cast<const P*>(src + r * a.sR);
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e])));
       }
@@ -383,7 +338,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
       const T* src = in + inOff + col;
 #pragma unroll 4
       for (I r = begin + ty; r < end; r += TY) {
-        const P v = *reinterpret_cast<const P*>(src + r * a.sR);
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<T>::up(v.v[e]);
