@@ -93,10 +93,13 @@ class Config(object):
         self.sets, self.run, self.check, self.kernel = sets, run, check, kernel
 
 
-def build_configs(thc, hip, which):
+def build_configs(thc, hip, which, only=None):
     rng = np.random.default_rng(0xC0FFEE)
     cfgs = []
     T = thc.Tensor
+
+    def want(*names):
+        return not only or any(n in only for n in names)
 
     def c2():
         n = 8192
@@ -127,7 +130,7 @@ def build_configs(thc, hip, which):
     # C1: contiguous 2^24, three rotating buffer sets (working set < Infinity Cache)
     n1 = 1 << 24
     sets1 = []
-    for _ in range(3):
+    for _ in range(3 if want('C1-add', 'C1-mul') else 0):
         a = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
         b = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
         sets1.append((a, b, T("float").resize((n1,))))
@@ -139,7 +142,7 @@ def build_configs(thc, hip, which):
     # C3a/b: 65536 x 1024, last dim
     r3, n3 = 65536, 1024
     sets3 = []
-    for _ in range(3):
+    for _ in range(3 if want('C3a-sum', 'C3b-max') else 0):
         x = rng.standard_normal((r3, n3), dtype=np.float32)
         dup = rng.integers(0, n3, (r3, 10))
         x[np.arange(r3)[:, None], dup] = x[np.arange(r3)[:, None], dup[:, ::-1]]
@@ -152,31 +155,33 @@ def build_configs(thc, hip, which):
 
     # C3c: reduceAll over 2^28
     n3c = 1 << 28
-    xa = T.from_numpy(rng.random(n3c, dtype=np.float32))
+    xa = T.from_numpy(rng.random(n3c if want('C3c-sumall') else 4, dtype=np.float32))
     cfgs.append(Config("C3c-sumall", "sumall over 2^28 fp32 (blocks on a 4-byte D2H copy)",
                        4 * n3c + 4, n3c, 1, lambda i: xa.sumall()))
 
     # C4: 64 x 4096 x 512, middle dim; fp32 and fp16
-    s4 = (64, 4096, 512)
+    s4 = (64, 4096, 512) if want('C4-sum-f32', 'C4-norm-f32', 'C4-sum-f16', 'C4-norm-f16') else (1, 4, 8)
     x4 = rng.uniform(-2, 2, s4).astype(np.float32)
     d4 = T.from_numpy(x4)
-    o4 = T("float").resize((64, 1, 512))
+    o4 = T("float").resize((s4[0], 1, s4[2]))
     n4 = int(np.prod(s4))
-    cfgs.append(Config("C4-sum-f32", "sum over middle dim of 64x4096x512 fp32", 4 * n4 + 4 * 64 * 512,
+    cfgs.append(Config("C4-sum-f32", "sum over middle dim of 64x4096x512 fp32", 4 * n4 + 4 * s4[0] * s4[2],
                        n4, 1, lambda i: o4.sum(d4, 1)))
     cfgs.append(Config("C4-norm-f32", "L2 norm over middle dim of 64x4096x512 fp32",
-                       4 * n4 + 4 * 64 * 512, n4, 1, lambda i: o4.norm(d4, 2.0, 1)))
+                       4 * n4 + 4 * s4[0] * s4[2], n4, 1, lambda i: o4.norm(d4, 2.0, 1)))
     sets4h = []
     for _ in range(3):
         h = T.from_numpy((x4 * np.float32(rng.uniform(0.5, 1.0))).astype(np.float16))
-        sets4h.append((h, T("half").resize((64, 1, 512))))
+        sets4h.append((h, T("half").resize((s4[0], 1, s4[2]))))
     cfgs.append(Config("C4-sum-f16", "sum over middle dim of 64x4096x512 fp16, fp32 accumulate",
-                       2 * n4 + 2 * 64 * 512, n4, 3, lambda i: sets4h[i % 3][1].sum(sets4h[i % 3][0], 1)))
+                       2 * n4 + 2 * s4[0] * s4[2], n4, 3, lambda i: sets4h[i % 3][1].sum(sets4h[i % 3][0], 1)))
     cfgs.append(Config("C4-norm-f16", "L2 norm over middle dim of 64x4096x512 fp16, fp32 accumulate",
-                       2 * n4 + 2 * 64 * 512, n4, 3,
+                       2 * n4 + 2 * s4[0] * s4[2], n4, 3,
                        lambda i: sets4h[i % 3][1].norm(sets4h[i % 3][0], 2.0, 1)))
 
     # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path
+    if not want('C5'):
+        return [c for c in cfgs if c is cfgs[0] or want(c.name)], host_c2
     block = rng.standard_normal(1 << 24, dtype=np.float32)
     a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
     b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), block[::-1].copy())
@@ -240,6 +245,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--configs", default="all", choices=["all", "primary"])
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated config names to measure")
+    ap.add_argument("--tune", action="append", default=[], help="engine tuning knob key=value")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)")
@@ -248,7 +255,13 @@ def main():
     thc.state()                      # raises if libTHC.so is missing or no GPU is visible
     hip = Hip()
     stream = thc.lib().THCState_getCurrentStream(thc.state())
-    cfgs, host_c2 = build_configs(thc, hip, args.configs)
+    for kv in args.tune:
+        k, v = kv.split("=")
+        thc.set_tuning(k, int(v))
+    only = set(args.only.split(",")) if args.only else None
+    cfgs, host_c2 = build_configs(thc, hip, args.configs, only)
+    if only:
+        cfgs = [cfgs[0]] + [c for c in cfgs[1:] if c.name in only]
     results = []
     for cfg in cfgs:
         steps = args.steps if cfg.name != "C5" else max(3, args.steps // 5)

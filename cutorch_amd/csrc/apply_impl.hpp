@@ -178,25 +178,37 @@ __global__ __launch_bounds__(kBlock) void apply_indexed_kernel(T* out, const T* 
 }
 
 // ------------------------------------------------------------------------
-// tiled: operands whose unit-stride dim is `p` meet operands whose
-// unit-stride dim is `q` in a TILE x TILE patch staged through LDS.
+// tiled: inputs whose unit-stride dim is `p` meet operands whose unit-stride
+// dim is `q` in a TP x TQ patch staged through LDS.
 // ------------------------------------------------------------------------
+constexpr int kMaxFuse = 4;
+
+// Tile bookkeeping is 32-bit (tile counts, coordinates inside p and q);
+// only the element offsets of the tile origin are of the index type I.
 template <typename I>
 struct TiledArgs {
-  int dims;
-  int p, q;
-  int staged[kMaxOps];             // operand k is accessed along p (through LDS)
-  I size[kMaxDims];
-  Divisor<I> bsize[kMaxDims];      // divisors of the batch dims (all but p, q)
-  I stride[kMaxOps][kMaxDims];
-  Divisor<I> tilesP, tilesQ;
-  I totalTiles;
+  int staged[kMaxOps];   // input k is read along p and goes through LDS
+  uint32_t sizeP, sizeQ; // extents of p and of the (possibly fused) q
+  I strideP[kMaxOps];    // per operand stride along p
+  I strideQ[kMaxOps];    // per operand stride along q (innermost fused dim)
+  // q may fuse nq >= 1 joint dims that are one contiguous run for every direct
+  // operand (e.g. the two inner dims of a dense output) while a staged
+  // operand sees them with unrelated strides: its row offset is recovered
+  // from the q coordinate by division.
+  int nq;
+  Divisor<uint32_t> qsub[kMaxFuse];      // sizes of the fused dims, innermost first
+  I qstride[kMaxOps][kMaxFuse];          // strides of the fused dims, innermost first
+  int nbatch;                            // remaining dims
+  Divisor<uint32_t> bsize[kMaxDims];
+  I bstride[kMaxOps][kMaxDims];
+  Divisor<uint32_t> tilesP, tilesQ;
+  uint32_t totalTiles;
 };
 
 // A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
-// Staged operands are read/written with LXP lanes along p, direct operands
-// with LXQ lanes along q, 16 bytes per lane. On MI355X the tile must be wide
-// in q (512-byte rows for the direct operands) and hold >= 32 KiB of a staged
+// Staged inputs are read with LXP lanes along p, direct operands with LXQ
+// lanes along q, 16 bytes per lane. On MI355X the tile must be wide in q
+// (512-byte rows for the direct operands) and hold >= 32 KiB of a staged
 // operand to reach streaming bandwidth: 64x128 and 128x128 fp32 tiles run at
 // the speed of a flat 3-read-1-write stream, 64x64 tiles ~20% below it.
 // MASK >= 0 fixes at compile time which inputs are staged (bit k-1 = input k);
@@ -217,8 +229,8 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
   T* lds = reinterpret_cast<T*>(lds_raw);
 
   const T* ptr[kMaxOps] = {out, in0, in1, in2};
-  const int lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
-  const int lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
+  const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
   bool staged[kMaxOps];
   int slot[kMaxOps];  // LDS slab of a staged operand
   {
@@ -235,39 +247,42 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
   // Thread-varying parts of the addresses are 32-bit element offsets inside a
   // tile (the host guarantees they fit); everything else is uniform and lives
   // in scalar registers, so a load is "scalar base + 32-bit lane offset".
-  uint32_t vo[kMaxOps];   // lane offset of operand k in its own access pattern
+  uint32_t vo[kMaxOps];     // lane offset of operand k in its own access pattern
   size_t rowStep[kMaxOps];  // uniform distance between two passes
 #pragma unroll
   for (int k = 0; k < NOPS; ++k) {
     if (staged[k]) {
-      vo[k] = (uint32_t)lyp * (uint32_t)args.stride[k][args.q] + lxp * VEC;
-      rowStep[k] = (size_t)ROWS_P * (size_t)args.stride[k][args.q];
+      vo[k] = lyp * (uint32_t)args.strideQ[k] + lxp * VEC;
+      rowStep[k] = (size_t)ROWS_P * (size_t)args.strideQ[k];
     } else {
-      vo[k] = (uint32_t)lyq * (uint32_t)args.stride[k][args.p] +
-              (uint32_t)(lxq * VEC) * (VEC > 1 ? 1u : (uint32_t)args.stride[k][args.q]);
-      rowStep[k] = (size_t)ROWS_Q * (size_t)args.stride[k][args.p];
+      vo[k] = lyq * (uint32_t)args.strideP[k] +
+              (lxq * VEC) * (VEC > 1 ? 1u : (uint32_t)args.strideQ[k]);
+      rowStep[k] = (size_t)ROWS_Q * (size_t)args.strideP[k];
     }
   }
+  const bool fused = args.nq > 1;
 
-  for (I tile = blockIdx.x; tile < args.totalTiles; tile += gridDim.x) {
-    I rest, tq, tp;
+  for (uint32_t tile = blockIdx.x; tile < args.totalTiles; tile += gridDim.x) {
+    uint32_t rest, tq, tp;
     args.tilesQ.divmod(tile, rest, tq);
     args.tilesP.divmod(rest, rest, tp);
     I base[kMaxOps] = {0, 0, 0, 0};
-    for (int d = args.dims - 1; d >= 0; --d) {
-      if (d == args.p || d == args.q) continue;
-      I r;
-      args.bsize[d].divmod(rest, rest, r);
+    for (int j = 0; j < args.nbatch; ++j) {
+      uint32_t r;
+      args.bsize[j].divmod(rest, rest, r);
 #pragma unroll
-      for (int k = 0; k < NOPS; ++k) base[k] += r * args.stride[k][d];
+      for (int k = 0; k < NOPS; ++k) base[k] += (I)r * args.bstride[k][j];
     }
-    const I p0 = tp * TP, q0 = tq * TQ;
-    const uint32_t pn = (uint32_t)min((I)TP, args.size[args.p] - p0);  // valid extent
-    const uint32_t qn = (uint32_t)min((I)TQ, args.size[args.q] - q0);
+    const uint32_t p0 = tp * TP, q0 = tq * TQ;
+    const uint32_t pn = min((uint32_t)TP, args.sizeP - p0);  // valid extent
+    const uint32_t qn = min((uint32_t)TQ, args.sizeQ - q0);
     const T* tbase[kMaxOps];  // uniform pointer to the tile origin of operand k
 #pragma unroll
-    for (int k = 0; k < NOPS; ++k)
-      tbase[k] = ptr[k] + (base[k] + p0 * args.stride[k][args.p] + q0 * args.stride[k][args.q]);
+    for (int k = 0; k < NOPS; ++k) {
+      I o = base[k] + (I)p0 * args.strideP[k];
+      if (!(staged[k] && fused)) o += (I)q0 * args.strideQ[k];
+      tbase[k] = ptr[k] + o;
+    }
 
     // Loads of a phase are issued as one batch (first loop) and consumed in a
     // second loop, so that 8 x 16 bytes per operand are in flight per lane.
@@ -282,11 +297,28 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
         if (!staged[k]) continue;
         T* slab = lds + slot[k] * (TQ * PITCH);
         P v[PASSES_P];
+        if (!fused) {
 #pragma unroll
-        for (int r = 0; r < PASSES_P; ++r) {
-          const uint32_t qi = lyp + r * ROWS_P;
-          if (FULL || (okP && qi < qn))
-            v[r] = load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
+          for (int r = 0; r < PASSES_P; ++r) {
+            const uint32_t qi = lyp + r * ROWS_P;
+            if (FULL || (okP && qi < qn))
+              v[r] = load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < PASSES_P; ++r) {
+            const uint32_t qi = lyp + r * ROWS_P;
+            if (FULL || (okP && qi < qn)) {
+              uint32_t qg = q0 + qi, c;
+              I off = lxp * VEC;
+              for (int j = 0; j < args.nq - 1; ++j) {
+                args.qsub[j].divmod(qg, qg, c);
+                off += (I)c * args.qstride[k][j];
+              }
+              off += (I)qg * args.qstride[k][args.nq - 1];
+              v[r] = load_pack<true>(reinterpret_cast<const P*>(tbase[k] + off));
+            }
+          }
         }
 #pragma unroll
         for (int r = 0; r < PASSES_P; ++r) {
@@ -495,24 +527,51 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
   const int64_t tileP = vec ? tpV : tS, tileQ = vec ? tqV : tS;
 
   TiledArgs<I> args{};
-  args.dims = nd;
-  args.p = p;
-  args.q = q;
-  int64_t batch = 1;
-  for (int d = 0; d < nd; ++d) {
-    args.size[d] = (I)pl.lay[0].size[d];
-    args.bsize[d].set((uint64_t)pl.lay[0].size[d]);
-    if (d != p && d != q) batch *= pl.lay[0].size[d];
-    for (int k = 0; k < pl.nops; ++k) args.stride[k][d] = (I)pl.lay[k].stride[d];
+  for (int k = 0; k < pl.nops; ++k) {
+    args.staged[k] = staged[k];
+    args.strideP[k] = (I)pl.lay[k].stride[p];
+    args.strideQ[k] = (I)pl.lay[k].stride[q];
   }
-  for (int k = 0; k < pl.nops; ++k) args.staged[k] = staged[k];
+  // Fuse into q the dims just outside it that continue q's run for every
+  // direct operand (vector variant only: there q has unit stride for them).
+  bool inQ[kMaxDims] = {};
+  inQ[q] = true;
+  int64_t sizeQ = pl.lay[0].size[q];
+  args.nq = 1;
+  args.qsub[0].set((uint64_t)sizeQ);
+  for (int k = 0; k < pl.nops; ++k) args.qstride[k][0] = (I)pl.lay[k].stride[q];
+  if (vec && tuning("apply.tiled.fuse_q", 1)) {
+    for (int d = q - 1; d >= 0 && d != p && args.nq < kMaxFuse; --d) {
+      bool ok = sizeQ * pl.lay[0].size[d] < kIndex32Limit;
+      for (int k = 0; k < pl.nops && ok; ++k)
+        if (!staged[k]) ok = pl.lay[k].stride[d] == sizeQ;
+      if (!ok) break;
+      args.qsub[args.nq].set((uint64_t)pl.lay[0].size[d]);
+      for (int k = 0; k < pl.nops; ++k) args.qstride[k][args.nq] = (I)pl.lay[k].stride[d];
+      ++args.nq;
+      inQ[d] = true;
+      sizeQ *= pl.lay[0].size[d];
+    }
+  }
+  if (pl.lay[0].size[p] >= kIndex32Limit || sizeQ >= kIndex32Limit) return false;
+  args.sizeP = (uint32_t)pl.lay[0].size[p];
+  args.sizeQ = (uint32_t)sizeQ;
+  int64_t batch = 1;
+  args.nbatch = 0;
+  for (int d = nd - 1; d >= 0; --d) {
+    if (d == p || inQ[d]) continue;
+    args.bsize[args.nbatch].set((uint64_t)pl.lay[0].size[d]);
+    for (int k = 0; k < pl.nops; ++k) args.bstride[k][args.nbatch] = (I)pl.lay[k].stride[d];
+    ++args.nbatch;
+    batch *= pl.lay[0].size[d];
+  }
   const int64_t tp = (pl.lay[0].size[p] + tileP - 1) / tileP;
-  const int64_t tq = (pl.lay[0].size[q] + tileQ - 1) / tileQ;
+  const int64_t tq = (sizeQ + tileQ - 1) / tileQ;
   args.tilesP.set((uint64_t)tp);
   args.tilesQ.set((uint64_t)tq);
   const int64_t total = batch * tp * tq;
-  if (sizeof(I) == 4 && total >= kIndex32Limit) return false;
-  args.totalTiles = (I)total;
+  if (total >= kIndex32Limit) return false;  // tile bookkeeping is 32-bit
+  args.totalTiles = (uint32_t)total;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, tuning("apply.tiled.max_grid", 1 << 22)));
   T* out = (T*)pl.ptr[0];
   const T* i0 = (const T*)pl.ptr[1];
@@ -533,7 +592,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
       default: return false;
     }
 #undef THC_TILED_CASE
-    note_kernel("tiled");
+    note_kernel(args.nq > 1 ? "tiled-fused" : "tiled");
   } else {
     hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, 1, 64, 64, -1>), dim3(grid), dim3(kBlock), ldsS,
                        st, out, i0, i1, i2, args, op);

@@ -105,7 +105,21 @@ hipStream_t current_stream(THCState* state);
 THCDeviceAllocator* state_allocator(THCState* state);  // THCGeneral.h.in:98-100
 int state_device(THCState* state);
 int num_compute_units(THCState* state);
-// Per-stream device scratch for partial results (THCGeneral.c:677-712).
+// Per-stream device scratch for partial results (THCGeneral.c:677-712):
+// `partials` for split reductions, a tail of zero-initialised arrival
+// counters (each kernel resets the ones it used), and a pinned host slot that
+// kernels can write the scalar result of an *all reduction into.
+constexpr size_t kScratchTailBytes = 64 * 1024;
+constexpr size_t kScratchCounters = (kScratchTailBytes - 256) / sizeof(unsigned);
+struct StreamScratch {
+  void* partials;
+  size_t partialBytes;
+  unsigned* counters;   // kScratchCounters arrival counters
+  float* result;        // device slot for a scalar result (last 256 bytes of the tail)
+  float* hostResult;    // pinned host memory ...
+  float* hostResultDev; // ... and its device-side address
+};
+const StreamScratch& stream_scratch(THCState* state);
 void* scratch_space(THCState* state, size_t* bytes);
 void check_same_gpu(THCState* state, int n, const AnyTensor* const* ts);
 void note_kernel(const char* name);  // for THCAmd_lastKernel

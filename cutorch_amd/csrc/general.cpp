@@ -19,7 +19,7 @@ struct THCState {
   int numCUs = 0;
   THCDeviceAllocator allocator{};
   std::mutex mu;
-  std::map<hipStream_t, void*> scratch;  // per stream, lazily allocated
+  std::map<hipStream_t, thc::StreamScratch> scratch;  // per stream, lazily allocated
   size_t scratchBytes = 0;
 };
 
@@ -96,17 +96,34 @@ int state_device(THCState* s) { return s->device; }
 
 int num_compute_units(THCState* s) { return s->numCUs > 0 ? s->numCUs : 256; }
 
-void* scratch_space(THCState* s, size_t* bytes) {
+const StreamScratch& stream_scratch(THCState* s) {
   hipStream_t st = current_stream(s);
   std::lock_guard<std::mutex> lk(s->mu);
-  if (bytes) *bytes = s->scratchBytes;
   auto it = s->scratch.find(st);
   if (it != s->scratch.end()) return it->second;
+  StreamScratch sc{};
   void* p = nullptr;
   THC_CHECK((hipError_t)s->allocator.malloc(s->allocator.state, &p, s->scratchBytes,
                                             (hipStream_t_)st));
-  s->scratch[st] = p;
-  return p;
+  sc.partials = p;
+  sc.partialBytes = s->scratchBytes - kScratchTailBytes;
+  sc.counters = reinterpret_cast<unsigned*>(static_cast<char*>(p) + sc.partialBytes);
+  sc.result = reinterpret_cast<float*>(static_cast<char*>(p) + s->scratchBytes - 256);
+  // Arrival counters start at zero and every kernel that uses one resets it.
+  THC_CHECK(hipMemsetAsync(sc.counters, 0, kScratchTailBytes, st));
+  THC_CHECK(hipStreamSynchronize(st));
+  // One pinned, device-mapped slot: *all reductions store their scalar there.
+  THC_CHECK(hipHostMalloc(reinterpret_cast<void**>(&sc.hostResult), 256, hipHostMallocMapped));
+  void* dv = nullptr;
+  THC_CHECK(hipHostGetDevicePointer(&dv, sc.hostResult, 0));
+  sc.hostResultDev = static_cast<float*>(dv);
+  return s->scratch[st] = sc;
+}
+
+void* scratch_space(THCState* s, size_t* bytes) {
+  const StreamScratch& sc = stream_scratch(s);
+  if (bytes) *bytes = sc.partialBytes;
+  return sc.partials;
 }
 
 void check_same_gpu(THCState* s, int n, const AnyTensor* const* ts) {
@@ -179,8 +196,11 @@ THC_API void THCudaInit(THCState* state) {
 THC_API void THCudaShutdown(THCState* state) {
   THC_GUARD_VOID({
     std::lock_guard<std::mutex> lk(state->mu);
-    for (auto& kv : state->scratch)
-      if (kv.second) THC_CHECK((hipError_t)state->allocator.free(state->allocator.state, kv.second));
+    for (auto& kv : state->scratch) {
+      if (kv.second.partials)
+        THC_CHECK((hipError_t)state->allocator.free(state->allocator.state, kv.second.partials));
+      if (kv.second.hostResult) THC_CHECK(hipHostFree(kv.second.hostResult));
+    }
     state->scratch.clear();
     state->initialised = false;
   })
@@ -197,7 +217,7 @@ THC_API void* THCState_getCurrentDeviceScratchSpace(THCState* state) {
   THC_GUARD_RET(nullptr, return scratch_space(state, nullptr))
 }
 THC_API size_t THCState_getCurrentDeviceScratchSpaceSize(THCState* state) {
-  return state->scratchBytes;
+  return state->scratchBytes - thc::kScratchTailBytes;
 }
 THC_API int THCudaMalloc(THCState* state, void** ptr, size_t size) {
   return state->allocator.malloc(state->allocator.state, ptr, size,

@@ -25,6 +25,7 @@
 // as in a sequential scan; the first NaN wins over everything.
 #include <cmath>
 #include <limits>
+#include <type_traits>
 
 #include "common.hpp"
 #include "device_util.hpp"
@@ -136,8 +137,24 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
       const I begin = s * chunk;
       const I end = min(R, begin + chunk);
       const TIn* src = in + inOff;
-#pragma unroll 4
-      for (I i = begin + lane * VEC; i < end; i += (I)G * VEC) {
+      // U loads are issued back to back before any of them is consumed.
+      constexpr int U = 8;
+      const I step = (I)G * VEC;
+      I i = begin + lane * VEC;
+      for (; i + (U - 1) * step < end; i += U * step) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(src + i + u * step));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float x = Cvt<TIn>::up(v[u].v[e]);
+            acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+          }
+        }
+      }
+      for (; i < end; i += step) {
         const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -183,8 +200,26 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
       oa.offsets(row, inOff, outOff);
       oaIdx.offsets(row, unused, idxOff);
       const T* src = in + inOff;
-#pragma unroll 4
-      for (I i = lane * VEC; i < R; i += (I)G * VEC) {
+      constexpr int U = 8;
+      const I step = (I)G * VEC;
+      I i = lane * VEC;
+      for (; i + (U - 1) * step < R; i += U * step) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(src + i + u * step));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float x = Cvt<T>::up(v[u].v[e]);
+            if (O::better(x, i + u * step + e, bv, bi)) {
+              bv = x;
+              bi = i + u * step + e;
+            }
+          }
+        }
+      }
+      for (; i < R; i += step) {
         const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
@@ -232,38 +267,24 @@ struct ColsArgs {
   uint32_t TX;          // lanes along the unit-stride dim (power of two <= 256)
 };
 
+// Split reductions run as two launches: workgroups publish fp32 partial planes
+// [S][outElems], a small second kernel folds the S planes in plane order. (A
+// single-launch variant in which the last workgroup to arrive folds the
+// partials needs agent-scope release/acquire fences; on MI355X each such
+// fence writes back the whole L2 of the XCD and made the kernel 5-10x slower.)
 template <typename TIn, typename TOut, typename F, typename I, int VEC>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restrict__ in,
                                                              TOut* __restrict__ out,
                                                              float* __restrict__ partial,
                                                              ColsArgs<I> a, I totalBlocks, Epi epi,
-                                                             F f) {
+                                                             F f, bool foldPass) {
   using P = Pack<TIn, VEC>;
   __shared__ float smem[kBlock * VEC];
   const uint32_t TX = a.TX, TY = kBlock / TX;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
-    I rest, s, ct;
-    a.S.divmod(b, rest, s);
-    a.colTiles.divmod(rest, rest, ct);
-    I inOff, outOff;
-    a.oa.offsets(rest, inOff, outOff);
-    const I col = (ct * TX + tx) * VEC;
-    float acc[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
-    if (col < a.C) {
-      const I begin = s * a.chunkR;
-      const I end = min(a.R, begin + a.chunkR);
-      const TIn* src = in + inOff + col;
-#pragma unroll 4
-      for (I r = begin + ty; r < end; r += TY) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e])));
-      }
-    }
-    // fold the TY thread rows (fixed tree)
+  // Fold the TY thread rows through LDS in a fixed tree; row 0 ends up with
+  // the result in smem[tx*VEC + e].
+  auto fold_rows = [&](const float (&acc)[VEC]) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) smem[(ty * TX + tx) * VEC + e] = acc[e];
     __syncthreads();
@@ -277,78 +298,78 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
       }
       __syncthreads();
     }
-    if (ty == 0 && col < a.C) {
+  };
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I group = b, s = 0, rest, ct;
+    if (!foldPass) a.S.divmod(b, group, s);
+    a.colTiles.divmod(group, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    float acc[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float r = smem[tx * VEC + e];
-        if (a.S.d > 1)
-          partial[s * a.outElems + rest * a.C + col + e] = r;
-        else
-          out[outOff + (col + e) * a.outInner] = epi.template finish<TOut>(r);
+    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+    float* plane = partial + rest * a.C + col;
+    if (foldPass) {
+      // second launch: one workgroup per group (S == 1 in the block index),
+      // thread row ty folds planes ty, ty+TY, ...
+      if (col < a.C) {
+        for (I sp = ty; sp < a.S.d; sp += TY) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], plane[sp * a.outElems + e]);
+        }
+      }
+    } else if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const TIn* src = in + inOff + col;
+      constexpr int U = 8;
+      I r = begin + ty;
+      for (; r + (U - 1) * TY < end; r += U * TY) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (r + u * TY) * a.sR));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v[u].v[e])));
+        }
+      }
+      for (; r < end; r += TY) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e])));
+      }
+    }
+    fold_rows(acc);
+    if (ty == 0 && col < a.C) {
+      if (foldPass || a.S.d == 1) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          out[outOff + (col + e) * a.outInner] = epi.template finish<TOut>(smem[tx * VEC + e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) plane[s * a.outElems + e] = smem[tx * VEC + e];
       }
     }
     __syncthreads();
   }
 }
 
-// Fold S partial planes [S][outElems] in plane order and store.
-template <typename TOut, typename F, typename I>
-__global__ __launch_bounds__(kBlock) void reduce_partials_kernel(const float* __restrict__ partial,
-                                                                 TOut* __restrict__ out,
-                                                                 ColsArgs<I> a, Epi epi, F f) {
-  const I step = (I)gridDim.x * kBlock;
-  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < a.outElems; o += step) {
-    float r = f.init();
-    for (I s = 0; s < a.S.d; ++s) r = f.combine(r, partial[s * a.outElems + o]);
-    const I outer = o / a.C, col = o - outer * a.C;
-    I inOff, outOff;
-    a.oa.offsets(outer, inOff, outOff);
-    out[outOff + col * a.outInner] = epi.template finish<TOut>(r);
-  }
-}
-
 template <typename T, typename I, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
     const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
-    float* __restrict__ partV, I* __restrict__ partI, ColsArgs<I> a, OuterArgs<I> oaIdx,
-    I idxInner, I totalBlocks) {
+    float* __restrict__ partV, I* __restrict__ partI, ColsArgs<I> a, OuterArgs<I> oaIdx, I idxInner,
+    I totalBlocks, bool foldPass) {
   using P = Pack<T, VEC>;
   using O = PairOrder<IS_MAX>;
   __shared__ float sv[kBlock * VEC];
   __shared__ I si[kBlock * VEC];
   const uint32_t TX = a.TX, TY = kBlock / TX;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
-    I rest, s, ct;
-    a.S.divmod(b, rest, s);
-    a.colTiles.divmod(rest, rest, ct);
-    I inOff, outOff;
-    a.oa.offsets(rest, inOff, outOff);
-    const I col = (ct * TX + tx) * VEC;
-    float bv[VEC];
-    I bi[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      bv[e] = O::worst();
-      bi[e] = ~(I)0;
-    }
-    if (col < a.C) {
-      const I begin = s * a.chunkR;
-      const I end = min(a.R, begin + a.chunkR);
-      const T* src = in + inOff + col;
-#pragma unroll 4
-      for (I r = begin + ty; r < end; r += TY) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const float x = Cvt<T>::up(v.v[e]);
-          if (O::better(x, r, bv[e], bi[e])) {
-            bv[e] = x;
-            bi[e] = r;
-          }
-        }
-      }
-    }
+  auto fold_rows = [&](const float (&bv)[VEC], const I (&bi)[VEC]) {
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       sv[(ty * TX + tx) * VEC + e] = bv[e];
@@ -368,19 +389,86 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
       }
       __syncthreads();
     }
-    if (ty == 0 && col < a.C) {
-      I unused, idxOff;
-      oaIdx.offsets(rest, unused, idxOff);
+  };
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I group = b, s = 0, rest, ct;
+    if (!foldPass) a.S.divmod(b, group, s);
+    a.colTiles.divmod(group, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    const I at = rest * a.C + col;
+    float bv[VEC];
+    I bi[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float v = sv[tx * VEC + e];
-        const I ix = si[tx * VEC + e];
-        if (a.S.d > 1) {
-          partV[s * a.outElems + rest * a.C + col + e] = v;
-          partI[s * a.outElems + rest * a.C + col + e] = ix;
-        } else {
-          outV[outOff + (col + e) * a.outInner] = Cvt<T>::down(v);
-          outI[idxOff + (col + e) * idxInner] = (long)ix + 1;
+    for (int e = 0; e < VEC; ++e) {
+      bv[e] = O::worst();
+      bi[e] = ~(I)0;
+    }
+    if (foldPass) {
+      if (col < a.C) {
+        for (I sp = ty; sp < a.S.d; sp += TY) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float v = partV[sp * a.outElems + at + e];
+            const I ix = partI[sp * a.outElems + at + e];
+            if (O::better(v, ix, bv[e], bi[e])) {
+              bv[e] = v;
+              bi[e] = ix;
+            }
+          }
+        }
+      }
+    } else if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const T* src = in + inOff + col;
+      constexpr int U = 8;
+      I r = begin + ty;
+      for (; r + (U - 1) * TY < end; r += U * TY) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (r + u * TY) * a.sR));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const float x = Cvt<T>::up(v[u].v[e]);
+            if (O::better(x, r + u * TY, bv[e], bi[e])) {
+              bv[e] = x;
+              bi[e] = r + u * TY;
+            }
+          }
+        }
+      }
+      for (; r < end; r += TY) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const float x = Cvt<T>::up(v.v[e]);
+          if (O::better(x, r, bv[e], bi[e])) {
+            bv[e] = x;
+            bi[e] = r;
+          }
+        }
+      }
+    }
+    fold_rows(bv, bi);
+    if (ty == 0 && col < a.C) {
+      if (foldPass || a.S.d == 1) {
+        I unused, idxOff;
+        oaIdx.offsets(rest, unused, idxOff);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          outV[outOff + (col + e) * a.outInner] = Cvt<T>::down(sv[tx * VEC + e]);
+          outI[idxOff + (col + e) * idxInner] = (long)si[tx * VEC + e] + 1;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          partV[s * a.outElems + at + e] = sv[tx * VEC + e];
+          partI[s * a.outElems + at + e] = si[tx * VEC + e];
         }
       }
     }
@@ -388,29 +476,77 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
   }
 }
 
-template <typename T, typename I, bool IS_MAX>
-__global__ __launch_bounds__(kBlock) void reduce_partials_index_kernel(
-    const float* __restrict__ partV, const I* __restrict__ partI, T* __restrict__ outV,
-    long* __restrict__ outI, ColsArgs<I> a, OuterArgs<I> oaIdx, I idxInner) {
-  using O = PairOrder<IS_MAX>;
-  const I step = (I)gridDim.x * kBlock;
-  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < a.outElems; o += step) {
-    float bv = O::worst();
-    I bi = ~(I)0;
-    for (I s = 0; s < a.S.d; ++s) {
-      const float v = partV[s * a.outElems + o];
-      const I ix = partI[s * a.outElems + o];
-      if (O::better(v, ix, bv, bi)) {
-        bv = v;
-        bi = ix;
+// ------------------------------------------------------------------- all --
+// Whole-tensor reduction of a dense run: every workgroup streams a contiguous
+// chunk, folds it (wave butterfly + LDS) and publishes one partial; a second
+// one-workgroup launch of the same kernel folds the partials in index order.
+// The final scalar goes to `result` (device scratch) and to `hostResult`
+// (pinned, device-mapped host memory, so no separate D2H copy is needed).
+template <typename F>
+__device__ __forceinline__ float block_fold(float r, float* red, F f) {
+  for (uint32_t o = 32; o > 0; o >>= 1) r = f.combine(r, __shfl_xor(r, o, 64));
+  const uint32_t wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = r;
+  __syncthreads();
+  float t = red[0];
+  for (uint32_t w = 1; w < kBlock / 64; ++w) t = f.combine(t, red[w]);
+  return t;
+}
+
+template <typename TIn, typename F, typename I, int VEC, bool FIRST>
+__global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restrict__ in, I n,
+                                                            I chunk, float* __restrict__ partial,
+                                                            float* result, float* hostResult,
+                                                            Epi epi, F f) {
+  using P = Pack<TIn, VEC>;
+  __shared__ float red[kBlock / 64];
+  float acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+  const I nv = n - n % VEC;  // packs cover [0, nv); the last workgroup adds the tail
+  const I begin = (I)blockIdx.x * chunk;
+  const I end = min(nv, begin + chunk);
+  constexpr int U = 8;
+  constexpr I step = (I)kBlock * VEC;
+  if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n) {
+    const float x = Cvt<TIn>::up(in[nv + threadIdx.x]);
+    acc[0] = f.combine(acc[0], FIRST ? f.modify(x) : x);
+  }
+  I i = begin + threadIdx.x * VEC;
+  for (; i + (U - 1) * step < end; i += U * step) {
+    P v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(in + i + u * step));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float x = Cvt<TIn>::up(v[u].v[e]);
+        acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
       }
     }
-    const I outer = o / a.C, col = o - outer * a.C;
-    I inOff, outOff, unused, idxOff;
-    a.oa.offsets(outer, inOff, outOff);
-    oaIdx.offsets(outer, unused, idxOff);
-    outV[outOff + col * a.outInner] = Cvt<T>::down(bv);
-    outI[idxOff + col * idxInner] = (long)bi + 1;
+  }
+  for (; i < end; i += step) {
+    const P v = load_pack<true>(reinterpret_cast<const P*>(in + i));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float x = Cvt<TIn>::up(v.v[e]);
+      acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+    }
+  }
+  float r = acc[0];
+#pragma unroll
+  for (int e = 1; e < VEC; ++e) r = f.combine(r, acc[e]);
+  r = block_fold(r, red, f);
+  if (threadIdx.x == 0) {
+    if (gridDim.x == 1) {
+      const float fin = epi.template finish<float>(r);
+      *result = fin;
+      *hostResult = fin;
+    } else {
+      partial[blockIdx.x] = r;
+    }
   }
 }
 
@@ -526,7 +662,7 @@ void launch_rows_pass(THCState* s, const TIn* in, TOut* out, float* partial, con
   constexpr int VEC = 16 / sizeof(TIn);
   const int pack = vec ? VEC : 1;
   const int64_t span = std::min(R, chunk);
-  const int64_t perLane = tuning("reduce.rows.packs_per_lane", 4);
+  const int64_t perLane = tuning("reduce.rows.packs_per_lane", 8);
   uint32_t G = pow2_ceil((uint64_t)((span + pack * perLane - 1) / (pack * perLane)));
   G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
   const int64_t groups = kBlock / G;
@@ -646,17 +782,18 @@ void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F 
   const bool split = p.a.S.d > 1;
   float* scratch = split ? (float*)scratch_space(s, nullptr) : nullptr;
   const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+  const int64_t groups = p.totalBlocks / (int64_t)p.a.S.d;
   hipStream_t st = current_stream(s);
-  if (p.vec)
-    hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, VEC>), dim3(grid), dim3(kBlock), 0, st, in,
-                       out, scratch, p.a, (I)p.totalBlocks, epi, f);
-  else
-    hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, 1>), dim3(grid), dim3(kBlock), 0, st, in, out,
-                       scratch, p.a, (I)p.totalBlocks, epi, f);
-  if (split) {
-    const int g2 = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.partials.blocks_per_cu", 8);
-    hipLaunchKernelGGL((reduce_partials_kernel<T, F, I>), dim3(g2), dim3(kBlock), 0, st, scratch, out,
-                       p.a, epi, f);
+  for (int pass = 0; pass < (split ? 2 : 1); ++pass) {
+    const bool fold = pass == 1;
+    const int gr = fold ? (int)groups : grid;
+    const I tb = fold ? (I)groups : (I)p.totalBlocks;
+    if (p.vec)
+      hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, VEC>), dim3(gr), dim3(kBlock), 0, st, in,
+                         out, scratch, p.a, tb, epi, f, fold);
+    else
+      hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, 1>), dim3(gr), dim3(kBlock), 0, st, in,
+                         out, scratch, p.a, tb, epi, f, fold);
   }
   note_kernel(split ? (p.vec ? "cols-split" : "cols-split-scalar") : (p.vec ? "cols" : "cols-scalar"));
 }
@@ -715,7 +852,7 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
     const int pack = vec ? VEC : 1;
     OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
-    const int64_t perLane = tuning("reduce.rows.packs_per_lane", 4);
+    const int64_t perLane = tuning("reduce.rows.packs_per_lane", 8);
     uint32_t G = pow2_ceil((uint64_t)((g.R + pack * perLane - 1) / (pack * perLane)));
     G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
     const int64_t groups = kBlock / G;
@@ -742,16 +879,17 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
       partV = (float*)(scratch + sizeof(I) * (size_t)p.a.S.d * (size_t)g.outElems);
     }
     const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
-    if (p.vec)
-      hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, VEC, IS_MAX>), dim3(grid), dim3(kBlock), 0,
-                         st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, (I)p.totalBlocks);
-    else
-      hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, 1, IS_MAX>), dim3(grid), dim3(kBlock), 0,
-                         st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, (I)p.totalBlocks);
-    if (split) {
-      const int g2 = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.partials.blocks_per_cu", 8);
-      hipLaunchKernelGGL((reduce_partials_index_kernel<T, I, IS_MAX>), dim3(g2), dim3(kBlock), 0, st,
-                         partV, partI, outV, outI, p.a, oaIdx, idxInner);
+    const int64_t groups = p.totalBlocks / (int64_t)p.a.S.d;
+    for (int pass = 0; pass < (split ? 2 : 1); ++pass) {
+      const bool fold = pass == 1;
+      const int gr = fold ? (int)groups : grid;
+      const I tb = fold ? (I)groups : (I)p.totalBlocks;
+      if (p.vec)
+        hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, VEC, IS_MAX>), dim3(gr), dim3(kBlock), 0,
+                           st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, tb, fold);
+      else
+        hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, 1, IS_MAX>), dim3(gr), dim3(kBlock), 0,
+                           st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, tb, fold);
     }
     note_kernel(split ? "cols-index-split" : "cols-index");
     return;
@@ -841,11 +979,6 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
   }
 }
 
-namespace {
-template <typename F>
-float identity_of(F f) { return f.init(); }
-}  // namespace
-
 bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result) {
   if (in->nDimension > kMaxDims) return false;  // THCReduceAll.cuh:249-251
   float init = 0.f;
@@ -890,10 +1023,9 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
 
   // Stage 1 (only if there are several rows): one fp32 partial per row, held
   // in a temporary; stage 2: fold the dense vector of partials (or the single
-  // row) to one value in scratch-backed two-pass form.
-  size_t scratchBytes = 0;
-  char* scratch = (char*)scratch_space(s, &scratchBytes);
-  float* devOut = (float*)(scratch + scratchBytes - 256);  // last 256 bytes hold the result
+  // row) to one value with the one-launch all-reduce kernel.
+  const StreamScratch& sc = stream_scratch(s);
+  float* devOut = sc.result;
   TensorRef rowPartials(s, nullptr);
   const void* src = tensor_data(in, dt);
   DType srcT = dt;
@@ -957,37 +1089,42 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
     Epi none{(int)Epilogue::None, 0.f};
     auto go = [&](auto idxTag) {
       using I = decltype(idxTag);
-      // float output regardless of the input type
-      const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
-      const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
-      int64_t S = 1, chunk = g.R;
-      if (g.R >= 2 * minChunk) {
-        S = std::min<int64_t>(target, g.R / minChunk);
-        S = std::min<int64_t>(S, (int64_t)((scratchBytes - 256) / sizeof(float)));
-        chunk = (g.R + S - 1) / S;
-        chunk = (chunk + 63) / 64 * 64;
-        S = (g.R + chunk - 1) / chunk;
-      }
-      OuterArgs<I> oa = make_outer<I>(g.in, g.out, 1);
-      float* part = (float*)scratch;
-      auto pass1 = [&](float* outp, float* partp, int64_t S_, int64_t chunk_) {
-        if (srcT == DType::F32) {
-          const bool vec = aligned16(src) && g.R % 4 == 0;
-          launch_rows_pass<float, float, F, I, true>(s, (const float*)src, outp, partp, oa, 1, g.R,
-                                                     S_, chunk_, vec, none, f);
-        } else {
-          const bool vec = aligned16(src) && g.R % 8 == 0;
-          launch_rows_pass<__half, float, F, I, true>(s, (const __half*)src, outp, partp, oa, 1, g.R,
-                                                      S_, chunk_, vec, none, f);
-        }
+      // Workgroups of 256 lanes stream chunks that are multiples of one full
+      // batch (256 lanes x 8 packs); about 8 workgroups per CU.
+      const int64_t pack = srcT == DType::F32 ? 4 : 8;
+      const int64_t batch = (int64_t)kBlock * pack * 8;
+      int64_t blocks = std::min<int64_t>((int64_t)num_compute_units(s) * tuning("reduce.all.blocks_per_cu", 8),
+                                         (g.R + batch - 1) / batch);
+      blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)(sc.partialBytes / sizeof(float))));
+      int64_t chunk = (g.R + blocks - 1) / blocks;
+      chunk = (chunk + batch - 1) / batch * batch;
+      blocks = (g.R + chunk - 1) / chunk;
+      hipStream_t st = current_stream(s);
+      float* part = (float*)sc.partials;
+      auto launch = [&](auto tag, auto vecTag, const void* sp, int64_t n, int64_t ch, int nb,
+                        bool first) {
+        using TI = decltype(tag);
+        constexpr int V = decltype(vecTag)::value;
+        if (first)
+          hipLaunchKernelGGL((reduce_all_kernel<TI, F, I, V, true>), dim3(nb), dim3(kBlock), 0, st,
+                             (const TI*)sp, (I)n, (I)ch, part, devOut, sc.hostResultDev, none, f);
+        else
+          hipLaunchKernelGGL((reduce_all_kernel<TI, F, I, V, false>), dim3(nb), dim3(kBlock), 0, st,
+                             (const TI*)sp, (I)n, (I)ch, part, devOut, sc.hostResultDev, none, f);
       };
-      if (S <= 1) {
-        pass1(devOut, nullptr, 1, g.R);
+      if (srcT == DType::F32) {
+        if (aligned16(src))
+          launch(float{}, std::integral_constant<int, 4>{}, src, g.R, chunk, (int)blocks, true);
+        else
+          launch(float{}, std::integral_constant<int, 1>{}, src, g.R, chunk, (int)blocks, true);
       } else {
-        pass1(nullptr, part, S, chunk);
-        launch_rows_pass<float, float, F, I, false>(s, part, devOut, nullptr, oa, 1, S, 1, S,
-                                                    S % 4 == 0, none, f);
+        if (aligned16(src))
+          launch(__half{}, std::integral_constant<int, 8>{}, src, g.R, chunk, (int)blocks, true);
+        else
+          launch(__half{}, std::integral_constant<int, 1>{}, src, g.R, chunk, (int)blocks, true);
       }
+      if (blocks > 1)  // fold the per-workgroup partials
+        launch(float{}, std::integral_constant<int, 1>{}, part, blocks, blocks, 1, false);
     };
     if (g.wide) go(uint64_t{}); else go(uint32_t{});
   };
@@ -1003,9 +1140,11 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
   }
   note_kernel(rows > 1 ? "all-rows" : "all");
   THC_CHECK(hipGetLastError());
-  // The one place the caller blocks on the device (THCReduceAll.cuh:333-335).
-  THC_CHECK(hipMemcpyAsync(result, devOut, sizeof(float), hipMemcpyDeviceToHost, current_stream(s)));
+  // The one place the caller blocks on the device (THCReduceAll.cuh:333-335):
+  // the kernel has stored the scalar into pinned host memory, so waiting for
+  // the stream is all that is left of the reference's synchronous D2H copy.
   THC_CHECK(hipStreamSynchronize(current_stream(s)));
+  *result = *sc.hostResult;
   return true;
 }
 
