@@ -10,9 +10,9 @@ the other benchmark configurations are measured in the same run and reported
 under "all_configs". Prints ONE JSON line.
 
   value               algorithmic bytes * steps / wall time of the timed region
-  roofline.achieved   algorithmic bytes / mean kernel time, from HIP events
-                      recorded around every launch of the timed region on the
-                      stream the engine launches on
+  roofline.achieved   algorithmic bytes / average launch duration, from two
+                      HIP events that bracket the K launches of the timed
+                      region on the stream the engine launches on
   cpu_baseline        the CPU restatement (oracle/) timed on this box's host
                       cores on the same workload, single thread; the all-core
                       figure is reported beside it
@@ -194,21 +194,33 @@ def build_configs(thc, hip, which, only=None):
 
 
 def time_config(hip, thc, cfg, steps, warmup, stream):
+    """Runs `steps` timed launches. Returns (wall seconds, event ms for the
+    whole region, per-step event ms of a second, separately instrumented
+    pass). The region-level events bracket the K launches on the engine's
+    stream, so event_ms / K is the average launch duration including the gaps
+    between back-to-back launches; the per-step pass gives min/median."""
     for i in range(warmup):
         cfg.run(i)
     hip.sync()
     cfg.kernel = thc.last_kernel()
-    evs = [(hip.event(), hip.event()) for _ in range(steps)]
+    e0, e1 = hip.event(), hip.event()
     hip.sync()
     t0 = time.perf_counter()
+    hip.record(e0, stream)
     for i in range(steps):
-        hip.record(evs[i][0], stream)
         cfg.run(warmup + i)
-        hip.record(evs[i][1], stream)
+    hip.record(e1, stream)
     hip.sync()
     wall = time.perf_counter() - t0
+    region_ms = hip.elapsed_ms(e0, e1)
+    evs = [(hip.event(), hip.event()) for _ in range(steps)]
+    for i in range(steps):
+        hip.record(evs[i][0], stream)
+        cfg.run(warmup + steps + i)
+        hip.record(evs[i][1], stream)
+    hip.sync()
     ms = np.array([hip.elapsed_ms(a, b) for a, b in evs])
-    return wall, ms
+    return wall, region_ms, ms
 
 
 def cpu_baseline(host, nbytes, budget_s=12.0):
@@ -246,6 +258,8 @@ def main():
     ap.add_argument("--configs", default="all", choices=["all", "primary"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated config names to measure")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 1-read-1-write stream of known size (counter calibration)")
     ap.add_argument("--tune", action="append", default=[], help="engine tuning knob key=value")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -262,12 +276,19 @@ def main():
     cfgs, host_c2 = build_configs(thc, hip, args.configs, only)
     if only:
         cfgs = [cfgs[0]] + [c for c in cfgs[1:] if c.name in only]
+    if args.calibrate:
+        # out = src + 0 on 2^26 contiguous fp32: reads 256 MiB, writes 256 MiB.
+        nc = 1 << 26
+        csrc = thc.Tensor.from_numpy(np.ones(nc, np.float32))
+        cdst = thc.Tensor("float").resize((nc,))
+        cfgs.append(Config("CAL-copy", "out = src + 0, 2^26 fp32 contiguous (1 read + 1 write of 256 MiB each)",
+                           8 * nc, nc, 1, lambda i: cdst.add(csrc, 0.0)))
     results = []
     for cfg in cfgs:
         steps = args.steps if cfg.name != "C5" else max(3, args.steps // 5)
-        wall, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
+        wall, region_ms, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
         ok = cfg.check() if cfg.check else None
-        mean_ms = float(ms.mean())
+        mean_ms = region_ms / steps
         results.append({
             "name": cfg.name, "desc": cfg.desc, "kernel": cfg.kernel, "steps": steps,
             "algorithmic_bytes": cfg.nbytes,

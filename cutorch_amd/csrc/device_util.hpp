@@ -36,9 +36,12 @@ struct RawBits<2> {
   typedef uint16_t type;
 };
 
-// Streaming access: every byte of these kernels is touched once, so loads and
-// stores carry the nontemporal hint (global_load/store ... nt). On MI355X this
-// is worth ~10% of achieved HBM bandwidth for 2-read-1-write streams.
+// Streaming access: every byte of these kernels is touched once. Measured on
+// MI355X with a flat 3-read-1-write fp32 stream over 1 GiB: plain loads and
+// stores 5.7 TB/s, nontemporal loads AND stores 6.5 TB/s, nontemporal loads
+// with plain (write-back cached) stores 7.1 TB/s. So inputs are loaded with
+// the nontemporal hint and outputs are stored normally, except where a kernel
+// says otherwise.
 template <bool NT, typename P>
 __device__ __forceinline__ P load_pack(const P* p) {
   if (NT) {

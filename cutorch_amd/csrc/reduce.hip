@@ -314,7 +314,22 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
       // second launch: one workgroup per group (S == 1 in the block index),
       // thread row ty folds planes ty, ty+TY, ...
       if (col < a.C) {
-        for (I sp = ty; sp < a.S.d; sp += TY) {
+        constexpr int UF = 8;  // planes fetched per batch
+        I sp = ty;
+        for (; sp + (UF - 1) * TY < a.S.d; sp += UF * TY) {
+          float v[UF][VEC];
+#pragma unroll
+          for (int u = 0; u < UF; ++u) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u][e] = plane[(sp + u * TY) * a.outElems + e];
+          }
+#pragma unroll
+          for (int u = 0; u < UF; ++u) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], v[u][e]);
+          }
+        }
+        for (; sp < a.S.d; sp += TY) {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], plane[sp * a.outElems + e]);
         }
@@ -746,7 +761,7 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   const int64_t colTiles = (C + (int64_t)TX * pack - 1) / ((int64_t)TX * pack);
   const int64_t outer = g.outElems / C;
   const int64_t base = outer * colTiles;
-  const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 8);
+  const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 1));
   const int64_t minRows = (int64_t)TY * tuning("reduce.cols.min_rows_per_thread", 8);
   int64_t S = 1;
   if (base < target && g.R >= 2 * minRows) {
@@ -1093,7 +1108,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
       // batch (256 lanes x 8 packs); about 8 workgroups per CU.
       const int64_t pack = srcT == DType::F32 ? 4 : 8;
       const int64_t batch = (int64_t)kBlock * pack * 8;
-      int64_t blocks = std::min<int64_t>((int64_t)num_compute_units(s) * tuning("reduce.all.blocks_per_cu", 8),
+      int64_t blocks = std::min<int64_t>((int64_t)num_compute_units(s) * tuning("reduce.all.blocks_per_cu", 2),
                                          (g.R + batch - 1) / batch);
       blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)(sc.partialBytes / sizeof(float))));
       int64_t chunk = (g.R + blocks - 1) / blocks;
