@@ -302,6 +302,12 @@ def main():
             "rotating_sets": cfg.sets, "parity_sample_ok": ok,
         })
     p = results[0]
+    traffic = None   # HBM bytes per launch from the committed rocprofv3 --pmc summary, if any
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            traffic = json.load(f).get(cfgs[0].name, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        pass
     line = {
         "metric": METRIC, "value": p["wall_gbps"], "unit": "GB/s", "n_gpus": 1,
         "steps": p["steps"], "warmup": args.warmup,
@@ -311,7 +317,7 @@ def main():
         "config": {"workload": p["desc"], "elements": cfgs[0].elements, "kernel": p["kernel"],
                    "parity_sample_ok": p["parity_sample_ok"]},
         "roofline": {"bound": "hbm", "achieved": p["gbps_mean"], "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": p["frac_of_peak"], "traffic": None},
+                     "frac": p["frac_of_peak"], "traffic": traffic},
         "all_configs": results,
     }
     if not args.no_cpu:
