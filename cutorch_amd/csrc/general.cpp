@@ -162,7 +162,16 @@ THC_API const char* THCAmd_lastError(void) {
 }
 THC_API void THCAmd_clearLastError(void) { t_last_error.clear(); }
 
-THC_API THCState* THCState_alloc(void) { return new THCState(); }
+THC_API THCState* THCState_alloc(void) {
+  THCState* state = new THCState();
+  state->allocator.malloc = default_malloc;
+  state->allocator.realloc = nullptr;
+  state->allocator.free = default_free;
+  state->allocator.emptyCache = default_empty_cache;
+  state->allocator.cacheInfo = nullptr;
+  state->allocator.state = nullptr;
+  return state;
+}
 
 THC_API void THCState_free(THCState* state) { delete state; }
 
@@ -179,12 +188,6 @@ THC_API void THCudaInit(THCState* state) {
     hipDeviceProp_t prop;
     THC_CHECK(hipGetDeviceProperties(&prop, state->device));
     state->numCUs = prop.multiProcessorCount;
-    state->allocator.malloc = default_malloc;
-    state->allocator.realloc = nullptr;
-    state->allocator.free = default_free;
-    state->allocator.emptyCache = default_empty_cache;
-    state->allocator.cacheInfo = nullptr;
-    state->allocator.state = nullptr;
     // Room for the partial results of a split reduction (a few MiB at the
     // largest shapes); the reference keeps 128 KiB (THCGeneral.c:12-17)
     // because its pass 1 is capped at 1024 partials.

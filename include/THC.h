@@ -238,6 +238,7 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
 /* Pointwise math on the apply engine.                                        */
 /*   tensor (op) scalar : generic/THCTensorMathPairwise.h:5-8                 */
 /*   tensor (op) tensor : generic/THCTensorMathPointwise.h:49-53,66-67        */
+/*   fill / zero        : generic/THCTensorMath.h:5-6                         */
 /* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
 /* ------------------------------------------------------------------------ */
 #define THC_AMD_DECLARE_MATH_API(Tensor, real, accreal)                        \

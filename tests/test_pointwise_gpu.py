@@ -10,7 +10,8 @@ Bar: add/sub/mul/div/cadd/addcmul/addcdiv and the scalar forms are bit-exact
 import numpy as np
 import pytest
 
-from tests.util import assert_bit_equal, contiguous_geometry, fill_storage, random_geometry
+from tests.util import (assert_bit_equal, contiguous_geometry, device_fill_from_block, fill_storage,
+                        random_geometry)
 
 pytestmark = pytest.mark.gpu
 
@@ -258,3 +259,32 @@ def test_large_transposed_roundtrip_property(thc):
     assert thc.last_kernel() == "tiled"
     back = thc.Tensor("float").cmul(out.t(), ones)
     assert_bit_equal(back.numpy(), x)
+
+
+def test_config5_full_size_64bit_index_path(thc):
+    """c = a + b on 2048 x 2048 x 520 fp32 (2.18e9 elements, 26 GB), a being a
+    permute(3,2,1) view of a dense 520 x 2048 x 2048 tensor. The operands repeat
+    a known block, so any element of the result can be predicted on the host:
+    a[i,j,k] = blockA[(k*2048*2048 + j*2048 + i) % L], b[i,j,k] = blockB[(i*2048*520 + j*520 + k) % L].
+    Whole (j,k) planes are checked bit for bit at the first, last and some
+    interior i, which covers offsets on both sides of 2^31 and 2^32."""
+    rng = np.random.default_rng(0xC0FFEE + 5)
+    L = (1 << 22) + 12345                          # block length coprime to the dims
+    ba = rng.standard_normal(L).astype(np.float32)
+    bb = rng.standard_normal(L).astype(np.float32)
+    a = device_fill_from_block(thc, (520, 2048, 2048), ba)
+    b = device_fill_from_block(thc, (2048, 2048, 520), bb)
+    av = a.view_as_strided(0, (2048, 2048, 520), (1, 2048, 2048 * 2048))
+    assert not av.is_contiguous()
+    c = thc.Tensor("float").cadd(av, 1.0, b)
+    assert thc.last_kernel().startswith("tiled") and c.shape == (2048, 2048, 520)
+    j = np.arange(2048, dtype=np.int64)[:, None]
+    k = np.arange(520, dtype=np.int64)[None, :]
+    for i in (0, 1, 63, 64, 1007, 1008, 2016, 2047):
+        want = ba[(k * 2048 * 2048 + j * 2048 + i) % L] + bb[(i * 2048 * 520 + j * 520 + k) % L]
+        assert_bit_equal(c.select(0, i).numpy(), want, "plane i=%d" % i)
+    # a plane across i (fixed j): strided gather on the device side as well
+    i = np.arange(2048, dtype=np.int64)[:, None]
+    for jj in (0, 2047):
+        want = ba[(k * 2048 * 2048 + jj * 2048 + i) % L] + bb[(i * 2048 * 520 + jj * 520 + k) % L]
+        assert_bit_equal(c.select(1, jj).numpy(), want, "plane j=%d" % jj)

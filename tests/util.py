@@ -58,3 +58,21 @@ def rel_err_rows(got, want, scale):
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     return float(np.max(np.abs(got - want) / scale)) if got.size else 0.0
+
+
+def device_fill_from_block(thc, shape, block):
+    """Device tensor of `shape` whose storage repeats the host array `block`
+    (device-to-device copies): sets up multi-GB operands in seconds. The
+    element at storage offset o is block[o % block.size]."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    t = thc.Tensor("float").resize(shape)
+    n = int(np.prod(shape))
+    blk = thc.Tensor.from_numpy(block)
+    base, done = t.data_ptr(), 0
+    while done < n:
+        m = min(block.size, n - done)
+        assert hip.hipMemcpy(base + 4 * done, blk.data_ptr(), 4 * m, 3) == 0
+        done += m
+    return t
