@@ -397,7 +397,6 @@ inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* 
 template <typename T, typename Op>
 void launch_contig(THCState* s, const Plan& pl, Op op) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int U = 4;
   bool vec = true;
   for (int k = 0; k < pl.nops; ++k) vec = vec && aligned16<T>(pl.ptr[k]);
   T* out = (T*)pl.ptr[0];
@@ -409,19 +408,29 @@ void launch_contig(THCState* s, const Plan& pl, Op op) {
   // One pass per workgroup (no persistent loop) measured best on MI355X; the
   // grid-stride loop only engages beyond 2^20 workgroups.
   const int64_t packs = vec ? (int64_t)(n / VEC) + 1 : (int64_t)n;
-  const int64_t blocks = (packs + kBlock * U - 1) / (kBlock * U);
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, tuning("apply.contig.max_grid", 1 << 20)));
   // Streaming hint only when the operands cannot stay cache resident anyway.
   const bool nt = (int64_t)n * (int64_t)sizeof(T) * pl.nops >= tuning("apply.contig.nt_bytes", 8 << 20);
-  if (vec && nt)
-    hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, U, true>), dim3(grid), dim3(kBlock), 0, st,
-                       out, i0, i1, i2, n, op);
-  else if (vec)
-    hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, U, false>), dim3(grid), dim3(kBlock), 0, st,
-                       out, i0, i1, i2, n, op);
+  const int64_t unroll = tuning("apply.contig.unroll", 2);
+  auto launch = [&](auto uTag) {
+    constexpr int UU = decltype(uTag)::value;
+    const int64_t blk = (packs + kBlock * UU - 1) / (kBlock * UU);
+    const int gr = (int)std::max<int64_t>(1, std::min<int64_t>(blk, tuning("apply.contig.max_grid", 1 << 20)));
+    if (vec && nt)
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true>), dim3(gr), dim3(kBlock), 0, st,
+                         out, i0, i1, i2, n, op);
+    else if (vec)
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, false>), dim3(gr), dim3(kBlock), 0, st,
+                         out, i0, i1, i2, n, op);
+    else
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, 1, UU, false>), dim3(gr), dim3(kBlock), 0, st,
+                         out, i0, i1, i2, n, op);
+  };
+  if (unroll >= 4)
+    launch(std::integral_constant<int, 4>{});
+  else if (unroll == 1)
+    launch(std::integral_constant<int, 1>{});
   else
-    hipLaunchKernelGGL((apply_contig_kernel<T, Op, 1, U, false>), dim3(grid), dim3(kBlock), 0, st,
-                       out, i0, i1, i2, n, op);
+    launch(std::integral_constant<int, 2>{});
   note_kernel(vec ? "contig" : "contig-scalar");
 }
 

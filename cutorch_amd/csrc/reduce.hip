@@ -756,12 +756,18 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   bool vec = aligned16(in) && C % VEC == 0 && g.sR % VEC == 0;
   for (int d = 0; d < nd - 1 && vec; ++d) vec = g.in.stride[d] % VEC == 0;
   const int pack = vec ? VEC : 1;
-  const uint32_t TX = std::min<uint32_t>(64, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
-  const uint32_t TY = kBlock / TX;
-  const int64_t colTiles = (C + (int64_t)TX * pack - 1) / ((int64_t)TX * pack);
-  const int64_t outer = g.outElems / C;
-  const int64_t base = outer * colTiles;
   const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 1));
+  const int64_t outer = g.outElems / C;
+  // Lanes along the unit-stride dim: a full wave if the dim is long enough, but
+  // narrower column tiles (down to 256-byte rows) are preferred over splitting
+  // the reduced dim when they already give every CU a workgroup.
+  uint32_t TX = std::min<uint32_t>(64, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
+  const uint32_t minTX = (uint32_t)tuning("reduce.cols.min_tx", 16);
+  auto tiles_for = [&](uint32_t tx) { return (C + (int64_t)tx * pack - 1) / ((int64_t)tx * pack); };
+  while (TX > minTX && outer * tiles_for(TX) < target) TX >>= 1;
+  const uint32_t TY = kBlock / TX;
+  const int64_t colTiles = tiles_for(TX);
+  const int64_t base = outer * colTiles;
   const int64_t minRows = (int64_t)TY * tuning("reduce.cols.min_rows_per_thread", 8);
   int64_t S = 1;
   if (base < target && g.R >= 2 * minRows) {
