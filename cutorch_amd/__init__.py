@@ -150,6 +150,18 @@ def _declare(l):
             f(T + "_" + name, None, P, TP, TP, TP)
         for name in ("addcmul", "addcdiv"):
             f(T + "_" + name, None, P, TP, TP, creal, TP, TP)
+        for name in ("sigmoid", "log", "lgamma", "log1p", "exp", "cos", "acos", "cosh", "sin", "asin",
+                     "sinh", "tan", "atan", "tanh", "sqrt", "rsqrt", "ceil", "floor", "round", "trunc",
+                     "frac", "cinv", "neg", "abs", "sign"):
+            f(T + "_" + name, None, P, TP, TP)
+        f(T + "_clamp", None, P, TP, TP, creal, creal)
+        f(T + "_tpow", None, P, TP, creal, TP)
+        for name in ("pow", "cmaxValue", "cminValue", "fmod", "remainder"):
+            f(T + "_" + name, None, P, TP, TP, creal)
+        for name in ("cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2"):
+            f(T + "_" + name, None, P, TP, TP, TP)
+        f(T + "_lerp", None, P, TP, TP, TP, creal)
+        f(T + "_equal", C.c_int, P, TP, TP)
         f(T + "_fill", None, P, TP, creal)
         f(T + "_zero", None, P, TP)
         for name in ("sum", "prod", "mean"):
@@ -347,6 +359,32 @@ class Tensor(object):
 
     def addcdiv(self, t, v, src1, src2):
         return self._call("addcdiv", self.h, t.h, self._real(v), src1.h, src2.h)
+
+    def unary(self, name, src):          # self = name(src): exp, log, abs, ...
+        return self._call(name, self.h, src.h)
+
+    def clamp(self, src, lo, hi):
+        return self._call("clamp", self.h, src.h, self._real(lo), self._real(hi))
+
+    def pow(self, src, v):
+        return self._call("pow", self.h, src.h, self._real(v))
+
+    def tpow(self, v, src):
+        return self._call("tpow", self.h, self._real(v), src.h)
+
+    def scalar2(self, name, src, v):     # cmaxValue, cminValue, fmod, remainder
+        return self._call(name, self.h, src.h, self._real(v))
+
+    def binary(self, name, src1, src2):  # cpow, cmax, cmin, cfmod, cremainder, atan2
+        return self._call(name, self.h, src1.h, src2.h)
+
+    def lerp(self, a, b, w):
+        return self._call("lerp", self.h, a.h, b.h, self._real(w))
+
+    def equal(self, other):
+        r = self._fn("equal")(self._st, self.h, other.h)
+        _check()
+        return bool(r)
 
     def sum(self, src, dim, keepdim=1):   # dim is 0-based, as at the C level
         return self._call("sum", self.h, src.h, dim, keepdim)

@@ -25,7 +25,7 @@ HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", "apply_plan.hpp", "app
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-unknown-pragmas",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-pragmas", "-Wno-pass-failed",
 ]
 
 

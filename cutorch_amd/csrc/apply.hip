@@ -16,15 +16,15 @@ int point_op_inputs(PointOp op) {
   switch (op) {
     case PointOp::Fill: return 0;
     case PointOp::Copy: case PointOp::AddC: case PointOp::SubC: case PointOp::MulC:
-    case PointOp::DivC: case PointOp::Pow: return 1;
+    case PointOp::DivC: case PointOp::Pow: case PointOp::Math1: return 1;
     case PointOp::Add: case PointOp::Sub: case PointOp::Mul: case PointOp::Div:
-    case PointOp::CAdd: return 2;
+    case PointOp::CAdd: case PointOp::Math2: case PointOp::Lerp: return 2;
     default: return 3;
   }
 }
 
 bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* out, AnyTensor* in0,
-                     AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap) {
+                     AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap, MathFn fn, float value2) {
   AnyTensor* t[kMaxOps] = {out, in0, in1, in2};
   const int nops = point_op_inputs(op) + 1;
   const ptrdiff_t n = tensor_numel(out);
@@ -38,7 +38,7 @@ bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* 
   // into a dense temporary and copied back, last writer wins (:472-489).
   if (!ignoreOverlap && overlapping(tensor_layout(out))) {
     TensorRef tmp(s, tensor_new_with_size(s, out->nDimension, out->size, dt));
-    if (!pointwise_apply(s, dt, op, value, tmp.t, in0, in1, in2, true)) return false;
+    if (!pointwise_apply(s, dt, op, value, tmp.t, in0, in1, in2, true, fn, value2)) return false;
     copy_tensor(s, dt, out, tmp.t, /*ignoreOverlap=*/true);
     return true;
   }
@@ -66,13 +66,13 @@ bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* 
   } else {
     const int g = op_group(op);
     if (dt == DType::F32) {
-      if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, op, value);
-      else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, op, value);
-      else apply_dispatch_group<float, 2>(s, pl, sameShape, op, value);
+      if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, op, value, fn, value2);
+      else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, op, value, fn, value2);
+      else apply_dispatch_group<float, 2>(s, pl, sameShape, op, value, fn, value2);
     } else {
-      if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, op, value);
-      else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, op, value);
-      else apply_dispatch_group<__half, 2>(s, pl, sameShape, op, value);
+      if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, op, value, fn, value2);
+      else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, op, value, fn, value2);
+      else apply_dispatch_group<__half, 2>(s, pl, sameShape, op, value, fn, value2);
     }
   }
   THC_CHECK(hipGetLastError());

@@ -2,5 +2,6 @@
 #include "apply_impl.hpp"
 
 namespace thc {
-template void apply_dispatch_group<__half, 1>(THCState*, Plan&, bool, PointOp, float);
+template void apply_dispatch_group<__half, 1>(THCState*, Plan&, bool, PointOp, float, MathFn,
+                                             float);
 }

@@ -75,7 +75,83 @@ THC_ARITH_OP(OpDiv, 2, a / b)
 THC_ARITH_OP(OpCAdd, 2, a + v * b)
 THC_ARITH_OP(OpAddCMul, 3, a + v * (b * c))
 THC_ARITH_OP(OpAddCDiv, 3, a + v * (b / c))
+THC_ARITH_OP(OpLerp, 2, a + v * (b - a))
 #undef THC_ARITH_OP
+
+__device__ __forceinline__ float math1(int fn, float x, float v, float w) {
+  switch (fn) {
+    case (int)MathFn::Sigmoid: return 1.0f / (1.0f + expf(-x));
+    case (int)MathFn::Log: return logf(x);
+    case (int)MathFn::Lgamma: return lgammaf(x);
+    case (int)MathFn::Log1p: return log1pf(x);
+    case (int)MathFn::Exp: return expf(x);
+    case (int)MathFn::Cos: return cosf(x);
+    case (int)MathFn::Acos: return acosf(x);
+    case (int)MathFn::Cosh: return coshf(x);
+    case (int)MathFn::Sin: return sinf(x);
+    case (int)MathFn::Asin: return asinf(x);
+    case (int)MathFn::Sinh: return sinhf(x);
+    case (int)MathFn::Tan: return tanf(x);
+    case (int)MathFn::Atan: return atanf(x);
+    case (int)MathFn::Tanh: return tanhf(x);
+    case (int)MathFn::Sqrt: return sqrtf(x);
+    case (int)MathFn::Rsqrt: return 1.0f / sqrtf(x);
+    case (int)MathFn::Ceil: return ceilf(x);
+    case (int)MathFn::Floor: return floorf(x);
+    case (int)MathFn::Round: return roundf(x);
+    case (int)MathFn::Trunc: return truncf(x);
+    case (int)MathFn::Frac: return x - truncf(x);
+    case (int)MathFn::Cinv: return 1.0f / x;
+    case (int)MathFn::Neg: return -x;
+    case (int)MathFn::Abs: return fabsf(x);
+    case (int)MathFn::Sign: return (float)((x > 0.f) - (x < 0.f));
+    case (int)MathFn::Clamp: return x < v ? v : (x > w ? w : x);
+    case (int)MathFn::PowScalar:
+      if (v == 1.f) return x;
+      if (v == 2.f) return x * x;
+      if (v == 3.f) return x * x * x;
+      if (v == -1.f) return 1.0f / x;
+      if (v == -2.f) return 1.0f / (x * x);
+      return powf(x, v);
+    case (int)MathFn::TPow: return powf(v, x);
+    case (int)MathFn::MaxValue: return x > v ? x : v;
+    case (int)MathFn::MinValue: return x < v ? x : v;
+    case (int)MathFn::FmodValue: return fmodf(x, v);
+    case (int)MathFn::RemainderValue: return v == 0.f ? NAN : x - v * floorf(x / v);
+    default: return x;
+  }
+}
+
+__device__ __forceinline__ float math2(int fn, float a, float b) {
+  switch (fn) {
+    case (int)MathFn::CPow: return powf(a, b);
+    case (int)MathFn::CMax: return a > b ? a : b;
+    case (int)MathFn::CMin: return a < b ? a : b;
+    case (int)MathFn::CFmod: return fmodf(a, b);
+    case (int)MathFn::CRemainder: return b == 0.f ? NAN : a - b * floorf(a / b);
+    case (int)MathFn::Atan2: return atan2f(a, b);
+    case (int)MathFn::Equal: return a == b ? 1.f : 0.f;
+    default: return a;
+  }
+}
+
+struct OpMath1 {
+  static constexpr int NIN = 1;
+  float v, w;
+  int fn;
+  template <typename T>
+  __device__ __forceinline__ T operator()(T a, T, T) const {
+    return Cvt<T>::down(math1(fn, Cvt<T>::up(a), v, w));
+  }
+};
+struct OpMath2 {
+  static constexpr int NIN = 2;
+  int fn;
+  template <typename T>
+  __device__ __forceinline__ T operator()(T a, T b, T) const {
+    return Cvt<T>::down(math2(fn, Cvt<T>::up(a), Cvt<T>::up(b)));
+  }
+};
 
 
 // ------------------------------------------------------------------------
@@ -658,7 +734,16 @@ void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
 
 // Operator groups: one translation unit per (element type, group).
 template <typename T, int GROUP>
-void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v) {
+void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
+                          float w) {
+  if (op == PointOp::Math1) {
+    if constexpr (GROUP == 0) run_plan<T>(s, pl, sameShape, OpMath1{v, w, (int)fn});
+    return;
+  }
+  if (op == PointOp::Math2) {
+    if constexpr (GROUP == 1) run_plan<T>(s, pl, sameShape, OpMath2{(int)fn});
+    return;
+  }
   switch (op) {
 #define THC_CASE(G, NAME)                                         \
   case PointOp::NAME:                                             \
@@ -667,6 +752,7 @@ void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, flo
     THC_CASE(0, Fill) THC_CASE(0, AddC) THC_CASE(0, SubC) THC_CASE(0, MulC) THC_CASE(0, DivC)
     THC_CASE(0, Pow)
     THC_CASE(1, Add) THC_CASE(1, Sub) THC_CASE(1, Mul) THC_CASE(1, Div) THC_CASE(1, CAdd)
+    THC_CASE(1, Lerp)
     THC_CASE(2, AddCMul) THC_CASE(2, AddCDiv)
 #undef THC_CASE
     default: raise_error("pointwise op not available for this element type");

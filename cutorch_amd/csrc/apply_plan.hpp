@@ -21,7 +21,8 @@ inline int op_group(PointOp op) {
 
 // Defined (explicitly instantiated) in the slices.
 template <typename T, int GROUP>
-void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v);
+void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
+                          float w);
 template <typename T>
 void apply_copy(THCState* s, Plan& pl, bool sameShape);
 

@@ -191,13 +191,31 @@ enum class PointOp : int {
   AddCDiv,  // out = in0 + v * (in1 / in2)
   Fill,     // out = v (no input)
   Pow,      // out = powf(in0, v)
+  Math1,    // out = f(in0 [, v, w]) with f chosen by a MathFn code
+  Math2,    // out = f(in0, in1) with f chosen by a MathFn code
+  Lerp,     // out = in0 + v * (in1 - in0)
+};
+
+// Function codes of the code-dispatched functors (one kernel set serves the
+// whole family; the switch is uniform and the kernels are memory-bound).
+enum class MathFn : int {
+  // unary (generic/THCTensorMathPointwise.cu:38-70,76-135)
+  Sigmoid, Log, Lgamma, Log1p, Exp, Cos, Acos, Cosh, Sin, Asin, Sinh, Tan, Atan, Tanh, Sqrt, Rsqrt,
+  Ceil, Floor, Round, Trunc, Frac, Cinv, Neg, Abs, Sign,
+  Clamp,      // v = min, w = max
+  PowScalar,  // x ^ v with the reference's special cases 1, 2, 3, -1, -2
+  TPow,       // v ^ x
+  MaxValue, MinValue, FmodValue, RemainderValue,   // x (op) v
+  // binary (generic/THCTensorMathPointwise.cu:345-560)
+  CPow, CMax, CMin, CFmod, CRemainder, Atan2, Equal
 };
 int point_op_inputs(PointOp op);
 
 // Returns false for the conditions on which the reference's engine returns
 // false (element-count mismatch, too many dims).
 bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* out,
-                     AnyTensor* in0, AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap = false);
+                     AnyTensor* in0, AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap = false,
+                     MathFn fn = MathFn::Abs, float value2 = 0.f);
 void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ignoreOverlap);
 void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src);
 

@@ -4,6 +4,9 @@
 //   generic/THCTensorMathPairwise.cu:5-81     add sub mul div (tensor, scalar)
 //   generic/THCTensorMathPointwise.cu:264-414 cadd csub cmul cdiv
 //   generic/THCTensorMathPointwise.cu:582-630 addcmul addcdiv
+//   generic/THCTensorMathPointwise.cu:5-255   unary math, sign, clamp, sigmoid, pow, tpow, lerp
+//   generic/THCTensorMathPointwise.cu:345-580 cpow cmax cmin cfmod cremainder cmaxValue cminValue
+//   generic/THCTensorMathPairwise.cu:116-258  fmod remainder equal
 //   generic/THCTensorMath.cu:5-36             fill zero
 //   generic/THCTensorMathReduce.cu:5-43       sum prod mean
 //   generic/THCTensorMathReduce.cu:160-232    norm normall
@@ -69,6 +72,40 @@ void ternary_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, Any
     THC_ARG_CHECK(tensor_numel(self) == tensor_numel(src1), 1, "sizes do not match");
   THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), 3, "sizes do not match");
   apply_or_throw(s, dt, op, v, self, t, src1, src2);
+}
+
+// self = f(src) for the code-dispatched unary family (in place when self == src)
+void unary_math(THCState* s, DType dt, MathFn fn, AnyTensor* self, AnyTensor* src, float v = 0.f,
+                float w = 0.f) {
+  same_gpu(s, {self, src});
+  if (self != src) tensor_resize_as(s, self, src, dt);
+  if (!pointwise_apply(s, dt, PointOp::Math1, v, self, src, nullptr, nullptr, false, fn, w))
+    raise_arg_error(2, "%s", kDimWarning);
+}
+
+// self = f(src1, src2)
+void binary_math(THCState* s, DType dt, MathFn fn, AnyTensor* self, AnyTensor* src1, AnyTensor* src2,
+                 int sizeArg) {
+  same_gpu(s, {self, src1, src2});
+  THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), sizeArg, "sizes do not match");
+  if (self != src1) tensor_resize_as(s, self, src1, dt);
+  if (!pointwise_apply(s, dt, PointOp::Math2, 0.f, self, src1, src2, nullptr, false, fn))
+    raise_arg_error(2, "%s", kDimWarning);
+}
+
+// generic/THCTensorMathPairwise.cu:235-258: same sizes and all elements equal
+int tensors_equal(THCState* s, DType dt, AnyTensor* a, AnyTensor* b) {
+  same_gpu(s, {a, b});
+  if (a->nDimension != b->nDimension) return 0;
+  for (int d = 0; d < a->nDimension; ++d)
+    if (a->size[d] != b->size[d]) return 0;
+  if (a->nDimension == 0) return 1;
+  TensorRef flags(s, tensor_new_with_size(s, a->nDimension, a->size, dt));
+  if (!pointwise_apply(s, dt, PointOp::Math2, 0.f, flags.t, a, b, nullptr, false, MathFn::Equal))
+    raise_arg_error(2, "%s", kDimWarning);
+  float r = 0.f;
+  if (!reduce_all(s, dt, ReduceOp::Min, 0.f, flags.t, &r)) raise_arg_error(1, "%s", kDimWarning);
+  return r != 0.f;
 }
 
 void reduce_or_throw(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* self,
@@ -158,6 +195,126 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
                                 Tensor* src2) {                                                    \
     THC_GUARD_VOID(ternary_op(s, DT, PointOp::AddCDiv, to_float(v), TN(self), TN(t), TN(src1),     \
                               TN(src2)))                                                           \
+  }                                                                                                \
+  THC_API void Tensor##_sigmoid(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Sigmoid, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_log(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Log, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_lgamma(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Lgamma, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_log1p(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Log1p, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_exp(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Exp, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_cos(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Cos, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_acos(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Acos, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_cosh(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Cosh, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_sin(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Sin, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_asin(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Asin, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_sinh(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Sinh, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_tan(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Tan, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_atan(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Atan, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_tanh(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Tanh, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_sqrt(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Sqrt, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_rsqrt(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Rsqrt, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_ceil(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Ceil, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_floor(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Floor, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_round(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Round, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_trunc(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Trunc, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_frac(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Frac, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_cinv(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Cinv, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_neg(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Neg, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_abs(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Abs, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_sign(THCState* s, Tensor* self, Tensor* src) {                              \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Sign, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_clamp(THCState* s, Tensor* self, Tensor* src, real lo, real hi) {          \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::Clamp, TN(self), TN(src), to_float(lo), to_float(hi))) \
+  }                                                                                                \
+  THC_API void Tensor##_pow(THCState* s, Tensor* self, Tensor* src, real v) {                      \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::PowScalar, TN(self), TN(src), to_float(v)))           \
+  }                                                                                                \
+  THC_API void Tensor##_tpow(THCState* s, Tensor* self, real v, Tensor* src) {                     \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::TPow, TN(self), TN(src), to_float(v)))                \
+  }                                                                                                \
+  THC_API void Tensor##_cmaxValue(THCState* s, Tensor* self, Tensor* src, real v) {                \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::MaxValue, TN(self), TN(src), to_float(v)))            \
+  }                                                                                                \
+  THC_API void Tensor##_cminValue(THCState* s, Tensor* self, Tensor* src, real v) {                \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::MinValue, TN(self), TN(src), to_float(v)))            \
+  }                                                                                                \
+  THC_API void Tensor##_fmod(THCState* s, Tensor* self, Tensor* src, real v) {                     \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::FmodValue, TN(self), TN(src), to_float(v)))           \
+  }                                                                                                \
+  THC_API void Tensor##_remainder(THCState* s, Tensor* self, Tensor* src, real v) {                \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::RemainderValue, TN(self), TN(src), to_float(v)))      \
+  }                                                                                                \
+  THC_API void Tensor##_cpow(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {              \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CPow, TN(self), TN(src1), TN(src2), 3))              \
+  }                                                                                                \
+  THC_API void Tensor##_cmax(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {              \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CMax, TN(self), TN(src1), TN(src2), 2))              \
+  }                                                                                                \
+  THC_API void Tensor##_cmin(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {              \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CMin, TN(self), TN(src1), TN(src2), 2))              \
+  }                                                                                                \
+  THC_API void Tensor##_cfmod(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {             \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CFmod, TN(self), TN(src1), TN(src2), 2))             \
+  }                                                                                                \
+  THC_API void Tensor##_cremainder(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {        \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CRemainder, TN(self), TN(src1), TN(src2), 2))        \
+  }                                                                                                \
+  THC_API void Tensor##_atan2(THCState* s, Tensor* self, Tensor* tx, Tensor* ty) {                 \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::Atan2, TN(self), TN(tx), TN(ty), 3))                 \
+  }                                                                                                \
+  THC_API void Tensor##_lerp(THCState* s, Tensor* self, Tensor* a, Tensor* b, real w) {            \
+    THC_GUARD_VOID(binary_op(s, DT, PointOp::Lerp, to_float(w), TN(self), TN(a), TN(b)))           \
+  }                                                                                                \
+  THC_API int Tensor##_equal(THCState* s, Tensor* self, Tensor* src) {                             \
+    THC_GUARD_RET(0, return tensors_equal(s, DT, TN(self), TN(src)))                               \
   }                                                                                                \
   THC_API void Tensor##_fill(THCState* s, Tensor* self, real v) {                                  \
     THC_GUARD_VOID(fill_tensor(s, DT, TN(self), to_float(v)))                                      \

@@ -238,6 +238,10 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
 /* Pointwise math on the apply engine.                                        */
 /*   tensor (op) scalar : generic/THCTensorMathPairwise.h:5-8                 */
 /*   tensor (op) tensor : generic/THCTensorMathPointwise.h:49-53,66-67        */
+/*   unary math, clamp, pow, tpow, lerp, atan2 :                              */
+/*                        generic/THCTensorMathPointwise.h:7-38,43-47          */
+/*   cpow cmax cmin cfmod cremainder cmaxValue cminValue : same file :52-63    */
+/*   fmod remainder equal : generic/THCTensorMathPairwise.h:11-12,18           */
 /*   fill / zero        : generic/THCTensorMath.h:5-6                         */
 /* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
 /* ------------------------------------------------------------------------ */
@@ -258,6 +262,57 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
                                 Tensor *src1, Tensor *src2);                   \
   THC_API void Tensor##_addcdiv(THCState *, Tensor *self, Tensor *t, real v,   \
                                 Tensor *src1, Tensor *src2);                   \
+  THC_API void Tensor##_sigmoid(THCState *, Tensor *self, Tensor *src);       \
+  THC_API void Tensor##_log(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_lgamma(THCState *, Tensor *self, Tensor *src);        \
+  THC_API void Tensor##_log1p(THCState *, Tensor *self, Tensor *src);         \
+  THC_API void Tensor##_exp(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_cos(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_acos(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_cosh(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_sin(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_asin(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_sinh(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_tan(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_atan(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_tanh(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_sqrt(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_rsqrt(THCState *, Tensor *self, Tensor *src);         \
+  THC_API void Tensor##_ceil(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_floor(THCState *, Tensor *self, Tensor *src);         \
+  THC_API void Tensor##_round(THCState *, Tensor *self, Tensor *src);         \
+  THC_API void Tensor##_trunc(THCState *, Tensor *self, Tensor *src);         \
+  THC_API void Tensor##_frac(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_cinv(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_neg(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_abs(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_sign(THCState *, Tensor *self, Tensor *src);          \
+  THC_API void Tensor##_clamp(THCState *, Tensor *self, Tensor *src, real lo,  \
+                              real hi);                                        \
+  THC_API void Tensor##_pow(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_tpow(THCState *, Tensor *self, real v, Tensor *src);   \
+  THC_API void Tensor##_cmaxValue(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_cminValue(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_fmod(THCState *, Tensor *self, Tensor *src, real v);   \
+  THC_API void Tensor##_remainder(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_cpow(THCState *, Tensor *self, Tensor *src1,           \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cmax(THCState *, Tensor *self, Tensor *src1,           \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cmin(THCState *, Tensor *self, Tensor *src1,           \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cfmod(THCState *, Tensor *self, Tensor *src1,          \
+                              Tensor *src2);                                   \
+  THC_API void Tensor##_cremainder(THCState *, Tensor *self, Tensor *src1,     \
+                                   Tensor *src2);                              \
+  THC_API void Tensor##_atan2(THCState *, Tensor *self, Tensor *tx,            \
+                              Tensor *ty);                                     \
+  THC_API void Tensor##_lerp(THCState *, Tensor *self, Tensor *a, Tensor *b,   \
+                             real w);                                          \
+  THC_API int Tensor##_equal(THCState *, Tensor *self, Tensor *src);           \
   THC_API void Tensor##_fill(THCState *, Tensor *self, real v);                \
   THC_API void Tensor##_zero(THCState *, Tensor *self);                        \
   THC_API void Tensor##_sum(THCState *, Tensor *self, Tensor *src, long dim,   \

@@ -57,7 +57,23 @@ typedef struct {
 enum {
   TH_OP_COPY = 0, TH_OP_ADDC, TH_OP_SUBC, TH_OP_MULC, TH_OP_DIVC,
   TH_OP_ADD, TH_OP_SUB, TH_OP_MUL, TH_OP_DIV, TH_OP_CADD,
-  TH_OP_ADDCMUL, TH_OP_ADDCDIV, TH_OP_FILL, TH_OP_POW
+  TH_OP_ADDCMUL, TH_OP_ADDCDIV, TH_OP_FILL, TH_OP_POW,
+  TH_OP_LERP,                 /* a + v * (b - a) */
+  TH_OP_MATH1 = 100,          /* TH_OP_MATH1 + fn: out = fn(a; v, w) */
+  TH_OP_MATH2 = 200           /* TH_OP_MATH2 + fn: out = fn(a, b) */
+};
+
+/* Function codes of the unary / binary math family; formulas as in
+ * lib/THC/THCNumerics.cuh:536-579 (float row) and
+ * lib/THC/THCTensorMathPointwise.cuh (sigmoid, sign, clamp, pow special
+ * cases 1, 2, 3, -1, -2, tpow, max/min, fmod/remainder, lerp). */
+enum {
+  TH_FN_SIGMOID = 0, TH_FN_LOG, TH_FN_LGAMMA, TH_FN_LOG1P, TH_FN_EXP, TH_FN_COS, TH_FN_ACOS,
+  TH_FN_COSH, TH_FN_SIN, TH_FN_ASIN, TH_FN_SINH, TH_FN_TAN, TH_FN_ATAN, TH_FN_TANH, TH_FN_SQRT,
+  TH_FN_RSQRT, TH_FN_CEIL, TH_FN_FLOOR, TH_FN_ROUND, TH_FN_TRUNC, TH_FN_FRAC, TH_FN_CINV,
+  TH_FN_NEG, TH_FN_ABS, TH_FN_SIGN, TH_FN_CLAMP, TH_FN_POWSCALAR, TH_FN_TPOW, TH_FN_MAXVALUE,
+  TH_FN_MINVALUE, TH_FN_FMODVALUE, TH_FN_REMAINDERVALUE,
+  TH_FN_CPOW, TH_FN_CMAX, TH_FN_CMIN, TH_FN_CFMOD, TH_FN_CREMAINDER, TH_FN_ATAN2, TH_FN_EQUAL
 };
 
 static int g_threads = 1;
@@ -155,7 +171,69 @@ void th_float2half_array(uint16_t *dst, const float *src, long n) {
 }
 
 /* ------------------------------------------------------------ pointwise -- */
+static float math1(int fn, float x, float v, float w) {
+  switch (fn) {
+    case TH_FN_SIGMOID: return 1.0f / (1.0f + expf(-x));
+    case TH_FN_LOG: return logf(x);
+    case TH_FN_LGAMMA: return lgammaf(x);
+    case TH_FN_LOG1P: return log1pf(x);
+    case TH_FN_EXP: return expf(x);
+    case TH_FN_COS: return cosf(x);
+    case TH_FN_ACOS: return acosf(x);
+    case TH_FN_COSH: return coshf(x);
+    case TH_FN_SIN: return sinf(x);
+    case TH_FN_ASIN: return asinf(x);
+    case TH_FN_SINH: return sinhf(x);
+    case TH_FN_TAN: return tanf(x);
+    case TH_FN_ATAN: return atanf(x);
+    case TH_FN_TANH: return tanhf(x);
+    case TH_FN_SQRT: return sqrtf(x);
+    case TH_FN_RSQRT: { float r = sqrtf(x); return 1.0f / r; }
+    case TH_FN_CEIL: return ceilf(x);
+    case TH_FN_FLOOR: return floorf(x);
+    case TH_FN_ROUND: return roundf(x);
+    case TH_FN_TRUNC: return truncf(x);
+    case TH_FN_FRAC: return x - truncf(x);
+    case TH_FN_CINV: return 1.0f / x;
+    case TH_FN_NEG: return -x;
+    case TH_FN_ABS: return fabsf(x);
+    case TH_FN_SIGN: return (float)((x > 0.f) - (x < 0.f));
+    case TH_FN_CLAMP: return x < v ? v : (x > w ? w : x);
+    case TH_FN_POWSCALAR:
+      if (v == 1.f) return x;
+      if (v == 2.f) return x * x;
+      if (v == 3.f) { float t = x * x; return t * x; }
+      if (v == -1.f) return 1.0f / x;
+      if (v == -2.f) { float t = x * x; return 1.0f / t; }
+      return powf(x, v);
+    case TH_FN_TPOW: return powf(v, x);
+    case TH_FN_MAXVALUE: return x > v ? x : v;
+    case TH_FN_MINVALUE: return x < v ? x : v;
+    case TH_FN_FMODVALUE: return fmodf(x, v);
+    case TH_FN_REMAINDERVALUE: { if (v == 0.f) return NAN; float q = x / v; q = floorf(q); q = v * q; return x - q; }
+  }
+  return x;
+}
+
+static float math2(int fn, float a, float b) {
+  switch (fn) {
+    case TH_FN_CPOW: return powf(a, b);
+    case TH_FN_CMAX: return a > b ? a : b;
+    case TH_FN_CMIN: return a < b ? a : b;
+    case TH_FN_CFMOD: return fmodf(a, b);
+    case TH_FN_CREMAINDER: { if (b == 0.f) return NAN; float q = a / b; q = floorf(q); q = b * q; return a - q; }
+    case TH_FN_ATAN2: return atan2f(a, b);
+    case TH_FN_EQUAL: return a == b ? 1.f : 0.f;
+  }
+  return a;
+}
+
+static float g_w = 0.f; /* second scalar of clamp, set through th_set_second_scalar */
+void th_set_second_scalar(float w) { g_w = w; }
+
 static inline float point_op(int op, float v, float a, float b, float c) {
+  if (op >= TH_OP_MATH2) return math2(op - TH_OP_MATH2, a, b);
+  if (op >= TH_OP_MATH1) return math1(op - TH_OP_MATH1, a, v, g_w);
   switch (op) {
     case TH_OP_COPY: return a;
     case TH_OP_ADDC: return a + v;
@@ -171,11 +249,15 @@ static inline float point_op(int op, float v, float a, float b, float c) {
     case TH_OP_ADDCDIV: { float t = b / c; t = v * t; return a + t; }
     case TH_OP_FILL: return v;
     case TH_OP_POW: return powf(a, v);
+    case TH_OP_LERP: { float t = b - a; t = v * t; return a + t; }
   }
   return 0.f;
 }
 
 static int op_inputs(int op) {
+  if (op >= TH_OP_MATH2) return 2;
+  if (op >= TH_OP_MATH1) return 1;
+  if (op == TH_OP_LERP) return 2;
   if (op == TH_OP_FILL) return 0;
   if (op <= TH_OP_DIVC || op == TH_OP_POW) return 1;
   if (op <= TH_OP_CADD) return 2;

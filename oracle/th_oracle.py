@@ -18,6 +18,13 @@ LIB_PATH = os.path.join(_HERE, "libth_oracle.so")
 
 OPS = {"copy": 0, "addc": 1, "subc": 2, "mulc": 3, "divc": 4, "add": 5, "sub": 6, "mul": 7,
        "div": 8, "cadd": 9, "addcmul": 10, "addcdiv": 11, "fill": 12, "pow": 13}
+FNS = ["sigmoid", "log", "lgamma", "log1p", "exp", "cos", "acos", "cosh", "sin", "asin", "sinh", "tan",
+       "atan", "tanh", "sqrt", "rsqrt", "ceil", "floor", "round", "trunc", "frac", "cinv", "neg", "abs",
+       "sign", "clamp", "pow", "tpow", "cmaxValue", "cminValue", "fmod", "remainder",
+       "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal"]
+OPS["lerp"] = 14
+for _i, _n in enumerate(FNS):
+    OPS["fn:" + _n] = (200 if _i >= FNS.index("cpow") else 100) + _i
 KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "norm": 4, "mean": 5}
 
 
@@ -57,6 +64,7 @@ def lib():
         l.th_half2float_array.argtypes = [C.c_void_p, C.c_void_p, C.c_long]
         l.th_float2half_array.argtypes = [C.c_void_p, C.c_void_p, C.c_long]
         l.th_set_num_threads.argtypes = [C.c_int]
+        l.th_set_second_scalar.argtypes = [C.c_float]
         _lib = l
     return _lib
 
@@ -113,7 +121,10 @@ def _ptr(v):
     return C.byref(v.c) if v is not None else None
 
 
-def pointwise(op, out, a=None, b=None, c=None, value=0.0):
+def pointwise(op, out, a=None, b=None, c=None, value=0.0, value2=0.0):
+    """op: a name from OPS; the math family is spelled "fn:<name>" (e.g.
+    "fn:exp", "fn:clamp" with value = min and value2 = max, "fn:cmax")."""
+    lib().th_set_second_scalar(value2)
     f = lib().th_pointwise_half if out.is_half else lib().th_pointwise_float
     rc = f(OPS[op], value, _ptr(out), _ptr(a), _ptr(b), _ptr(c))
     if rc:
