@@ -70,6 +70,9 @@ def state():
     if _state is None:
         l = lib()
         st = l.THCState_alloc()
+        # as cutorch's init.c:1037-1042: caching allocator unless THC_CACHING_ALLOCATOR=0
+        if os.environ.get("THC_CACHING_ALLOCATOR", "1") != "0":
+            l.THCState_setDeviceAllocator(C.c_void_p(st), l.THCCachingAllocator_get())
         l.THCudaInit(st)
         _check()
         _state = st
@@ -86,6 +89,11 @@ _TYPES = {
 def _declare(l):
     P = C.c_void_p
     l.THCState_alloc.restype = P
+    l.THCCachingAllocator_get.restype = P
+    l.THCState_setDeviceAllocator.argtypes = [P, P]
+    l.THCState_isCachingAllocatorEnabled.argtypes = [P]
+    l.THCudaMemGetInfoCached.argtypes = [P, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t),
+                                         C.POINTER(C.c_size_t)]
     l.THCudaInit.argtypes = [P]
     l.THCudaShutdown.argtypes = [P]
     l.THCState_free.argtypes = [P]
@@ -431,6 +439,15 @@ class Tensor(object):
 
     def maxall(self):
         return self._real_out(self._scalar("maxall"))
+
+
+def cached_memory():
+    """(free incl. parked blocks, total, largest block) from THCudaMemGetInfoCached."""
+    f, t, b = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+    err = lib().THCudaMemGetInfoCached(state(), C.byref(f), C.byref(t), C.byref(b))
+    if err:
+        raise THCError("THCudaMemGetInfoCached failed: %d" % err)
+    return f.value, t.value, b.value
 
 
 def last_kernel():

@@ -3,6 +3,7 @@
 // engines touch on one GPU: the state, the current stream, per-stream scratch
 // (THCGeneral.c:677-712), THCudaMalloc/Free (:842-860) and THCudaCheck
 // (:714-726).
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -17,7 +18,8 @@ struct THCState {
   int numDevices = 0;
   int device = 0;
   int numCUs = 0;
-  THCDeviceAllocator allocator{};
+  THCDeviceAllocator allocator{};            // plain hipMalloc / hipFree
+  THCDeviceAllocator* active = &allocator;    // what storages and scratch use
   std::mutex mu;
   std::map<hipStream_t, thc::StreamScratch> scratch;  // per stream, lazily allocated
   size_t scratchBytes = 0;
@@ -34,11 +36,16 @@ thread_local std::string t_last_error;
 thread_local const char* t_last_kernel = "";
 thread_local hipStream_t t_stream = nullptr;
 int g_force64 = 0;
-std::mutex g_tune_mu;
-std::map<std::string, long>& tune_map() {
-  static std::map<std::string, long> m;
-  return m;
-}
+
+// Tuning knobs: a small append-only table, read without locks on every launch.
+struct Knob {
+  char name[56];
+  std::atomic<long> value;
+};
+constexpr int kMaxKnobs = 64;
+Knob g_knobs[kMaxKnobs];
+std::atomic<int> g_numKnobs{0};
+std::mutex g_tune_mu;  // writers only
 
 std::string vformat(const char* fmt, va_list ap) {
   char buf[2048];
@@ -91,7 +98,7 @@ void hip_check(hipError_t err, const char* file, int line) {
 }
 
 hipStream_t current_stream(THCState*) { return t_stream; }
-THCDeviceAllocator* state_allocator(THCState* s) { return &s->allocator; }
+THCDeviceAllocator* state_allocator(THCState* s) { return s->active; }
 int state_device(THCState* s) { return s->device; }
 
 int num_compute_units(THCState* s) { return s->numCUs > 0 ? s->numCUs : 256; }
@@ -104,7 +111,7 @@ const StreamScratch& stream_scratch(THCState* s) {
   StreamScratch sc{};
   void* p = nullptr;
   THC_CHECK((hipError_t)s->allocator.malloc(s->allocator.state, &p, s->scratchBytes,
-                                            (hipStream_t_)st));
+                                            (hipStream_t_)st));  // scratch stays with hipMalloc
   sc.partials = p;
   sc.partialBytes = s->scratchBytes - kScratchTailBytes;
   sc.counters = reinterpret_cast<unsigned*>(static_cast<char*>(p) + sc.partialBytes);
@@ -139,10 +146,10 @@ void note_kernel(const char* name) { t_last_kernel = name; }
 bool force_64bit_index() { return g_force64 != 0; }
 
 long tuning(const char* key, long fallback) {
-  std::lock_guard<std::mutex> lk(g_tune_mu);
-  auto& m = tune_map();
-  auto it = m.find(key);
-  return it == m.end() ? fallback : it->second;
+  const int n = g_numKnobs.load(std::memory_order_acquire);
+  for (int i = 0; i < n; ++i)
+    if (strcmp(g_knobs[i].name, key) == 0) return g_knobs[i].value.load(std::memory_order_relaxed);
+  return fallback;
 }
 
 }  // namespace thc
@@ -199,6 +206,7 @@ THC_API void THCudaInit(THCState* state) {
 THC_API void THCudaShutdown(THCState* state) {
   THC_GUARD_VOID({
     std::lock_guard<std::mutex> lk(state->mu);
+    if (state->active->emptyCache) state->active->emptyCache(state->active->state);
     for (auto& kv : state->scratch) {
       if (kv.second.partials)
         THC_CHECK((hipError_t)state->allocator.free(state->allocator.state, kv.second.partials));
@@ -223,11 +231,30 @@ THC_API size_t THCState_getCurrentDeviceScratchSpaceSize(THCState* state) {
   return state->scratchBytes - thc::kScratchTailBytes;
 }
 THC_API int THCudaMalloc(THCState* state, void** ptr, size_t size) {
-  return state->allocator.malloc(state->allocator.state, ptr, size,
-                                 (hipStream_t_)current_stream(state));
+  return state->active->malloc(state->active->state, ptr, size,
+                               (hipStream_t_)current_stream(state));
 }
 THC_API int THCudaFree(THCState* state, void* ptr) {
-  return state->allocator.free(state->allocator.state, ptr);
+  return state->active->free(state->active->state, ptr);
+}
+THC_API THCDeviceAllocator* THCState_getDeviceAllocator(THCState* state) { return state->active; }
+THC_API void THCState_setDeviceAllocator(THCState* state, THCDeviceAllocator* allocator) {
+  state->active = allocator ? allocator : &state->allocator;
+}
+THC_API int THCState_isCachingAllocatorEnabled(THCState* state) {
+  return state->active == THCCachingAllocator_get();
+}
+THC_API int THCudaMemGetInfoCached(THCState* state, size_t* freeBytes, size_t* totalBytes,
+                                   size_t* largestBlock) {
+  size_t cached = 0;
+  *largestBlock = 0;
+  hipError_t e = hipMemGetInfo(freeBytes, totalBytes);
+  if (e != hipSuccess) return (int)e;
+  *largestBlock = *freeBytes;  // the driver's free memory is the largest thing one can ask for
+  if (state->active->cacheInfo)
+    state->active->cacheInfo(state->active->state, state->device, &cached, largestBlock);
+  *freeBytes += cached;        // parked blocks are free for the next request
+  return 0;
 }
 THC_API void __THCudaCheck(int err, const char* file, const int line) {
   THC_GUARD_VOID(hip_check((hipError_t)err, file, line))
@@ -237,7 +264,17 @@ THC_API void THCAmd_setForce64BitIndex(int enable) { g_force64 = enable; }
 THC_API const char* THCAmd_lastKernel(void) { return t_last_kernel; }
 THC_API int THCAmd_setTuning(const char* key, long value) {
   std::lock_guard<std::mutex> lk(g_tune_mu);
-  tune_map()[key] = value;
+  const int n = g_numKnobs.load(std::memory_order_relaxed);
+  for (int i = 0; i < n; ++i) {
+    if (strcmp(g_knobs[i].name, key) == 0) {
+      g_knobs[i].value.store(value, std::memory_order_relaxed);
+      return 1;
+    }
+  }
+  if (n == kMaxKnobs || strlen(key) >= sizeof(g_knobs[0].name)) return 0;
+  strcpy(g_knobs[n].name, key);
+  g_knobs[n].value.store(value, std::memory_order_relaxed);
+  g_numKnobs.store(n + 1, std::memory_order_release);
   return 1;
 }
 THC_API long THCAmd_getTuning(const char* key) { return tuning(key, -1); }

@@ -66,6 +66,19 @@ THC_API int THCudaMalloc(THCState *state, void **ptr, size_t size);    /* :213 *
 THC_API int THCudaFree(THCState *state, void *ptr);                    /* :214 */
 THC_API void __THCudaCheck(int err, const char *file, const int line); /* :208 */
 
+/* Allocator selection. THCGeneral.h.in:155-157,215-216; the caching allocator
+ * replaces lib/THC/THCCachingAllocator.h:11. Storages remember the allocator
+ * they came from. cutorch's init.c:1037-1042 installs the caching allocator
+ * unless THC_CACHING_ALLOCATOR=0; a host does the same with
+ * THCState_setDeviceAllocator(state, THCCachingAllocator_get()). */
+struct _THCDeviceAllocator;
+THC_API struct _THCDeviceAllocator *THCState_getDeviceAllocator(THCState *state);
+THC_API void THCState_setDeviceAllocator(THCState *state, struct _THCDeviceAllocator *allocator);
+THC_API int THCState_isCachingAllocatorEnabled(THCState *state);
+THC_API struct _THCDeviceAllocator *THCCachingAllocator_get(void);
+THC_API int THCudaMemGetInfoCached(THCState *state, size_t *freeBytes, size_t *totalBytes,
+                                   size_t *largestBlock);
+
 /* Diagnostics with no counterpart in the reference. */
 THC_API int THCAmd_getNumComputeUnits(THCState *state);
 /* Force the 64-bit index kernels even when 32 bits would do (tests). */
@@ -73,7 +86,7 @@ THC_API void THCAmd_setForce64BitIndex(int enable);
 /* Kernel family chosen by the last apply / reduce call on this thread
  * ("contig", "strided", "tiled", "generic", "rows", "cols", ...). */
 THC_API const char *THCAmd_lastKernel(void);
-/* Launch-shape tuning knobs, by name; returns 0 if the key is unknown. */
+/* Launch-shape tuning knobs, by name; returns 0 if the knob table is full. */
 THC_API int THCAmd_setTuning(const char *key, long value);
 THC_API long THCAmd_getTuning(const char *key);
 
