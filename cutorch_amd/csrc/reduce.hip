@@ -83,6 +83,12 @@ struct PairOrder {
     if (an || bn) return an && (!bn || ai < bi);
     return (IS_MAX ? av > bv : av < bv) || (av == bv && ai < bi);
   }
+  // Same decision when `a` is known to come after `b` in index order (a lane
+  // scanning its elements front to back): ties never replace, a NaN replaces
+  // only a non-NaN.
+  static __device__ __forceinline__ bool better_later(float av, float bv) {
+    return (IS_MAX ? av > bv : av < bv) || ((av != av) && (bv == bv));
+  }
 };
 
 // Coordinates of an output element / a row in the joint (input, output)
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             const float x = Cvt<T>::up(v[u].v[e]);
-            if (O::better(x, i + u * step + e, bv, bi)) {
+            if (O::better_later(x, bv)) {
               bv = x;
               bi = i + u * step + e;
             }
@@ -224,7 +230,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<T>::up(v.v[e]);
-          if (O::better(x, i + e, bv, bi)) {
+          if (O::better_later(x, bv)) {
             bv = x;
             bi = i + e;
           }
@@ -247,6 +253,9 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
       }
     }
     if (active && lane == 0) {
+      // No element beat the start value: the whole row equals it (all -inf for
+      // max, all +inf for min), and the first occurrence is element 0.
+      if (bi == ~(I)0) bi = 0;
       outV[outOff] = Cvt<T>::down(bv);
       outI[idxOff] = (long)bi + 1;  // 1-based (TH_INDEX_BASE)
     }
@@ -450,7 +459,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             const float x = Cvt<T>::up(v[u].v[e]);
-            if (O::better(x, r + u * TY, bv[e], bi[e])) {
+            if (O::better_later(x, bv[e])) {
               bv[e] = x;
               bi[e] = r + u * TY;
             }
@@ -462,7 +471,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<T>::up(v.v[e]);
-          if (O::better(x, r, bv[e], bi[e])) {
+          if (O::better_later(x, bv[e])) {
             bv[e] = x;
             bi[e] = r;
           }
@@ -476,8 +485,9 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
         oaIdx.offsets(rest, unused, idxOff);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
+          const I ix = si[tx * VEC + e] == ~(I)0 ? 0 : si[tx * VEC + e];  // column of start values
           outV[outOff + (col + e) * a.outInner] = Cvt<T>::down(sv[tx * VEC + e]);
-          outI[idxOff + (col + e) * idxInner] = (long)si[tx * VEC + e] + 1;
+          outI[idxOff + (col + e) * idxInner] = (long)ix + 1;
         }
       } else {
 #pragma unroll
