@@ -179,6 +179,11 @@ def _declare(l):
             f(T + "_" + name, None, P, TP, LT, TP, C.c_long, C.c_int)
         for name in ("sumall", "prodall", "meanall"):
             f(T + "_" + name, C.c_float, P, TP)
+        for name in ("var", "std"):
+            f(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int, C.c_int)
+        for name in ("varall", "stdall"):
+            f(T + "_" + name, C.c_float, P, TP, C.c_int)
+        f(T + "_dist", C.c_float, P, TP, TP, creal)
         f(T + "_normall", C.c_float, P, TP, creal)
         for name in ("minall", "maxall"):
             f(T + "_" + name, creal, P, TP)
@@ -405,6 +410,23 @@ class Tensor(object):
 
     def norm(self, src, p, dim, keepdim=1):
         return self._call("norm", self.h, src.h, self._real(p), dim, keepdim)
+
+    def var(self, src, dim, biased=0, keepdim=1):
+        return self._call("var", self.h, src.h, dim, biased, keepdim)
+
+    def std(self, src, dim, biased=0, keepdim=1):
+        return self._call("std", self.h, src.h, dim, biased, keepdim)
+
+    def varall(self, biased=0):
+        return self._scalar("varall", biased)
+
+    def stdall(self, biased=0):
+        return self._scalar("stdall", biased)
+
+    def dist(self, other, p):
+        r = self._fn("dist")(self._st, self.h, other.h, self._real(p))
+        _check()
+        return r
 
     def max(self, indices, src, dim, keepdim=1):  # self = values
         return self._call("max", self.h, indices.h, src.h, dim, keepdim)

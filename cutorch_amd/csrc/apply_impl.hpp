@@ -106,6 +106,7 @@ __device__ __forceinline__ float math1(int fn, float x, float v, float w) {
     case (int)MathFn::Abs: return fabsf(x);
     case (int)MathFn::Sign: return (float)((x > 0.f) - (x < 0.f));
     case (int)MathFn::Clamp: return x < v ? v : (x > w ? w : x);
+    case (int)MathFn::SqDiffValue: return (x - v) * (x - v);
     case (int)MathFn::PowScalar:
       if (v == 1.f) return x;
       if (v == 2.f) return x * x;
@@ -131,6 +132,7 @@ __device__ __forceinline__ float math2(int fn, float a, float b) {
     case (int)MathFn::CRemainder: return b == 0.f ? NAN : a - b * floorf(a / b);
     case (int)MathFn::Atan2: return atan2f(a, b);
     case (int)MathFn::Equal: return a == b ? 1.f : 0.f;
+    case (int)MathFn::SqDiff: return (a - b) * (a - b);
     default: return a;
   }
 }

@@ -203,11 +203,13 @@ enum class MathFn : int {
   Sigmoid, Log, Lgamma, Log1p, Exp, Cos, Acos, Cosh, Sin, Asin, Sinh, Tan, Atan, Tanh, Sqrt, Rsqrt,
   Ceil, Floor, Round, Trunc, Frac, Cinv, Neg, Abs, Sign,
   Clamp,      // v = min, w = max
+  SqDiffValue,  // (x - v)^2
   PowScalar,  // x ^ v with the reference's special cases 1, 2, 3, -1, -2
   TPow,       // v ^ x
   MaxValue, MinValue, FmodValue, RemainderValue,   // x (op) v
   // binary (generic/THCTensorMathPointwise.cu:345-560)
-  CPow, CMax, CMin, CFmod, CRemainder, Atan2, Equal
+  CPow, CMax, CMin, CFmod, CRemainder, Atan2, Equal,
+  SqDiff      // (a - b)^2
 };
 int point_op_inputs(PointOp op);
 
@@ -220,8 +222,10 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
 void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src);
 
 // --------------------------------------------------------- reduce engine --
-enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP };
-enum class Epilogue : int { None, Sqrt, PowInv, DivN };
+// SqDev: sum of (x - p)^2 (second pass of varall, generic/THCTensorMathReduce.cu:122-144)
+enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev };
+// DivBy / DivBySqrt take their divisor from the `p` argument of reduce_dim.
+enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 
 // out[..., 0, ...] = reduce over dim (THC_reduceDim, lib/THC/THCReduce.cuh:263-453)
 bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* out,

@@ -10,6 +10,7 @@
 //   generic/THCTensorMath.cu:5-36             fill zero
 //   generic/THCTensorMathReduce.cu:5-43       sum prod mean
 //   generic/THCTensorMathReduce.cu:160-232    norm normall
+//   generic/THCTensorMathReduce.cu:70-144,234-259  var std varall stdall dist
 //   generic/THCTensorMathReduce.cu:261-333    sumall prodall meanall minall maxall
 //   generic/THCTensorMathReduce.cu:400-436    max min
 #include <cfloat>
@@ -139,6 +140,46 @@ float norm_all(THCState* s, DType dt, float p, AnyTensor* self) {
   if (p == 1.f) return all_or_throw(s, dt, ReduceOp::Norm1, p, self);
   if (p == 2.f) return sqrtf(all_or_throw(s, dt, ReduceOp::Norm2, p, self));
   return powf(all_or_throw(s, dt, ReduceOp::NormP, p, self), 1.0f / p);
+}
+
+// var / std along a dim (generic/THCTensorMathReduce.cu:70-120), two-pass for
+// accuracy in fp32: m = mean over dim; t = (src - m)^2 with m broadcast along
+// dim (stride 0); self = sum(t) / (n - !biased) [sqrt for std].
+void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* src, long dim,
+             int biased, int keepdim) {
+  same_gpu(s, {self, src});
+  THC_ARG_CHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
+  const long n = src->size[dim];
+  TensorRef mean(s, tensor_new(s));
+  if (!reduce_dim(s, dt, ReduceOp::Sum, Epilogue::DivN, 0.f, mean.t, src, (int)dim, 1))
+    raise_arg_error(2, "%s", kDimWarning);
+  TensorRef wide(s, tensor_new_with_tensor(s, mean.t, dt));  // mean viewed with src's shape
+  wide.t->size[dim] = n;
+  wide.t->stride[dim] = 0;
+  TensorRef dev(s, tensor_new_with_size(s, src->nDimension, src->size, dt));
+  if (!pointwise_apply(s, dt, PointOp::Math2, 0.f, dev.t, src, wide.t, nullptr, false, MathFn::SqDiff))
+    raise_arg_error(2, "%s", kDimWarning);
+  const float div = (float)(biased ? n : n - 1);
+  if (!reduce_dim(s, dt, ReduceOp::Sum, wantStd ? Epilogue::DivBySqrt : Epilogue::DivBy, div, self,
+                  dev.t, (int)dim, keepdim))
+    raise_arg_error(2, "%s", kDimWarning);
+}
+
+float var_all(THCState* s, DType dt, AnyTensor* self, int biased) {
+  THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");
+  const float n = (float)tensor_numel(self);
+  const float mean = all_or_throw(s, dt, ReduceOp::Sum, 0.f, self) / n;
+  return all_or_throw(s, dt, ReduceOp::SqDev, mean, self) / (n - (biased ? 0.f : 1.f));
+}
+
+// dist(a, b, p) = (sum |a - b|^p)^(1/p)  (generic/THCTensorMathReduce.cu:234-259)
+float dist_all(THCState* s, DType dt, AnyTensor* a, AnyTensor* b, float p) {
+  same_gpu(s, {a, b});
+  THC_ARG_CHECK(tensor_numel(a) == tensor_numel(b), 2, "sizes do not match");
+  if (a->nDimension == 0) return 0.f;
+  TensorRef diff(s, tensor_new_with_size(s, a->nDimension, a->size, dt));
+  apply_or_throw(s, dt, PointOp::Sub, 0.f, diff.t, a, b);
+  return powf(all_or_throw(s, dt, ReduceOp::NormP, p, diff.t), 1.0f / p);
 }
 
 void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
@@ -351,6 +392,23 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
       same_gpu(s, {values, indices, src});                                                         \
       reduce_dim_index(s, DT, false, TN(values), TN(indices), TN(src), (int)dim, keepdim);         \
     })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_var(THCState* s, Tensor* self, Tensor* src, long dim, int biased,          \
+                            int keepdim) {                                                         \
+    THC_GUARD_VOID(var_dim(s, DT, false, TN(self), TN(src), dim, biased, keepdim))                 \
+  }                                                                                                \
+  THC_API void Tensor##_std(THCState* s, Tensor* self, Tensor* src, long dim, int biased,          \
+                            int keepdim) {                                                         \
+    THC_GUARD_VOID(var_dim(s, DT, true, TN(self), TN(src), dim, biased, keepdim))                  \
+  }                                                                                                \
+  THC_API float Tensor##_varall(THCState* s, Tensor* self, int biased) {                           \
+    THC_GUARD_RET(0.f, return var_all(s, DT, TN(self), biased))                                    \
+  }                                                                                                \
+  THC_API float Tensor##_stdall(THCState* s, Tensor* self, int biased) {                           \
+    THC_GUARD_RET(0.f, return sqrtf(var_all(s, DT, TN(self), biased)))                             \
+  }                                                                                                \
+  THC_API float Tensor##_dist(THCState* s, Tensor* self, Tensor* src, real p) {                    \
+    THC_GUARD_RET(0.f, return dist_all(s, DT, TN(self), TN(src), to_float(p)))                     \
   }                                                                                                \
   THC_API float Tensor##_sumall(THCState* s, Tensor* self) {                                       \
     THC_GUARD_RET(0.f, return all_or_throw(s, DT, ReduceOp::Sum, 0.f, TN(self)))                   \

@@ -44,6 +44,8 @@ struct Epi {
       case (int)Epilogue::Sqrt: return Cvt<T>::down(sqrtf(acc));
       case (int)Epilogue::PowInv: return Cvt<T>::down(powf(acc, arg));
       case (int)Epilogue::DivN: return Cvt<T>::down(Cvt<T>::up(Cvt<T>::down(acc)) / arg);
+      case (int)Epilogue::DivBy: return Cvt<T>::down(acc / arg);
+      case (int)Epilogue::DivBySqrt: return Cvt<T>::down(sqrtf(acc / arg));
       default: return Cvt<T>::down(acc);
     }
   }
@@ -71,6 +73,7 @@ THC_REDUCE_FUNCTOR(FNorm0, 0.f, (x != 0.f ? 1.f : 0.f), a + b)
 THC_REDUCE_FUNCTOR(FNorm1, 0.f, fabsf(x), a + b)
 THC_REDUCE_FUNCTOR(FNorm2, 0.f, x * x, a + b)
 THC_REDUCE_FUNCTOR(FNormP, 0.f, powf(fabsf(x), p), a + b)
+THC_REDUCE_FUNCTOR(FSqDev, 0.f, (x - p) * (x - p), a + b)
 #undef THC_REDUCE_FUNCTOR
 
 // (value, index) pairs. `better(a, b)`: a must replace b.
@@ -868,6 +871,7 @@ void dispatch_reduce(THCState* s, const ReduceGeom& g, const void* in, void* out
     case ReduceOp::Norm1: run_dim<T>(s, g, in, out, epi, FNorm1{p}); break;
     case ReduceOp::Norm2: run_dim<T>(s, g, in, out, epi, FNorm2{p}); break;
     case ReduceOp::NormP: run_dim<T>(s, g, in, out, epi, FNormP{p}); break;
+    case ReduceOp::SqDev: run_dim<T>(s, g, in, out, epi, FSqDev{p}); break;
   }
 }
 
@@ -969,6 +973,7 @@ bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTen
   Epi epi{(int)ep, 0.f};
   if (ep == Epilogue::PowInv) epi.arg = 1.0f / p;
   if (ep == Epilogue::DivN) epi.arg = (float)g.R;
+  if (ep == Epilogue::DivBy || ep == Epilogue::DivBySqrt) epi.arg = p;
   const void* ip = tensor_data(in, dt);
   void* opn = tensor_data(out, dt);
   if (dt == DType::F32)
@@ -1102,6 +1107,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
       case ReduceOp::Norm1: stage1(FNorm1{p}); op2 = ReduceOp::Sum; break;
       case ReduceOp::Norm2: stage1(FNorm2{p}); op2 = ReduceOp::Sum; break;
       case ReduceOp::NormP: stage1(FNormP{p}); op2 = ReduceOp::Sum; break;
+      case ReduceOp::SqDev: stage1(FSqDev{p}); op2 = ReduceOp::Sum; break;
     }
     src = rp;
     srcT = DType::F32;
@@ -1168,6 +1174,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
     case ReduceOp::Norm1: stage2(FNorm1{p}); break;
     case ReduceOp::Norm2: stage2(FNorm2{p}); break;
     case ReduceOp::NormP: stage2(FNormP{p}); break;
+    case ReduceOp::SqDev: stage2(FSqDev{p}); break;
   }
   note_kernel(rows > 1 ? "all-rows" : "all");
   THC_CHECK(hipGetLastError());

@@ -342,6 +342,14 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
   THC_API void Tensor##_min(THCState *, Tensor *values,                        \
                             THCudaLongTensor *indices, Tensor *src, long dim,  \
                             int keepdim);                                      \
+  THC_API void Tensor##_var(THCState *, Tensor *self, Tensor *src, long dim,   \
+                            int biased, int keepdim);                          \
+  THC_API void Tensor##_std(THCState *, Tensor *self, Tensor *src, long dim,   \
+                            int biased, int keepdim);                          \
+  THC_API accreal Tensor##_varall(THCState *, Tensor *self, int biased);       \
+  THC_API accreal Tensor##_stdall(THCState *, Tensor *self, int biased);       \
+  THC_API accreal Tensor##_dist(THCState *, Tensor *self, Tensor *src,         \
+                                real p);                                       \
   THC_API accreal Tensor##_sumall(THCState *, Tensor *self);                   \
   THC_API accreal Tensor##_prodall(THCState *, Tensor *self);                  \
   THC_API accreal Tensor##_meanall(THCState *, Tensor *self);                  \

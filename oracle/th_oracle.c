@@ -71,9 +71,10 @@ enum {
   TH_FN_SIGMOID = 0, TH_FN_LOG, TH_FN_LGAMMA, TH_FN_LOG1P, TH_FN_EXP, TH_FN_COS, TH_FN_ACOS,
   TH_FN_COSH, TH_FN_SIN, TH_FN_ASIN, TH_FN_SINH, TH_FN_TAN, TH_FN_ATAN, TH_FN_TANH, TH_FN_SQRT,
   TH_FN_RSQRT, TH_FN_CEIL, TH_FN_FLOOR, TH_FN_ROUND, TH_FN_TRUNC, TH_FN_FRAC, TH_FN_CINV,
-  TH_FN_NEG, TH_FN_ABS, TH_FN_SIGN, TH_FN_CLAMP, TH_FN_POWSCALAR, TH_FN_TPOW, TH_FN_MAXVALUE,
+  TH_FN_NEG, TH_FN_ABS, TH_FN_SIGN, TH_FN_CLAMP, TH_FN_SQDIFFVALUE, TH_FN_POWSCALAR, TH_FN_TPOW, TH_FN_MAXVALUE,
   TH_FN_MINVALUE, TH_FN_FMODVALUE, TH_FN_REMAINDERVALUE,
-  TH_FN_CPOW, TH_FN_CMAX, TH_FN_CMIN, TH_FN_CFMOD, TH_FN_CREMAINDER, TH_FN_ATAN2, TH_FN_EQUAL
+  TH_FN_CPOW, TH_FN_CMAX, TH_FN_CMIN, TH_FN_CFMOD, TH_FN_CREMAINDER, TH_FN_ATAN2, TH_FN_EQUAL,
+  TH_FN_SQDIFF
 };
 
 static int g_threads = 1;
@@ -199,6 +200,7 @@ static float math1(int fn, float x, float v, float w) {
     case TH_FN_ABS: return fabsf(x);
     case TH_FN_SIGN: return (float)((x > 0.f) - (x < 0.f));
     case TH_FN_CLAMP: return x < v ? v : (x > w ? w : x);
+    case TH_FN_SQDIFFVALUE: { float t = x - v; return t * t; }
     case TH_FN_POWSCALAR:
       if (v == 1.f) return x;
       if (v == 2.f) return x * x;
@@ -224,6 +226,7 @@ static float math2(int fn, float a, float b) {
     case TH_FN_CREMAINDER: { if (b == 0.f) return NAN; float q = a / b; q = floorf(q); q = b * q; return a - q; }
     case TH_FN_ATAN2: return atan2f(a, b);
     case TH_FN_EQUAL: return a == b ? 1.f : 0.f;
+    case TH_FN_SQDIFF: { float t = a - b; return t * t; }
   }
   return a;
 }
@@ -330,7 +333,10 @@ int th_pointwise_half(int op, float v, const th_view *out, const th_view *a, con
 }
 
 /* ----------------------------------------------------------- reductions -- */
-enum { TH_R_SUM = 0, TH_R_PROD, TH_R_MIN, TH_R_MAX, TH_R_NORM, TH_R_MEAN };
+/* VAR / STD (+ their unbiased forms) follow TH's one-sweep formula in double:
+ * sum and sum of squares, then E[x^2] - E[x]^2 with the n/(n-1) correction. */
+enum { TH_R_SUM = 0, TH_R_PROD, TH_R_MIN, TH_R_MAX, TH_R_NORM, TH_R_MEAN,
+       TH_R_VAR_BIASED, TH_R_VAR, TH_R_STD_BIASED, TH_R_STD };
 
 static inline float load_elem(const void *base, long off, int is_half) {
   return is_half ? th_half2float(((const uint16_t *)base)[off]) : ((const float *)base)[off];
@@ -350,6 +356,25 @@ static double reduce_slice(int kind, double p, const void *base, long off, long 
       acc = 1;
       for (long i = 0; i < n; ++i) acc *= load_elem(base, off + i * stride, is_half);
       return acc;
+    case TH_R_VAR_BIASED: case TH_R_VAR: case TH_R_STD_BIASED: case TH_R_STD: {
+      double sum = 0, sum2 = 0;
+      for (long i = 0; i < n; ++i) {
+        const double z = load_elem(base, off + i * stride, is_half);
+        sum += z;
+        sum2 += z * z;
+      }
+      const int biased = kind == TH_R_VAR_BIASED || kind == TH_R_STD_BIASED;
+      sum /= (double)n;
+      if (biased) {
+        sum2 /= (double)n;
+        sum2 -= sum * sum;
+      } else {
+        sum2 /= (double)(n - 1);
+        sum2 -= ((double)n) / ((double)(n - 1)) * sum * sum;
+      }
+      if (sum2 < 0) sum2 = 0;
+      return (kind == TH_R_STD_BIASED || kind == TH_R_STD) ? sqrt(sum2) : sum2;
+    }
     case TH_R_NORM:
       acc = 0;
       if (p == 0) {
@@ -527,6 +552,24 @@ static double reduce_all_impl(int kind, double p, const th_view *in, int is_half
   }
   return acc;
 }
+
+/* varall: mean first, then the sum of squared deviations (two sweeps, as
+ * lib/THC/generic/THCTensorMathReduce.cu:122-144), divided by n or n-1. */
+static double var_all_impl(const th_view *in, int biased, int is_half) {
+  const long n = th_numel(in);
+  const double mean = reduce_all_impl(TH_R_SUM, 0, in, is_half) / (double)n;
+  th_odo o;
+  odo_seek(&o, in, 0);
+  double acc = 0;
+  for (long i = 0; i < n; ++i) {
+    const double d = load_elem(in->data, o.off, is_half) - mean;
+    acc += d * d;
+    odo_next(&o, in);
+  }
+  return acc / (double)(n - (biased ? 0 : 1));
+}
+double th_var_all_float(const th_view *in, int biased) { return var_all_impl(in, biased, 0); }
+double th_var_all_half(const th_view *in, int biased) { return var_all_impl(in, biased, 1); }
 
 double th_reduce_all_float(int kind, double p, const th_view *in) {
   return reduce_all_impl(kind, p, in, 0);

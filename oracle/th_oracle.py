@@ -20,12 +20,13 @@ OPS = {"copy": 0, "addc": 1, "subc": 2, "mulc": 3, "divc": 4, "add": 5, "sub": 6
        "div": 8, "cadd": 9, "addcmul": 10, "addcdiv": 11, "fill": 12, "pow": 13}
 FNS = ["sigmoid", "log", "lgamma", "log1p", "exp", "cos", "acos", "cosh", "sin", "asin", "sinh", "tan",
        "atan", "tanh", "sqrt", "rsqrt", "ceil", "floor", "round", "trunc", "frac", "cinv", "neg", "abs",
-       "sign", "clamp", "pow", "tpow", "cmaxValue", "cminValue", "fmod", "remainder",
-       "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal"]
+       "sign", "clamp", "sqdiffValue", "pow", "tpow", "cmaxValue", "cminValue", "fmod", "remainder",
+       "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal", "sqdiff"]
 OPS["lerp"] = 14
 for _i, _n in enumerate(FNS):
     OPS["fn:" + _n] = (200 if _i >= FNS.index("cpow") else 100) + _i
-KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "norm": 4, "mean": 5}
+KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "norm": 4, "mean": 5, "var_biased": 6, "var": 7,
+         "std_biased": 8, "std": 9}
 
 
 class _CView(C.Structure):
@@ -56,6 +57,9 @@ def lib():
                 f.restype = C.c_int
             f = getattr(l, "th_reduce_all_" + suffix)
             f.argtypes = [C.c_int, C.c_double, VP]
+            f.restype = C.c_double
+            f = getattr(l, "th_var_all_" + suffix)
+            f.argtypes = [VP, C.c_int]
             f.restype = C.c_double
         l.th_half2float.argtypes = [C.c_uint16]
         l.th_half2float.restype = C.c_float
@@ -160,6 +164,11 @@ def minmax_dim(which, src, dim, values=None, indices=None):
 def reduce_all(kind, src, p=0.0):
     f = lib().th_reduce_all_half if src.is_half else lib().th_reduce_all_float
     return f(KINDS[kind], p, _ptr(src))
+
+
+def var_all(src, biased=False):
+    f = lib().th_var_all_half if src.is_half else lib().th_var_all_float
+    return f(_ptr(src), 1 if biased else 0)
 
 
 def set_num_threads(n):

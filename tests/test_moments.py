@@ -1,0 +1,76 @@
+"""var / std / varall / stdall / dist (sibling reductions on the reduce engine:
+generic/THCTensorMathReduce.cu:70-144,234-259). The oracle is pinned against
+numpy's float64 var/std (ddof 0 and 1); the HIP path, which centres the data
+first (two sweeps), must agree with it to 1e-5 relative."""
+import numpy as np
+import pytest
+
+from tests.util import contiguous_geometry, fill_storage, random_geometry
+
+
+def _np_view(st, off, size, stride):
+    return np.lib.stride_tricks.as_strided(st[off:], shape=size, strides=tuple(4 * s for s in stride))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_oracle_var_std_match_numpy(oracle, seed):
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(1, 4))
+    shape = tuple(int(x) for x in rng.integers(2, 9, nd))
+    dim = int(rng.integers(0, nd))
+    n, off, size, stride = random_geometry(rng, shape)
+    st = (fill_storage(rng, n) * 3 + 5).astype(np.float32)
+    src = oracle.View(st, off, size, stride)
+    x = _np_view(st, off, size, stride).astype(np.float64)
+    for kind, f, ddof in (("var", np.var, 1), ("var_biased", np.var, 0), ("std", np.std, 1),
+                          ("std_biased", np.std, 0)):
+        got = oracle.reduce_dim(kind, src, dim).numpy()
+        np.testing.assert_allclose(got, f(x, axis=dim, ddof=ddof, keepdims=True), rtol=2e-6)
+    assert abs(oracle.var_all(src) - x.var(ddof=1)) <= 1e-12 * x.var()
+    assert abs(oracle.var_all(src, biased=True) - x.var()) <= 1e-12 * x.var()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_gpu_var_std(thc, oracle, kind):
+    rng = np.random.default_rng(7)
+    tol = 1e-5 if kind == "float" else 2e-3
+    dtype = np.float32 if kind == "float" else np.float16
+    for shape, dim in (((64, 1024), 1), ((300, 7), 1), ((16, 500, 24), 1), ((9, 33), 0), ((5, 6, 7), 2)):
+        geom = contiguous_geometry(shape) if len(shape) == 2 else random_geometry(rng, shape)
+        st = (rng.standard_normal(geom[0]) * 2 + 3).astype(dtype)     # mean 3, sd 2
+        dev = thc.Tensor.from_storage(st, *geom[1:], kind=kind)
+        ref = oracle.View(st.copy(), *geom[1:])
+        for biased in (0, 1):
+            for name in ("var", "std"):
+                out = getattr(thc.Tensor(kind), name)(dev, dim, biased)
+                want = oracle.reduce_dim(name + ("_biased" if biased else ""), ref, dim).numpy()
+                assert out.shape == want.shape
+                np.testing.assert_allclose(out.numpy().astype(np.float64), want.astype(np.float64),
+                                           rtol=tol, err_msg="%s %s dim %d" % (name, shape, dim))
+        out = thc.Tensor(kind).var(dev, dim, 0, 0)
+        assert out.shape == tuple(s for d, s in enumerate(shape) if d != dim)
+
+
+@pytest.mark.gpu
+def test_gpu_varall_stdall_dist(thc, oracle):
+    rng = np.random.default_rng(8)
+    for shape in ((1000,), (257, 129), (1 << 20,)):
+        geom = random_geometry(rng, shape) if len(shape) == 2 else contiguous_geometry(shape)
+        st = (rng.standard_normal(geom[0]) * 2 + 10).astype(np.float32)
+        dev = thc.Tensor.from_storage(st, *geom[1:])
+        ref = oracle.View(st.copy(), *geom[1:])
+        for biased in (0, 1):
+            want = oracle.var_all(ref, bool(biased))
+            assert abs(dev.varall(biased) - want) <= 1e-5 * want
+            assert abs(dev.stdall(biased) - np.sqrt(want)) <= 1e-5 * np.sqrt(want)
+        st2 = rng.standard_normal(geom[0]).astype(np.float32)
+        other = thc.Tensor.from_storage(st2, *geom[1:])
+        x = ref.numpy().astype(np.float64)
+        y = oracle.View(st2.copy(), *geom[1:]).numpy().astype(np.float64)
+        for p in (1.0, 2.0, 3.0):
+            want = (np.abs(x - y) ** p).sum() ** (1 / p)
+            assert abs(dev.dist(other, p) - want) <= 1e-5 * want
+    e = thc.Tensor("float")
+    with pytest.raises(thc.THCError, match="empty Tensor"):
+        e.varall()
