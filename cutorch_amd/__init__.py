@@ -179,6 +179,8 @@ def _declare(l):
             f(T + "_" + name, None, P, TP, LT, TP, C.c_long, C.c_int)
         for name in ("sumall", "prodall", "meanall"):
             f(T + "_" + name, C.c_float, P, TP)
+        for name in ("cumsum", "cumprod"):
+            f(T + "_" + name, None, P, TP, TP, C.c_long)
         for name in ("var", "std"):
             f(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int, C.c_int)
         for name in ("varall", "stdall"):
@@ -410,6 +412,12 @@ class Tensor(object):
 
     def norm(self, src, p, dim, keepdim=1):
         return self._call("norm", self.h, src.h, self._real(p), dim, keepdim)
+
+    def cumsum(self, src, dim):
+        return self._call("cumsum", self.h, src.h, dim)
+
+    def cumprod(self, src, dim):
+        return self._call("cumprod", self.h, src.h, dim)
 
     def var(self, src, dim, biased=0, keepdim=1):
         return self._call("var", self.h, src.h, dim, biased, keepdim)

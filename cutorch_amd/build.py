@@ -18,7 +18,7 @@ BUILD = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libTHC.so")
 SOURCES = ["general.cpp", "tensor.cpp", "math.cpp", "caching_allocator.cpp", "apply.hip", "apply_f32_0.hip", "apply_f32_1.hip",
            "apply_f32_2.hip", "apply_f16_0.hip", "apply_f16_1.hip", "apply_f16_2.hip", "apply_raw.hip",
-           "reduce.hip"]
+           "reduce.hip", "scan.hip"]
 HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", "apply_plan.hpp", "apply_impl.hpp",
            os.path.join("..", "..", "include", "THC.h")]
 

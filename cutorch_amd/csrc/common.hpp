@@ -238,4 +238,8 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
 // (THC_reduceAll, lib/THC/THCReduceAll.cuh:239-342)
 bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result);
 
+// Inclusive prefix sum / product along `dim` (THCTensor_(scanDim),
+// lib/THC/generic/THCTensorMathScan.cu:76-110)
+void scan_dim(THCState* s, DType dt, bool product, AnyTensor* self, AnyTensor* src, int dim);
+
 }  // namespace thc

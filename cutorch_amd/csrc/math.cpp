@@ -13,6 +13,7 @@
 //   generic/THCTensorMathReduce.cu:70-144,234-259  var std varall stdall dist
 //   generic/THCTensorMathReduce.cu:261-333    sumall prodall meanall minall maxall
 //   generic/THCTensorMathReduce.cu:400-436    max min
+//   generic/THCTensorMathScan.cu:76-126       cumsum cumprod
 #include <cfloat>
 #include <cmath>
 
@@ -409,6 +410,18 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
   }                                                                                                \
   THC_API float Tensor##_dist(THCState* s, Tensor* self, Tensor* src, real p) {                    \
     THC_GUARD_RET(0.f, return dist_all(s, DT, TN(self), TN(src), to_float(p)))                     \
+  }                                                                                                \
+  THC_API void Tensor##_cumsum(THCState* s, Tensor* self, Tensor* src, long dim) {                 \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {self, src});                                                                    \
+      scan_dim(s, DT, false, TN(self), TN(src), (int)dim);                                         \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_cumprod(THCState* s, Tensor* self, Tensor* src, long dim) {                \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {self, src});                                                                    \
+      scan_dim(s, DT, true, TN(self), TN(src), (int)dim);                                          \
+    })                                                                                             \
   }                                                                                                \
   THC_API float Tensor##_sumall(THCState* s, Tensor* self) {                                       \
     THC_GUARD_RET(0.f, return all_or_throw(s, DT, ReduceOp::Sum, 0.f, TN(self)))                   \

@@ -257,6 +257,7 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
 /*   fmod remainder equal : generic/THCTensorMathPairwise.h:11-12,18           */
 /*   fill / zero        : generic/THCTensorMath.h:5-6                         */
 /* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
+/* Scans: generic/THCTensorMathScan.h (cumsum, cumprod)                       */
 /* ------------------------------------------------------------------------ */
 #define THC_AMD_DECLARE_MATH_API(Tensor, real, accreal)                        \
   THC_API void Tensor##_add(THCState *, Tensor *self, Tensor *src, real v);    \
@@ -350,6 +351,10 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
   THC_API accreal Tensor##_stdall(THCState *, Tensor *self, int biased);       \
   THC_API accreal Tensor##_dist(THCState *, Tensor *self, Tensor *src,         \
                                 real p);                                       \
+  THC_API void Tensor##_cumsum(THCState *, Tensor *self, Tensor *src,          \
+                               long dim);                                      \
+  THC_API void Tensor##_cumprod(THCState *, Tensor *self, Tensor *src,         \
+                                long dim);                                     \
   THC_API accreal Tensor##_sumall(THCState *, Tensor *self);                   \
   THC_API accreal Tensor##_prodall(THCState *, Tensor *self);                  \
   THC_API accreal Tensor##_meanall(THCState *, Tensor *self);                  \

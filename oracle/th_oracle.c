@@ -441,6 +441,46 @@ int th_reduce_dim_half(int kind, double p, const th_view *out, const th_view *in
   return reduce_dim_impl(kind, p, out, in, dim, 1);
 }
 
+/* Inclusive prefix sum (product = 0) or product (product = 1) along dim with
+ * a sequential double accumulator, rounded per output element (TH's cumsum /
+ * cumprod loops; entry semantics lib/THC/generic/THCTensorMathScan.cu:76-126).
+ * `out` has the shape of `in`. */
+static int scan_dim_impl(int product, const th_view *out, const th_view *in, int dim, int is_half) {
+  if (in->nd == 0) return 0;
+  if (out->nd != in->nd || dim < 0 || dim >= in->nd) return 1;
+  long osz[TH_MAX_DIMS];
+  for (int d = 0; d < in->nd; ++d) {
+    if (out->size[d] != in->size[d]) return 1;
+    osz[d] = d == dim ? 1 : in->size[d];
+  }
+  th_view il = *in, ol = *out;
+  il.size = osz;
+  ol.size = osz;
+  const long lines = th_numel(&il), n = in->size[dim];
+  th_odo oi, oo;
+  odo_seek(&oi, &il, 0);
+  odo_seek(&oo, &ol, 0);
+  for (long l = 0; l < lines; ++l) {
+    double acc = product ? 1.0 : 0.0;
+    for (long i = 0; i < n; ++i) {
+      const double x = load_elem(in->data, oi.off + i * in->stride[dim], is_half);
+      acc = product ? acc * x : acc + x;
+      const long at = oo.off + i * out->stride[dim];
+      if (is_half) ((uint16_t *)out->data)[at] = th_float2half((float)acc);
+      else ((float *)out->data)[at] = (float)acc;
+    }
+    odo_next(&oi, &il);
+    odo_next(&oo, &ol);
+  }
+  return 0;
+}
+int th_scan_dim_float(int product, const th_view *out, const th_view *in, int dim) {
+  return scan_dim_impl(product, out, in, dim, 0);
+}
+int th_scan_dim_half(int product, const th_view *out, const th_view *in, int dim) {
+  return scan_dim_impl(product, out, in, dim, 1);
+}
+
 /* (value, 1-based index) of the max / min along dim; first occurrence wins,
  * the first NaN wins over everything and ends the scan. */
 static int minmax_dim_impl(int is_max, const th_view *val, const th_view *idx, const th_view *in,

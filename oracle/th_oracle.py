@@ -58,6 +58,9 @@ def lib():
             f = getattr(l, "th_reduce_all_" + suffix)
             f.argtypes = [C.c_int, C.c_double, VP]
             f.restype = C.c_double
+            f = getattr(l, "th_scan_dim_" + suffix)
+            f.argtypes = [C.c_int, VP, VP, C.c_int]
+            f.restype = C.c_int
             f = getattr(l, "th_var_all_" + suffix)
             f.argtypes = [VP, C.c_int]
             f.restype = C.c_double
@@ -164,6 +167,15 @@ def minmax_dim(which, src, dim, values=None, indices=None):
 def reduce_all(kind, src, p=0.0):
     f = lib().th_reduce_all_half if src.is_half else lib().th_reduce_all_float
     return f(KINDS[kind], p, _ptr(src))
+
+
+def scan_dim(src, dim, product=False, out=None):
+    if out is None:
+        out = View.empty(src.size, src.storage.dtype)
+    f = lib().th_scan_dim_half if src.is_half else lib().th_scan_dim_float
+    if f(1 if product else 0, _ptr(out), _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return out
 
 
 def var_all(src, biased=False):

@@ -1,0 +1,59 @@
+"""cumsum / cumprod (lib/THC/generic/THCTensorMathScan.cu:76-126). Oracle
+pinned against numpy.cumsum/cumprod in float64 (and bit-exactly on
+integer-valued data); HIP path against the oracle: integer-valued data
+bit-exact, random data within 1e-5 of the running mass."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal, contiguous_geometry, fill_storage, random_geometry
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_oracle_scan_matches_numpy(oracle, seed):
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(1, 4))
+    shape = tuple(int(x) for x in rng.integers(1, 9, nd))
+    dim = int(rng.integers(0, nd))
+    n, off, size, stride = random_geometry(rng, shape)
+    st = fill_storage(rng, n, dist="uniform")
+    src = oracle.View(st, off, size, stride)
+    x = src.numpy().astype(np.float64)
+    np.testing.assert_allclose(oracle.scan_dim(src, dim).numpy(), np.cumsum(x, axis=dim), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oracle.scan_dim(src, dim, product=True).numpy(), np.cumprod(x, axis=dim),
+                               rtol=1e-6, atol=1e-30)
+    xi = rng.integers(-9, 10, shape).astype(np.float32)
+    assert_bit_equal(oracle.scan_dim(oracle.View.of(xi), dim).numpy(), np.cumsum(xi.astype(np.int64), axis=dim).astype(np.float32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_gpu_scan(thc, oracle, kind):
+    rng = np.random.default_rng(17)
+    dtype = np.float32 if kind == "float" else np.float16
+    tol = 1e-5 if kind == "float" else 2e-3
+    for shape, dim in (((7, 1000), 1), ((3, 257), 1), ((300, 5), 1), ((50, 64), 0), ((4, 33, 20), 1),
+                       ((2, 3, 4, 130), 3), ((1,), 0), ((9000,), 0), ((6, 5, 1), 1)):
+        geom = random_geometry(rng, shape) if len(shape) == 3 else contiguous_geometry(shape)
+        st = rng.uniform(-1, 1, geom[0]).astype(dtype)
+        dev = thc.Tensor.from_storage(st, *geom[1:], kind=kind)
+        ref = oracle.View(st.copy(), *geom[1:])
+        got = thc.Tensor(kind).cumsum(dev, dim)
+        assert got.shape == tuple(shape)
+        want = oracle.scan_dim(ref, dim).numpy().astype(np.float64)
+        mass = np.cumsum(np.abs(ref.numpy().astype(np.float64)), axis=dim)
+        err = np.abs(got.numpy().astype(np.float64) - want) / np.maximum(np.abs(want), mass * 2.0 ** -6 + 1e-30)
+        assert err.max() <= tol, (shape, dim, err.max())
+        stp = rng.uniform(0.9, 1.1, geom[0]).astype(dtype)
+        devp = thc.Tensor.from_storage(stp, *geom[1:], kind=kind)
+        gotp = thc.Tensor(kind).cumprod(devp, dim).numpy().astype(np.float64)
+        wantp = oracle.scan_dim(oracle.View(stp.copy(), *geom[1:]), dim, product=True).numpy().astype(np.float64)
+        np.testing.assert_allclose(gotp, wantp, rtol=max(tol, 2e-5) * 4)
+    xi = rng.integers(-9, 10, (37, 700)).astype(np.float32)
+    for dim in (0, 1):
+        got = thc.Tensor("float").cumsum(thc.Tensor.from_numpy(xi), dim)
+        assert_bit_equal(got.numpy(), np.cumsum(xi.astype(np.int64), axis=dim).astype(np.float32))
+    t = thc.Tensor.from_numpy(xi)
+    t.cumsum(t, 1)                                               # in place
+    assert_bit_equal(t.numpy(), np.cumsum(xi.astype(np.int64), axis=1).astype(np.float32))
+    with pytest.raises(thc.THCError, match="out of range"):
+        thc.Tensor("float").cumsum(thc.Tensor.from_numpy(xi), 2)
