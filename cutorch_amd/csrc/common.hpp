@@ -223,7 +223,9 @@ void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor
 
 // --------------------------------------------------------- reduce engine --
 // SqDev: sum of (x - p)^2 (second pass of varall, generic/THCTensorMathReduce.cu:122-144)
-enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev };
+// SqDevOut: sum of (x - c)^2 where c is what the output element holds on entry (the slice's
+//           mean: second sweep of var/std along a dim, THCTensorMathReduce.cuh:268-445)
+enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev, SqDevOut };
 // DivBy / DivBySqrt take their divisor from the `p` argument of reduce_dim.
 enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 

@@ -143,9 +143,9 @@ float norm_all(THCState* s, DType dt, float p, AnyTensor* self) {
   return powf(all_or_throw(s, dt, ReduceOp::NormP, p, self), 1.0f / p);
 }
 
-// var / std along a dim (generic/THCTensorMathReduce.cu:70-120), two-pass for
-// accuracy in fp32: m = mean over dim; t = (src - m)^2 with m broadcast along
-// dim (stride 0); self = sum(t) / (n - !biased) [sqrt for std].
+// var / std along a dim (generic/THCTensorMathReduce.cu:70-120), two sweeps
+// for accuracy in fp32: m = mean over dim; self = sum((src - m)^2) /
+// (n - !biased) [sqrt for std].
 void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* src, long dim,
              int biased, int keepdim) {
   same_gpu(s, {self, src});
@@ -154,16 +154,16 @@ void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* sr
   TensorRef mean(s, tensor_new(s));
   if (!reduce_dim(s, dt, ReduceOp::Sum, Epilogue::DivN, 0.f, mean.t, src, (int)dim, 1))
     raise_arg_error(2, "%s", kDimWarning);
-  TensorRef wide(s, tensor_new_with_tensor(s, mean.t, dt));  // mean viewed with src's shape
-  wide.t->size[dim] = n;
-  wide.t->stride[dim] = 0;
-  TensorRef dev(s, tensor_new_with_size(s, src->nDimension, src->size, dt));
-  if (!pointwise_apply(s, dt, PointOp::Math2, 0.f, dev.t, src, wide.t, nullptr, false, MathFn::SqDiff))
-    raise_arg_error(2, "%s", kDimWarning);
+  // Second sweep: sum of (x - mean)^2 per slice. The kernels take each slice's
+  // centre from the output element itself, so the sweep runs in place on the
+  // tensor of means (no temporary of the input's size, input read twice in all).
   const float div = (float)(biased ? n : n - 1);
-  if (!reduce_dim(s, dt, ReduceOp::Sum, wantStd ? Epilogue::DivBySqrt : Epilogue::DivBy, div, self,
-                  dev.t, (int)dim, keepdim))
+  if (!reduce_dim(s, dt, ReduceOp::SqDevOut, wantStd ? Epilogue::DivBySqrt : Epilogue::DivBy, div,
+                  mean.t, src, (int)dim, 1))
     raise_arg_error(2, "%s", kDimWarning);
+  tensor_resize_as(s, self, mean.t, dt);
+  copy_tensor(s, dt, self, mean.t, false);
+  if (!keepdim) tensor_squeeze1d(s, self, nullptr, (int)dim, dt);
 }
 
 float var_all(THCState* s, DType dt, AnyTensor* self, int biased) {

@@ -58,22 +58,32 @@ __device__ __forceinline__ float nan_min(float a, float b) {
   return (a != a) ? a : ((b != b) ? b : fminf(a, b));
 }
 
-#define THC_REDUCE_FUNCTOR(Name, INIT, MODIFY, COMBINE)                              \
+// modify(x, c): c is the centre of the output element that x belongs to. Only
+// a CENTRED functor looks at it; for those the kernels read c from the output
+// location itself before they overwrite it (the caller stores the centres
+// there), which is how var/std subtract a per-slice mean without an extra
+// operand or a temporary of the input's size.
+#define THC_REDUCE_FUNCTOR(Name, CENTRED, INIT, MODIFY, COMBINE)                     \
   struct Name {                                                                      \
+    static constexpr bool kCentred = CENTRED;                                        \
     float p;                                                                         \
     __host__ __device__ __forceinline__ float init() const { return INIT; }          \
-    __device__ __forceinline__ float modify(float x) const { return MODIFY; }        \
+    __device__ __forceinline__ float modify(float x, float c) const {                \
+      (void)c;                                                                       \
+      return MODIFY;                                                                 \
+    }                                                                                \
     __device__ __forceinline__ float combine(float a, float b) const { return COMBINE; } \
   };
-THC_REDUCE_FUNCTOR(FSum, 0.f, x, a + b)
-THC_REDUCE_FUNCTOR(FProd, 1.f, x, a * b)
-THC_REDUCE_FUNCTOR(FMax, -INFINITY, x, nan_max(a, b))
-THC_REDUCE_FUNCTOR(FMin, INFINITY, x, nan_min(a, b))
-THC_REDUCE_FUNCTOR(FNorm0, 0.f, (x != 0.f ? 1.f : 0.f), a + b)
-THC_REDUCE_FUNCTOR(FNorm1, 0.f, fabsf(x), a + b)
-THC_REDUCE_FUNCTOR(FNorm2, 0.f, x * x, a + b)
-THC_REDUCE_FUNCTOR(FNormP, 0.f, powf(fabsf(x), p), a + b)
-THC_REDUCE_FUNCTOR(FSqDev, 0.f, (x - p) * (x - p), a + b)
+THC_REDUCE_FUNCTOR(FSum, false, 0.f, x, a + b)
+THC_REDUCE_FUNCTOR(FProd, false, 1.f, x, a * b)
+THC_REDUCE_FUNCTOR(FMax, false, -INFINITY, x, nan_max(a, b))
+THC_REDUCE_FUNCTOR(FMin, false, INFINITY, x, nan_min(a, b))
+THC_REDUCE_FUNCTOR(FNorm0, false, 0.f, (x != 0.f ? 1.f : 0.f), a + b)
+THC_REDUCE_FUNCTOR(FNorm1, false, 0.f, fabsf(x), a + b)
+THC_REDUCE_FUNCTOR(FNorm2, false, 0.f, x * x, a + b)
+THC_REDUCE_FUNCTOR(FNormP, false, 0.f, powf(fabsf(x), p), a + b)
+THC_REDUCE_FUNCTOR(FSqDev, false, 0.f, (x - p) * (x - p), a + b)
+THC_REDUCE_FUNCTOR(FSqDevOut, true, 0.f, (x - c) * (x - c), a + b)
 #undef THC_REDUCE_FUNCTOR
 
 // (value, index) pairs. `better(a, b)`: a must replace b.
@@ -125,8 +135,10 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
                                                              TOut* __restrict__ out,
                                                              float* __restrict__ partial,
                                                              OuterArgs<I> oa, I numRows, I R,
-                                                             Divisor<I> S, I chunk, uint32_t G,
-                                                             Epi epi, F f) {
+                                                             I sR, Divisor<I> S, I chunk,
+                                                             uint32_t G, Epi epi, F f) {
+  // sR (element stride of the reduced dim) is honoured by the VEC == 1
+  // instantiation only; packs need sR == 1.
   using P = Pack<TIn, VEC>;
   const uint32_t groups = kBlock / G;
   const uint32_t lane = threadIdx.x % G;
@@ -146,6 +158,9 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
       const I begin = s * chunk;
       const I end = min(R, begin + chunk);
       const TIn* src = in + inOff;
+      float c = 0.f;
+      if constexpr (F::kCentred && FIRST) c = Cvt<TOut>::up(out[outOff]);
+      const I es = VEC == 1 ? sR : (I)1;  // element stride
       // U loads are issued back to back before any of them is consumed.
       constexpr int U = 8;
       const I step = (I)G * VEC;
@@ -153,22 +168,23 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
       for (; i + (U - 1) * step < end; i += U * step) {
         P v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(src + i + u * step));
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             const float x = Cvt<TIn>::up(v[u].v[e]);
-            acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+            acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
           }
         }
       }
       for (; i < end; i += step) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<TIn>::up(v.v[e]);
-          acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+          acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
         }
       }
     }
@@ -185,37 +201,45 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
   }
 }
 
-// max/min with index along a unit-stride dim: one group of G lanes per row.
+// max/min with index: one group of G lanes per row, or per chunk of a row
+// (virtual row vr = row * S + s, as in reduce_rows_kernel) when few long rows
+// must feed the whole chip. S > 1 publishes (value, index) partials with
+// indices relative to the whole row; fold_pairs_kernel finishes. The VEC == 1
+// instantiation honours the element stride sR of the reduced dim.
 template <typename T, typename I, int VEC, bool IS_MAX>
-__global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __restrict__ in,
-                                                                   T* __restrict__ outV,
-                                                                   long* __restrict__ outI,
-                                                                   OuterArgs<I> oa,
-                                                                   OuterArgs<I> oaIdx, I numRows,
-                                                                   I R, uint32_t G) {
+__global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
+    float* __restrict__ partV, I* __restrict__ partI, OuterArgs<I> oa, OuterArgs<I> oaIdx,
+    I numRows, I R, I sR, Divisor<I> S, I chunk, uint32_t G) {
   using P = Pack<T, VEC>;
   using O = PairOrder<IS_MAX>;
   const uint32_t groups = kBlock / G;
   const uint32_t lane = threadIdx.x % G;
   const uint32_t grp = threadIdx.x / G;
-  for (I r0 = (I)blockIdx.x * groups; r0 < numRows; r0 += (I)gridDim.x * groups) {
-    const I row = r0 + grp;
-    const bool active = row < numRows;
+  const I total = numRows * S.d;
+  for (I r0 = (I)blockIdx.x * groups; r0 < total; r0 += (I)gridDim.x * groups) {
+    const I vr = r0 + grp;
+    const bool active = vr < total;
     float bv = O::worst();
     I bi = ~(I)0;
     I outOff = 0, idxOff = 0;
     if (active) {
-      I inOff, unused;
+      I row, sp, inOff, unused;
+      S.divmod(vr, row, sp);
       oa.offsets(row, inOff, outOff);
       oaIdx.offsets(row, unused, idxOff);
       const T* src = in + inOff;
+      const I begin = sp * chunk;
+      const I end = min(R, begin + chunk);
+      const I es = VEC == 1 ? sR : (I)1;
       constexpr int U = 8;
       const I step = (I)G * VEC;
-      I i = lane * VEC;
-      for (; i + (U - 1) * step < R; i += U * step) {
+      I i = begin + lane * VEC;
+      for (; i + (U - 1) * step < end; i += U * step) {
         P v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(src + i + u * step));
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -228,8 +252,8 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
           }
         }
       }
-      for (; i < R; i += step) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i));
+      for (; i < end; i += step) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
           const float x = Cvt<T>::up(v.v[e]);
@@ -256,11 +280,67 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(const T* __re
       }
     }
     if (active && lane == 0) {
-      // No element beat the start value: the whole row equals it (all -inf for
-      // max, all +inf for min), and the first occurrence is element 0.
+      if (S.d > 1) {
+        partV[vr] = bv;
+        partI[vr] = bi;
+      } else {
+        // No element beat the start value: the whole row equals it (all -inf
+        // for max, all +inf for min), and the first occurrence is element 0.
+        if (bi == ~(I)0) bi = 0;
+        outV[outOff] = Cvt<T>::down(bv);
+        outI[idxOff] = (long)bi + 1;  // 1-based (TH_INDEX_BASE)
+      }
+    }
+  }
+}
+
+// Second launch of a split max/min along rows: one wave per row folds that
+// row's S (value, index) partials.
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const float* __restrict__ partV,
+                                                            const I* __restrict__ partI,
+                                                            T* __restrict__ outV,
+                                                            long* __restrict__ outI,
+                                                            OuterArgs<I> oa, OuterArgs<I> oaIdx,
+                                                            I numRows, I S) {
+  using O = PairOrder<IS_MAX>;
+  const uint32_t lane = threadIdx.x & 63;
+  const I wavesPerGrid = (I)gridDim.x * (kBlock / 64);
+  // every wave runs the same number of rounds (row is wave-uniform)
+  for (I row = (I)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); row < numRows;
+       row += wavesPerGrid) {
+    float bv = O::worst();
+    I bi = ~(I)0;
+    for (I sp = lane; sp < S; sp += 64) {
+      const float v = partV[row * S + sp];
+      const I ix = partI[row * S + sp];
+      if (O::better(v, ix, bv, bi)) {
+        bv = v;
+        bi = ix;
+      }
+    }
+    for (uint32_t o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      I oi;
+      if (sizeof(I) == 8) {
+        const uint32_t lo = __shfl_xor((uint32_t)bi, o, 64);
+        const uint32_t hi = __shfl_xor((uint32_t)((uint64_t)bi >> 32), o, 64);
+        oi = (I)(((uint64_t)hi << 32) | lo);
+      } else {
+        oi = (I)__shfl_xor((uint32_t)bi, o, 64);
+      }
+      if (O::better(ov, oi, bv, bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (lane == 0) {
+      I unusedA, unusedB, outOff, idxOff;
+      oa.offsets(row, unusedA, outOff);
+      oaIdx.offsets(row, unusedB, idxOff);
       if (bi == ~(I)0) bi = 0;
       outV[outOff] = Cvt<T>::down(bv);
-      outI[idxOff] = (long)bi + 1;  // 1-based (TH_INDEX_BASE)
+      outI[idxOff] = (long)bi + 1;
     }
   }
 }
@@ -350,6 +430,12 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
       const I begin = s * a.chunkR;
       const I end = min(a.R, begin + a.chunkR);
       const TIn* src = in + inOff + col;
+      float c[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        c[e] = 0.f;
+        if constexpr (F::kCentred) c[e] = Cvt<TOut>::up(out[outOff + (col + e) * a.outInner]);
+      }
       constexpr int U = 8;
       I r = begin + ty;
       for (; r + (U - 1) * TY < end; r += U * TY) {
@@ -361,13 +447,14 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
         for (int u = 0; u < U; ++u) {
 #pragma unroll
           for (int e = 0; e < VEC; ++e)
-            acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v[u].v[e])));
+            acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v[u].v[e]), c[e]));
         }
       }
       for (; r < end; r += TY) {
         const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e])));
+        for (int e = 0; e < VEC; ++e)
+          acc[e] = f.combine(acc[e], f.modify(Cvt<TIn>::up(v.v[e]), c[e]));
       }
     }
     fold_rows(acc);
@@ -539,7 +626,7 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
   constexpr I step = (I)kBlock * VEC;
   if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n) {
     const float x = Cvt<TIn>::up(in[nv + threadIdx.x]);
-    acc[0] = f.combine(acc[0], FIRST ? f.modify(x) : x);
+    acc[0] = f.combine(acc[0], FIRST ? f.modify(x, 0.f) : x);
   }
   I i = begin + threadIdx.x * VEC;
   for (; i + (U - 1) * step < end; i += U * step) {
@@ -551,7 +638,7 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         const float x = Cvt<TIn>::up(v[u].v[e]);
-        acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+        acc[e] = f.combine(acc[e], FIRST ? f.modify(x, 0.f) : x);
       }
     }
   }
@@ -560,7 +647,7 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
       const float x = Cvt<TIn>::up(v.v[e]);
-      acc[e] = f.combine(acc[e], FIRST ? f.modify(x) : x);
+      acc[e] = f.combine(acc[e], FIRST ? f.modify(x, 0.f) : x);
     }
   }
   float r = acc[0];
@@ -575,46 +662,6 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
     } else {
       partial[blockIdx.x] = r;
     }
-  }
-}
-
-// --------------------------------------------------------------- generic --
-template <typename TIn, typename TOut, typename F, typename I>
-__global__ __launch_bounds__(kBlock) void reduce_generic_kernel(const TIn* __restrict__ in,
-                                                                TOut* __restrict__ out,
-                                                                OuterArgs<I> oa, I outElems, I R,
-                                                                I sR, Epi epi, F f) {
-  const I step = (I)gridDim.x * kBlock;
-  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < outElems; o += step) {
-    I inOff, outOff;
-    oa.offsets(o, inOff, outOff);
-    float r = f.init();
-    for (I i = 0; i < R; ++i) r = f.combine(r, f.modify(Cvt<TIn>::up(in[inOff + i * sR])));
-    out[outOff] = epi.template finish<TOut>(r);
-  }
-}
-
-template <typename T, typename I, bool IS_MAX>
-__global__ __launch_bounds__(kBlock) void reduce_generic_index_kernel(
-    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI, OuterArgs<I> oa,
-    OuterArgs<I> oaIdx, I outElems, I R, I sR) {
-  using O = PairOrder<IS_MAX>;
-  const I step = (I)gridDim.x * kBlock;
-  for (I o = (I)blockIdx.x * kBlock + threadIdx.x; o < outElems; o += step) {
-    I inOff, outOff, unused, idxOff;
-    oa.offsets(o, inOff, outOff);
-    oaIdx.offsets(o, unused, idxOff);
-    float bv = O::worst();
-    I bi = ~(I)0;
-    for (I i = 0; i < R; ++i) {
-      const float x = Cvt<T>::up(in[inOff + i * sR]);
-      if (O::better(x, i, bv, bi)) {
-        bv = x;
-        bi = i;
-      }
-    }
-    outV[outOff] = Cvt<T>::down(bv);
-    outI[idxOff] = (long)bi + 1;
   }
 }
 
@@ -685,8 +732,8 @@ ReduceGeom make_geom(AnyTensor* in, AnyTensor* out, AnyTensor* idxT, int dim) {
 
 template <typename TIn, typename TOut, typename F, typename I, bool FIRST>
 void launch_rows_pass(THCState* s, const TIn* in, TOut* out, float* partial, const OuterArgs<I>& oa,
-                      int64_t numRows, int64_t R, int64_t S, int64_t chunk, bool vec, Epi epi,
-                      F f) {
+                      int64_t numRows, int64_t R, int64_t sR, int64_t S, int64_t chunk, bool vec,
+                      Epi epi, F f) {
   constexpr int VEC = 16 / sizeof(TIn);
   const int pack = vec ? VEC : 1;
   const int64_t span = std::min(R, chunk);
@@ -701,18 +748,20 @@ void launch_rows_pass(THCState* s, const TIn* in, TOut* out, float* partial, con
   hipStream_t st = current_stream(s);
   if (vec)
     hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, VEC, FIRST>), dim3(grid), dim3(kBlock),
-                       0, st, in, out, partial, oa, (I)numRows, (I)R, Sd, (I)chunk, G, epi, f);
+                       0, st, in, out, partial, oa, (I)numRows, (I)R, (I)1, Sd, (I)chunk, G, epi,
+                       f);
   else
     hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, 1, FIRST>), dim3(grid), dim3(kBlock), 0,
-                       st, in, out, partial, oa, (I)numRows, (I)R, Sd, (I)chunk, G, epi, f);
+                       st, in, out, partial, oa, (I)numRows, (I)R, (I)sR, Sd, (I)chunk, G, epi, f);
 }
 
-// rows: reduced dim has unit stride.
+// rows: a group of lanes per output. Packs when the reduced dim has unit stride
+// and everything is 16-byte aligned, scalar strided loads otherwise.
 template <typename T, typename F, typename I>
 void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
   constexpr int VEC = 16 / sizeof(T);
   const int64_t rows = g.outElems;
-  bool vec = aligned16(in) && g.R % VEC == 0;
+  bool vec = g.sR == 1 && aligned16(in) && g.R % VEC == 0;
   for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
   OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
 
@@ -732,12 +781,12 @@ void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F 
     S = (g.R + chunk - 1) / chunk;
   }
   if (S == 1) {
-    launch_rows_pass<T, T, F, I, true>(s, in, out, nullptr, oa, rows, g.R, 1, g.R, vec, epi, f);
-    note_kernel(vec ? "rows" : "rows-scalar");
+    launch_rows_pass<T, T, F, I, true>(s, in, out, nullptr, oa, rows, g.R, g.sR, 1, g.R, vec, epi, f);
+    note_kernel(vec ? "rows" : (g.sR == 1 ? "rows-scalar" : "rows-strided"));
     return;
   }
   float* scratch = (float*)scratch_space(s, &scratchBytes);
-  launch_rows_pass<T, T, F, I, true>(s, in, (T*)nullptr, scratch, oa, rows, g.R, S, chunk, vec,
+  launch_rows_pass<T, T, F, I, true>(s, in, out, scratch, oa, rows, g.R, g.sR, S, chunk, vec,
                                      Epi{(int)Epilogue::None, 0.f}, f);
   // pass 2: partial[row*S + s] is a dense rows x S matrix
   Layout pin = g.in;
@@ -747,9 +796,9 @@ void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F 
     run *= pin.size[d];
   }
   OuterArgs<I> oa2 = make_outer<I>(pin, g.out, pin.dims);
-  launch_rows_pass<float, T, F, I, false>(s, scratch, out, nullptr, oa2, rows, S, 1, S,
+  launch_rows_pass<float, T, F, I, false>(s, scratch, out, nullptr, oa2, rows, S, 1, 1, S,
                                           S % 4 == 0, epi, f);
-  note_kernel(vec ? "rows-split" : "rows-split-scalar");
+  note_kernel(vec ? "rows-split" : (g.sR == 1 ? "rows-split-scalar" : "rows-split-strided"));
 }
 
 template <typename I>
@@ -833,22 +882,11 @@ void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F 
 }
 
 template <typename T, typename F, typename I>
-void run_generic(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
-  OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
-  const int grid = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.generic.blocks_per_cu", 32);
-  hipLaunchKernelGGL((reduce_generic_kernel<T, T, F, I>), dim3(grid), dim3(kBlock), 0,
-                     current_stream(s), in, out, oa, (I)g.outElems, (I)g.R, (I)g.sR, epi, f);
-  note_kernel("reduce-generic");
-}
-
-template <typename T, typename F, typename I>
 void run_dim_typed(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi epi, F f) {
-  if (g.sR == 1)
-    run_rows<T, F, I>(s, g, in, out, epi, f);
-  else if (g.in.stride[g.in.dims - 1] == 1 && g.in.size[g.in.dims - 1] > 1)
+  if (g.sR != 1 && g.in.stride[g.in.dims - 1] == 1 && g.in.size[g.in.dims - 1] > 1)
     run_cols<T, F, I>(s, g, in, out, epi, f);
   else
-    run_generic<T, F, I>(s, g, in, out, epi, f);
+    run_rows<T, F, I>(s, g, in, out, epi, f);  // unit stride: packs; otherwise its scalar form
 }
 
 template <typename T, typename F>
@@ -872,6 +910,7 @@ void dispatch_reduce(THCState* s, const ReduceGeom& g, const void* in, void* out
     case ReduceOp::Norm2: run_dim<T>(s, g, in, out, epi, FNorm2{p}); break;
     case ReduceOp::NormP: run_dim<T>(s, g, in, out, epi, FNormP{p}); break;
     case ReduceOp::SqDev: run_dim<T>(s, g, in, out, epi, FSqDev{p}); break;
+    case ReduceOp::SqDevOut: run_dim<T>(s, g, in, out, epi, FSqDevOut{p}); break;
   }
 }
 
@@ -881,27 +920,62 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
   constexpr int VEC = 16 / sizeof(T);
   hipStream_t st = current_stream(s);
   const int nd = g.in.dims;
-  if (g.sR == 1) {
-    bool vec = aligned16(in) && g.R % VEC == 0;
+  const bool colsShape = g.sR != 1 && g.in.stride[nd - 1] == 1 && g.in.size[nd - 1] > 1;
+  if (!colsShape) {
+    bool vec = g.sR == 1 && aligned16(in) && g.R % VEC == 0;
     for (int d = 0; d < nd && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
     const int pack = vec ? VEC : 1;
     OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
+    const int64_t rows = g.outElems;
+    // Few long rows: cut them as run_rows does.
+    const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+    const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
+    int64_t S = 1, chunk = g.R;
+    float* partV = nullptr;
+    I* partI = nullptr;
+    if (rows < target && g.R >= 2 * minChunk) {
+      size_t scratchBytes = 0;
+      char* scratch = (char*)scratch_space(s, &scratchBytes);
+      S = std::min<int64_t>((target + rows - 1) / rows, g.R / minChunk);
+      S = std::min<int64_t>(S, (int64_t)(scratchBytes / (sizeof(float) + sizeof(I))) / std::max<int64_t>(rows, 1));
+      if (S < 2) S = 1;
+      chunk = (g.R + S - 1) / S;
+      chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
+      S = (g.R + chunk - 1) / chunk;
+      if (S > 1) {
+        partI = (I*)scratch;  // 8-byte aligned part first
+        partV = (float*)(scratch + sizeof(I) * (size_t)S * (size_t)rows);
+      }
+    }
+    const int64_t span = std::min(g.R, chunk);
     const int64_t perLane = tuning("reduce.rows.packs_per_lane", 8);
-    uint32_t G = pow2_ceil((uint64_t)((g.R + pack * perLane - 1) / (pack * perLane)));
+    uint32_t G = pow2_ceil((uint64_t)((span + pack * perLane - 1) / (pack * perLane)));
     G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
     const int64_t groups = kBlock / G;
-    const int grid = capped_grid(s, (g.outElems + groups - 1) / groups, "reduce.rows.blocks_per_cu", 64);
+    const int grid = capped_grid(s, (rows * S + groups - 1) / groups, "reduce.rows.blocks_per_cu", 64);
+    Divisor<I> Sd;
+    Sd.set((uint64_t)S);
     if (vec)
       hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, VEC, IS_MAX>), dim3(grid), dim3(kBlock), 0,
-                         st, in, outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, G);
+                         st, in, outV, outI, partV, partI, oa, oaIdx, (I)rows, (I)g.R, (I)1, Sd,
+                         (I)chunk, G);
     else
       hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, 1, IS_MAX>), dim3(grid), dim3(kBlock), 0,
-                         st, in, outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, G);
-    note_kernel(vec ? "rows-index" : "rows-index-scalar");
+                         st, in, outV, outI, partV, partI, oa, oaIdx, (I)rows, (I)g.R, (I)g.sR, Sd,
+                         (I)chunk, G);
+    if (S > 1) {
+      const int fgrid = capped_grid(s, (rows + kBlock / 64 - 1) / (kBlock / 64), "reduce.rows.blocks_per_cu", 64);
+      hipLaunchKernelGGL((fold_pairs_kernel<T, I, IS_MAX>), dim3(fgrid), dim3(kBlock), 0, st, partV,
+                         partI, outV, outI, oa, oaIdx, (I)rows, (I)S);
+    }
+    if (S > 1)
+      note_kernel(vec ? "rows-index-split" : (g.sR == 1 ? "rows-index-split-scalar" : "rows-index-split-strided"));
+    else
+      note_kernel(vec ? "rows-index" : (g.sR == 1 ? "rows-index-scalar" : "rows-index-strided"));
     return;
   }
-  if (g.in.stride[nd - 1] == 1 && g.in.size[nd - 1] > 1) {
+  {
     ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(float) + sizeof(I));
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
     const I idxInner = (I)g.idx.stride[nd - 1];
@@ -927,14 +1001,7 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
                            st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, tb, fold);
     }
     note_kernel(split ? "cols-index-split" : "cols-index");
-    return;
   }
-  OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
-  OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
-  const int grid = capped_grid(s, (g.outElems + kBlock - 1) / kBlock, "reduce.generic.blocks_per_cu", 32);
-  hipLaunchKernelGGL((reduce_generic_index_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock), 0, st, in,
-                     outV, outI, oa, oaIdx, (I)g.outElems, (I)g.R, (I)g.sR);
-  note_kernel("generic-index");
 }
 
 template <typename T>
@@ -1088,12 +1155,12 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
           bool vec = aligned16(src) && g.R % 4 == 0;
           for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % 4 == 0 || g.in.size[d] == 1;
           launch_rows_pass<float, float, F, I, true>(s, (const float*)src, rp, nullptr, oa, rows, g.R,
-                                                     1, g.R, vec, none, f);
+                                                     1, 1, g.R, vec, none, f);
         } else {
           bool vec = aligned16(src) && g.R % 8 == 0;
           for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % 8 == 0 || g.in.size[d] == 1;
           launch_rows_pass<__half, float, F, I, true>(s, (const __half*)src, rp, nullptr, oa, rows,
-                                                      g.R, 1, g.R, vec, none, f);
+                                                      g.R, 1, 1, g.R, vec, none, f);
         }
       };
       if (g.wide) go(uint64_t{}); else go(uint32_t{});
@@ -1108,6 +1175,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
       case ReduceOp::Norm2: stage1(FNorm2{p}); op2 = ReduceOp::Sum; break;
       case ReduceOp::NormP: stage1(FNormP{p}); op2 = ReduceOp::Sum; break;
       case ReduceOp::SqDev: stage1(FSqDev{p}); op2 = ReduceOp::Sum; break;
+      case ReduceOp::SqDevOut: raise_error("centred reduction needs a dim");
     }
     src = rp;
     srcT = DType::F32;
@@ -1175,6 +1243,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
     case ReduceOp::Norm2: stage2(FNorm2{p}); break;
     case ReduceOp::NormP: stage2(FNormP{p}); break;
     case ReduceOp::SqDev: stage2(FSqDev{p}); break;
+    case ReduceOp::SqDevOut: raise_error("centred reduction needs a dim");
   }
   note_kernel(rows > 1 ? "all-rows" : "all");
   THC_CHECK(hipGetLastError());

@@ -311,3 +311,52 @@ def test_sumall_2pow28_uniform(thc, oracle):
     got = dev.sumall()
     assert abs(got - want) <= 1e-5 * abs(want), (got, want)
     assert abs(dev.normall(2.0) - oracle.reduce_all("norm", oracle.View(x[:1 << 20]), p=2)) >= 0  # smoke
+
+
+# ------------------------------------------------ strided and long-row shapes --
+def test_strided_reduced_dim_without_unit_stride_sibling(thc, oracle):
+    """A column of a matrix (one output over a strided dim) and a strided slice
+    whose other dim is strided too: lanes share each output instead of one
+    thread walking it."""
+    rng = np.random.default_rng(51)
+    n, w = 70000, 3
+    st = rng.uniform(-1, 1, n * w).astype(np.float32)
+    for kind_name, fn in (("sum", "sum"), ("norm2", "norm2")):
+        dev = thc.Tensor.from_storage(st, 1, (n, 1), (w, 1))
+        ref = oracle.View(st.copy(), 1, (n, 1), (w, 1))
+        assert run_reduce(thc, oracle, fn, dev, ref, 0).startswith("rows-split-strided")
+    dev = thc.Tensor.from_storage(st, 0, (100, 300), (2100, 7))     # both dims strided
+    ref = oracle.View(st.copy(), 0, (100, 300), (2100, 7))
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1) == "rows-strided"
+    assert run_reduce(thc, oracle, "sum", dev, ref, 0) == "rows-strided"
+    sti = rng.integers(-50, 50, n * w).astype(np.float32)
+    devi = thc.Tensor.from_storage(sti, 2, (n, 1), (w, 1))
+    refi = oracle.View(sti.copy(), 2, (n, 1), (w, 1))
+    for which in ("max", "min"):
+        assert run_minmax(thc, oracle, which, devi, refi, 0) == "rows-index-split-strided"
+    devi = thc.Tensor.from_storage(sti, 0, (100, 300), (2100, 7))
+    refi = oracle.View(sti.copy(), 0, (100, 300), (2100, 7))
+    assert run_minmax(thc, oracle, "max", devi, refi, 1) == "rows-index-strided"
+    assert run_minmax(thc, oracle, "min", devi, refi, 0) == "rows-index-strided"
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_minmax_of_few_long_rows_is_split(thc, oracle, kind):
+    rng = np.random.default_rng(52)
+    for shape in ((3, 1 << 18), (1, 300001), (2, 5, 40000)):
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "ints")
+        for which in ("max", "min"):
+            k = run_minmax(thc, oracle, which, dev, ref, len(shape) - 1, kind)
+            assert k.startswith("rows-index-split"), k
+    x = np.full((2, 100000), -np.inf, np.float32)                  # nothing beats the start value
+    x[1, 77777] = np.nan
+    vals, idx = thc.Tensor("float"), thc.Tensor("long")
+    vals.max(idx, thc.Tensor.from_numpy(x), 1)
+    assert idx.numpy().ravel().tolist() == [1, 77778]
+    assert vals.numpy()[0, 0] == -np.inf and np.isnan(vals.numpy()[1, 0])
+    thc.force_64bit_index(True)
+    try:
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((2, 70000)), "float", "ints")
+        assert run_minmax(thc, oracle, "max", dev, ref, 1) == "rows-index-split"
+    finally:
+        thc.force_64bit_index(False)
