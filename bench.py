@@ -155,12 +155,12 @@ def build_configs(thc, hip, which, only=None):
 
     # C3c: reduceAll over 2^28
     n3c = 1 << 28
-    xa = T.from_numpy(rng.random(n3c if want('C3c-sumall') else 4, dtype=np.float32))
+    xa = T.from_numpy(rng.random(n3c if want('C3c-sumall', 'N-fill') else 4, dtype=np.float32))
     cfgs.append(Config("C3c-sumall", "sumall over 2^28 fp32 (blocks on a 4-byte D2H copy)",
                        4 * n3c + 4, n3c, 1, lambda i: xa.sumall()))
 
     # C4: 64 x 4096 x 512, middle dim; fp32 and fp16
-    s4 = (64, 4096, 512) if want('C4-sum-f32', 'C4-norm-f32', 'C4-sum-f16', 'C4-norm-f16') else (1, 4, 8)
+    s4 = (64, 4096, 512) if want('C4-sum-f32', 'C4-norm-f32', 'C4-sum-f16', 'C4-norm-f16', 'N-std-cols', 'N-cumsum-cols') else (1, 4, 8)
     x4 = rng.uniform(-2, 2, s4).astype(np.float32)
     d4 = T.from_numpy(x4)
     o4 = T("float").resize((s4[0], 1, s4[2]))
@@ -178,6 +178,40 @@ def build_configs(thc, hip, which, only=None):
     cfgs.append(Config("C4-norm-f16", "L2 norm over middle dim of 64x4096x512 fp16, fp32 accumulate",
                        2 * n4 + 2 * s4[0] * s4[2], n4, 3,
                        lambda i: sets4h[i % 3][1].norm(sets4h[i % 3][0], 2.0, 1)))
+
+    # Neighbours of the hot path on the same engines (same operands where possible).
+    nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
+                      "N-cumsum-cols", "N-dist", "N-varall") if (only and n in only) or (not only and which == "all")]
+    if nx:
+        ne = 1 << 26
+        e_src = T.from_numpy(rng.uniform(-1, 1, ne).astype(np.float32))
+        e_dst = T("float").resize((ne,))
+        sq = T.from_numpy(rng.standard_normal((8192, 8192), dtype=np.float32))
+        sq_t, sq_out = sq.t(), T("float").resize((8192, 8192))
+        x3 = sets3[0][0] if sets3 else T.from_numpy(rng.standard_normal((r3, n3), dtype=np.float32))
+        o3 = T("float").resize((r3, 1))
+        s3 = T("float").resize((r3, n3))
+        s4o = T("float").resize(s4)
+        big = 1 << 28
+        table = {
+            "N-copy-t": ("out:copy(a:t()), 8192x8192 fp32", 8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.copy(sq_t)),
+            "N-fill": ("fill of 2^28 fp32", 4 * big, big, lambda i: xa.fill(0.5) if xa.numel() == big else e_dst.fill(0.5)),
+            "N-exp": ("out = exp(x), 2^26 fp32 contiguous", 8 * ne, ne, lambda i: e_dst.unary("exp", e_src)),
+            "N-var-rows": ("var over last dim of 65536x1024 fp32 (input counted once)", 4 * r3 * n3 + 4 * r3,
+                           r3 * n3, lambda i: o3.var(x3, 1)),
+            "N-std-cols": ("std over middle dim of 64x4096x512 fp32 (input counted once)",
+                           4 * n4 + 4 * s4[0] * s4[2], n4, lambda i: o4.std(d4, 1)),
+            "N-cumsum-rows": ("cumsum over last dim of 65536x1024 fp32", 8 * r3 * n3, r3 * n3,
+                              lambda i: s3.cumsum(x3, 1)),
+            "N-cumsum-cols": ("cumsum over middle dim of 64x4096x512 fp32", 8 * n4, n4, lambda i: s4o.cumsum(d4, 1)),
+            "N-dist": ("dist(a, b, 2) over 2^26 fp32", 8 * ne, ne, lambda i: e_src.dist(e_dst, 2.0)),
+            "N-varall": ("varall over 2^26 fp32 (input counted once)", 4 * ne, ne, lambda i: e_src.varall()),
+        }
+        if "N-fill" in nx and xa.numel() != big:
+            table["N-fill"] = ("fill of 2^26 fp32", 4 * ne, ne, lambda i: e_dst.fill(0.5))
+        for n in nx:
+            d, nb, el, fn = table[n]
+            cfgs.append(Config(n, d, nb, el, 1, fn))
 
     # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path
     if not want('C5'):

@@ -3,12 +3,13 @@
 // Role of THCTensor_(scanDim) and its kernels (lib/THC/THCTensorMathScan.cu:
 // 23-110, generic/THCTensorMathScan.cu:1-128). Operands are made dense first,
 // as in the reference, and viewed as [outer][R][inner]:
-//   inner == 1  one wave64 per row: every lane owns 4 consecutive elements
-//               (one 16-byte load), scans them in registers, the wave combines
-//               the lane totals with shuffle-up steps, and a running carry
-//               links the 256-element chunks of a long row;
-//   inner  > 1  lanes run along the unit-stride inner dim (coalesced) and each
-//               walks the scanned dim sequentially.
+//   inner == 1  one wave64 per row: every lane owns one 16-byte pack of each
+//               chunk, scans it in registers, the wave combines the lane
+//               totals with shuffle-up steps, and a running carry links the
+//               chunks of a long row;
+//   inner  > 1  lanes run along the unit-stride inner dim (coalesced), thread
+//               rows split the scanned dim into register-resident segments
+//               and exchange segment totals through LDS.
 // Accumulation is fp32 (also for half tensors, rounded per output element).
 #include "common.hpp"
 #include "device_util.hpp"
@@ -25,11 +26,15 @@ struct ScanMul {
   static __device__ __forceinline__ float op(float a, float b) { return a * b; }
 };
 
-template <typename T, typename Op>
+// One wave64 per row. A lane owns VEC consecutive elements of each
+// 64*VEC-element chunk; U chunks are loaded before the first is consumed.
+template <typename T, typename Op, int VEC>
 __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t numRows, uint64_t R) {
-  constexpr int K = 4;  // elements per lane per chunk
+  using P = Pack<T, VEC>;
+  constexpr int U = 4;
+  constexpr uint64_t kChunk = 64 * VEC;
   const uint32_t lane = threadIdx.x & 63;
   const uint64_t wavesPerGrid = (uint64_t)gridDim.x * (kBlock / 64);
   for (uint64_t row = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); row < numRows;
@@ -37,64 +42,176 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
     const T* src = in + row * R;
     T* dst = out + row * R;
     float carry = Op::id();
-    for (uint64_t base = 0; base < R; base += 64 * K) {
-      const uint64_t i0 = base + (uint64_t)lane * K;
-      float x[K];
+    for (uint64_t base = 0; base < R; base += U * kChunk) {
+      float x[U][VEC];
 #pragma unroll
-      for (int k = 0; k < K; ++k) x[k] = i0 + k < R ? Cvt<T>::up(src[i0 + k]) : Op::id();
+      for (int u = 0; u < U; ++u) {
+        const uint64_t i0 = base + u * kChunk + (uint64_t)lane * VEC;
+        if (VEC > 1) {
+          // rows are whole packs (R % VEC == 0), so a pack is inside or outside
+          if (i0 < R) {
+            const P v = load_pack<true>(reinterpret_cast<const P*>(src + i0));
 #pragma unroll
-      for (int k = 1; k < K; ++k) x[k] = Op::op(x[k - 1], x[k]);
-      // inclusive scan of the lane totals across the wave
-      float t = x[K - 1];
+            for (int k = 0; k < VEC; ++k) x[u][k] = Cvt<T>::up(v.v[k]);
+          } else {
 #pragma unroll
-      for (uint32_t o = 1; o < 64; o <<= 1) {
-        const float y = __shfl_up(t, o, 64);
-        if (lane >= o) t = Op::op(y, t);
+            for (int k = 0; k < VEC; ++k) x[u][k] = Op::id();
+          }
+        } else {
+          x[u][0] = i0 < R ? Cvt<T>::up(src[i0]) : Op::id();
+        }
       }
-      float before = __shfl_up(t, 1, 64);  // exclusive prefix of this lane
-      if (lane == 0) before = Op::id();
-      const float offset = Op::op(carry, before);
 #pragma unroll
-      for (int k = 0; k < K; ++k)
-        if (i0 + k < R) dst[i0 + k] = Cvt<T>::down(Op::op(offset, x[k]));
-      carry = Op::op(carry, __shfl(t, 63, 64));
+      for (int u = 0; u < U; ++u) {
+        const uint64_t i0 = base + u * kChunk + (uint64_t)lane * VEC;
+#pragma unroll
+        for (int k = 1; k < VEC; ++k) x[u][k] = Op::op(x[u][k - 1], x[u][k]);
+        // inclusive scan of the lane totals across the wave
+        float t = x[u][VEC - 1];
+#pragma unroll
+        for (uint32_t o = 1; o < 64; o <<= 1) {
+          const float y = __shfl_up(t, o, 64);
+          if (lane >= o) t = Op::op(y, t);
+        }
+        float before = __shfl_up(t, 1, 64);  // exclusive prefix of this lane
+        if (lane == 0) before = Op::id();
+        const float offset = Op::op(carry, before);
+        if (i0 < R) {
+          if (VEC > 1) {
+            P v;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v.v[k] = Cvt<T>::down(Op::op(offset, x[u][k]));
+            *reinterpret_cast<P*>(dst + i0) = v;
+          } else {
+            dst[i0] = Cvt<T>::down(Op::op(offset, x[u][0]));
+          }
+        }
+        carry = Op::op(carry, __shfl(t, 63, 64));
+      }
     }
   }
 }
 
-template <typename T, typename Op>
+// Scan along a strided dim of a dense [outer][R][inner] block. A workgroup
+// owns one `outer` index and TX*VEC adjacent columns and walks R in segments
+// of TY*U rows: thread row ty holds U consecutive rows of the segment in
+// registers, scans them locally, the thread rows exchange their totals
+// through LDS, and a per-column carry links the segments. The input is read
+// once and the output written once.
+template <typename T, typename Op, int VEC>
 __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t outer, uint64_t R,
-                                                           uint64_t inner) {
-  const uint64_t lines = outer * inner;
-  const uint64_t step = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t l = (uint64_t)blockIdx.x * kBlock + threadIdx.x; l < lines; l += step) {
-    const uint64_t o = l / inner, c = l - o * inner;
-    const uint64_t base = o * R * inner + c;
-    float acc = Op::id();
-    for (uint64_t r = 0; r < R; ++r) {
-      acc = Op::op(acc, Cvt<T>::up(in[base + r * inner]));
-      out[base + r * inner] = Cvt<T>::down(acc);
+                                                           uint64_t inner, uint32_t TX,
+                                                           uint64_t colTiles) {
+  using P = Pack<T, VEC>;
+  constexpr int U = 8;
+  __shared__ float totals[2][kBlock * VEC];
+  const uint32_t TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const uint64_t blocks = outer * colTiles;
+  for (uint64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
+    const uint64_t o = b / colTiles, ct = b - o * colTiles;
+    const uint64_t col = (ct * TX + tx) * VEC;
+    const bool live = col < inner;  // inner % VEC == 0 for VEC > 1
+    const T* src = in + o * R * inner + col;
+    T* dst = out + o * R * inner + col;
+    float carry[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) carry[e] = Op::id();
+    uint32_t flip = 0;
+    for (uint64_t seg = 0; seg < R; seg += (uint64_t)TY * U, flip ^= 1) {
+      const uint64_t r0 = seg + (uint64_t)ty * U;
+      float x[U][VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (live && r0 + u < R) {
+          const P v = load_pack<true>(reinterpret_cast<const P*>(src + (r0 + u) * inner));
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) x[u][e] = Cvt<T>::up(v.v[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) x[u][e] = Op::id();
+        }
+      }
+#pragma unroll
+      for (int u = 1; u < U; ++u) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[u][e] = Op::op(x[u - 1][e], x[u][e]);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) totals[flip][(ty * TX + tx) * VEC + e] = x[U - 1][e];
+      __syncthreads();  // the other buffer is free again after the next barrier
+      float offset[VEC], running[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        running[e] = Op::id();
+        offset[e] = Op::id();
+      }
+      for (uint32_t t = 0; t < TY; ++t) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          if (t == ty) offset[e] = running[e];
+          running[e] = Op::op(running[e], totals[flip][(t * TX + tx) * VEC + e]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) offset[e] = Op::op(carry[e], offset[e]);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (live && r0 + u < R) {
+          P v;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) v.v[e] = Cvt<T>::down(Op::op(offset[e], x[u][e]));
+          *reinterpret_cast<P*>(dst + (r0 + u) * inner) = v;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) carry[e] = Op::op(carry[e], running[e]);
     }
+    __syncthreads();  // both LDS buffers are idle before the next tile
   }
+}
+
+uint32_t pow2_at_least(uint64_t x) {
+  uint32_t p = 1;
+  while (p < x && p < 64) p <<= 1;
+  return p;
 }
 
 template <typename T, typename Op>
 void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int64_t inner) {
+  constexpr int VEC = 16 / sizeof(T);
   hipStream_t st = current_stream(s);
-  const int64_t cap = (int64_t)num_compute_units(s) * 32;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
   if (inner == 1) {
+    const int64_t cap = (int64_t)num_compute_units(s) * 32;
     const int64_t blocks = (outer + (kBlock / 64) - 1) / (kBlock / 64);
     const int grid = (int)std::max<int64_t>(1, std::min(blocks, cap));
-    hipLaunchKernelGGL((scan_rows_kernel<T, Op>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                       (uint64_t)outer, (uint64_t)R);
+    if (aligned && R % VEC == 0)
+      hipLaunchKernelGGL((scan_rows_kernel<T, Op, VEC>), dim3(grid), dim3(kBlock), 0, st, out, in,
+                         (uint64_t)outer, (uint64_t)R);
+    else
+      hipLaunchKernelGGL((scan_rows_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
+                         (uint64_t)outer, (uint64_t)R);
     note_kernel("scan-rows");
   } else {
-    const int64_t blocks = (outer * inner + kBlock - 1) / kBlock;
-    const int grid = (int)std::max<int64_t>(1, std::min(blocks, cap));
-    hipLaunchKernelGGL((scan_cols_kernel<T, Op>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                       (uint64_t)outer, (uint64_t)R, (uint64_t)inner);
+    const bool vec = aligned && inner % VEC == 0;
+    const int64_t pack = vec ? VEC : 1;
+    const int64_t packs = (inner + pack - 1) / pack;
+    // 16..64 lanes along the unit-stride dim: narrower tiles when that is what
+    // gives every CU a workgroup
+    uint32_t TX = std::max<uint32_t>(16, pow2_at_least((uint64_t)packs));
+    const int64_t want = 2 * (int64_t)num_compute_units(s);
+    while (TX > 16 && outer * ((packs + TX - 1) / TX) < want) TX >>= 1;
+    const int64_t colTiles = (packs + TX - 1) / TX;
+    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * colTiles, 1 << 30));
+    if (vec)
+      hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC>), dim3(grid), dim3(kBlock), 0, st, out, in,
+                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles);
+    else
+      hipLaunchKernelGGL((scan_cols_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
+                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles);
     note_kernel("scan-cols");
   }
 }

@@ -32,7 +32,8 @@ def test_gpu_scan(thc, oracle, kind):
     dtype = np.float32 if kind == "float" else np.float16
     tol = 1e-5 if kind == "float" else 2e-3
     for shape, dim in (((7, 1000), 1), ((3, 257), 1), ((300, 5), 1), ((50, 64), 0), ((4, 33, 20), 1),
-                       ((2, 3, 4, 130), 3), ((1,), 0), ((9000,), 0), ((6, 5, 1), 1)):
+                       ((2, 3, 4, 130), 3), ((1,), 0), ((9000,), 0), ((6, 5, 1), 1), ((2, 1000, 24), 1),
+                       ((3, 300, 7), 1), ((1, 5000, 136), 1), ((700, 2), 0), ((5, 2049), 1), ((2, 130, 8, 16), 1)):
         geom = random_geometry(rng, shape) if len(shape) == 3 else contiguous_geometry(shape)
         st = rng.uniform(-1, 1, geom[0]).astype(dtype)
         dev = thc.Tensor.from_storage(st, *geom[1:], kind=kind)
