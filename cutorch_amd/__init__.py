@@ -83,7 +83,15 @@ _TYPES = {
     "float": ("THCudaTensor", "THCudaStorage", C.c_float, np.float32),
     "half": ("THCudaHalfTensor", "THCudaHalfStorage", C.c_uint16, np.float16),
     "long": ("THCudaLongTensor", "THCudaLongStorage", C.c_long, np.int64),
+    "byte": ("THCudaByteTensor", "THCudaByteStorage", C.c_ubyte, np.uint8),
+    "char": ("THCudaCharTensor", "THCudaCharStorage", C.c_byte, np.int8),
+    "short": ("THCudaShortTensor", "THCudaShortStorage", C.c_short, np.int16),
+    "int": ("THCudaIntTensor", "THCudaIntStorage", C.c_int, np.int32),
+    "double": ("THCudaDoubleTensor", "THCudaDoubleStorage", C.c_double, np.float64),
 }
+_COPY_SUFFIX = {"byte": "Byte", "char": "Char", "short": "Short", "int": "Int", "long": "Long",
+                "float": "Float", "double": "Double", "half": "Half"}
+_FLOAT_KINDS = ("float", "half")
 
 
 def _declare(l):
@@ -147,31 +155,40 @@ def _declare(l):
         f(T + "_nElement", C.c_ssize_t, P, TP)
         f(T + "_data", P, P, TP)
         f(T + "_squeeze1d", None, P, TP, TP, C.c_int)
-        if kind == "long":
-            continue
+        for other in _TYPES:
+            f(T + "_copyCuda" + _COPY_SUFFIX[other], None, P, TP, TP)
+        for cmp in ("lt", "gt", "le", "ge", "eq", "ne"):
+            f(T + "_" + cmp + "Value", None, P, TP, TP, creal)
+            f(T + "_" + cmp + "ValueT", None, P, TP, TP, creal)
+            f(T + "_" + cmp + "Tensor", None, P, TP, TP, TP)
+            f(T + "_" + cmp + "TensorT", None, P, TP, TP, TP)
+
+        def opt(name, res, *args):      # declared when the type has the entry point
+            if hasattr(l, name):
+                f(name, res, *args)
         LT = TP
-        for name in ("add", "sub", "mul", "div"):
-            f(T + "_" + name, None, P, TP, TP, creal)
+        for name in ("add", "sub", "mul", "div", "pow", "cmaxValue", "cminValue", "fmod", "remainder",
+                     "lshift", "rshift", "bitand", "bitor", "bitxor"):
+            opt(T + "_" + name, None, P, TP, TP, creal)
         for name in ("cadd", "csub"):
-            f(T + "_" + name, None, P, TP, TP, creal, TP)
-        for name in ("cmul", "cdiv"):
-            f(T + "_" + name, None, P, TP, TP, TP)
+            opt(T + "_" + name, None, P, TP, TP, creal, TP)
+        for name in ("cmul", "cdiv", "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "clshift",
+                     "crshift", "cbitand", "cbitor", "cbitxor"):
+            opt(T + "_" + name, None, P, TP, TP, TP)
         for name in ("addcmul", "addcdiv"):
-            f(T + "_" + name, None, P, TP, TP, creal, TP, TP)
+            opt(T + "_" + name, None, P, TP, TP, creal, TP, TP)
         for name in ("sigmoid", "log", "lgamma", "log1p", "exp", "cos", "acos", "cosh", "sin", "asin",
                      "sinh", "tan", "atan", "tanh", "sqrt", "rsqrt", "ceil", "floor", "round", "trunc",
                      "frac", "cinv", "neg", "abs", "sign"):
-            f(T + "_" + name, None, P, TP, TP)
-        f(T + "_clamp", None, P, TP, TP, creal, creal)
-        f(T + "_tpow", None, P, TP, creal, TP)
-        for name in ("pow", "cmaxValue", "cminValue", "fmod", "remainder"):
-            f(T + "_" + name, None, P, TP, TP, creal)
-        for name in ("cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2"):
-            f(T + "_" + name, None, P, TP, TP, TP)
-        f(T + "_lerp", None, P, TP, TP, TP, creal)
-        f(T + "_equal", C.c_int, P, TP, TP)
-        f(T + "_fill", None, P, TP, creal)
-        f(T + "_zero", None, P, TP)
+            opt(T + "_" + name, None, P, TP, TP)
+        opt(T + "_clamp", None, P, TP, TP, creal, creal)
+        opt(T + "_tpow", None, P, TP, creal, TP)
+        opt(T + "_lerp", None, P, TP, TP, TP, creal)
+        opt(T + "_equal", C.c_int, P, TP, TP)
+        opt(T + "_fill", None, P, TP, creal)
+        opt(T + "_zero", None, P, TP)
+        if kind not in _FLOAT_KINDS:
+            continue
         for name in ("sum", "prod", "mean"):
             f(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int)
         f(T + "_norm", None, P, TP, TP, creal, C.c_long, C.c_int)
@@ -189,7 +206,6 @@ def _declare(l):
         f(T + "_normall", C.c_float, P, TP, creal)
         for name in ("minall", "maxall"):
             f(T + "_" + name, creal, P, TP)
-    l.THCudaTensor_copyCudaHalf.argtypes = [P, TP, TP]
     l.THCudaHalfTensor_copyCuda.argtypes = [P, TP, TP]
 
 
@@ -233,8 +249,7 @@ class Tensor(object):
         """Contiguous device tensor with the shape and values of `arr`."""
         arr = np.ascontiguousarray(arr)
         if kind is None:
-            kind = {np.dtype(np.float32): "float", np.dtype(np.float16): "half",
-                    np.dtype(np.int64): "long"}[arr.dtype]
+            kind = {np.dtype(t[3]): k for k, t in _TYPES.items()}[arr.dtype]
         t = cls(kind)
         if arr.ndim > 0 and arr.size > 0:
             t.resize(arr.shape)
@@ -395,6 +410,18 @@ class Tensor(object):
 
     def lerp(self, a, b, w):
         return self._call("lerp", self.h, a.h, b.h, self._real(w))
+
+    def copy_from(self, src):            # type-converting copy, any kind to any kind
+        return self._call("copyCuda" + _COPY_SUFFIX[src.kind], self.h, src.h)
+
+    def compare_value(self, cmp, src, v, same_type=False):
+        """self = src (cmp) v as 0/1; self is a Byte tensor unless same_type."""
+        return getattr(lib(), "%s_%sValue%s" % (src.T, cmp, "T" if same_type else ""))(
+            self._st, self.h, src.h, src._real(v)) or _check() or self
+
+    def compare_tensor(self, cmp, a, b, same_type=False):
+        return getattr(lib(), "%s_%sTensor%s" % (a.T, cmp, "T" if same_type else ""))(
+            self._st, self.h, a.h, b.h) or _check() or self
 
     def equal(self, other):
         r = self._fn("equal")(self._st, self.h, other.h)

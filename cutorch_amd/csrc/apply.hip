@@ -16,17 +16,40 @@ int point_op_inputs(PointOp op) {
   switch (op) {
     case PointOp::Fill: return 0;
     case PointOp::Copy: case PointOp::AddC: case PointOp::SubC: case PointOp::MulC:
-    case PointOp::DivC: case PointOp::Pow: case PointOp::Math1: return 1;
+    case PointOp::DivC: case PointOp::Pow: case PointOp::Math1: case PointOp::CmpValue: return 1;
     case PointOp::Add: case PointOp::Sub: case PointOp::Mul: case PointOp::Div:
-    case PointOp::CAdd: case PointOp::Math2: case PointOp::Lerp: return 2;
+    case PointOp::CAdd: case PointOp::Math2: case PointOp::Lerp: case PointOp::CmpTensor: return 2;
     default: return 3;
   }
 }
 
 bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* out, AnyTensor* in0,
                      AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap, MathFn fn, float value2) {
+  const ApplyDesc d{dt, dt, op, (int)fn, scalar_of(value), scalar_of(value2), ignoreOverlap};
+  return pointwise_apply(s, d, out, in0, in1, in2);
+}
+
+namespace {
+// Ops on byte/char/short/int/long/double, and Math ops outside the float
+// family's own code range, run on the code-dispatched functors.
+template <typename Fn>
+void for_wide_type(DType dt, Fn&& fn) {
+  switch (dt) {
+    case DType::U8: fn(uint8_t{}); break;
+    case DType::I8: fn(int8_t{}); break;
+    case DType::I16: fn(int16_t{}); break;
+    case DType::I32: fn(int32_t{}); break;
+    case DType::I64: fn(int64_t{}); break;
+    case DType::F64: fn(double{}); break;
+    default: raise_error("unexpected element type");
+  }
+}
+}  // namespace
+
+bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor* in0, AnyTensor* in1,
+                     AnyTensor* in2) {
   AnyTensor* t[kMaxOps] = {out, in0, in1, in2};
-  const int nops = point_op_inputs(op) + 1;
+  const int nops = point_op_inputs(d.op) + 1;
   const ptrdiff_t n = tensor_numel(out);
   for (int k = 0; k < nops; ++k) {
     if (tensor_numel(t[k]) != n) return false;          // THCApply.cuh:434-439
@@ -36,10 +59,12 @@ bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* 
 
   // An output that addresses one element through several indices is computed
   // into a dense temporary and copied back, last writer wins (:472-489).
-  if (!ignoreOverlap && overlapping(tensor_layout(out))) {
-    TensorRef tmp(s, tensor_new_with_size(s, out->nDimension, out->size, dt));
-    if (!pointwise_apply(s, dt, op, value, tmp.t, in0, in1, in2, true, fn, value2)) return false;
-    copy_tensor(s, dt, out, tmp.t, /*ignoreOverlap=*/true);
+  if (!d.ignoreOverlap && overlapping(tensor_layout(out))) {
+    TensorRef tmp(s, tensor_new_with_size(s, out->nDimension, out->size, d.outDt));
+    ApplyDesc inner = d;
+    inner.ignoreOverlap = true;
+    if (!pointwise_apply(s, inner, tmp.t, in0, in1, in2)) return false;
+    copy_tensor(s, d.outDt, out, tmp.t, /*ignoreOverlap=*/true);
     return true;
   }
 
@@ -48,32 +73,49 @@ bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* 
   pl.numel = n;
   bool sameShape = true;
   for (int k = 0; k < nops; ++k) {
-    pl.ptr[k] = tensor_data(t[k], dt);
+    pl.ptr[k] = tensor_data(t[k], k == 0 ? d.outDt : d.dt);
     pl.lay[k] = tensor_layout(t[k]);
     if (!pl.ptr[k]) raise_error("pointwise apply on a tensor without storage");
     if (k > 0) {
       sameShape = sameShape && pl.lay[k].dims == pl.lay[0].dims;
-      for (int d = 0; sameShape && d < pl.lay[0].dims; ++d)
-        sameShape = pl.lay[k].size[d] == pl.lay[0].size[d];
+      for (int d2 = 0; sameShape && d2 < pl.lay[0].dims; ++d2)
+        sameShape = pl.lay[k].size[d2] == pl.lay[0].size[d2];
     }
   }
-  if (op == PointOp::Copy) {
-    if (dt == DType::F32) apply_copy<uint32_t>(s, pl, sameShape);
-    else if (dt == DType::F16) apply_copy<uint16_t>(s, pl, sameShape);
-    else apply_copy<uint64_t>(s, pl, sameShape);
-  } else if (dt == DType::I64) {
-    raise_error("only copy is available for long tensors");
-  } else {
-    const int g = op_group(op);
-    if (dt == DType::F32) {
-      if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, op, value, fn, value2);
-      else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, op, value, fn, value2);
-      else apply_dispatch_group<float, 2>(s, pl, sameShape, op, value, fn, value2);
-    } else {
-      if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, op, value, fn, value2);
-      else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, op, value, fn, value2);
-      else apply_dispatch_group<__half, 2>(s, pl, sameShape, op, value, fn, value2);
+  const DType dt = d.dt;
+  const bool floatFamilyFn =
+      (d.op != PointOp::Math1 && d.op != PointOp::Math2) || d.fn <= (int)MathFn::SqDiff;
+  if (d.op == PointOp::Copy) {
+    switch (dtype_size(dt)) {
+      case 1: apply_copy<uint8_t>(s, pl, sameShape); break;
+      case 2: apply_copy<uint16_t>(s, pl, sameShape); break;
+      case 4: apply_copy<uint32_t>(s, pl, sameShape); break;
+      default: apply_copy<uint64_t>(s, pl, sameShape); break;
     }
+  } else if (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor) {
+    if (d.outDt != dt && d.outDt != DType::U8) raise_error("comparison output must be Byte or the input type");
+    if (dt == DType::F32) apply_cmp<float>(s, pl, sameShape, d);
+    else if (dt == DType::F16) apply_cmp<__half>(s, pl, sameShape, d);
+    else for_wide_type(dt, [&](auto tag) { apply_cmp<decltype(tag)>(s, pl, sameShape, d); });
+  } else if (d.outDt != dt) {
+    raise_error("pointwise op cannot change the element type");
+  } else if ((dt == DType::F32 || dt == DType::F16) && floatFamilyFn) {
+    const int g = op_group(d.op);
+    const float value = (float)d.v.f, value2 = (float)d.w.f;
+    const MathFn fn = (MathFn)d.fn;
+    if (dt == DType::F32) {
+      if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, d.op, value, fn, value2);
+      else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, d.op, value, fn, value2);
+      else apply_dispatch_group<float, 2>(s, pl, sameShape, d.op, value, fn, value2);
+    } else {
+      if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, d.op, value, fn, value2);
+      else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, d.op, value, fn, value2);
+      else apply_dispatch_group<__half, 2>(s, pl, sameShape, d.op, value, fn, value2);
+    }
+  } else if (dt == DType::F32 || dt == DType::F16) {
+    raise_error("pointwise op not available for this element type");
+  } else {
+    for_wide_type(dt, [&](auto tag) { apply_wide<decltype(tag)>(s, pl, sameShape, d); });
   }
   THC_CHECK(hipGetLastError());
   return true;
@@ -91,40 +133,6 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
   }
   if (!pointwise_apply(s, dt, PointOp::Copy, 0.f, dst, src, nullptr, nullptr, ignoreOverlap))
     raise_arg_error(2, "%s", kDimWarning);
-}
-
-// ------------------------------------------------------------------------
-// fp16 <-> fp32 copies
-// ------------------------------------------------------------------------
-template <typename D, typename S>
-__global__ __launch_bounds__(kBlock) void convert_kernel(D* dst, const S* src, uint64_t n) {
-  const uint64_t step = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += step)
-    dst[i] = Cvt<D>::down(Cvt<S>::up(src[i]));
-}
-
-void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src) {
-  const ptrdiff_t n = tensor_numel(dst);
-  THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");
-  if (n == 0) return;
-  TensorRef cs(s, tensor_new_contiguous(s, src, srcT));
-  const bool direct = tensor_is_contiguous(dst);
-  TensorRef cd(s, direct ? (tensor_retain(dst), dst)
-                         : tensor_new_with_size(s, dst->nDimension, dst->size, dstT));
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((n + kBlock * 4 - 1) / (kBlock * 4), 1 << 20));
-  hipStream_t st = current_stream(s);
-  if (dstT == DType::F32 && srcT == DType::F16)
-    hipLaunchKernelGGL((convert_kernel<float, __half>), dim3(grid), dim3(kBlock), 0, st,
-                       (float*)tensor_data(cd.t, dstT), (const __half*)tensor_data(cs.t, srcT),
-                       (uint64_t)n);
-  else if (dstT == DType::F16 && srcT == DType::F32)
-    hipLaunchKernelGGL((convert_kernel<__half, float>), dim3(grid), dim3(kBlock), 0, st,
-                       (__half*)tensor_data(cd.t, dstT), (const float*)tensor_data(cs.t, srcT),
-                       (uint64_t)n);
-  else
-    raise_error("unsupported conversion");
-  THC_CHECK(hipGetLastError());
-  if (!direct) copy_tensor(s, dstT, dst, cd.t, false);
 }
 
 }  // namespace thc

@@ -159,10 +159,13 @@ struct OpMath2 {
 // ------------------------------------------------------------------------
 // contig: flat streaming, one 16-byte pack per operand per step
 // ------------------------------------------------------------------------
-template <typename T, typename Op, int VEC, int UNROLL, bool NT>
-__global__ __launch_bounds__(kBlock) void apply_contig_kernel(T* out, const T* in0, const T* in1,
+// TOut differs from T only for ops that change the element type (comparisons
+// into a Byte tensor); the output pack then has VEC elements of TOut.
+template <typename T, typename Op, int VEC, int UNROLL, bool NT, typename TOut = T>
+__global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T* in0, const T* in1,
                                                               const T* in2, uint64_t n, Op op) {
   using P = Pack<T, VEC>;
+  using PO = Pack<TOut, VEC>;
   const uint64_t npack = n / VEC;
   const uint64_t step = (uint64_t)gridDim.x * (kBlock * UNROLL);
   for (uint64_t base = (uint64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x; base < npack;
@@ -181,10 +184,10 @@ __global__ __launch_bounds__(kBlock) void apply_contig_kernel(T* out, const T* i
     for (int u = 0; u < UNROLL; ++u) {
       const uint64_t i = base + (uint64_t)u * kBlock;
       if (i < npack) {
-        P r;
+        PO r;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) r.v[e] = op(a[u].v[e], b[u].v[e], c[u].v[e]);
-        store_pack<false>(reinterpret_cast<P*>(out) + i, r);
+        store_pack<false>(reinterpret_cast<PO*>(out) + i, r);
       }
     }
   }
@@ -211,11 +214,12 @@ struct IndexedArgs {
 
 // JOINT = all operands share sizes (one division chain); VEC packs along the
 // innermost dim (then that dim's size is already divided by VEC on the host).
-template <typename T, typename Op, typename I, int VEC, bool JOINT>
-__global__ __launch_bounds__(kBlock) void apply_indexed_kernel(T* out, const T* in0, const T* in1,
+template <typename T, typename Op, typename I, int VEC, bool JOINT, typename TOut = T>
+__global__ __launch_bounds__(kBlock) void apply_indexed_kernel(TOut* out, const T* in0, const T* in1,
                                                                const T* in2, I total,
                                                                IndexedArgs<I> args, Op op) {
   using P = Pack<T, VEC>;
+  using PO = Pack<TOut, VEC>;
   constexpr int NOPS = Op::NIN + 1;
   const I step = (I)gridDim.x * kBlock;
   for (I lin = (I)blockIdx.x * kBlock + threadIdx.x; lin < total; lin += step) {
@@ -248,10 +252,10 @@ __global__ __launch_bounds__(kBlock) void apply_indexed_kernel(T* out, const T* 
     if (Op::NIN > 0) a = load_pack<true>(reinterpret_cast<const P*>(in0 + off[1]));
     if (Op::NIN > 1) b = load_pack<true>(reinterpret_cast<const P*>(in1 + off[2]));
     if (Op::NIN > 2) c = load_pack<true>(reinterpret_cast<const P*>(in2 + off[3]));
-    P r;
+    PO r;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) r.v[e] = op(a.v[e], b.v[e], c.v[e]);
-    store_pack<false>(reinterpret_cast<P*>(out + off[0]), r);
+    store_pack<false>(reinterpret_cast<PO*>(out + off[0]), r);
   }
 }
 
@@ -465,6 +469,13 @@ template <typename T>
 inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }
+// Operand k of a plan whose inputs are T and whose output (k == 0) is TOut:
+// aligned for packs of 16 / sizeof(T) elements.
+template <typename T, typename TOut>
+inline bool pack_aligned(const Plan& pl, int k) {
+  const size_t bytes = (16 / sizeof(T)) * (k == 0 ? sizeof(TOut) : sizeof(T));
+  return (reinterpret_cast<uintptr_t>(pl.ptr[k]) & (bytes - 1)) == 0;
+}
 
 inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* key, int default_per_cu) {
   const int64_t blocks = (work_items + per_block - 1) / per_block;
@@ -472,12 +483,13 @@ inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* 
   return (int)std::max<int64_t>(1, std::min(blocks, cap));
 }
 
-template <typename T, typename Op>
+// LEAN: one unroll variant only (element types off the hot path).
+template <typename T, typename Op, typename TOut = T, bool LEAN = false>
 void launch_contig(THCState* s, const Plan& pl, Op op) {
   constexpr int VEC = 16 / sizeof(T);
   bool vec = true;
-  for (int k = 0; k < pl.nops; ++k) vec = vec && aligned16<T>(pl.ptr[k]);
-  T* out = (T*)pl.ptr[0];
+  for (int k = 0; k < pl.nops; ++k) vec = vec && pack_aligned<T, TOut>(pl, k);
+  TOut* out = (TOut*)pl.ptr[0];
   const T* i0 = (const T*)pl.ptr[1];
   const T* i1 = (const T*)pl.ptr[2];
   const T* i2 = (const T*)pl.ptr[3];
@@ -494,25 +506,30 @@ void launch_contig(THCState* s, const Plan& pl, Op op) {
     const int64_t blk = (packs + kBlock * UU - 1) / (kBlock * UU);
     const int gr = (int)std::max<int64_t>(1, std::min<int64_t>(blk, tuning("apply.contig.max_grid", 1 << 20)));
     if (vec && nt)
-      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true>), dim3(gr), dim3(kBlock), 0, st,
-                         out, i0, i1, i2, n, op);
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut>), dim3(gr), dim3(kBlock),
+                         0, st, out, i0, i1, i2, n, op);
     else if (vec)
-      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, false>), dim3(gr), dim3(kBlock), 0, st,
-                         out, i0, i1, i2, n, op);
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, false, TOut>), dim3(gr), dim3(kBlock),
+                         0, st, out, i0, i1, i2, n, op);
     else
-      hipLaunchKernelGGL((apply_contig_kernel<T, Op, 1, UU, false>), dim3(gr), dim3(kBlock), 0, st,
-                         out, i0, i1, i2, n, op);
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, 1, UU, false, TOut>), dim3(gr), dim3(kBlock), 0,
+                         st, out, i0, i1, i2, n, op);
   };
-  if (unroll >= 4)
-    launch(std::integral_constant<int, 4>{});
-  else if (unroll == 1)
-    launch(std::integral_constant<int, 1>{});
-  else
+  if constexpr (LEAN) {
+    (void)unroll;
     launch(std::integral_constant<int, 2>{});
+  } else {
+    if (unroll >= 4)
+      launch(std::integral_constant<int, 4>{});
+    else if (unroll == 1)
+      launch(std::integral_constant<int, 1>{});
+    else
+      launch(std::integral_constant<int, 2>{});
+  }
   note_kernel(vec ? "contig" : "contig-scalar");
 }
 
-template <typename T, typename Op, typename I, bool JOINT>
+template <typename T, typename Op, typename I, bool JOINT, typename TOut = T>
 void launch_indexed(THCState* s, const Plan& pl, Op op) {
   constexpr int VEC = 16 / sizeof(T);
   IndexedArgs<I> args{};
@@ -521,7 +538,7 @@ void launch_indexed(THCState* s, const Plan& pl, Op op) {
     const int nd = pl.lay[0].dims;
     vec = vec && pl.lay[0].size[nd - 1] % VEC == 0;
     for (int k = 0; k < pl.nops && vec; ++k) {
-      vec = aligned16<T>(pl.ptr[k]) && pl.lay[k].stride[nd - 1] == 1;
+      vec = pack_aligned<T, TOut>(pl, k) && pl.lay[k].stride[nd - 1] == 1;
       for (int d = 0; d < nd - 1 && vec; ++d) vec = pl.lay[k].stride[d] % VEC == 0;
     }
   }
@@ -543,17 +560,17 @@ void launch_indexed(THCState* s, const Plan& pl, Op op) {
   const int64_t total = pl.numel / pack;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((total + kBlock - 1) / kBlock,
                                                                tuning("apply.indexed.max_grid", 1 << 22)));
-  T* out = (T*)pl.ptr[0];
+  TOut* out = (TOut*)pl.ptr[0];
   const T* i0 = (const T*)pl.ptr[1];
   const T* i1 = (const T*)pl.ptr[2];
   const T* i2 = (const T*)pl.ptr[3];
   hipStream_t st = current_stream(s);
   if (vec) {
-    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, VEC, JOINT>), dim3(grid), dim3(kBlock), 0, st,
-                       out, i0, i1, i2, (I)total, args, op);
+    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, VEC, JOINT, TOut>), dim3(grid), dim3(kBlock),
+                       0, st, out, i0, i1, i2, (I)total, args, op);
   } else {
-    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, 1, JOINT>), dim3(grid), dim3(kBlock), 0, st,
-                       out, i0, i1, i2, (I)total, args, op);
+    hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, 1, JOINT, TOut>), dim3(grid), dim3(kBlock), 0,
+                       st, out, i0, i1, i2, (I)total, args, op);
   }
   note_kernel(JOINT ? (vec ? "strided" : "strided-scalar") : "generic");
 }
@@ -702,7 +719,10 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
   return true;
 }
 
-template <typename T, typename Op>
+// TILED = false keeps an op off the LDS-tiled kernels (transposed operands then
+// go through the strided kernel); LEAN trims launch variants. Both exist to
+// bound the number of kernels built for element types off the hot path.
+template <typename T, typename Op, typename TOut = T, bool TILED = true, bool LEAN = false>
 void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
   bool wide = force_64bit_index();
   for (int k = 0; k < pl.nops; ++k) {
@@ -713,24 +733,26 @@ void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
     bool flat = pl.lay[0].dims == 1;
     for (int k = 0; k < pl.nops && flat; ++k) flat = pl.lay[k].stride[0] == 1;
     if (flat) {
-      launch_contig<T>(s, pl, op);
+      launch_contig<T, Op, TOut, LEAN>(s, pl, op);
       return;
     }
-    if (tuning("apply.tiled.enable", 1)) {
-      if (wide ? launch_tiled<T, Op, uint64_t>(s, pl, op) : launch_tiled<T, Op, uint32_t>(s, pl, op))
-        return;
+    if constexpr (TILED && std::is_same<T, TOut>::value) {
+      if (tuning("apply.tiled.enable", 1)) {
+        if (wide ? launch_tiled<T, Op, uint64_t>(s, pl, op) : launch_tiled<T, Op, uint32_t>(s, pl, op))
+          return;
+      }
     }
     if (wide)
-      launch_indexed<T, Op, uint64_t, true>(s, pl, op);
+      launch_indexed<T, Op, uint64_t, true, TOut>(s, pl, op);
     else
-      launch_indexed<T, Op, uint32_t, true>(s, pl, op);
+      launch_indexed<T, Op, uint32_t, true, TOut>(s, pl, op);
     return;
   }
   for (int k = 0; k < pl.nops; ++k) collapse(pl.lay[k]);
   if (wide)
-    launch_indexed<T, Op, uint64_t, false>(s, pl, op);
+    launch_indexed<T, Op, uint64_t, false, TOut>(s, pl, op);
   else
-    launch_indexed<T, Op, uint32_t, false>(s, pl, op);
+    launch_indexed<T, Op, uint32_t, false, TOut>(s, pl, op);
 }
 
 

@@ -25,5 +25,11 @@ void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, flo
                           float w);
 template <typename T>
 void apply_copy(THCState* s, Plan& pl, bool sameShape);
+// Code-dispatched functors for the element types without dedicated slices
+// (apply_w_*.hip) and the comparison ops of every type.
+template <typename T>
+void apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d);
+template <typename T>
+void apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d);
 
 }  // namespace thc

@@ -1,0 +1,7 @@
+// Apply-engine slice: element type double (arithmetic family and comparisons).
+#include "apply_wide.hpp"
+
+namespace thc {
+template void apply_wide<double>(THCState*, Plan&, bool, const ApplyDesc&);
+template void apply_cmp<double>(THCState*, Plan&, bool, const ApplyDesc&);
+}

@@ -1,0 +1,7 @@
+// Apply-engine slice: element type int32_t (arithmetic family and comparisons).
+#include "apply_wide.hpp"
+
+namespace thc {
+template void apply_wide<int32_t>(THCState*, Plan&, bool, const ApplyDesc&);
+template void apply_cmp<int32_t>(THCState*, Plan&, bool, const ApplyDesc&);
+}

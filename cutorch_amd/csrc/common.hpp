@@ -58,10 +58,29 @@ constexpr const char* kDimWarning =
     "tensor too large or too many (>25) dimensions";  // THCTensorInfo.cuh:14-16
 
 // ------------------------------------------------------------ data types --
-enum class DType : int { F32 = 0, F16 = 1, I64 = 2 };
+// The eight element types of the reference (THCGenerateAllTypes.h:9-16).
+enum class DType : int { F32 = 0, F16 = 1, I64 = 2, U8 = 3, I8 = 4, I16 = 5, I32 = 6, F64 = 7 };
+constexpr int kNumDTypes = 8;
 inline size_t dtype_size(DType t) {
-  return t == DType::F32 ? 4 : (t == DType::F16 ? 2 : 8);
+  switch (t) {
+    case DType::U8: case DType::I8: return 1;
+    case DType::F16: case DType::I16: return 2;
+    case DType::F32: case DType::I32: return 4;
+    default: return 8;
+  }
 }
+inline bool dtype_is_float(DType t) { return t == DType::F32 || t == DType::F16 || t == DType::F64; }
+
+// A scalar argument (`real value`) carried in both forms, so that integer
+// types keep all 64 bits and floating types keep double precision.
+struct Scalar {
+  double f;
+  int64_t i;
+};
+inline Scalar scalar_of(double v) { return Scalar{v, (int64_t)v}; }
+inline Scalar scalar_of(float v) { return Scalar{(double)v, (int64_t)v}; }
+inline Scalar scalar_of(long v) { return Scalar{(double)v, (int64_t)v}; }
+inline Scalar scalar_of(int v) { return Scalar{(double)v, (int64_t)v}; }
 
 // Type-erased views of THCuda*Storage / THCuda*Tensor (all element types
 // share one field layout, generic/THCStorage.h:9-19, generic/THCTensor.h:7-19).
@@ -194,7 +213,11 @@ enum class PointOp : int {
   Math1,    // out = f(in0 [, v, w]) with f chosen by a MathFn code
   Math2,    // out = f(in0, in1) with f chosen by a MathFn code
   Lerp,     // out = in0 + v * (in1 - in0)
+  CmpValue,   // out = in0 (cmp) v  as 0/1, cmp chosen by a CmpFn code; out may be a Byte tensor
+  CmpTensor,  // out = in0 (cmp) in1
 };
+// Comparison codes (THCTensorMathCompare.cuh:10-74, THCTensorMathCompareT.cuh:10-66)
+enum class CmpFn : int { LT, GT, LE, GE, EQ, NE };
 
 // Function codes of the code-dispatched functors (one kernel set serves the
 // whole family; the switch is uniform and the kernels are memory-bound).
@@ -209,7 +232,10 @@ enum class MathFn : int {
   MaxValue, MinValue, FmodValue, RemainderValue,   // x (op) v
   // binary (generic/THCTensorMathPointwise.cu:345-560)
   CPow, CMax, CMin, CFmod, CRemainder, Atan2, Equal,
-  SqDiff      // (a - b)^2
+  SqDiff,     // (a - b)^2
+  // shifts and bitwise ops (THCTensorMathPairwise.cu:408-560, THCTensorMathPointwise.cuh:462-620)
+  LShiftValue, RShiftValue, BitAndValue, BitOrValue, BitXorValue,   // x (op) v
+  CLShift, CRShift, CBitAnd, CBitOr, CBitXor                        // a (op) b
 };
 int point_op_inputs(PointOp op);
 
@@ -218,7 +244,22 @@ int point_op_inputs(PointOp op);
 bool pointwise_apply(THCState* s, DType dt, PointOp op, float value, AnyTensor* out,
                      AnyTensor* in0, AnyTensor* in1, AnyTensor* in2, bool ignoreOverlap = false,
                      MathFn fn = MathFn::Abs, float value2 = 0.f);
+// General form: any element type, scalars at full width, and an output type
+// that may differ from the inputs' (comparisons into a Byte tensor). `fn` is a
+// MathFn or, for the Cmp ops, a CmpFn code.
+struct ApplyDesc {
+  DType dt;           // element type of the inputs
+  DType outDt;        // element type of the output
+  PointOp op;
+  int fn;
+  Scalar v, w;
+  bool ignoreOverlap;
+};
+bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor* in0, AnyTensor* in1,
+                     AnyTensor* in2);
 void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ignoreOverlap);
+// dst = (dst's type) src, C conversion rules, half through float
+// (THC_copyTensor with differing types, lib/THC/THCTensorCopy.cu:24-205)
 void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src);
 
 // --------------------------------------------------------- reduce engine --

@@ -1,0 +1,110 @@
+// Type-converting copies between any two of the eight element types.
+//
+// Role of THC_copyTensor with differing source and destination types
+// (lib/THC/THCTensorCopy.cu:24-205, the copyCuda<Type> entries of
+// generic/THCTensorCopy.h:16-24). The conversion itself is a flat streaming
+// kernel over dense operands; strided operands are densified or scattered by
+// the same-type copy of the apply engine (which owns the transposing kernels),
+// so a strided conversion costs up to two extra passes instead of 64 more
+// instantiations of every strided kernel.
+// Values convert as C casts do (float -> integer truncates toward zero), half
+// goes through float.
+#include <type_traits>
+
+#include "common.hpp"
+#include "device_util.hpp"
+
+namespace thc {
+namespace {
+
+template <typename D, typename S>
+__device__ __forceinline__ D convert_value(S x) {
+  if constexpr (std::is_same<S, __half>::value) {
+    const float f = __half2float(x);
+    if constexpr (std::is_same<D, __half>::value) return x;
+    else return (D)f;
+  } else if constexpr (std::is_same<D, __half>::value) {
+    return __float2half_rn((float)x);
+  } else {
+    return (D)x;
+  }
+}
+
+// N consecutive elements per lane as one load and one store.
+template <typename D, typename S, int N>
+__global__ __launch_bounds__(kBlock) void convert_kernel(D* __restrict__ dst,
+                                                         const S* __restrict__ src, uint64_t n) {
+  using PS = Pack<S, N>;
+  using PD = Pack<D, N>;
+  const uint64_t packs = n / N;
+  const uint64_t step = (uint64_t)gridDim.x * kBlock;
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < packs; i += step) {
+    const PS v = reinterpret_cast<const PS*>(src)[i];
+    PD r;
+#pragma unroll
+    for (int e = 0; e < N; ++e) r.v[e] = convert_value<D, S>(v.v[e]);
+    reinterpret_cast<PD*>(dst)[i] = r;
+  }
+  const uint64_t tail = packs * N + (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (N > 1 && tail < n) dst[tail] = convert_value<D, S>(src[tail]);
+}
+
+template <typename D, typename S>
+void launch_convert(THCState* s, void* dst, const void* src, int64_t n) {
+  constexpr int N = 8;
+  const bool vec = (reinterpret_cast<uintptr_t>(dst) % (N * sizeof(D)) == 0) &&
+                   (reinterpret_cast<uintptr_t>(src) % (N * sizeof(S)) == 0);
+  const int64_t items = vec ? n / N + 1 : n;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((items + kBlock - 1) / kBlock, 1 << 20));
+  hipStream_t st = current_stream(s);
+  if (vec)
+    hipLaunchKernelGGL((convert_kernel<D, S, N>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
+                       (const S*)src, (uint64_t)n);
+  else
+    hipLaunchKernelGGL((convert_kernel<D, S, 1>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
+                       (const S*)src, (uint64_t)n);
+}
+
+template <typename Fn>
+void with_type(DType dt, Fn&& fn) {
+  switch (dt) {
+    case DType::U8: fn(uint8_t{}); break;
+    case DType::I8: fn(int8_t{}); break;
+    case DType::I16: fn(int16_t{}); break;
+    case DType::I32: fn(int32_t{}); break;
+    case DType::I64: fn(int64_t{}); break;
+    case DType::F16: fn(__half{}); break;
+    case DType::F32: fn(float{}); break;
+    case DType::F64: fn(double{}); break;
+  }
+}
+
+}  // namespace
+
+void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor* src) {
+  if (dstT == srcT) {
+    copy_tensor(s, dstT, dst, src, false);
+    return;
+  }
+  const ptrdiff_t n = tensor_numel(dst);
+  THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
+  if (n == 0) return;
+  // The flat kernel pairs elements by logical linear index, which is what a
+  // dense tensor's memory order is.
+  TensorRef cs(s, tensor_new_contiguous(s, src, srcT));
+  const bool direct = tensor_is_contiguous(dst);
+  TensorRef cd(s, direct ? (tensor_retain(dst), dst)
+                         : tensor_new_with_size(s, dst->nDimension, dst->size, dstT));
+  void* dp = tensor_data(cd.t, dstT);
+  const void* sp = tensor_data(cs.t, srcT);
+  with_type(dstT, [&](auto dtag) {
+    with_type(srcT, [&](auto stag) {
+      launch_convert<decltype(dtag), decltype(stag)>(s, dp, sp, (int64_t)n);
+    });
+  });
+  THC_CHECK(hipGetLastError());
+  note_kernel("convert");
+  if (!direct) copy_tensor(s, dstT, dst, cd.t, false);
+}
+
+}  // namespace thc

@@ -35,6 +35,10 @@ template <>
 struct RawBits<2> {
   typedef uint16_t type;
 };
+template <>
+struct RawBits<1> {
+  typedef uint8_t type;
+};
 
 // Streaming access: every byte of these kernels is touched once. Measured on
 // MI355X with a flat 3-read-1-write fp32 stream over 1 GiB: plain loads and

@@ -547,9 +547,46 @@ THC_AMD_DEFINE_TENSOR_API(THCudaStorage, THCudaTensor, float, DType::F32)
 THC_AMD_DEFINE_TENSOR_API(THCudaHalfStorage, THCudaHalfTensor, THHalf, DType::F16)
 THC_AMD_DEFINE_TENSOR_API(THCudaLongStorage, THCudaLongTensor, long, DType::I64)
 
-THC_API void THCudaTensor_copyCudaHalf(THCState* s, THCudaTensor* self, THCudaHalfTensor* src) {
-  THC_GUARD_VOID(convert_copy(s, DType::F32, TN(self), DType::F16, TN(src)))
-}
+THC_AMD_DEFINE_TENSOR_API(THCudaByteStorage, THCudaByteTensor, unsigned char, DType::U8)
+THC_AMD_DEFINE_TENSOR_API(THCudaCharStorage, THCudaCharTensor, char, DType::I8)
+THC_AMD_DEFINE_TENSOR_API(THCudaShortStorage, THCudaShortTensor, short, DType::I16)
+THC_AMD_DEFINE_TENSOR_API(THCudaIntStorage, THCudaIntTensor, int, DType::I32)
+THC_AMD_DEFINE_TENSOR_API(THCudaDoubleStorage, THCudaDoubleTensor, double, DType::F64)
+
+#define THC_AMD_DEFINE_COPY_API(Tensor, DT)                                                        \
+  THC_API void Tensor##_copyCudaByte(THCState* s, Tensor* self, THCudaByteTensor* src) {           \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::U8, TN(src)))                              \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaChar(THCState* s, Tensor* self, THCudaCharTensor* src) {           \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::I8, TN(src)))                              \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaShort(THCState* s, Tensor* self, THCudaShortTensor* src) {         \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::I16, TN(src)))                             \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaInt(THCState* s, Tensor* self, THCudaIntTensor* src) {             \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::I32, TN(src)))                             \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaLong(THCState* s, Tensor* self, THCudaLongTensor* src) {           \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::I64, TN(src)))                             \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaFloat(THCState* s, Tensor* self, THCudaTensor* src) {              \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::F32, TN(src)))                             \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaDouble(THCState* s, Tensor* self, THCudaDoubleTensor* src) {       \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::F64, TN(src)))                             \
+  }                                                                                                \
+  THC_API void Tensor##_copyCudaHalf(THCState* s, Tensor* self, THCudaHalfTensor* src) {           \
+    THC_GUARD_VOID(convert_copy(s, DT, TN(self), DType::F16, TN(src)))                             \
+  }
+THC_AMD_DEFINE_COPY_API(THCudaByteTensor, DType::U8)
+THC_AMD_DEFINE_COPY_API(THCudaCharTensor, DType::I8)
+THC_AMD_DEFINE_COPY_API(THCudaShortTensor, DType::I16)
+THC_AMD_DEFINE_COPY_API(THCudaIntTensor, DType::I32)
+THC_AMD_DEFINE_COPY_API(THCudaLongTensor, DType::I64)
+THC_AMD_DEFINE_COPY_API(THCudaTensor, DType::F32)
+THC_AMD_DEFINE_COPY_API(THCudaDoubleTensor, DType::F64)
+THC_AMD_DEFINE_COPY_API(THCudaHalfTensor, DType::F16)
+
 THC_API void THCudaHalfTensor_copyCuda(THCState* s, THCudaHalfTensor* self, THCudaTensor* src) {
   THC_GUARD_VOID(convert_copy(s, DType::F16, TN(self), DType::F32, TN(src)))
 }

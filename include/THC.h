@@ -153,6 +153,11 @@ typedef struct _THCDeviceAllocator {          /* THCGeneral.h.in:48-55 */
 THC_AMD_DECLARE_STRUCTS(THCudaStorage, THCudaTensor, float)
 THC_AMD_DECLARE_STRUCTS(THCudaHalfStorage, THCudaHalfTensor, THHalf)
 THC_AMD_DECLARE_STRUCTS(THCudaLongStorage, THCudaLongTensor, long)
+THC_AMD_DECLARE_STRUCTS(THCudaByteStorage, THCudaByteTensor, unsigned char)
+THC_AMD_DECLARE_STRUCTS(THCudaCharStorage, THCudaCharTensor, char)
+THC_AMD_DECLARE_STRUCTS(THCudaShortStorage, THCudaShortTensor, short)
+THC_AMD_DECLARE_STRUCTS(THCudaIntStorage, THCudaIntTensor, int)
+THC_AMD_DECLARE_STRUCTS(THCudaDoubleStorage, THCudaDoubleTensor, double)
 
 /* ------------------------------------------------------------------------ */
 /* Storage and tensor management. generic/THCStorage.h:22-61,                 */
@@ -242,9 +247,34 @@ THC_AMD_DECLARE_STRUCTS(THCudaLongStorage, THCudaLongTensor, long)
 THC_AMD_DECLARE_TENSOR_API(THCudaStorage, THCudaTensor, float)
 THC_AMD_DECLARE_TENSOR_API(THCudaHalfStorage, THCudaHalfTensor, THHalf)
 THC_AMD_DECLARE_TENSOR_API(THCudaLongStorage, THCudaLongTensor, long)
+THC_AMD_DECLARE_TENSOR_API(THCudaByteStorage, THCudaByteTensor, unsigned char)
+THC_AMD_DECLARE_TENSOR_API(THCudaCharStorage, THCudaCharTensor, char)
+THC_AMD_DECLARE_TENSOR_API(THCudaShortStorage, THCudaShortTensor, short)
+THC_AMD_DECLARE_TENSOR_API(THCudaIntStorage, THCudaIntTensor, int)
+THC_AMD_DECLARE_TENSOR_API(THCudaDoubleStorage, THCudaDoubleTensor, double)
 
-/* Type-converting device copies. generic/THCTensorCopy.h:14-24 */
-THC_API void THCudaTensor_copyCudaHalf(THCState *, THCudaTensor *self, THCudaHalfTensor *src);
+/* Type-converting device copies, every destination type from every source  */
+/* type: THCTensor_(copyCudaByte) ... (copyCudaHalf),                        */
+/* generic/THCTensorCopy.h:16-24. Values convert as C casts do; half goes    */
+/* through float. (THCudaTensor_copyCudaFloat etc. are plain copies.)        */
+#define THC_AMD_DECLARE_COPY_API(Tensor)                                       \
+  THC_API void Tensor##_copyCudaByte(THCState *, Tensor *self, THCudaByteTensor *src);     \
+  THC_API void Tensor##_copyCudaChar(THCState *, Tensor *self, THCudaCharTensor *src);     \
+  THC_API void Tensor##_copyCudaShort(THCState *, Tensor *self, THCudaShortTensor *src);   \
+  THC_API void Tensor##_copyCudaInt(THCState *, Tensor *self, THCudaIntTensor *src);       \
+  THC_API void Tensor##_copyCudaLong(THCState *, Tensor *self, THCudaLongTensor *src);     \
+  THC_API void Tensor##_copyCudaFloat(THCState *, Tensor *self, THCudaTensor *src);        \
+  THC_API void Tensor##_copyCudaDouble(THCState *, Tensor *self, THCudaDoubleTensor *src); \
+  THC_API void Tensor##_copyCudaHalf(THCState *, Tensor *self, THCudaHalfTensor *src);
+THC_AMD_DECLARE_COPY_API(THCudaByteTensor)
+THC_AMD_DECLARE_COPY_API(THCudaCharTensor)
+THC_AMD_DECLARE_COPY_API(THCudaShortTensor)
+THC_AMD_DECLARE_COPY_API(THCudaIntTensor)
+THC_AMD_DECLARE_COPY_API(THCudaLongTensor)
+THC_AMD_DECLARE_COPY_API(THCudaTensor)
+THC_AMD_DECLARE_COPY_API(THCudaDoubleTensor)
+THC_AMD_DECLARE_COPY_API(THCudaHalfTensor)
+/* generic/THCTensorCopy.h:35 for the half tensor */
 THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCudaTensor *src);
 
 /* ------------------------------------------------------------------------ */
@@ -361,6 +391,131 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
   THC_API accreal Tensor##_normall(THCState *, Tensor *self, real p);          \
   THC_API real Tensor##_minall(THCState *, Tensor *self);                      \
   THC_API real Tensor##_maxall(THCState *, Tensor *self);
+
+/* ------------------------------------------------------------------------ */
+/* Comparisons, every element type. Output 0/1 in a Byte tensor             */
+/* (generic/THCTensorMathCompare.h:5-10, generic/THCTensorMathCompareT.h:5-10) */
+/* or in a tensor of the input type (the ...T forms, same files :12-17).     */
+/* The output is resized to the input's sizes.                               */
+/* ------------------------------------------------------------------------ */
+#define THC_AMD_DECLARE_ONE_COMPARE(TT, real, name)                        \
+  THC_API void TT##_##name##Value(THCState *, THCudaByteTensor *self,      \
+                                      TT *src, real value);                \
+  THC_API void TT##_##name##ValueT(THCState *, TT *self, TT *src,  \
+                                       real value);                            \
+  THC_API void TT##_##name##Tensor(THCState *, THCudaByteTensor *self,     \
+                                       TT *src1, TT *src2);            \
+  THC_API void TT##_##name##TensorT(THCState *, TT *self, TT *src1,\
+                                        TT *src2);
+#define THC_AMD_DECLARE_COMPARE_API(Tensor, real)                              \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, lt)                                \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, gt)                                \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, le)                                \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, ge)                                \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, eq)                                \
+  THC_AMD_DECLARE_ONE_COMPARE(Tensor, real, ne)
+THC_AMD_DECLARE_COMPARE_API(THCudaByteTensor, unsigned char)
+THC_AMD_DECLARE_COMPARE_API(THCudaCharTensor, char)
+THC_AMD_DECLARE_COMPARE_API(THCudaShortTensor, short)
+THC_AMD_DECLARE_COMPARE_API(THCudaIntTensor, int)
+THC_AMD_DECLARE_COMPARE_API(THCudaLongTensor, long)
+THC_AMD_DECLARE_COMPARE_API(THCudaTensor, float)
+THC_AMD_DECLARE_COMPARE_API(THCudaDoubleTensor, double)
+THC_AMD_DECLARE_COMPARE_API(THCudaHalfTensor, THHalf)
+
+/* ------------------------------------------------------------------------ */
+/* Pointwise math of the integer types and double: the per-type expansion    */
+/* of generic/THCTensorMathPairwise.h:5-15 (scalar forms),                   */
+/* generic/THCTensorMathPointwise.h:40-67 (tensor forms, addcmul/addcdiv)    */
+/* and generic/THCTensorMath.h:5-6 (fill, zero). Integer arithmetic wraps    */
+/* in the element type as C does; fmod takes the sign of the dividend,       */
+/* remainder the sign of the divisor.                                        */
+/* ------------------------------------------------------------------------ */
+#define THC_AMD_DECLARE_WIDE_API(Tensor, real)                                 \
+  THC_API void Tensor##_add(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_sub(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_mul(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_div(THCState *, Tensor *self, Tensor *src, real v);    \
+  THC_API void Tensor##_fmod(THCState *, Tensor *self, Tensor *src, real v);   \
+  THC_API void Tensor##_remainder(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_lshift(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_rshift(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_cmaxValue(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_cminValue(THCState *, Tensor *self, Tensor *src,       \
+                                  real v);                                     \
+  THC_API void Tensor##_abs(THCState *, Tensor *self, Tensor *src);            \
+  THC_API void Tensor##_sign(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_clamp(THCState *, Tensor *self, Tensor *src, real lo,  \
+                              real hi);                                        \
+  THC_API void Tensor##_cadd(THCState *, Tensor *self, Tensor *src1, real v,   \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_csub(THCState *, Tensor *self, Tensor *src1, real v,   \
+                             Tensor *src2);                                    \
+  THC_API void Tensor##_cmul(THCState *, Tensor *self, Tensor *a, Tensor *b);  \
+  THC_API void Tensor##_cdiv(THCState *, Tensor *self, Tensor *a, Tensor *b);  \
+  THC_API void Tensor##_cpow(THCState *, Tensor *self, Tensor *a, Tensor *b);  \
+  THC_API void Tensor##_cmax(THCState *, Tensor *self, Tensor *a, Tensor *b);  \
+  THC_API void Tensor##_cmin(THCState *, Tensor *self, Tensor *a, Tensor *b);  \
+  THC_API void Tensor##_cfmod(THCState *, Tensor *self, Tensor *a, Tensor *b); \
+  THC_API void Tensor##_cremainder(THCState *, Tensor *self, Tensor *a,        \
+                                   Tensor *b);                                 \
+  THC_API void Tensor##_clshift(THCState *, Tensor *self, Tensor *a,           \
+                                Tensor *b);                                    \
+  THC_API void Tensor##_crshift(THCState *, Tensor *self, Tensor *a,           \
+                                Tensor *b);                                    \
+  THC_API void Tensor##_addcmul(THCState *, Tensor *self, Tensor *t, real v,   \
+                                Tensor *src1, Tensor *src2);                   \
+  THC_API void Tensor##_addcdiv(THCState *, Tensor *self, Tensor *t, real v,   \
+                                Tensor *src1, Tensor *src2);                   \
+  THC_API void Tensor##_fill(THCState *, Tensor *self, real v);                \
+  THC_API void Tensor##_zero(THCState *, Tensor *self);
+#define THC_AMD_DECLARE_BITS_API(Tensor, real)                                 \
+  THC_API void Tensor##_bitand(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_bitor(THCState *, Tensor *self, Tensor *src, real v);  \
+  THC_API void Tensor##_bitxor(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_cbitand(THCState *, Tensor *self, Tensor *a,           \
+                                Tensor *b);                                    \
+  THC_API void Tensor##_cbitor(THCState *, Tensor *self, Tensor *a, Tensor *b);\
+  THC_API void Tensor##_cbitxor(THCState *, Tensor *self, Tensor *a,           \
+                                Tensor *b);
+THC_AMD_DECLARE_WIDE_API(THCudaByteTensor, unsigned char)
+THC_AMD_DECLARE_WIDE_API(THCudaCharTensor, char)
+THC_AMD_DECLARE_WIDE_API(THCudaShortTensor, short)
+THC_AMD_DECLARE_WIDE_API(THCudaIntTensor, int)
+THC_AMD_DECLARE_WIDE_API(THCudaLongTensor, long)
+THC_AMD_DECLARE_WIDE_API(THCudaDoubleTensor, double)
+THC_AMD_DECLARE_BITS_API(THCudaByteTensor, unsigned char)
+THC_AMD_DECLARE_BITS_API(THCudaCharTensor, char)
+THC_AMD_DECLARE_BITS_API(THCudaShortTensor, short)
+THC_AMD_DECLARE_BITS_API(THCudaIntTensor, int)
+THC_AMD_DECLARE_BITS_API(THCudaLongTensor, long)
+/* neg: signed types only (generic/THCTensorMathPointwise.h:37-42) */
+THC_API void THCudaCharTensor_neg(THCState *, THCudaCharTensor *self, THCudaCharTensor *src);
+THC_API void THCudaShortTensor_neg(THCState *, THCudaShortTensor *self, THCudaShortTensor *src);
+THC_API void THCudaIntTensor_neg(THCState *, THCudaIntTensor *self, THCudaIntTensor *src);
+THC_API void THCudaLongTensor_neg(THCState *, THCudaLongTensor *self, THCudaLongTensor *src);
+THC_API void THCudaDoubleTensor_neg(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src);
+/* double: the floating-point family (generic/THCTensorMathPointwise.h:5-35) */
+#define THC_AMD_DECLARE_DOUBLE_UNARY(name)                                     \
+  THC_API void THCudaDoubleTensor_##name(THCState *, THCudaDoubleTensor *self, \
+                                         THCudaDoubleTensor *src);
+THC_AMD_DECLARE_DOUBLE_UNARY(sigmoid) THC_AMD_DECLARE_DOUBLE_UNARY(log)
+THC_AMD_DECLARE_DOUBLE_UNARY(lgamma) THC_AMD_DECLARE_DOUBLE_UNARY(log1p)
+THC_AMD_DECLARE_DOUBLE_UNARY(exp) THC_AMD_DECLARE_DOUBLE_UNARY(cos)
+THC_AMD_DECLARE_DOUBLE_UNARY(acos) THC_AMD_DECLARE_DOUBLE_UNARY(cosh)
+THC_AMD_DECLARE_DOUBLE_UNARY(sin) THC_AMD_DECLARE_DOUBLE_UNARY(asin)
+THC_AMD_DECLARE_DOUBLE_UNARY(sinh) THC_AMD_DECLARE_DOUBLE_UNARY(tan)
+THC_AMD_DECLARE_DOUBLE_UNARY(atan) THC_AMD_DECLARE_DOUBLE_UNARY(tanh)
+THC_AMD_DECLARE_DOUBLE_UNARY(sqrt) THC_AMD_DECLARE_DOUBLE_UNARY(rsqrt)
+THC_AMD_DECLARE_DOUBLE_UNARY(ceil) THC_AMD_DECLARE_DOUBLE_UNARY(floor)
+THC_AMD_DECLARE_DOUBLE_UNARY(round) THC_AMD_DECLARE_DOUBLE_UNARY(trunc)
+THC_AMD_DECLARE_DOUBLE_UNARY(frac) THC_AMD_DECLARE_DOUBLE_UNARY(cinv)
+THC_API void THCudaDoubleTensor_pow(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, double v);
+THC_API void THCudaDoubleTensor_tpow(THCState *, THCudaDoubleTensor *self, double v, THCudaDoubleTensor *src);
+THC_API void THCudaDoubleTensor_atan2(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *tx, THCudaDoubleTensor *ty);
+THC_API void THCudaDoubleTensor_lerp(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *a, THCudaDoubleTensor *b, double w);
 
 THC_AMD_DECLARE_MATH_API(THCudaTensor, float, float)
 THC_AMD_DECLARE_MATH_API(THCudaHalfTensor, THHalf, float)

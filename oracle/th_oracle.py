@@ -18,13 +18,21 @@ LIB_PATH = os.path.join(_HERE, "libth_oracle.so")
 
 OPS = {"copy": 0, "addc": 1, "subc": 2, "mulc": 3, "divc": 4, "add": 5, "sub": 6, "mul": 7,
        "div": 8, "cadd": 9, "addcmul": 10, "addcdiv": 11, "fill": 12, "pow": 13}
+DTYPES = {"float": 0, "half": 1, "long": 2, "byte": 3, "char": 4, "short": 5, "int": 6, "double": 7}
+NP_OF = {"float": np.float32, "half": np.float16, "long": np.int64, "byte": np.uint8, "char": np.int8,
+         "short": np.int16, "int": np.int32, "double": np.float64}
+KIND_OF = {np.dtype(v): k for k, v in NP_OF.items()}
+CMPS = {"lt": 0, "gt": 1, "le": 2, "ge": 3, "eq": 4, "ne": 5}
 FNS = ["sigmoid", "log", "lgamma", "log1p", "exp", "cos", "acos", "cosh", "sin", "asin", "sinh", "tan",
        "atan", "tanh", "sqrt", "rsqrt", "ceil", "floor", "round", "trunc", "frac", "cinv", "neg", "abs",
        "sign", "clamp", "sqdiffValue", "pow", "tpow", "cmaxValue", "cminValue", "fmod", "remainder",
-       "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal", "sqdiff"]
+       "cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal", "sqdiff",
+       "lshift", "rshift", "bitand", "bitor", "bitxor", "clshift", "crshift", "cbitand", "cbitor", "cbitxor"]
+BINARY_FNS = {"cpow", "cmax", "cmin", "cfmod", "cremainder", "atan2", "equal", "sqdiff", "clshift", "crshift",
+              "cbitand", "cbitor", "cbitxor"}
 OPS["lerp"] = 14
 for _i, _n in enumerate(FNS):
-    OPS["fn:" + _n] = (200 if _i >= FNS.index("cpow") else 100) + _i
+    OPS["fn:" + _n] = (200 if _n in BINARY_FNS else 100) + _i
 KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "norm": 4, "mean": 5, "var_biased": 6, "var": 7,
          "std_biased": 8, "std": 9}
 
@@ -64,6 +72,10 @@ def lib():
             f = getattr(l, "th_var_all_" + suffix)
             f.argtypes = [VP, C.c_int]
             f.restype = C.c_double
+        l.th_typed_pointwise.argtypes = [C.c_int, C.c_int, C.c_int, C.c_double, C.c_long, C.c_double, C.c_long,
+                                         VP, VP, VP, VP]
+        l.th_typed_compare.argtypes = [C.c_int, C.c_int, C.c_int, C.c_double, C.c_long, VP, VP, VP]
+        l.th_typed_convert.argtypes = [C.c_int, VP, C.c_int, VP]
         l.th_half2float.argtypes = [C.c_uint16]
         l.th_half2float.restype = C.c_float
         l.th_float2half.argtypes = [C.c_float]
@@ -77,7 +89,7 @@ def lib():
 
 
 class View(object):
-    """A strided view on a host storage array (float32, float16 or int64)."""
+    """A strided view on a host storage array (any of the eight element types)."""
 
     def __init__(self, storage, offset=0, size=None, stride=None):
         assert storage.flags["C_CONTIGUOUS"] and storage.ndim == 1
@@ -114,6 +126,10 @@ class View(object):
     def is_half(self):
         return self.storage.dtype == np.float16
 
+    @property
+    def kind(self):
+        return KIND_OF[self.storage.dtype]
+
     def numpy(self):
         """Logical contents, gathered through numpy's own stride machinery."""
         if not self.size:
@@ -137,6 +153,48 @@ def pointwise(op, out, a=None, b=None, c=None, value=0.0, value2=0.0):
     if rc:
         raise ValueError("sizes do not match")
     return out
+
+
+def _int_scalar(kind, v):
+    """The scalar as the element type holds it (wrapped), as a Python int."""
+    if kind in ("float", "half", "double"):
+        return 0
+    return int(np.array(int(v)).astype(NP_OF[kind]))
+
+
+def typed_pointwise(op, out, a=None, b=None, c=None, value=0, value2=0):
+    """Pointwise op on byte/char/short/int/long/double views. `op` as for
+    pointwise(): a name from OPS or "fn:<name>"."""
+    kind = out.kind
+    code = OPS[op]
+    fn = 0
+    if code >= 200:
+        code, fn = 200, code - 200
+    elif code >= 100:
+        code, fn = 100, code - 100
+    rc = lib().th_typed_pointwise(DTYPES[kind], code, fn, float(value), _int_scalar(kind, value),
+                                  float(value2), _int_scalar(kind, value2), _ptr(out), _ptr(a), _ptr(b),
+                                  _ptr(c))
+    if rc:
+        raise ValueError("sizes do not match")
+    return out
+
+
+def typed_compare(cmp, out, a, b=None, value=0):
+    """out = a (cmp) (b or value) as 0/1; out is a byte view or one of a's kind."""
+    kind = a.kind
+    vf = float(np.float16(value)) if kind == "half" else (float(np.float32(value)) if kind == "float" else float(value))
+    rc = lib().th_typed_compare(DTYPES[kind], DTYPES[out.kind], CMPS[cmp], vf, _int_scalar(kind, value),
+                                _ptr(out), _ptr(a), _ptr(b))
+    if rc:
+        raise ValueError("sizes do not match")
+    return out
+
+
+def typed_convert(dst, src):
+    if lib().th_typed_convert(DTYPES[dst.kind], _ptr(dst), DTYPES[src.kind], _ptr(src)):
+        raise ValueError("sizes do not match")
+    return dst
 
 
 def reduced_shape(shape, dim):

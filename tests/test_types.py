@@ -1,0 +1,395 @@
+"""The element types beyond float/half (byte, char, short, int, long, double):
+pointwise arithmetic, comparisons of all eight types, and type-converting
+copies (the per-type expansion of generic/THCTensorMathPairwise.cu,
+generic/THCTensorMathPointwise.cu, generic/THCTensorMathCompare{,T}.cu and the
+copyCuda<Type> entries of generic/THCTensorCopy.h:16-24).
+
+CPU half: the oracle (oracle/th_oracle_types.c) is pinned against numpy's
+fixed-width integer arithmetic, float64 ufuncs and astype casts.
+GPU half: the engine against the oracle, bit for bit on whole storages
+(transcendental double functions within 4 ulp)."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal, contiguous_geometry, random_geometry
+
+INT_KINDS = ["byte", "char", "short", "int", "long"]
+WIDE_KINDS = INT_KINDS + ["double"]
+ALL_KINDS = WIDE_KINDS + ["float", "half"]
+
+
+def np_of(oracle, kind):
+    return oracle.NP_OF[kind]
+
+
+def minus_one(dt):
+    return np.array(-1, np.int64).astype(dt)
+
+
+def rand_storage(rng, kind, n, oracle, small=False):
+    dt = np_of(oracle, kind)
+    if kind in ("double", "float", "half"):
+        return rng.uniform(-4, 4, n).astype(dt)
+    info = np.iinfo(dt)
+    if small:
+        return rng.integers(max(info.min, -9), min(info.max, 9) + 1, n).astype(dt)
+    pick = rng.integers(0, 3, n)
+    wide = rng.integers(info.min, info.max, n, dtype=np.int64 if dt != np.uint8 else np.int64).astype(dt)
+    narrow = rng.integers(max(info.min, -100), min(info.max, 100) + 1, n).astype(dt)
+    edge = rng.choice(np.array([info.min, info.max, 0, 1, info.max - 1], dtype=dt), n)
+    return np.where(pick == 0, wide, np.where(pick == 1, narrow, edge)).astype(dt)
+
+
+def trunc_div(a, b):
+    """C integer division (toward zero) on numpy integer arrays, exact."""
+    a64, b64 = a.astype(object), b.astype(object) if isinstance(b, np.ndarray) else int(b)
+    q = np.frompyfunc(lambda x, y: 0 if y == 0 else (abs(x) // abs(y)) * (1 if (x < 0) == (y < 0) else -1), 2, 1)(a64, b64)
+    return np.array(q, dtype=object)
+
+
+def wrap(obj_arr, dt):
+    bits = np.iinfo(dt).bits
+    m = np.frompyfunc(lambda x: int(x) & ((1 << bits) - 1), 1, 1)(obj_arr)
+    return np.array(m, dtype=np.uint64).astype({8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]).view(
+        {8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]).astype(dt) if dt == np.uint8 else \
+        np.array(m, dtype=np.uint64).astype({8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[bits]).view(dt)
+
+
+# --------------------------------------------------------------- oracle pins --
+@pytest.mark.parametrize("kind", INT_KINDS)
+def test_oracle_integer_arithmetic_matches_numpy(oracle, kind):
+    rng = np.random.default_rng(7)
+    dt = np_of(oracle, kind)
+    n = 4000
+    a, b, c = (rand_storage(rng, kind, n, oracle) for _ in range(3))
+    bnz = np.where(b == 0, dt(3), b)
+    V = oracle.View
+    v = int(dt(7))
+
+    def run(op, *ins, **kw):
+        return oracle.typed_pointwise(op, V(np.zeros(n, dt)), *[V(x.copy()) for x in ins], **kw).storage
+
+    with np.errstate(over="ignore"):
+        assert_bit_equal(run("add", a, b), a + b)
+        assert_bit_equal(run("sub", a, b), a - b)
+        assert_bit_equal(run("mul", a, b), a * b)
+        assert_bit_equal(run("addc", a, value=v), a + dt(v))
+        assert_bit_equal(run("mulc", a, value=v), a * dt(v))
+        assert_bit_equal(run("cadd", a, b, value=v), a + dt(v) * b)
+        assert_bit_equal(run("addcmul", a, b, c, value=v), a + dt(v) * (b * c))
+        assert_bit_equal(run("div", a, bnz), wrap(trunc_div(a, bnz), dt))
+        assert_bit_equal(run("divc", a, value=v), wrap(trunc_div(a, v), dt))
+        assert_bit_equal(run("addcdiv", a, b, bnz, value=v), a + dt(v) * wrap(trunc_div(b, bnz), dt))
+        # numpy has the same two conventions: fmod = sign of dividend, remainder = sign of divisor
+        safe = bnz if kind == "byte" else np.where(bnz == -1, dt(5), bnz)
+        assert_bit_equal(run("fn:cfmod", a, safe), np.fmod(a, safe))
+        assert_bit_equal(run("fn:cremainder", a, safe), np.remainder(a, safe))
+        assert_bit_equal(run("fn:fmod", a, value=v), np.fmod(a, dt(v)))
+        assert_bit_equal(run("fn:remainder", a, value=v), np.remainder(a, dt(v)))
+        assert_bit_equal(run("fn:cmax", a, b), np.maximum(a, b))
+        assert_bit_equal(run("fn:cmin", a, b), np.minimum(a, b))
+        assert_bit_equal(run("fn:cmaxValue", a, value=v), np.maximum(a, dt(v)))
+        assert_bit_equal(run("fn:clamp", a, value=2, value2=50), np.clip(a, dt(2), dt(50)))
+        assert_bit_equal(run("fn:abs", a), np.abs(a))
+        assert_bit_equal(run("fn:sign", a), np.sign(a).astype(dt))
+        if kind != "byte":
+            assert_bit_equal(run("fn:neg", a), -a)
+        assert_bit_equal(run("fn:bitand", a, value=v), a & dt(v))
+        assert_bit_equal(run("fn:bitor", a, value=v), a | dt(v))
+        assert_bit_equal(run("fn:cbitxor", a, b), a ^ b)
+        assert_bit_equal(run("fn:lshift", a, value=3), np.left_shift(a, 3))
+        assert_bit_equal(run("fn:rshift", a, value=2), np.right_shift(a, 2))
+        e = rng.integers(0, 6, n).astype(dt)
+        assert_bit_equal(run("fn:cpow", a, e), np.power(a, e))
+        assert_bit_equal(run("fill", value=v), np.full(n, v, dt))
+
+
+def test_oracle_double_arithmetic_matches_numpy(oracle):
+    rng = np.random.default_rng(8)
+    n = 3000
+    a, b, c = (rng.uniform(-3, 3, n) for _ in range(3))
+    V = oracle.View
+
+    def run(op, *ins, **kw):
+        return oracle.typed_pointwise(op, V(np.zeros(n)), *[V(x.copy()) for x in ins], **kw).storage
+
+    assert_bit_equal(run("add", a, b), a + b)
+    assert_bit_equal(run("div", a, b), a / b)
+    assert_bit_equal(run("cadd", a, b, value=0.3), a + 0.3 * b)
+    assert_bit_equal(run("addcmul", a, b, c, value=0.7), a + 0.7 * (b * c))
+    assert_bit_equal(run("lerp", a, b, value=0.25), a + 0.25 * (b - a))
+    assert_bit_equal(run("fn:sqrt", np.abs(a)), np.sqrt(np.abs(a)))
+    assert_bit_equal(run("fn:floor", a), np.floor(a))
+    assert_bit_equal(run("fn:cfmod", a, b), np.fmod(a, b))
+    assert_bit_equal(run("fn:cremainder", a, b), a - b * np.floor(a / b))
+    assert_bit_equal(run("fn:clamp", a, value=-1.0, value2=0.5), np.clip(a, -1.0, 0.5))
+    np.testing.assert_allclose(run("fn:exp", a), np.exp(a), rtol=4e-16)
+    np.testing.assert_allclose(run("fn:tanh", a), np.tanh(a), rtol=1e-15, atol=1e-300)
+    np.testing.assert_allclose(run("fn:atan2", a, b), np.arctan2(a, b), rtol=1e-15)
+    np.testing.assert_allclose(run("fn:cpow", np.abs(a), b), np.power(np.abs(a), b), rtol=1e-14)
+
+
+@pytest.mark.parametrize("kind", ALL_KINDS)
+def test_oracle_compare_matches_numpy(oracle, kind):
+    rng = np.random.default_rng(9)
+    dt = np_of(oracle, kind)
+    n = 2000
+    a = rand_storage(rng, kind, n, oracle, small=True)
+    b = rand_storage(rng, kind, n, oracle, small=True)
+    ops = {"lt": np.less, "gt": np.greater, "le": np.less_equal, "ge": np.greater_equal, "eq": np.equal,
+           "ne": np.not_equal}
+    v = dt(2)
+    for name, f in ops.items():
+        got = oracle.typed_compare(name, oracle.View(np.zeros(n, np.uint8)), oracle.View(a), oracle.View(b))
+        assert_bit_equal(got.storage, f(a, b).astype(np.uint8), name)
+        got = oracle.typed_compare(name, oracle.View(np.zeros(n, dt)), oracle.View(a), value=v)
+        assert_bit_equal(got.storage, f(a, v).astype(dt), name + " value")
+
+
+def conv_source(rng, oracle, src, dst, n):
+    """Values of kind `src` that convert to `dst` without undefined behaviour."""
+    sdt, ddt = np_of(oracle, src), np_of(oracle, dst)
+    if src in ("float", "double", "half"):
+        if dst in ("float", "double", "half"):
+            return rng.uniform(-1000, 1000, n).astype(sdt)
+        lo, hi = (0, 200) if dst == "byte" else (-100, 100)
+        return rng.uniform(lo, hi, n).astype(sdt)
+    return rand_storage(rng, src, n, oracle, small=(dst == "half"))
+
+
+@pytest.mark.parametrize("src", ALL_KINDS)
+def test_oracle_convert_matches_numpy_astype(oracle, src):
+    rng = np.random.default_rng(10)
+    n = 1500
+    for dst in ALL_KINDS:
+        x = conv_source(rng, oracle, src, dst, n)
+        got = oracle.typed_convert(oracle.View(np.zeros(n, np_of(oracle, dst))), oracle.View(x.copy())).storage
+        if dst == "half" and src == "double":
+            want = x.astype(np.float32).astype(np.float16)      # through float, as the reference does
+        elif dst == "half" and src in INT_KINDS:
+            want = x.astype(np.float32).astype(np.float16)
+        else:
+            want = x.astype(np_of(oracle, dst))
+        assert_bit_equal(got, want, "%s -> %s" % (src, dst))
+
+
+# ------------------------------------------------------------------ GPU parity --
+def dev_ref(thc, oracle, rng, kind, geom, small=False):
+    st = rand_storage(rng, kind, geom[0], oracle, small)
+    return thc.Tensor.from_storage(st, *geom[1:], kind=kind), oracle.View(st.copy(), *geom[1:])
+
+
+def whole(dev, ref, what, ulp=0):
+    got, want = dev.storage_numpy(), ref.storage
+    if ulp == 0:
+        assert_bit_equal(got, want, what)
+    else:
+        ok = np.isclose(got, want, rtol=ulp * 2.3e-16, atol=0, equal_nan=True)
+        assert ok.all(), (what, got[~ok][:3], want[~ok][:3])
+
+
+BIN_OPS = ["add", "sub", "mul", "div", "fn:cmax", "fn:cmin", "fn:cfmod", "fn:cremainder", "fn:cpow",
+           "fn:clshift", "fn:crshift"]
+BIT_OPS = ["fn:cbitand", "fn:cbitor", "fn:cbitxor"]
+GPU_NAME = {"add": "cadd", "sub": "csub", "mul": "cmul", "div": "cdiv"}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_gpu_binary_ops_random_geometry(thc, oracle, kind):
+    rng = np.random.default_rng(100)
+    ops = BIN_OPS + (BIT_OPS if kind != "double" else [])
+    for trial in range(6):
+        nd = int(rng.integers(1, 4))
+        shape = tuple(int(x) for x in rng.integers(1, 40, nd))
+        for op in ops:
+            small = op in ("fn:cpow", "fn:clshift", "fn:crshift")
+            ga, gb, go = (random_geometry(rng, shape, permute=trial % 2 == 1) for _ in range(3))
+            da, ra = dev_ref(thc, oracle, rng, kind, ga, small)
+            db, rb = dev_ref(thc, oracle, rng, kind, gb, small)
+            do, ro = dev_ref(thc, oracle, rng, kind, go)
+            if small and kind != "double":       # exponents / shift counts 0..5
+                stb = rng.integers(0, 6, gb[0]).astype(np_of(oracle, kind))
+                db, rb = thc.Tensor.from_storage(stb, *gb[1:], kind=kind), oracle.View(stb.copy(), *gb[1:])
+            if kind == "double" and op == "fn:cpow":
+                sta = np.abs(ra.storage) + 0.1
+                da, ra = thc.Tensor.from_storage(sta, *ga[1:], kind=kind), oracle.View(sta.copy(), *ga[1:])
+            if op in ("div", "fn:cfmod", "fn:cremainder") and kind != "double":   # keep away from x/0, x%-1
+                stb = rb.storage.copy()
+                stb[(stb == 0) | (stb == minus_one(np_of(oracle, kind)))] = 3
+                db, rb = thc.Tensor.from_storage(stb, *gb[1:], kind=kind), oracle.View(stb.copy(), *gb[1:])
+            name = GPU_NAME.get(op, op.replace("fn:", ""))
+            if name in ("cadd", "csub"):
+                getattr(do, name)(da, 1, db)
+            else:
+                do.binary(name, da, db)
+            oracle.typed_pointwise(op, ro, ra, rb)
+            whole(do, ro, "%s %s %s" % (kind, op, shape), ulp=4 if (kind == "double" and small) else 0)     # pow() on the device vs libm
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_gpu_scalar_unary_ternary_ops(thc, oracle, kind):
+    rng = np.random.default_rng(101)
+    dt = np_of(oracle, kind)
+    v = 3 if kind != "double" else 1.75
+    for trial in range(4):
+        shape = tuple(int(x) for x in rng.integers(1, 50, int(rng.integers(1, 4))))
+        geoms = [random_geometry(rng, shape, permute=trial % 2 == 1) for _ in range(4)]
+        for op, call in (("addc", lambda o, a: o.add(a, v)), ("subc", lambda o, a: o.sub(a, v)),
+                         ("mulc", lambda o, a: o.mul(a, v)), ("divc", lambda o, a: o.div(a, v)),
+                         ("fn:fmod", lambda o, a: o.scalar2("fmod", a, v)),
+                         ("fn:remainder", lambda o, a: o.scalar2("remainder", a, v)),
+                         ("fn:cmaxValue", lambda o, a: o.scalar2("cmaxValue", a, v)),
+                         ("fn:cminValue", lambda o, a: o.scalar2("cminValue", a, v)),
+                         ("fn:lshift", lambda o, a: o.scalar2("lshift", a, v if kind != "double" else 3)),
+                         ("fn:rshift", lambda o, a: o.scalar2("rshift", a, v if kind != "double" else 3))):
+            da, ra = dev_ref(thc, oracle, rng, kind, geoms[0])
+            do, ro = dev_ref(thc, oracle, rng, kind, geoms[1])
+            call(do, da)
+            vv = 3 if (kind == "double" and "shift" in op) else v
+            oracle.typed_pointwise(op, ro, ra, value=vv)
+            whole(do, ro, "%s %s" % (kind, op))
+        for fn in ("abs", "sign") + (("neg",) if kind != "byte" else ()):
+            da, ra = dev_ref(thc, oracle, rng, kind, geoms[0])
+            do, ro = dev_ref(thc, oracle, rng, kind, geoms[1])
+            do.unary(fn, da)
+            oracle.typed_pointwise("fn:" + fn, ro, ra)
+            whole(do, ro, "%s %s" % (kind, fn))
+        da, ra = dev_ref(thc, oracle, rng, kind, geoms[0])
+        do, ro = dev_ref(thc, oracle, rng, kind, geoms[1])
+        do.clamp(da, 2, 60)
+        oracle.typed_pointwise("fn:clamp", ro, ra, value=2, value2=60)
+        whole(do, ro, kind + " clamp")
+        if kind != "double":
+            for name in ("bitand", "bitor", "bitxor"):
+                do.scalar2(name, da, 0x35)
+                oracle.typed_pointwise("fn:" + name, ro, ra, value=0x35)
+                whole(do, ro, kind + " " + name)
+        # cadd / csub with a value, addcmul / addcdiv (out of place and in place on t)
+        db, rb = dev_ref(thc, oracle, rng, kind, geoms[2])
+        dc, rc = dev_ref(thc, oracle, rng, kind, geoms[3])
+        if kind != "double":
+            stc = rc.storage.copy()
+            stc[(stc == 0) | (stc == minus_one(dt))] = 5
+            dc, rc = thc.Tensor.from_storage(stc, *geoms[3][1:], kind=kind), oracle.View(stc.copy(), *geoms[3][1:])
+        do.cadd(da, v, db)
+        oracle.typed_pointwise("cadd", ro, ra, rb, value=v)
+        whole(do, ro, kind + " cadd v")
+        do.csub(da, v, db)
+        oracle.typed_pointwise("cadd", ro, ra, rb, value=-v)
+        whole(do, ro, kind + " csub v")
+        do.addcmul(da, v, db, dc)
+        oracle.typed_pointwise("addcmul", ro, ra, rb, rc, value=v)
+        whole(do, ro, kind + " addcmul")
+        da.addcdiv(da, v, db, dc)
+        oracle.typed_pointwise("addcdiv", ra, ra, rb, rc, value=v)
+        whole(da, ra, kind + " addcdiv in place")
+        do.fill(v)
+        oracle.typed_pointwise("fill", ro, value=v)
+        whole(do, ro, kind + " fill")
+        do.zero()
+        oracle.typed_pointwise("fill", ro, value=0)
+        whole(do, ro, kind + " zero")
+
+
+@pytest.mark.gpu
+def test_gpu_double_math_family(thc, oracle):
+    rng = np.random.default_rng(102)
+    geom = random_geometry(rng, (37, 29))
+    pos = ("log", "sqrt", "rsqrt", "lgamma", "log1p")
+    unit = ("acos", "asin")
+    exact = ("sqrt", "ceil", "floor", "round", "trunc", "frac", "cinv", "neg", "abs", "sign", "rsqrt")
+    for fn in oracle.FNS[:oracle.FNS.index("clamp")]:
+        st = rng.uniform(-3, 3, geom[0])
+        if fn in pos:
+            st = np.abs(st) + 0.05
+        if fn in unit:
+            st = rng.uniform(-1, 1, geom[0])
+        da = thc.Tensor.from_storage(st, *geom[1:], kind="double")
+        ra = oracle.View(st.copy(), *geom[1:])
+        do, ro = dev_ref(thc, oracle, rng, "double", contiguous_geometry((37, 29)))
+        do.unary(fn, da)
+        oracle.typed_pointwise("fn:" + fn, ro, ra)
+        whole(do, ro, "double " + fn, ulp=0 if fn in exact else 8)
+    da, ra = dev_ref(thc, oracle, rng, "double", geom)
+    db, rb = dev_ref(thc, oracle, rng, "double", geom)
+    do, ro = dev_ref(thc, oracle, rng, "double", geom)
+    do.binary("atan2", da, db)
+    oracle.typed_pointwise("fn:atan2", ro, ra, rb)
+    whole(do, ro, "atan2", ulp=8)
+    do.lerp(da, db, 0.3)
+    oracle.typed_pointwise("lerp", ro, ra, rb, value=0.3)
+    whole(do, ro, "lerp")
+    do.pow(da, 2.0)
+    oracle.typed_pointwise("mul", ro, ra, ra)
+    whole(do, ro, "pow 2")
+    do.tpow(1.7, da)
+    oracle.typed_pointwise("fn:tpow", ro, ra, value=1.7)
+    whole(do, ro, "tpow", ulp=8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ALL_KINDS)
+def test_gpu_compare_ops(thc, oracle, kind):
+    rng = np.random.default_rng(103)
+    dt = np_of(oracle, kind)
+    for trial in range(3):
+        shape = tuple(int(x) for x in rng.integers(1, 60, int(rng.integers(1, 4))))
+        ga, gb = (random_geometry(rng, shape, permute=trial == 1) for _ in range(2))
+        da, ra = dev_ref(thc, oracle, rng, kind, ga, small=True)
+        db, rb = dev_ref(thc, oracle, rng, kind, gb, small=True)
+        if kind in ("double", "float", "half"):          # make ties likely
+            sta = np.round(ra.storage * 2) / 2
+            stb = np.round(rb.storage * 2) / 2
+            da, ra = thc.Tensor.from_storage(sta, *ga[1:], kind=kind), oracle.View(sta.astype(dt), *ga[1:])
+            db, rb = thc.Tensor.from_storage(stb, *gb[1:], kind=kind), oracle.View(stb.astype(dt), *gb[1:])
+        for cmp in ("lt", "gt", "le", "ge", "eq", "ne"):
+            out = thc.Tensor("byte").compare_tensor(cmp, da, db)
+            assert out.shape == shape
+            want = oracle.typed_compare(cmp, oracle.View.empty(shape, np.uint8), ra, rb)
+            assert_bit_equal(out.numpy(), want.numpy(), "%s %sTensor" % (kind, cmp))
+            out = thc.Tensor(kind).compare_tensor(cmp, da, db, same_type=True)
+            want = oracle.typed_compare(cmp, oracle.View.empty(shape, dt), ra, rb)
+            assert_bit_equal(out.numpy(), want.numpy(), "%s %sTensorT" % (kind, cmp))
+            out = thc.Tensor("byte").compare_value(cmp, da, 1)
+            want = oracle.typed_compare(cmp, oracle.View.empty(shape, np.uint8), ra, value=1)
+            assert_bit_equal(out.numpy(), want.numpy(), "%s %sValue" % (kind, cmp))
+            out = thc.Tensor(kind).compare_value(cmp, da, 1, same_type=True)
+            want = oracle.typed_compare(cmp, oracle.View.empty(shape, dt), ra, value=1)
+            assert_bit_equal(out.numpy(), want.numpy(), "%s %sValueT" % (kind, cmp))
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("byte").compare_tensor("lt", thc.Tensor.from_numpy(np.zeros(4, dt)),
+                                          thc.Tensor.from_numpy(np.zeros(5, dt)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("src", ALL_KINDS)
+def test_gpu_converting_copies(thc, oracle, src):
+    rng = np.random.default_rng(104)
+    for dst in ALL_KINDS:
+        for shape, strided in (((1000,), False), ((13, 21), True), ((4099,), False)):
+            gs = random_geometry(rng, shape) if strided else contiguous_geometry(shape)
+            gd = random_geometry(rng, shape) if strided else contiguous_geometry(shape)
+            st = conv_source(rng, oracle, src, dst, gs[0])
+            dsrc = thc.Tensor.from_storage(st, *gs[1:], kind=src)
+            rsrc = oracle.View(st.copy(), *gs[1:])
+            std = rand_storage(rng, dst, gd[0], oracle)
+            ddst = thc.Tensor.from_storage(std, *gd[1:], kind=dst)
+            rdst = oracle.View(std.copy(), *gd[1:])
+            ddst.copy_from(dsrc)
+            oracle.typed_convert(rdst, rsrc)
+            assert_bit_equal(ddst.storage_numpy(), rdst.storage, "%s -> %s %s" % (src, dst, shape))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["byte", "short", "int", "double"])
+def test_gpu_same_type_copy_of_transposed_tensors(thc, oracle, kind):
+    rng = np.random.default_rng(105)
+    dt = np_of(oracle, kind)
+    x = rand_storage(rng, kind, 300 * 260, oracle).reshape(300, 260)
+    d = thc.Tensor.from_numpy(x)
+    out = thc.Tensor(kind).resize((260, 300))
+    out.copy(d.t())
+    assert_bit_equal(out.numpy(), np.ascontiguousarray(x.T))
+    assert thc.last_kernel().startswith("tiled")

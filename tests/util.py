@@ -6,7 +6,7 @@ import numpy as np
 
 def bits(a):
     a = np.ascontiguousarray(a)
-    return a.view({2: np.uint16, 4: np.uint32, 8: np.uint64}[a.itemsize])
+    return a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.itemsize])
 
 
 def assert_bit_equal(got, want, what=""):
