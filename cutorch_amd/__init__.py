@@ -187,25 +187,27 @@ def _declare(l):
         opt(T + "_equal", C.c_int, P, TP, TP)
         opt(T + "_fill", None, P, TP, creal)
         opt(T + "_zero", None, P, TP)
-        if kind not in _FLOAT_KINDS:
-            continue
+        acc = C.c_float if kind in _FLOAT_KINDS else (C.c_double if kind == "double" else C.c_long)
         for name in ("sum", "prod", "mean"):
-            f(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int)
-        f(T + "_norm", None, P, TP, TP, creal, C.c_long, C.c_int)
+            opt(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int)
+        opt(T + "_norm", None, P, TP, TP, creal, C.c_long, C.c_int)
         for name in ("max", "min"):
-            f(T + "_" + name, None, P, TP, LT, TP, C.c_long, C.c_int)
+            opt(T + "_" + name, None, P, TP, LT, TP, C.c_long, C.c_int)
         for name in ("sumall", "prodall", "meanall"):
-            f(T + "_" + name, C.c_float, P, TP)
+            opt(T + "_" + name, acc, P, TP)
         for name in ("cumsum", "cumprod"):
-            f(T + "_" + name, None, P, TP, TP, C.c_long)
+            opt(T + "_" + name, None, P, TP, TP, C.c_long)
         for name in ("var", "std"):
-            f(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int, C.c_int)
+            opt(T + "_" + name, None, P, TP, TP, C.c_long, C.c_int, C.c_int)
         for name in ("varall", "stdall"):
-            f(T + "_" + name, C.c_float, P, TP, C.c_int)
-        f(T + "_dist", C.c_float, P, TP, TP, creal)
-        f(T + "_normall", C.c_float, P, TP, creal)
+            opt(T + "_" + name, acc, P, TP, C.c_int)
+        opt(T + "_dist", acc, P, TP, TP, creal)
+        opt(T + "_normall", acc, P, TP, creal)
         for name in ("minall", "maxall"):
-            f(T + "_" + name, creal, P, TP)
+            opt(T + "_" + name, creal, P, TP)
+        opt(T + "_renorm", None, P, TP, TP, creal, C.c_long, creal)
+    l.THCudaByteTensor_logicalall.argtypes = [P, TP]
+    l.THCudaByteTensor_logicalany.argtypes = [P, TP]
     l.THCudaHalfTensor_copyCuda.argtypes = [P, TP, TP]
 
 
@@ -489,6 +491,16 @@ class Tensor(object):
     def _real_out(self, r):
         if self.kind == "half":
             return float(np.array(r, dtype=np.uint16).view(np.float16))
+        return r
+
+    def logicalall(self):
+        r = lib().THCudaByteTensor_logicalall(self._st, self.h)
+        _check()
+        return r
+
+    def logicalany(self):
+        r = lib().THCudaByteTensor_logicalany(self._st, self.h)
+        _check()
         return r
 
     def minall(self):

@@ -266,12 +266,13 @@ void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor
 // SqDev: sum of (x - p)^2 (second pass of varall, generic/THCTensorMathReduce.cu:122-144)
 // SqDevOut: sum of (x - c)^2 where c is what the output element holds on entry (the slice's
 //           mean: second sweep of var/std along a dim, THCTensorMathReduce.cuh:268-445)
-enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev, SqDevOut };
+// All / Any: logical and / or of a Byte tensor (THCTensorMathReduce.cuh:118-130)
+enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev, SqDevOut, All, Any };
 // DivBy / DivBySqrt take their divisor from the `p` argument of reduce_dim.
 enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 
 // out[..., 0, ...] = reduce over dim (THC_reduceDim, lib/THC/THCReduce.cuh:263-453)
-bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* out,
+bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTensor* out,
                 AnyTensor* in, int dim, int keepdim);
 // (value, 1-based index) of the max/min along dim, lowest index on ties
 // (THC_reduceDimIndex, lib/THC/THCTensorMathReduce.cuh:619-661)
@@ -280,6 +281,9 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
 // Whole-tensor reduction returned on the host; blocks on a 4-byte D2H copy
 // (THC_reduceAll, lib/THC/THCReduceAll.cuh:239-342)
 bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result);
+// Any element type; the result arrives as accreal: .f for the floating types,
+// .i for the integer types (long accumulation).
+bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Scalar* result);
 
 // Inclusive prefix sum / product along `dim` (THCTensor_(scanDim),
 // lib/THC/generic/THCTensorMathScan.cu:76-110)

@@ -15,6 +15,7 @@
 //   generic/THCTensorMathReduce.cu:400-436    max min
 //   generic/THCTensorMathScan.cu:76-126       cumsum cumprod
 #include <cfloat>
+#include <climits>
 #include <cmath>
 
 #include "common.hpp"
@@ -110,14 +111,14 @@ int tensors_equal(THCState* s, DType dt, AnyTensor* a, AnyTensor* b) {
   return r != 0.f;
 }
 
-void reduce_or_throw(THCState* s, DType dt, ReduceOp op, Epilogue ep, float p, AnyTensor* self,
+void reduce_or_throw(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTensor* self,
                      AnyTensor* src, long dim, int keepdim) {
   same_gpu(s, {self, src});
   if (!reduce_dim(s, dt, op, ep, p, self, src, (int)dim, keepdim))
     raise_arg_error(2, "%s", kDimWarning);
 }
 
-void norm_dim(THCState* s, DType dt, float p, AnyTensor* self, AnyTensor* src, long dim,
+void norm_dim(THCState* s, DType dt, double p, AnyTensor* self, AnyTensor* src, long dim,
               int keepdim) {
   if (p == 0.f)
     reduce_or_throw(s, dt, ReduceOp::Norm0, Epilogue::None, p, self, src, dim, keepdim);
@@ -157,7 +158,7 @@ void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* sr
   // Second sweep: sum of (x - mean)^2 per slice. The kernels take each slice's
   // centre from the output element itself, so the sweep runs in place on the
   // tensor of means (no temporary of the input's size, input read twice in all).
-  const float div = (float)(biased ? n : n - 1);
+  const double div = (double)(biased ? n : n - 1);
   if (!reduce_dim(s, dt, ReduceOp::SqDevOut, wantStd ? Epilogue::DivBySqrt : Epilogue::DivBy, div,
                   mean.t, src, (int)dim, 1))
     raise_arg_error(2, "%s", kDimWarning);
@@ -453,3 +454,148 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
 
 THC_AMD_DEFINE_MATH_API(THCudaTensor, float, DType::F32, FLT_MAX)
 THC_AMD_DEFINE_MATH_API(THCudaHalfTensor, THHalf, DType::F16, 65504.f)
+
+// ------------------------------------------------------------------------
+// Reductions of the integer types and double: the per-type expansion of
+// generic/THCTensorMathReduce.h:18-45 (sum prod mean, the *all forms, min max
+// with indices, minall maxall, dist), generic/THCTensorMathPairwise.h:17
+// (equal) and, for double, :5-16 (norm, var, std and their *all forms).
+// accreal is long for the integer types (sums wrap in 64 bits, the stored
+// result wraps in the element type) and double for double.
+// ------------------------------------------------------------------------
+namespace {
+
+Scalar all_scalar(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* self) {
+  same_gpu(s, {self});
+  Scalar r{0.0, 0};
+  if (!reduce_all(s, dt, op, p, self, &r)) raise_arg_error(1, "%s", kDimWarning);
+  return r;
+}
+template <typename R>
+R pick(const Scalar& v);
+template <>
+inline long pick<long>(const Scalar& v) { return (long)v.i; }
+template <>
+inline double pick<double>(const Scalar& v) { return v.f; }
+
+double norm_all_d(THCState* s, AnyTensor* self, double p) {
+  const DType dt = DType::F64;
+  if (p == 0.0) return all_scalar(s, dt, ReduceOp::Norm0, p, self).f;
+  if (p == 1.0) return all_scalar(s, dt, ReduceOp::Norm1, p, self).f;
+  if (p == 2.0) return std::sqrt(all_scalar(s, dt, ReduceOp::Norm2, p, self).f);
+  return std::pow(all_scalar(s, dt, ReduceOp::NormP, p, self).f, 1.0 / p);
+}
+double var_all_d(THCState* s, AnyTensor* self, int biased) {
+  THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");
+  const double n = (double)tensor_numel(self);
+  const double mean = all_scalar(s, DType::F64, ReduceOp::Sum, 0.0, self).f / n;
+  return all_scalar(s, DType::F64, ReduceOp::SqDev, mean, self).f / (n - (biased ? 0.0 : 1.0));
+}
+double dist_all_d(THCState* s, AnyTensor* a, AnyTensor* b, double p) {
+  same_gpu(s, {a, b});
+  THC_ARG_CHECK(tensor_numel(a) == tensor_numel(b), 2, "sizes do not match");
+  if (a->nDimension == 0) return 0.0;
+  TensorRef diff(s, tensor_new_with_size(s, a->nDimension, a->size, DType::F64));
+  apply_or_throw(s, DType::F64, PointOp::Sub, 0.f, diff.t, a, b);
+  return std::pow(all_scalar(s, DType::F64, ReduceOp::NormP, p, diff.t).f, 1.0 / p);
+}
+
+}  // namespace
+
+#define THC_AMD_DEFINE_WIDE_REDUCE_API(Tensor, real, accreal, DT, REAL_LOWEST, REAL_MAX)           \
+  THC_API void Tensor##_sum(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {       \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Sum, Epilogue::None, 0.0, TN(self), TN(src),   \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_prod(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {      \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Prod, Epilogue::None, 0.0, TN(self), TN(src),  \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_mean(THCState* s, Tensor* self, Tensor* src, long dim, int keepdim) {      \
+    THC_GUARD_VOID(reduce_or_throw(s, DT, ReduceOp::Sum, Epilogue::DivN, 0.0, TN(self), TN(src),   \
+                                   dim, keepdim))                                                  \
+  }                                                                                                \
+  THC_API void Tensor##_max(THCState* s, Tensor* values, THCudaLongTensor* indices, Tensor* src,   \
+                            long dim, int keepdim) {                                               \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {values, indices, src});                                                         \
+      reduce_dim_index(s, DT, true, TN(values), TN(indices), TN(src), (int)dim, keepdim);          \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_min(THCState* s, Tensor* values, THCudaLongTensor* indices, Tensor* src,   \
+                            long dim, int keepdim) {                                               \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {values, indices, src});                                                         \
+      reduce_dim_index(s, DT, false, TN(values), TN(indices), TN(src), (int)dim, keepdim);         \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API accreal Tensor##_sumall(THCState* s, Tensor* self) {                                     \
+    THC_GUARD_RET((accreal)0, return pick<accreal>(all_scalar(s, DT, ReduceOp::Sum, 0.0, TN(self)))) \
+  }                                                                                                \
+  THC_API accreal Tensor##_prodall(THCState* s, Tensor* self) {                                    \
+    THC_GUARD_RET((accreal)0, return pick<accreal>(all_scalar(s, DT, ReduceOp::Prod, 0.0, TN(self)))) \
+  }                                                                                                \
+  THC_API accreal Tensor##_meanall(THCState* s, Tensor* self) {                                    \
+    THC_GUARD_RET((accreal)0, {                                                                    \
+      THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");                                      \
+      return pick<accreal>(all_scalar(s, DT, ReduceOp::Sum, 0.0, TN(self))) /                      \
+             (accreal)tensor_numel(TN(self));                                                      \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API real Tensor##_minall(THCState* s, Tensor* self) {                                        \
+    THC_GUARD_RET((real)0, {                                                                       \
+      if (self->nDimension == 0) return (real)REAL_MAX;                                            \
+      return (real)pick<accreal>(all_scalar(s, DT, ReduceOp::Min, 0.0, TN(self)));                 \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API real Tensor##_maxall(THCState* s, Tensor* self) {                                        \
+    THC_GUARD_RET((real)0, {                                                                       \
+      if (self->nDimension == 0) return (real)REAL_LOWEST;                                         \
+      return (real)pick<accreal>(all_scalar(s, DT, ReduceOp::Max, 0.0, TN(self)));                 \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API int Tensor##_equal(THCState* s, Tensor* self, Tensor* src) {                             \
+    THC_GUARD_RET(0, return tensors_equal(s, DT, TN(self), TN(src)))                               \
+  }
+
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaByteTensor, unsigned char, long, DType::U8, 0, 255)
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaCharTensor, char, long, DType::I8, -128, 127)
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaShortTensor, short, long, DType::I16, -32768, 32767)
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaIntTensor, int, long, DType::I32, INT_MIN, INT_MAX)
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaLongTensor, long, long, DType::I64, LONG_MIN, LONG_MAX)
+THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaDoubleTensor, double, double, DType::F64, -DBL_MAX, DBL_MAX)
+
+// lib/THC/THCTensorMathReduce.cu:3-32
+THC_API int THCudaByteTensor_logicalall(THCState* s, THCudaByteTensor* self) {
+  THC_GUARD_RET(0, return (int)all_scalar(s, DType::U8, ReduceOp::All, 0.0, TN(self)).i)
+}
+THC_API int THCudaByteTensor_logicalany(THCState* s, THCudaByteTensor* self) {
+  THC_GUARD_RET(0, return (int)all_scalar(s, DType::U8, ReduceOp::Any, 0.0, TN(self)).i)
+}
+
+// double: the floating-point reductions
+THC_API void THCudaDoubleTensor_norm(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
+                                     double p, long dim, int keepdim) {
+  THC_GUARD_VOID(norm_dim(s, DType::F64, p, TN(self), TN(src), dim, keepdim))
+}
+THC_API void THCudaDoubleTensor_var(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
+                                    long dim, int biased, int keepdim) {
+  THC_GUARD_VOID(var_dim(s, DType::F64, false, TN(self), TN(src), dim, biased, keepdim))
+}
+THC_API void THCudaDoubleTensor_std(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
+                                    long dim, int biased, int keepdim) {
+  THC_GUARD_VOID(var_dim(s, DType::F64, true, TN(self), TN(src), dim, biased, keepdim))
+}
+THC_API double THCudaDoubleTensor_normall(THCState* s, THCudaDoubleTensor* self, double p) {
+  THC_GUARD_RET(0.0, return norm_all_d(s, TN(self), p))
+}
+THC_API double THCudaDoubleTensor_varall(THCState* s, THCudaDoubleTensor* self, int biased) {
+  THC_GUARD_RET(0.0, return var_all_d(s, TN(self), biased))
+}
+THC_API double THCudaDoubleTensor_stdall(THCState* s, THCudaDoubleTensor* self, int biased) {
+  THC_GUARD_RET(0.0, return std::sqrt(var_all_d(s, TN(self), biased)))
+}
+THC_API double THCudaDoubleTensor_dist(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
+                                       double p) {
+  THC_GUARD_RET(0.0, return dist_all_d(s, TN(self), TN(src), p))
+}

@@ -1,0 +1,9 @@
+// Reduce-engine slice: element type __half.
+#include "reduce_impl.hpp"
+
+namespace thc {
+template void reduce_dim_type<__half>(THCState*, const ReduceGeom&, const void*, void*, ReduceOp, Epilogue,
+                                  double, double);
+template void reduce_index_type<__half>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
+template void reduce_all_type<__half>(THCState*, ReduceGeom, const void*, ReduceOp, double, Scalar*);
+}

@@ -1,0 +1,1229 @@
+// Dimension and whole-tensor reductions for gfx950 (wave64).
+//
+// Role of THC_reduceDim / THC_reduceAll / THC_reduceDimIndex and their kernels
+// (lib/THC/THCReduce.cuh:35-453, THCReduceAll.cuh:28-342,
+// THCTensorMathReduce.cuh:453-661). Redesigned around three access shapes:
+//
+//   rows   the reduced dim has stride 1. A group of G lanes (G = 1..64, a power
+//          of two chosen from the row length) owns one row, streams it with
+//          16-byte loads and finishes with an xor-butterfly inside the wave.
+//          Long rows with few siblings are cut into chunks ("virtual rows");
+//          the per-chunk partials land in scratch and a second launch of the
+//          same kernel folds them. reduceAll is the one-row case of this.
+//   cols   the reduced dim is strided and another dim has stride 1 (reducing
+//          a non-innermost dim of a dense tensor). Lanes run along the
+//          unit-stride dim with 16-byte loads, thread rows and, if the output
+//          is too small to fill 256 CUs, extra workgroups split the reduced
+//          dim; LDS folds the thread rows, a tiny second kernel folds the
+//          workgroup partials in a fixed order (bit-reproducible).
+//   generic  anything else: one thread per output walks the reduced dim.
+//
+// Accumulation is fp32 for float and half input (accreal = float,
+// THCGenerateFloatType.h:5-8, THCGenerateHalfType.h:9-10); results are rounded
+// once on store. max/min carry (value, index) pairs whose combine step prefers
+// the lower index on equal values at every level, so the first occurrence wins
+// as in a sequential scan; the first NaN wins over everything.
+#pragma once
+#include <cmath>
+#include <limits>
+#include <type_traits>
+
+#include "common.hpp"
+#include "device_util.hpp"
+#include "reduce_plan.hpp"
+
+namespace thc {
+
+namespace {
+
+// ----------------------------------------------------- accumulator types --
+// accreal of the reference (THCGenerate*Type.h): float for float and half,
+// double for double, long for the integer types.
+template <typename T>
+struct Acc {
+  using type = int64_t;
+};
+template <>
+struct Acc<float> {
+  using type = float;
+};
+template <>
+struct Acc<__half> {
+  using type = float;
+};
+template <>
+struct Acc<double> {
+  using type = double;
+};
+
+template <typename A, typename T>
+__device__ __forceinline__ A acc_up(T x) {
+  if constexpr (std::is_same<T, __half>::value) return (A)__half2float(x);
+  else return (A)x;
+}
+template <typename T, typename A>
+__device__ __forceinline__ T acc_down(A a) {
+  if constexpr (std::is_same<T, __half>::value) return __float2half_rn((float)a);
+  else return (T)a;
+}
+__device__ __forceinline__ float sqrt_any(float x) { return sqrtf(x); }
+__device__ __forceinline__ double sqrt_any(double x) { return sqrt(x); }
+__device__ __forceinline__ int64_t sqrt_any(int64_t x) { return x; }
+__device__ __forceinline__ float pow_any(float x, float y) { return powf(x, y); }
+__device__ __forceinline__ double pow_any(double x, double y) { return pow(x, y); }
+__device__ __forceinline__ int64_t pow_any(int64_t x, int64_t) { return x; }
+__device__ __forceinline__ float abs_any(float x) { return fabsf(x); }
+__device__ __forceinline__ double abs_any(double x) { return fabs(x); }
+__device__ __forceinline__ int64_t abs_any(int64_t x) { return x < 0 ? -x : x; }
+// Sums and products of integer types wrap (two's complement).
+template <typename A>
+__device__ __forceinline__ A add_any(A a, A b) {
+  if constexpr (std::is_integral<A>::value) return (A)((uint64_t)a + (uint64_t)b);
+  else return a + b;
+}
+template <typename A>
+__device__ __forceinline__ A mul_any(A a, A b) {
+  if constexpr (std::is_integral<A>::value) return (A)((uint64_t)a * (uint64_t)b);
+  else return a * b;
+}
+// Exchange across lanes; 8-byte values go as two 32-bit halves.
+template <typename A>
+__device__ __forceinline__ A shfl_xor_any(A v, uint32_t o) {
+  if constexpr (sizeof(A) == 8) {
+    uint64_t bits;
+    __builtin_memcpy(&bits, &v, 8);
+    const uint32_t lo = __shfl_xor((uint32_t)bits, o, 64);
+    const uint32_t hi = __shfl_xor((uint32_t)(bits >> 32), o, 64);
+    bits = ((uint64_t)hi << 32) | lo;
+    A r;
+    __builtin_memcpy(&r, &bits, 8);
+    return r;
+  } else {
+    return __shfl_xor(v, o, 64);
+  }
+}
+
+// --------------------------------------------------------------- functors --
+template <typename A>
+struct Epi {
+  int kind;  // Epilogue
+  A arg;     // 1/p for PowInv, n for DivN
+  template <typename T>
+  __device__ __forceinline__ T finish(A acc) const {
+    switch (kind) {
+      case (int)Epilogue::Sqrt: return acc_down<T>(sqrt_any(acc));
+      case (int)Epilogue::PowInv: return acc_down<T>(pow_any(acc, arg));
+      // the sum is rounded (or wrapped) to the element type before the division,
+      // as sum followed by div does (generic/THCTensorMathReduce.cu:37-43)
+      case (int)Epilogue::DivN: return acc_down<T>(acc_up<A>(acc_down<T>(acc)) / arg);
+      case (int)Epilogue::DivBy: return acc_down<T>(acc / arg);
+      case (int)Epilogue::DivBySqrt: return acc_down<T>(sqrt_any(acc / arg));
+      default: return acc_down<T>(acc);
+    }
+  }
+};
+
+template <typename A>
+__device__ __forceinline__ A nan_max(A a, A b) {
+  return (a != a) ? a : ((b != b) ? b : (a > b ? a : b));
+}
+template <typename A>
+__device__ __forceinline__ A nan_min(A a, A b) {
+  return (a != a) ? a : ((b != b) ? b : (a < b ? a : b));
+}
+template <typename A>
+__host__ __device__ __forceinline__ A lowest_of() {
+  if constexpr (std::is_integral<A>::value) return std::numeric_limits<A>::lowest();
+  else return (A)-INFINITY;
+}
+template <typename A>
+__host__ __device__ __forceinline__ A highest_of() {
+  if constexpr (std::is_integral<A>::value) return std::numeric_limits<A>::max();
+  else return (A)INFINITY;
+}
+
+// modify(x, c): c is the centre of the output element that x belongs to. Only
+// a CENTRED functor looks at it; for those the kernels read c from the output
+// location itself before they overwrite it (the caller stores the centres
+// there), which is how var/std subtract a per-slice mean without an extra
+// operand or a temporary of the input's size.
+#define THC_REDUCE_FUNCTOR(Name, CENTRED, INIT, MODIFY, COMBINE)                     \
+  template <typename A_>                                                             \
+  struct Name {                                                                      \
+    using A = A_;                                                                    \
+    static constexpr bool kCentred = CENTRED;                                        \
+    A p;                                                                             \
+    __host__ __device__ __forceinline__ A init() const { return INIT; }              \
+    __device__ __forceinline__ A modify(A x, A c) const {                            \
+      (void)c;                                                                       \
+      return MODIFY;                                                                 \
+    }                                                                                \
+    __device__ __forceinline__ A combine(A a, A b) const { return COMBINE; }         \
+  };
+THC_REDUCE_FUNCTOR(FSum, false, (A)0, x, add_any(a, b))
+THC_REDUCE_FUNCTOR(FProd, false, (A)1, x, mul_any(a, b))
+THC_REDUCE_FUNCTOR(FMax, false, lowest_of<A>(), x, nan_max(a, b))
+THC_REDUCE_FUNCTOR(FMin, false, highest_of<A>(), x, nan_min(a, b))
+THC_REDUCE_FUNCTOR(FNorm0, false, (A)0, (x != (A)0 ? (A)1 : (A)0), a + b)
+THC_REDUCE_FUNCTOR(FNorm1, false, (A)0, abs_any(x), a + b)
+THC_REDUCE_FUNCTOR(FNorm2, false, (A)0, x * x, a + b)
+THC_REDUCE_FUNCTOR(FNormP, false, (A)0, pow_any(abs_any(x), p), a + b)
+THC_REDUCE_FUNCTOR(FSqDev, false, (A)0, (x - p) * (x - p), a + b)
+THC_REDUCE_FUNCTOR(FSqDevOut, true, (A)0, (x - c) * (x - c), a + b)
+// logical all / any of a Byte tensor (THCTensorMathReduce.cuh:118-130)
+THC_REDUCE_FUNCTOR(FAll, false, (A)1, (x != (A)0 ? (A)1 : (A)0), (A)((a != (A)0) && (b != (A)0)))
+THC_REDUCE_FUNCTOR(FAny, false, (A)0, (x != (A)0 ? (A)1 : (A)0), (A)((a != (A)0) || (b != (A)0)))
+#undef THC_REDUCE_FUNCTOR
+
+// (value, index) pairs. `better(a, b)`: a must replace b.
+template <bool IS_MAX, typename V>
+struct PairOrder {
+  static __device__ __forceinline__ V worst() { return IS_MAX ? lowest_of<V>() : highest_of<V>(); }
+  template <typename X>
+  static __device__ __forceinline__ bool better(V av, X ai, V bv, X bi) {
+    const bool an = av != av, bn = bv != bv;
+    if (an || bn) return an && (!bn || ai < bi);
+    return (IS_MAX ? av > bv : av < bv) || (av == bv && ai < bi);
+  }
+  // Same decision when `a` is known to come after `b` in index order (a lane
+  // scanning its elements front to back): ties never replace, a NaN replaces
+  // only a non-NaN.
+  static __device__ __forceinline__ bool better_later(V av, V bv) {
+    return (IS_MAX ? av > bv : av < bv) || ((av != av) && (bv == bv));
+  }
+};
+
+// Coordinates of an output element / a row in the joint (input, output)
+// space of the non-reduced dims.
+template <typename I>
+struct OuterArgs {
+  int dims;
+  Divisor<I> size[kMaxDims];
+  I inStride[kMaxDims];
+  I outStride[kMaxDims];
+  __device__ __forceinline__ void offsets(I lin, I& inOff, I& outOff) const {
+    inOff = 0;
+    outOff = 0;
+    for (int d = dims - 1; d > 0; --d) {
+      I r;
+      size[d].divmod(lin, lin, r);
+      inOff += r * inStride[d];
+      outOff += r * outStride[d];
+    }
+    inOff += lin * inStride[0];
+    outOff += lin * outStride[0];
+  }
+};
+
+// ------------------------------------------------------------------ rows --
+// Virtual row vr = row * S + s covers [s*chunk, min(R, (s+1)*chunk)) of `row`.
+// S == 1: the result goes to out at the row's output offset (with epilogue).
+// S  > 1: the fp32 partial goes to partial[vr].
+template <typename TIn, typename TOut, typename F, typename I, int VEC, bool FIRST>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restrict__ in,
+                                                             TOut* __restrict__ out,
+                                                             typename F::A* __restrict__ partial,
+                                                             OuterArgs<I> oa, I numRows, I R,
+                                                             I sR, Divisor<I> S, I chunk,
+                                                             uint32_t G, Epi<typename F::A> epi, F f) {
+  // sR (element stride of the reduced dim) is honoured by the VEC == 1
+  // instantiation only; packs need sR == 1.
+  using P = Pack<TIn, VEC>;
+  using A = typename F::A;
+  const uint32_t groups = kBlock / G;
+  const uint32_t lane = threadIdx.x % G;
+  const uint32_t grp = threadIdx.x / G;
+  const I total = numRows * S.d;
+  for (I vr0 = (I)blockIdx.x * groups; vr0 < total; vr0 += (I)gridDim.x * groups) {
+    const I vr = vr0 + grp;
+    const bool active = vr < total;
+    A acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+    I outOff = 0;
+    if (active) {
+      I row, s, inOff;
+      S.divmod(vr, row, s);
+      oa.offsets(row, inOff, outOff);
+      const I begin = s * chunk;
+      const I end = min(R, begin + chunk);
+      const TIn* src = in + inOff;
+      A c = (A)0;
+      if constexpr (F::kCentred && FIRST) c = acc_up<A>(out[outOff]);
+      const I es = VEC == 1 ? sR : (I)1;  // element stride
+      // U loads are issued back to back before any of them is consumed.
+      constexpr int U = 8;
+      const I step = (I)G * VEC;
+      I i = begin + lane * VEC;
+      for (; i + (U - 1) * step < end; i += U * step) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
+          }
+        }
+      }
+      for (; i < end; i += step) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const A x = acc_up<A>(v.v[e]);
+          acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
+        }
+      }
+    }
+    A r = acc[0];
+#pragma unroll
+    for (int e = 1; e < VEC; ++e) r = f.combine(r, acc[e]);
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) r = f.combine(r, shfl_xor_any(r, o));
+    if (active && lane == 0) {
+      if (S.d > 1)
+        partial[vr] = r;
+      else
+        out[outOff] = epi.template finish<TOut>(r);
+    }
+  }
+}
+
+// max/min with index: one group of G lanes per row, or per chunk of a row
+// (virtual row vr = row * S + s, as in reduce_rows_kernel) when few long rows
+// must feed the whole chip. S > 1 publishes (value, index) partials with
+// indices relative to the whole row; fold_pairs_kernel finishes. The VEC == 1
+// instantiation honours the element stride sR of the reduced dim.
+template <typename T, typename I, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
+    typename Acc<T>::type* __restrict__ partV, I* __restrict__ partI, OuterArgs<I> oa,
+    OuterArgs<I> oaIdx, I numRows, I R, I sR, Divisor<I> S, I chunk, uint32_t G) {
+  using P = Pack<T, VEC>;
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  const uint32_t groups = kBlock / G;
+  const uint32_t lane = threadIdx.x % G;
+  const uint32_t grp = threadIdx.x / G;
+  const I total = numRows * S.d;
+  for (I r0 = (I)blockIdx.x * groups; r0 < total; r0 += (I)gridDim.x * groups) {
+    const I vr = r0 + grp;
+    const bool active = vr < total;
+    A bv = O::worst();
+    I bi = ~(I)0;
+    I outOff = 0, idxOff = 0;
+    if (active) {
+      I row, sp, inOff, unused;
+      S.divmod(vr, row, sp);
+      oa.offsets(row, inOff, outOff);
+      oaIdx.offsets(row, unused, idxOff);
+      const T* src = in + inOff;
+      const I begin = sp * chunk;
+      const I end = min(R, begin + chunk);
+      const I es = VEC == 1 ? sR : (I)1;
+      constexpr int U = 8;
+      const I step = (I)G * VEC;
+      I i = begin + lane * VEC;
+      for (; i + (U - 1) * step < end; i += U * step) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            if (O::better_later(x, bv)) {
+              bv = x;
+              bi = i + u * step + e;
+            }
+          }
+        }
+      }
+      for (; i < end; i += step) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const A x = acc_up<A>(v.v[e]);
+          if (O::better_later(x, bv)) {
+            bv = x;
+            bi = i + e;
+          }
+        }
+      }
+    }
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) {
+      const A ov = shfl_xor_any(bv, o);
+      I oi;
+      if (sizeof(I) == 8) {
+        const uint32_t lo = __shfl_xor((uint32_t)bi, o, 64);
+        const uint32_t hi = __shfl_xor((uint32_t)((uint64_t)bi >> 32), o, 64);
+        oi = (I)(((uint64_t)hi << 32) | lo);
+      } else {
+        oi = (I)__shfl_xor((uint32_t)bi, o, 64);
+      }
+      if (O::better(ov, oi, bv, bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (active && lane == 0) {
+      if (S.d > 1) {
+        partV[vr] = bv;
+        partI[vr] = bi;
+      } else {
+        // No element beat the start value: the whole row equals it (all -inf
+        // for max, all +inf for min), and the first occurrence is element 0.
+        if (bi == ~(I)0) bi = 0;
+        outV[outOff] = acc_down<T>(bv);
+        outI[idxOff] = (long)bi + 1;  // 1-based (TH_INDEX_BASE)
+      }
+    }
+  }
+}
+
+// Second launch of a split max/min along rows: one wave per row folds that
+// row's S (value, index) partials.
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T>::type* __restrict__ partV,
+                                                            const I* __restrict__ partI,
+                                                            T* __restrict__ outV,
+                                                            long* __restrict__ outI,
+                                                            OuterArgs<I> oa, OuterArgs<I> oaIdx,
+                                                            I numRows, I S) {
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  const uint32_t lane = threadIdx.x & 63;
+  const I wavesPerGrid = (I)gridDim.x * (kBlock / 64);
+  // every wave runs the same number of rounds (row is wave-uniform)
+  for (I row = (I)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); row < numRows;
+       row += wavesPerGrid) {
+    A bv = O::worst();
+    I bi = ~(I)0;
+    for (I sp = lane; sp < S; sp += 64) {
+      const A v = partV[row * S + sp];
+      const I ix = partI[row * S + sp];
+      if (O::better(v, ix, bv, bi)) {
+        bv = v;
+        bi = ix;
+      }
+    }
+    for (uint32_t o = 32; o > 0; o >>= 1) {
+      const A ov = shfl_xor_any(bv, o);
+      I oi;
+      if (sizeof(I) == 8) {
+        const uint32_t lo = __shfl_xor((uint32_t)bi, o, 64);
+        const uint32_t hi = __shfl_xor((uint32_t)((uint64_t)bi >> 32), o, 64);
+        oi = (I)(((uint64_t)hi << 32) | lo);
+      } else {
+        oi = (I)__shfl_xor((uint32_t)bi, o, 64);
+      }
+      if (O::better(ov, oi, bv, bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (lane == 0) {
+      I unusedA, unusedB, outOff, idxOff;
+      oa.offsets(row, unusedA, outOff);
+      oaIdx.offsets(row, unusedB, idxOff);
+      if (bi == ~(I)0) bi = 0;
+      outV[outOff] = acc_down<T>(bv);
+      outI[idxOff] = (long)bi + 1;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ cols --
+template <typename I>
+struct ColsArgs {
+  OuterArgs<I> oa;      // dims other than the reduced one and the unit-stride one
+  I C;                  // length of the unit-stride dim
+  I R, sR;              // reduced dim: length, input stride
+  I outInner;           // output stride along the unit-stride dim
+  I chunkR;             // rows of the reduced dim per workgroup
+  Divisor<I> S;         // workgroups along the reduced dim
+  Divisor<I> colTiles;  // workgroups along the unit-stride dim
+  I outElems;           // number of outputs (stride between partial planes)
+  uint32_t TX;          // lanes along the unit-stride dim (power of two <= 256)
+};
+
+// Split reductions run as two launches: workgroups publish fp32 partial planes
+// [S][outElems], a small second kernel folds the S planes in plane order. (A
+// single-launch variant in which the last workgroup to arrive folds the
+// partials needs agent-scope release/acquire fences; on MI355X each such
+// fence writes back the whole L2 of the XCD and made the kernel 5-10x slower.)
+template <typename TIn, typename TOut, typename F, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restrict__ in,
+                                                             TOut* __restrict__ out,
+                                                             typename F::A* __restrict__ partial,
+                                                             ColsArgs<I> a, I totalBlocks, Epi<typename F::A> epi,
+                                                             F f, bool foldPass) {
+  using P = Pack<TIn, VEC>;
+  using A = typename F::A;
+  __shared__ A smem[kBlock * VEC];
+  const uint32_t TX = a.TX, TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  // Fold the TY thread rows through LDS in a fixed tree; row 0 ends up with
+  // the result in smem[tx*VEC + e].
+  auto fold_rows = [&](const A (&acc)[VEC]) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) smem[(ty * TX + tx) * VEC + e] = acc[e];
+    __syncthreads();
+    for (uint32_t h = TY >> 1; h > 0; h >>= 1) {
+      if (ty < h) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const uint32_t i = (ty * TX + tx) * VEC + e;
+          smem[i] = f.combine(smem[i], smem[i + h * TX * VEC]);
+        }
+      }
+      __syncthreads();
+    }
+  };
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I group = b, s = 0, rest, ct;
+    if (!foldPass) a.S.divmod(b, group, s);
+    a.colTiles.divmod(group, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    A acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+    A* plane = partial + rest * a.C + col;
+    if (foldPass) {
+      // second launch: one workgroup per group (S == 1 in the block index),
+      // thread row ty folds planes ty, ty+TY, ...
+      if (col < a.C) {
+        constexpr int UF = 8;  // planes fetched per batch
+        I sp = ty;
+        for (; sp + (UF - 1) * TY < a.S.d; sp += UF * TY) {
+          A v[UF][VEC];
+#pragma unroll
+          for (int u = 0; u < UF; ++u) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[u][e] = plane[(sp + u * TY) * a.outElems + e];
+          }
+#pragma unroll
+          for (int u = 0; u < UF; ++u) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], v[u][e]);
+          }
+        }
+        for (; sp < a.S.d; sp += TY) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], plane[sp * a.outElems + e]);
+        }
+      }
+    } else if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const TIn* src = in + inOff + col;
+      A c[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        c[e] = (A)0;
+        if constexpr (F::kCentred) c[e] = acc_up<A>(out[outOff + (col + e) * a.outInner]);
+      }
+      constexpr int U = 8;
+      I r = begin + ty;
+      for (; r + (U - 1) * TY < end; r += U * TY) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (r + u * TY) * a.sR));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            acc[e] = f.combine(acc[e], f.modify(acc_up<A>(v[u].v[e]), c[e]));
+        }
+      }
+      for (; r < end; r += TY) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          acc[e] = f.combine(acc[e], f.modify(acc_up<A>(v.v[e]), c[e]));
+      }
+    }
+    fold_rows(acc);
+    if (ty == 0 && col < a.C) {
+      if (foldPass || a.S.d == 1) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          out[outOff + (col + e) * a.outInner] = epi.template finish<TOut>(smem[tx * VEC + e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) plane[s * a.outElems + e] = smem[tx * VEC + e];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T, typename I, int VEC, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
+    typename Acc<T>::type* __restrict__ partV, I* __restrict__ partI, ColsArgs<I> a,
+    OuterArgs<I> oaIdx, I idxInner, I totalBlocks, bool foldPass) {
+  using P = Pack<T, VEC>;
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  __shared__ A sv[kBlock * VEC];
+  __shared__ I si[kBlock * VEC];
+  const uint32_t TX = a.TX, TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  auto fold_rows = [&](const A (&bv)[VEC], const I (&bi)[VEC]) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      sv[(ty * TX + tx) * VEC + e] = bv[e];
+      si[(ty * TX + tx) * VEC + e] = bi[e];
+    }
+    __syncthreads();
+    for (uint32_t h = TY >> 1; h > 0; h >>= 1) {
+      if (ty < h) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const uint32_t i = (ty * TX + tx) * VEC + e, j = i + h * TX * VEC;
+          if (O::better(sv[j], si[j], sv[i], si[i])) {
+            sv[i] = sv[j];
+            si[i] = si[j];
+          }
+        }
+      }
+      __syncthreads();
+    }
+  };
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I group = b, s = 0, rest, ct;
+    if (!foldPass) a.S.divmod(b, group, s);
+    a.colTiles.divmod(group, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    const I at = rest * a.C + col;
+    A bv[VEC];
+    I bi[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      bv[e] = O::worst();
+      bi[e] = ~(I)0;
+    }
+    if (foldPass) {
+      if (col < a.C) {
+        for (I sp = ty; sp < a.S.d; sp += TY) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A v = partV[sp * a.outElems + at + e];
+            const I ix = partI[sp * a.outElems + at + e];
+            if (O::better(v, ix, bv[e], bi[e])) {
+              bv[e] = v;
+              bi[e] = ix;
+            }
+          }
+        }
+      }
+    } else if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const T* src = in + inOff + col;
+      constexpr int U = 8;
+      I r = begin + ty;
+      for (; r + (U - 1) * TY < end; r += U * TY) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (r + u * TY) * a.sR));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            if (O::better_later(x, bv[e])) {
+              bv[e] = x;
+              bi[e] = r + u * TY;
+            }
+          }
+        }
+      }
+      for (; r < end; r += TY) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const A x = acc_up<A>(v.v[e]);
+          if (O::better_later(x, bv[e])) {
+            bv[e] = x;
+            bi[e] = r;
+          }
+        }
+      }
+    }
+    fold_rows(bv, bi);
+    if (ty == 0 && col < a.C) {
+      if (foldPass || a.S.d == 1) {
+        I unused, idxOff;
+        oaIdx.offsets(rest, unused, idxOff);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const I ix = si[tx * VEC + e] == ~(I)0 ? 0 : si[tx * VEC + e];  // column of start values
+          outV[outOff + (col + e) * a.outInner] = acc_down<T>(sv[tx * VEC + e]);
+          outI[idxOff + (col + e) * idxInner] = (long)ix + 1;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          partV[s * a.outElems + at + e] = sv[tx * VEC + e];
+          partI[s * a.outElems + at + e] = si[tx * VEC + e];
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------- all --
+// Whole-tensor reduction of a dense run: every workgroup streams a contiguous
+// chunk, folds it (wave butterfly + LDS) and publishes one partial; a second
+// one-workgroup launch of the same kernel folds the partials in index order.
+// The final scalar goes to `result` (device scratch) and to `hostResult`
+// (pinned, device-mapped host memory, so no separate D2H copy is needed).
+template <typename F>
+__device__ __forceinline__ typename F::A block_fold(typename F::A r, typename F::A* red, F f) {
+  for (uint32_t o = 32; o > 0; o >>= 1) r = f.combine(r, shfl_xor_any(r, o));
+  const uint32_t wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[wave] = r;
+  __syncthreads();
+  typename F::A t = red[0];
+  for (uint32_t w = 1; w < kBlock / 64; ++w) t = f.combine(t, red[w]);
+  return t;
+}
+
+template <typename TIn, typename F, typename I, int VEC, bool FIRST>
+__global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restrict__ in, I n,
+                                                            I chunk,
+                                                            typename F::A* __restrict__ partial,
+                                                            typename F::A* result,
+                                                            typename F::A* hostResult,
+                                                            Epi<typename F::A> epi, F f) {
+  using P = Pack<TIn, VEC>;
+  using A = typename F::A;
+  __shared__ A red[kBlock / 64];
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+  const I nv = n - n % VEC;  // packs cover [0, nv); the last workgroup adds the tail
+  const I begin = (I)blockIdx.x * chunk;
+  const I end = min(nv, begin + chunk);
+  constexpr int U = 8;
+  constexpr I step = (I)kBlock * VEC;
+  if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n) {
+    const A x = acc_up<A>(in[nv + threadIdx.x]);
+    acc[0] = f.combine(acc[0], FIRST ? f.modify(x, (A)0) : x);
+  }
+  I i = begin + threadIdx.x * VEC;
+  for (; i + (U - 1) * step < end; i += U * step) {
+    P v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(in + i + u * step));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const A x = acc_up<A>(v[u].v[e]);
+        acc[e] = f.combine(acc[e], FIRST ? f.modify(x, (A)0) : x);
+      }
+    }
+  }
+  for (; i < end; i += step) {
+    const P v = load_pack<true>(reinterpret_cast<const P*>(in + i));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const A x = acc_up<A>(v.v[e]);
+      acc[e] = f.combine(acc[e], FIRST ? f.modify(x, (A)0) : x);
+    }
+  }
+  A r = acc[0];
+#pragma unroll
+  for (int e = 1; e < VEC; ++e) r = f.combine(r, acc[e]);
+  r = block_fold(r, red, f);
+  if (threadIdx.x == 0) {
+    if (gridDim.x == 1) {
+      const A fin = epi.template finish<A>(r);
+      *result = fin;
+      *hostResult = fin;
+    } else {
+      partial[blockIdx.x] = r;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+uint32_t pow2_ceil(uint64_t x) {
+  uint32_t p = 1;
+  while (p < x && p < (1u << 30)) p <<= 1;
+  return p;
+}
+
+template <typename I>
+OuterArgs<I> make_outer(const Layout& in, const Layout& out, int dims) {
+  OuterArgs<I> oa{};
+  oa.dims = dims < 1 ? 1 : dims;
+  if (dims < 1) {
+    oa.size[0].set(1);
+    oa.inStride[0] = 0;
+    oa.outStride[0] = 0;
+    return oa;
+  }
+  for (int d = 0; d < dims; ++d) {
+    oa.size[d].set((uint64_t)in.size[d]);
+    oa.inStride[d] = (I)in.stride[d];
+    oa.outStride[d] = (I)out.stride[d];
+  }
+  return oa;
+}
+
+int capped_grid(THCState* s, int64_t blocks, const char* key, int defaultPerCu) {
+  const int64_t cap = (int64_t)num_compute_units(s) * tuning(key, defaultPerCu);
+  return (int)std::max<int64_t>(1, std::min(blocks, cap));
+}
+
+template <typename TIn, typename TOut, typename F, typename I, bool FIRST>
+void launch_rows_pass(THCState* s, const TIn* in, TOut* out, typename F::A* partial,
+                      const OuterArgs<I>& oa, int64_t numRows, int64_t R, int64_t sR, int64_t S,
+                      int64_t chunk, bool vec, Epi<typename F::A> epi, F f) {
+  constexpr int VEC = 16 / sizeof(TIn);
+  const int pack = vec ? VEC : 1;
+  const int64_t span = std::min(R, chunk);
+  const int64_t perLane = tuning("reduce.rows.packs_per_lane", 8);
+  uint32_t G = pow2_ceil((uint64_t)((span + pack * perLane - 1) / (pack * perLane)));
+  G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+  const int64_t groups = kBlock / G;
+  const int64_t blocks = (numRows * S + groups - 1) / groups;
+  const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+  Divisor<I> Sd;
+  Sd.set((uint64_t)S);
+  hipStream_t st = current_stream(s);
+  if (vec)
+    hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, VEC, FIRST>), dim3(grid), dim3(kBlock),
+                       0, st, in, out, partial, oa, (I)numRows, (I)R, (I)1, Sd, (I)chunk, G, epi,
+                       f);
+  else
+    hipLaunchKernelGGL((reduce_rows_kernel<TIn, TOut, F, I, 1, FIRST>), dim3(grid), dim3(kBlock), 0,
+                       st, in, out, partial, oa, (I)numRows, (I)R, (I)sR, Sd, (I)chunk, G, epi, f);
+}
+
+// rows: a group of lanes per output. Packs when the reduced dim has unit stride
+// and everything is 16-byte aligned, scalar strided loads otherwise.
+template <typename T, typename F, typename I>
+void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  constexpr int VEC = 16 / sizeof(T);
+  const int64_t rows = g.outElems;
+  bool vec = g.sR == 1 && aligned16(in) && g.R % VEC == 0;
+  for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+  OuterArgs<I> oa = make_outer<I>(g.in, g.out, g.in.dims);
+
+  // Few long rows: cut them so that about `target` waves have work.
+  const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+  const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
+  size_t scratchBytes = 0;
+  int64_t S = 1, chunk = g.R;
+  if (rows < target && g.R >= 2 * minChunk) {
+    S = std::min<int64_t>((target + rows - 1) / rows, g.R / minChunk);
+    scratch_space(s, &scratchBytes);
+    S = std::min<int64_t>(S, (int64_t)(scratchBytes / sizeof(A)) / std::max<int64_t>(rows, 1));
+    if (S < 2) S = 1;
+    chunk = (g.R + S - 1) / S;
+    chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
+    S = (g.R + chunk - 1) / chunk;
+  }
+  if (S == 1) {
+    launch_rows_pass<T, T, F, I, true>(s, in, out, nullptr, oa, rows, g.R, g.sR, 1, g.R, vec, epi, f);
+    note_kernel(vec ? "rows" : (g.sR == 1 ? "rows-scalar" : "rows-strided"));
+    return;
+  }
+  A* scratch = (A*)scratch_space(s, &scratchBytes);
+  launch_rows_pass<T, T, F, I, true>(s, in, out, scratch, oa, rows, g.R, g.sR, S, chunk, vec,
+                                     Epi<A>{(int)Epilogue::None, (A)0}, f);
+  // pass 2: partial[row*S + s] is a dense rows x S matrix
+  Layout pin = g.in;
+  int64_t run = S;
+  for (int d = pin.dims - 1; d >= 0; --d) {
+    pin.stride[d] = run;
+    run *= pin.size[d];
+  }
+  OuterArgs<I> oa2 = make_outer<I>(pin, g.out, pin.dims);
+  launch_rows_pass<A, T, F, I, false>(s, scratch, out, nullptr, oa2, rows, S, 1, 1, S,
+                                      S % (16 / sizeof(A)) == 0, epi, f);
+  note_kernel(vec ? "rows-split" : (g.sR == 1 ? "rows-split-scalar" : "rows-split-strided"));
+}
+
+template <typename I>
+struct ColsPlan {
+  ColsArgs<I> a;
+  int64_t totalBlocks;
+  bool vec;
+};
+
+// cols: reduced dim strided, innermost joint dim has unit input stride.
+template <typename T, typename I>
+ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t partialElemBytes) {
+  constexpr int VEC = 16 / sizeof(T);
+  ColsPlan<I> p{};
+  const int nd = g.in.dims;
+  const int64_t C = g.in.size[nd - 1];
+  bool vec = aligned16(in) && C % VEC == 0 && g.sR % VEC == 0;
+  for (int d = 0; d < nd - 1 && vec; ++d) vec = g.in.stride[d] % VEC == 0;
+  const int pack = vec ? VEC : 1;
+  const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 1));
+  const int64_t outer = g.outElems / C;
+  // Lanes along the unit-stride dim: a full wave if the dim is long enough, but
+  // narrower column tiles (down to 256-byte rows) are preferred over splitting
+  // the reduced dim when they already give every CU a workgroup.
+  uint32_t TX = std::min<uint32_t>(64, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
+  const uint32_t minTX = (uint32_t)tuning("reduce.cols.min_tx", 16);
+  auto tiles_for = [&](uint32_t tx) { return (C + (int64_t)tx * pack - 1) / ((int64_t)tx * pack); };
+  while (TX > minTX && outer * tiles_for(TX) < target) TX >>= 1;
+  const uint32_t TY = kBlock / TX;
+  const int64_t colTiles = tiles_for(TX);
+  const int64_t base = outer * colTiles;
+  const int64_t minRows = (int64_t)TY * tuning("reduce.cols.min_rows_per_thread", 8);
+  int64_t S = 1;
+  if (base < target && g.R >= 2 * minRows) {
+    S = std::min<int64_t>((target + base - 1) / base, g.R / minRows);
+    size_t scratchBytes = 0;
+    scratch_space(s, &scratchBytes);
+    S = std::min<int64_t>(S, (int64_t)(scratchBytes / partialElemBytes) / std::max<int64_t>(g.outElems, 1));
+    if (S < 2) S = 1;
+  }
+  const int64_t forced = tuning("reduce.cols.force_split", 0);
+  if (forced > 0) S = std::min<int64_t>(forced, g.R);
+  int64_t chunk = (g.R + S - 1) / S;
+  S = (g.R + chunk - 1) / chunk;
+  p.vec = vec;
+  p.a.oa = make_outer<I>(g.in, g.out, nd - 1);
+  p.a.C = (I)C;
+  p.a.R = (I)g.R;
+  p.a.sR = (I)g.sR;
+  p.a.outInner = (I)g.out.stride[nd - 1];
+  p.a.chunkR = (I)chunk;
+  p.a.S.set((uint64_t)S);
+  p.a.colTiles.set((uint64_t)colTiles);
+  p.a.outElems = (I)g.outElems;
+  p.a.TX = TX;
+  p.totalBlocks = base * S;
+  return p;
+}
+
+template <typename T, typename F, typename I>
+void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  constexpr int VEC = 16 / sizeof(T);
+  ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(A));
+  const bool split = p.a.S.d > 1;
+  A* scratch = split ? (A*)scratch_space(s, nullptr) : nullptr;
+  const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+  const int64_t groups = p.totalBlocks / (int64_t)p.a.S.d;
+  hipStream_t st = current_stream(s);
+  for (int pass = 0; pass < (split ? 2 : 1); ++pass) {
+    const bool fold = pass == 1;
+    const int gr = fold ? (int)groups : grid;
+    const I tb = fold ? (I)groups : (I)p.totalBlocks;
+    if (p.vec)
+      hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, VEC>), dim3(gr), dim3(kBlock), 0, st, in,
+                         out, scratch, p.a, tb, epi, f, fold);
+    else
+      hipLaunchKernelGGL((reduce_cols_kernel<T, T, F, I, 1>), dim3(gr), dim3(kBlock), 0, st, in,
+                         out, scratch, p.a, tb, epi, f, fold);
+  }
+  note_kernel(split ? (p.vec ? "cols-split" : "cols-split-scalar") : (p.vec ? "cols" : "cols-scalar"));
+}
+
+template <typename T, typename F, typename I>
+void run_dim_typed(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi,
+                   F f) {
+  if (g.sR != 1 && g.in.stride[g.in.dims - 1] == 1 && g.in.size[g.in.dims - 1] > 1)
+    run_cols<T, F, I>(s, g, in, out, epi, f);
+  else
+    run_rows<T, F, I>(s, g, in, out, epi, f);  // unit stride: packs; otherwise its scalar form
+}
+
+template <typename T, typename F>
+void run_dim(THCState* s, const ReduceGeom& g, const void* in, void* out, Epi<typename F::A> epi, F f) {
+  if (g.wide)
+    run_dim_typed<T, F, uint64_t>(s, g, (const T*)in, (T*)out, epi, f);
+  else
+    run_dim_typed<T, F, uint32_t>(s, g, (const T*)in, (T*)out, epi, f);
+}
+
+// ---------------------------------------------------------------- index --
+template <typename T, typename I, bool IS_MAX>
+void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, long* outI) {
+  using A = typename Acc<T>::type;
+  constexpr int VEC = 16 / sizeof(T);
+  hipStream_t st = current_stream(s);
+  const int nd = g.in.dims;
+  const bool colsShape = g.sR != 1 && g.in.stride[nd - 1] == 1 && g.in.size[nd - 1] > 1;
+  if (!colsShape) {
+    bool vec = g.sR == 1 && aligned16(in) && g.R % VEC == 0;
+    for (int d = 0; d < nd && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+    const int pack = vec ? VEC : 1;
+    OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
+    OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
+    const int64_t rows = g.outElems;
+    // Few long rows: cut them as run_rows does.
+    const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+    const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
+    int64_t S = 1, chunk = g.R;
+    A* partV = nullptr;
+    I* partI = nullptr;
+    if (rows < target && g.R >= 2 * minChunk) {
+      size_t scratchBytes = 0;
+      char* scratch = (char*)scratch_space(s, &scratchBytes);
+      S = std::min<int64_t>((target + rows - 1) / rows, g.R / minChunk);
+      S = std::min<int64_t>(S, (int64_t)(scratchBytes / 16) / std::max<int64_t>(rows, 1));
+      if (S < 2) S = 1;
+      chunk = (g.R + S - 1) / S;
+      chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
+      S = (g.R + chunk - 1) / chunk;
+      if (S > 1) {
+        partI = (I*)scratch;  // both parts start 8-byte aligned
+        partV = (A*)(scratch + 8 * (size_t)S * (size_t)rows);
+      }
+    }
+    const int64_t span = std::min(g.R, chunk);
+    const int64_t perLane = tuning("reduce.rows.packs_per_lane", 8);
+    uint32_t G = pow2_ceil((uint64_t)((span + pack * perLane - 1) / (pack * perLane)));
+    G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+    const int64_t groups = kBlock / G;
+    const int grid = capped_grid(s, (rows * S + groups - 1) / groups, "reduce.rows.blocks_per_cu", 64);
+    Divisor<I> Sd;
+    Sd.set((uint64_t)S);
+    if (vec)
+      hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, VEC, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, partV, partI, oa, oaIdx, (I)rows, (I)g.R, (I)1, Sd,
+                         (I)chunk, G);
+    else
+      hipLaunchKernelGGL((reduce_rows_index_kernel<T, I, 1, IS_MAX>), dim3(grid), dim3(kBlock), 0,
+                         st, in, outV, outI, partV, partI, oa, oaIdx, (I)rows, (I)g.R, (I)g.sR, Sd,
+                         (I)chunk, G);
+    if (S > 1) {
+      const int fgrid = capped_grid(s, (rows + kBlock / 64 - 1) / (kBlock / 64), "reduce.rows.blocks_per_cu", 64);
+      hipLaunchKernelGGL((fold_pairs_kernel<T, I, IS_MAX>), dim3(fgrid), dim3(kBlock), 0, st, partV,
+                         partI, outV, outI, oa, oaIdx, (I)rows, (I)S);
+    }
+    if (S > 1)
+      note_kernel(vec ? "rows-index-split" : (g.sR == 1 ? "rows-index-split-scalar" : "rows-index-split-strided"));
+    else
+      note_kernel(vec ? "rows-index" : (g.sR == 1 ? "rows-index-scalar" : "rows-index-strided"));
+    return;
+  }
+  {
+    ColsPlan<I> p = plan_cols<T, I>(s, g, in, 16);
+    OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
+    const I idxInner = (I)g.idx.stride[nd - 1];
+    const bool split = p.a.S.d > 1;
+    A* partV = nullptr;
+    I* partI = nullptr;
+    if (split) {
+      char* scratch = (char*)scratch_space(s, nullptr);
+      partI = (I*)scratch;  // both parts start 8-byte aligned
+      partV = (A*)(scratch + 8 * (size_t)p.a.S.d * (size_t)g.outElems);
+    }
+    const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+    const int64_t groups = p.totalBlocks / (int64_t)p.a.S.d;
+    for (int pass = 0; pass < (split ? 2 : 1); ++pass) {
+      const bool fold = pass == 1;
+      const int gr = fold ? (int)groups : grid;
+      const I tb = fold ? (I)groups : (I)p.totalBlocks;
+      if (p.vec)
+        hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, VEC, IS_MAX>), dim3(gr), dim3(kBlock), 0,
+                           st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, tb, fold);
+      else
+        hipLaunchKernelGGL((reduce_cols_index_kernel<T, I, 1, IS_MAX>), dim3(gr), dim3(kBlock), 0,
+                           st, in, outV, outI, partV, partI, p.a, oaIdx, idxInner, tb, fold);
+    }
+    note_kernel(split ? "cols-index-split" : "cols-index");
+  }
+}
+
+}  // namespace
+
+// Entry of a per-type slice: every reduction op the element type has.
+template <typename T>
+void reduce_dim_type(THCState* s, const ReduceGeom& g, const void* in, void* out, ReduceOp op,
+                     Epilogue ep, double epArg, double p_) {
+  using A = typename Acc<T>::type;
+  const A p = (A)p_;
+  const Epi<A> epi{(int)ep, (A)epArg};
+  switch (op) {
+    case ReduceOp::Sum: run_dim<T>(s, g, in, out, epi, FSum<A>{p}); return;
+    case ReduceOp::Prod: run_dim<T>(s, g, in, out, epi, FProd<A>{p}); return;
+    case ReduceOp::Min: run_dim<T>(s, g, in, out, epi, FMin<A>{p}); return;
+    case ReduceOp::Max: run_dim<T>(s, g, in, out, epi, FMax<A>{p}); return;
+    default: break;
+  }
+  if constexpr (!std::is_integral<A>::value) {
+    switch (op) {
+      case ReduceOp::Norm0: run_dim<T>(s, g, in, out, epi, FNorm0<A>{p}); return;
+      case ReduceOp::Norm1: run_dim<T>(s, g, in, out, epi, FNorm1<A>{p}); return;
+      case ReduceOp::Norm2: run_dim<T>(s, g, in, out, epi, FNorm2<A>{p}); return;
+      case ReduceOp::NormP: run_dim<T>(s, g, in, out, epi, FNormP<A>{p}); return;
+      case ReduceOp::SqDev: run_dim<T>(s, g, in, out, epi, FSqDev<A>{p}); return;
+      case ReduceOp::SqDevOut: run_dim<T>(s, g, in, out, epi, FSqDevOut<A>{p}); return;
+      default: break;
+    }
+  }
+  raise_error("reduction not available for this element type");
+}
+
+template <typename T>
+void reduce_index_type(THCState* s, const ReduceGeom& g, bool isMax, const void* in, void* outV,
+                       long* outI) {
+  if (g.wide) {
+    if (isMax) run_index_typed<T, uint64_t, true>(s, g, (const T*)in, (T*)outV, outI);
+    else run_index_typed<T, uint64_t, false>(s, g, (const T*)in, (T*)outV, outI);
+  } else {
+    if (isMax) run_index_typed<T, uint32_t, true>(s, g, (const T*)in, (T*)outV, outI);
+    else run_index_typed<T, uint32_t, false>(s, g, (const T*)in, (T*)outV, outI);
+  }
+}
+
+
+// ------------------------------------------------------------------- all --
+template <typename A>
+constexpr DType acc_dtype() {
+  return std::is_same<A, float>::value ? DType::F32
+                                       : (std::is_same<A, double>::value ? DType::F64 : DType::I64);
+}
+
+namespace {
+template <typename T, typename F>
+void reduce_all_with(THCState* s, ReduceGeom g, const void* src, F f1, bool sumSecond,
+                     Scalar* result) {
+  using A = typename F::A;
+  const int64_t rows = g.outElems;
+  const StreamScratch& sc = stream_scratch(s);
+  A* devOut = reinterpret_cast<A*>(sc.result);
+  A* hostDev = reinterpret_cast<A*>(sc.hostResultDev);
+  const Epi<A> none{(int)Epilogue::None, (A)0};
+  TensorRef rowPartials(s, nullptr);
+  bool partialsAreInput = false;  // stage 2 reads accumulator-typed partials
+  // Stage 1 (only if there are several rows): one partial per row, held in a
+  // temporary; stage 2 folds the dense vector of partials (or the single row).
+  if (rows > 1) {
+    long n1 = rows;
+    rowPartials.t = tensor_new_with_size(s, 1, &n1, acc_dtype<A>());
+    g.out = g.in;  // dense row-major output
+    int64_t run = 1;
+    for (int d = g.out.dims - 1; d >= 0; --d) {
+      g.out.stride[d] = run;
+      run *= g.out.size[d];
+    }
+    A* rp = (A*)tensor_data(rowPartials.t, acc_dtype<A>());
+    constexpr int VEC = 16 / sizeof(T);
+    bool vec = aligned16(src) && g.R % VEC == 0;
+    for (int d = 0; d < g.in.dims && vec; ++d) vec = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+    if (g.wide) {
+      OuterArgs<uint64_t> oa = make_outer<uint64_t>(g.in, g.out, g.in.dims);
+      launch_rows_pass<T, A, F, uint64_t, true>(s, (const T*)src, rp, nullptr, oa, rows, g.R, 1, 1,
+                                                g.R, vec, none, f1);
+    } else {
+      OuterArgs<uint32_t> oa = make_outer<uint32_t>(g.in, g.out, g.in.dims);
+      launch_rows_pass<T, A, F, uint32_t, true>(s, (const T*)src, rp, nullptr, oa, rows, g.R, 1, 1,
+                                                g.R, vec, none, f1);
+    }
+    src = rp;
+    partialsAreInput = true;
+    g.R = rows;
+    g.wide = force_64bit_index() || rows >= kIndex32Limit;
+  }
+  // Workgroups of 256 lanes stream chunks that are multiples of one full
+  // batch (256 lanes x 8 packs); a few workgroups per CU.
+  auto stage2 = [&](auto srcTag, auto f, auto idxTag) {
+    using TI = decltype(srcTag);
+    using F2 = decltype(f);
+    using I = decltype(idxTag);
+    constexpr int V = 16 / sizeof(TI);
+    const int64_t batch = (int64_t)kBlock * V * 8;
+    int64_t blocks = std::min<int64_t>((int64_t)num_compute_units(s) * tuning("reduce.all.blocks_per_cu", 2),
+                                       (g.R + batch - 1) / batch);
+    blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)(sc.partialBytes / sizeof(A))));
+    int64_t chunk = (g.R + blocks - 1) / blocks;
+    chunk = (chunk + batch - 1) / batch * batch;
+    blocks = (g.R + chunk - 1) / chunk;
+    hipStream_t st = current_stream(s);
+    A* part = (A*)sc.partials;
+    if (aligned16(src))
+      hipLaunchKernelGGL((reduce_all_kernel<TI, F2, I, V, true>), dim3((int)blocks), dim3(kBlock), 0,
+                         st, (const TI*)src, (I)g.R, (I)chunk, part, devOut, hostDev, none, f);
+    else
+      hipLaunchKernelGGL((reduce_all_kernel<TI, F2, I, 1, true>), dim3((int)blocks), dim3(kBlock), 0,
+                         st, (const TI*)src, (I)g.R, (I)chunk, part, devOut, hostDev, none, f);
+    if (blocks > 1)  // fold the per-workgroup partials
+      hipLaunchKernelGGL((reduce_all_kernel<A, F2, I, 1, false>), dim3(1), dim3(kBlock), 0, st,
+                         (const A*)part, (I)blocks, (I)blocks, part, devOut, hostDev, none, f);
+  };
+  auto pick_index = [&](auto srcTag, auto f) {
+    if (g.wide) stage2(srcTag, f, uint64_t{});
+    else stage2(srcTag, f, uint32_t{});
+  };
+  if (partialsAreInput) {
+    // the row partials are already modified values: fold them with the plain
+    // combine (a sum for the norm / deviation family)
+    if (sumSecond) pick_index(A{}, FSum<A>{(A)0});
+    else pick_index(A{}, f1);
+  } else {
+    pick_index(T{}, f1);
+  }
+  note_kernel(rows > 1 ? "all-rows" : "all");
+  THC_CHECK(hipGetLastError());
+  // The one place the caller blocks on the device (THCReduceAll.cuh:333-335):
+  // the kernel has stored the scalar into pinned host memory, so waiting for
+  // the stream is all that is left of the reference's synchronous D2H copy.
+  THC_CHECK(hipStreamSynchronize(current_stream(s)));
+  const A r = *reinterpret_cast<const volatile A*>(sc.hostResult);
+  result->f = (double)r;
+  result->i = (int64_t)r;
+}
+}  // namespace
+
+template <typename T>
+void reduce_all_type(THCState* s, ReduceGeom g, const void* src, ReduceOp op, double p_,
+                     Scalar* result) {
+  using A = typename Acc<T>::type;
+  const A p = (A)p_;
+  switch (op) {
+    case ReduceOp::Sum: reduce_all_with<T>(s, g, src, FSum<A>{p}, false, result); return;
+    case ReduceOp::Prod: reduce_all_with<T>(s, g, src, FProd<A>{p}, false, result); return;
+    case ReduceOp::Min: reduce_all_with<T>(s, g, src, FMin<A>{p}, false, result); return;
+    case ReduceOp::Max: reduce_all_with<T>(s, g, src, FMax<A>{p}, false, result); return;
+    default: break;
+  }
+  if constexpr (!std::is_integral<A>::value) {
+    switch (op) {
+      case ReduceOp::Norm0: reduce_all_with<T>(s, g, src, FNorm0<A>{p}, true, result); return;
+      case ReduceOp::Norm1: reduce_all_with<T>(s, g, src, FNorm1<A>{p}, true, result); return;
+      case ReduceOp::Norm2: reduce_all_with<T>(s, g, src, FNorm2<A>{p}, true, result); return;
+      case ReduceOp::NormP: reduce_all_with<T>(s, g, src, FNormP<A>{p}, true, result); return;
+      case ReduceOp::SqDev: reduce_all_with<T>(s, g, src, FSqDev<A>{p}, true, result); return;
+      default: break;
+    }
+  }
+  if constexpr (std::is_same<T, uint8_t>::value) {
+    if (op == ReduceOp::All) { reduce_all_with<T>(s, g, src, FAll<A>{p}, false, result); return; }
+    if (op == ReduceOp::Any) { reduce_all_with<T>(s, g, src, FAny<A>{p}, false, result); return; }
+  }
+  raise_error("reduction not available for this element type");
+}
+
+}  // namespace thc

@@ -1,0 +1,32 @@
+// Interface between the type-independent reduction front end (reduce.hip) and
+// the per-type kernel slices (reduce_f32.hip, reduce_f16.hip, reduce_w_*.hip).
+#pragma once
+#include "common.hpp"
+
+namespace thc {
+
+// What a reduction looks like after the non-reduced dims of input and output
+// were brought into one joint space (input = operand 0 decides the order).
+struct ReduceGeom {
+  Layout in, out;     // non-reduced dims, jointly collapsed (same sizes)
+  Layout idx;         // optional second output with the same joint sizes
+  int64_t R, sR;      // reduced dim
+  int64_t outElems;
+  bool wide;
+};
+
+// Defined (explicitly instantiated) in the slices.
+template <typename T>
+void reduce_dim_type(THCState* s, const ReduceGeom& g, const void* in, void* out, ReduceOp op,
+                     Epilogue ep, double epArg, double p);
+template <typename T>
+void reduce_index_type(THCState* s, const ReduceGeom& g, bool isMax, const void* in, void* outV,
+                       long* outI);
+// Whole-tensor reduction of a tensor whose innermost collapsed dim has unit
+// stride (`g.R` long, `g.in` = the remaining dims = rows). Blocks until the
+// scalar is on the host.
+template <typename T>
+void reduce_all_type(THCState* s, ReduceGeom g, const void* src, ReduceOp op, double p,
+                     Scalar* result);
+
+}  // namespace thc

@@ -1,0 +1,9 @@
+// Reduce-engine slice: element type double.
+#include "reduce_impl.hpp"
+
+namespace thc {
+template void reduce_dim_type<double>(THCState*, const ReduceGeom&, const void*, void*, ReduceOp, Epilogue,
+                                  double, double);
+template void reduce_index_type<double>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
+template void reduce_all_type<double>(THCState*, ReduceGeom, const void*, ReduceOp, double, Scalar*);
+}

@@ -1,0 +1,9 @@
+// Reduce-engine slice: element type int32_t.
+#include "reduce_impl.hpp"
+
+namespace thc {
+template void reduce_dim_type<int32_t>(THCState*, const ReduceGeom&, const void*, void*, ReduceOp, Epilogue,
+                                  double, double);
+template void reduce_index_type<int32_t>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
+template void reduce_all_type<int32_t>(THCState*, ReduceGeom, const void*, ReduceOp, double, Scalar*);
+}

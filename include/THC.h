@@ -517,6 +517,46 @@ THC_API void THCudaDoubleTensor_tpow(THCState *, THCudaDoubleTensor *self, doubl
 THC_API void THCudaDoubleTensor_atan2(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *tx, THCudaDoubleTensor *ty);
 THC_API void THCudaDoubleTensor_lerp(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *a, THCudaDoubleTensor *b, double w);
 
+/* Reductions of the integer types and double: the per-type expansion of     */
+/* generic/THCTensorMathReduce.h:18-36 and generic/THCTensorMathPairwise.h:17. */
+/* accreal is long for the integer types, double for double.                  */
+#define THC_AMD_DECLARE_WIDE_REDUCE_API(Tensor, real, accreal)                 \
+  THC_API void Tensor##_sum(THCState *, Tensor *self, Tensor *src, long dim,   \
+                            int keepdim);                                      \
+  THC_API void Tensor##_prod(THCState *, Tensor *self, Tensor *src, long dim,  \
+                             int keepdim);                                     \
+  THC_API void Tensor##_mean(THCState *, Tensor *self, Tensor *src, long dim,  \
+                             int keepdim);                                     \
+  THC_API void Tensor##_max(THCState *, Tensor *values,                        \
+                            THCudaLongTensor *indices, Tensor *src, long dim,  \
+                            int keepdim);                                      \
+  THC_API void Tensor##_min(THCState *, Tensor *values,                        \
+                            THCudaLongTensor *indices, Tensor *src, long dim,  \
+                            int keepdim);                                      \
+  THC_API accreal Tensor##_sumall(THCState *, Tensor *self);                   \
+  THC_API accreal Tensor##_prodall(THCState *, Tensor *self);                  \
+  THC_API accreal Tensor##_meanall(THCState *, Tensor *self);                  \
+  THC_API real Tensor##_minall(THCState *, Tensor *self);                      \
+  THC_API real Tensor##_maxall(THCState *, Tensor *self);                      \
+  THC_API int Tensor##_equal(THCState *, Tensor *self, Tensor *src);
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaByteTensor, unsigned char, long)
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaCharTensor, char, long)
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaShortTensor, short, long)
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaIntTensor, int, long)
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaLongTensor, long, long)
+THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaDoubleTensor, double, double)
+/* lib/THC/THCTensorMath.h:52-53 */
+THC_API int THCudaByteTensor_logicalall(THCState *, THCudaByteTensor *self);
+THC_API int THCudaByteTensor_logicalany(THCState *, THCudaByteTensor *self);
+/* double: generic/THCTensorMathReduce.h:7-14,44-45 */
+THC_API void THCudaDoubleTensor_norm(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, double p, long dim, int keepdim);
+THC_API void THCudaDoubleTensor_var(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, long dim, int biased, int keepdim);
+THC_API void THCudaDoubleTensor_std(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, long dim, int biased, int keepdim);
+THC_API double THCudaDoubleTensor_normall(THCState *, THCudaDoubleTensor *self, double p);
+THC_API double THCudaDoubleTensor_varall(THCState *, THCudaDoubleTensor *self, int biased);
+THC_API double THCudaDoubleTensor_stdall(THCState *, THCudaDoubleTensor *self, int biased);
+THC_API double THCudaDoubleTensor_dist(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, double p);
+
 THC_AMD_DECLARE_MATH_API(THCudaTensor, float, float)
 THC_AMD_DECLARE_MATH_API(THCudaHalfTensor, THHalf, float)
 

@@ -76,6 +76,10 @@ def lib():
                                          VP, VP, VP, VP]
         l.th_typed_compare.argtypes = [C.c_int, C.c_int, C.c_int, C.c_double, C.c_long, VP, VP, VP]
         l.th_typed_convert.argtypes = [C.c_int, VP, C.c_int, VP]
+        l.th_typed_reduce_dim.argtypes = [C.c_int, C.c_int, VP, VP, C.c_int]
+        l.th_typed_minmax_dim.argtypes = [C.c_int, C.c_int, VP, VP, VP, C.c_int]
+        l.th_typed_reduce_all.argtypes = [C.c_int, C.c_int, VP, C.POINTER(C.c_long)]
+        l.th_typed_reduce_all.restype = C.c_double
         l.th_half2float.argtypes = [C.c_uint16]
         l.th_half2float.restype = C.c_float
         l.th_float2half.argtypes = [C.c_float]
@@ -195,6 +199,34 @@ def typed_convert(dst, src):
     if lib().th_typed_convert(DTYPES[dst.kind], _ptr(dst), DTYPES[src.kind], _ptr(src)):
         raise ValueError("sizes do not match")
     return dst
+
+
+TYPED_KINDS = {"sum": 0, "prod": 1, "min": 2, "max": 3, "mean": 4}
+
+
+def typed_reduce_dim(kind, src, dim, out=None):
+    """sum / prod / min / max / mean along dim for byte..long and double views."""
+    if out is None:
+        out = View.empty(reduced_shape(src.size, dim), src.storage.dtype)
+    if lib().th_typed_reduce_dim(DTYPES[src.kind], TYPED_KINDS[kind], _ptr(out), _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return out
+
+
+def typed_minmax_dim(which, src, dim):
+    shape = reduced_shape(src.size, dim)
+    values, indices = View.empty(shape, src.storage.dtype), View.empty(shape, np.int64)
+    if lib().th_typed_minmax_dim(DTYPES[src.kind], 1 if which == "max" else 0, _ptr(values), _ptr(indices),
+                                 _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return values, indices
+
+
+def typed_reduce_all(kind, src):
+    """accreal result: a Python int for the integer kinds, a float for double."""
+    ri = C.c_long(0)
+    rf = lib().th_typed_reduce_all(DTYPES[src.kind], TYPED_KINDS[kind], _ptr(src), C.byref(ri))
+    return rf if src.kind == "double" else ri.value
 
 
 def reduced_shape(shape, dim):

@@ -386,3 +386,161 @@ int th_typed_convert(int dstT, const th_view *dst, int srcT, const th_view *src)
   }
   return 0;
 }
+
+/* ------------------------------------------------------------ reductions -- */
+/* Integer types accumulate in long (accreal = long, lib/THC/THCGenerate*Type.h)
+ * with two's complement wrap-around; the stored result wraps in the element
+ * type. Double accumulates sequentially in long double and rounds once, which
+ * pins a sum to within half an ulp of the exact value. mean = sum converted to
+ * the element type, divided by the size converted to the element type
+ * (lib/THC/generic/THCTensorMathReduce.cu:37-43). */
+enum { RK_SUM = 0, RK_PROD, RK_MIN, RK_MAX, RK_MEAN };
+
+static void reduce_slice_typed(int t, int kind, const void *base, long off, long n, long stride,
+                               int64_t *ri, double *rf) {
+  if (t == T_F64) {
+    long double acc = kind == RK_PROD ? 1.0L : 0.0L;
+    double best = 0;
+    for (long i = 0; i < n; ++i) {
+      const double x = ((const double *)base)[off + i * stride];
+      if (kind == RK_SUM || kind == RK_MEAN) acc += x;
+      else if (kind == RK_PROD) acc *= x;
+      else if (i == 0) best = x;
+      else if (best == best) { /* the first NaN stays */
+        if (x != x) best = x;
+        else if (kind == RK_MIN ? x < best : x > best) best = x;
+      }
+    }
+    if (kind == RK_MIN || kind == RK_MAX) *rf = best;
+    else if (kind == RK_MEAN) *rf = (double)acc / (double)n;
+    else *rf = (double)acc;
+    return;
+  }
+  uint64_t acc = kind == RK_PROD ? 1 : 0;
+  int64_t best = 0;
+  for (long i = 0; i < n; ++i) {
+    const int64_t x = load_i(t, base, off + i * stride);
+    if (kind == RK_SUM || kind == RK_MEAN) acc += (uint64_t)x;
+    else if (kind == RK_PROD) acc *= (uint64_t)x;
+    else if (i == 0) best = x;
+    else if (kind == RK_MIN ? x < best : x > best) best = x;
+  }
+  *ri = (kind == RK_MIN || kind == RK_MAX) ? best : (int64_t)acc;
+}
+
+/* truncate v to the element type and widen again */
+static int64_t as_type(int t, int64_t v) {
+  switch (t) {
+    case T_U8: return (uint8_t)v;
+    case T_I8: return (int8_t)v;
+    case T_I16: return (int16_t)v;
+    case T_I32: return (int32_t)v;
+    default: return v;
+  }
+}
+
+int th_typed_reduce_dim(int t, int kind, const th_view *out, const th_view *in, int dim) {
+  if (in->nd == 0) return 0;
+  if (out->nd != in->nd || dim < 0 || dim >= in->nd) return 1;
+  long osz[TH_MAX_DIMS];
+  for (int d = 0; d < in->nd; ++d) {
+    osz[d] = d == dim ? 1 : in->size[d];
+    if (out->size[d] != osz[d]) return 1;
+  }
+  th_view il = *in;
+  il.size = osz;
+  const long lines = numel(out), n = in->size[dim];
+  odo oi, oo;
+  odo_start(&oi);
+  odo_start(&oo);
+  for (long l = 0; l < lines; ++l) {
+    int64_t ri = 0;
+    double rf = 0;
+    reduce_slice_typed(t, kind, in->data, oi.off, n, in->stride[dim], &ri, &rf);
+    if (t == T_F64) store_f(t, out->data, oo.off, rf);
+    else if (kind == RK_MEAN) store_i(t, out->data, oo.off, as_type(t, ri) / as_type(t, n));
+    else store_i(t, out->data, oo.off, ri);
+    odo_next(&oi, &il);
+    odo_next(&oo, out);
+  }
+  return 0;
+}
+
+/* (value, 1-based index of the first occurrence) of the max / min along dim */
+int th_typed_minmax_dim(int t, int is_max, const th_view *val, const th_view *idx, const th_view *in,
+                        int dim) {
+  if (in->nd == 0) return 0;
+  if (val->nd != in->nd || idx->nd != in->nd || dim < 0 || dim >= in->nd) return 1;
+  long osz[TH_MAX_DIMS];
+  for (int d = 0; d < in->nd; ++d) osz[d] = d == dim ? 1 : in->size[d];
+  th_view il = *in;
+  il.size = osz;
+  const long lines = numel(val), n = in->size[dim], st = in->stride[dim];
+  odo oi, ov, ox;
+  odo_start(&oi);
+  odo_start(&ov);
+  odo_start(&ox);
+  for (long l = 0; l < lines; ++l) {
+    long at = 0;
+    if (t == T_F64) {
+      double best = ((const double *)in->data)[oi.off];
+      for (long i = 1; i < n && best == best; ++i) {
+        const double x = ((const double *)in->data)[oi.off + i * st];
+        if (x != x || (is_max ? x > best : x < best)) { best = x; at = i; }
+      }
+      ((double *)val->data)[ov.off] = best;
+    } else {
+      int64_t best = load_i(t, in->data, oi.off);
+      for (long i = 1; i < n; ++i) {
+        const int64_t x = load_i(t, in->data, oi.off + i * st);
+        if (is_max ? x > best : x < best) { best = x; at = i; }
+      }
+      store_i(t, val->data, ov.off, best);
+    }
+    ((int64_t *)idx->data)[ox.off] = at + 1;
+    odo_next(&oi, &il);
+    odo_next(&ov, val);
+    odo_next(&ox, idx);
+  }
+  return 0;
+}
+
+/* Whole-tensor reduction in logical order; integer result in *ri (accreal =
+ * long), double result returned. */
+double th_typed_reduce_all(int t, int kind, const th_view *in, long *ri_out) {
+  const long n = numel(in);
+  odo o;
+  odo_start(&o);
+  long double acc = kind == RK_PROD ? 1.0L : 0.0L;
+  uint64_t iacc = kind == RK_PROD ? 1 : 0;
+  double bestf = 0;
+  int64_t besti = 0;
+  for (long i = 0; i < n; ++i) {
+    if (t == T_F64) {
+      const double x = ((const double *)in->data)[o.off];
+      if (kind == RK_SUM || kind == RK_MEAN) acc += x;
+      else if (kind == RK_PROD) acc *= x;
+      else if (i == 0) bestf = x;
+      else if (bestf == bestf) {
+        if (x != x) bestf = x;
+        else if (kind == RK_MIN ? x < bestf : x > bestf) bestf = x;
+      }
+    } else {
+      const int64_t x = load_i(t, in->data, o.off);
+      if (kind == RK_SUM || kind == RK_MEAN) iacc += (uint64_t)x;
+      else if (kind == RK_PROD) iacc *= (uint64_t)x;
+      else if (i == 0) besti = x;
+      else if (kind == RK_MIN ? x < besti : x > besti) besti = x;
+    }
+    odo_next(&o, in);
+  }
+  if (t == T_F64) {
+    if (kind == RK_MIN || kind == RK_MAX) return bestf;
+    if (kind == RK_MEAN) return (double)acc / (double)n;
+    return (double)acc;
+  }
+  int64_t r = (kind == RK_MIN || kind == RK_MAX) ? besti : (int64_t)iacc;
+  if (kind == RK_MEAN) r = r / n;   /* accreal division (sumall / nElement) */
+  *ri_out = r;
+  return (double)r;
+}

@@ -393,3 +393,138 @@ def test_gpu_same_type_copy_of_transposed_tensors(thc, oracle, kind):
     out.copy(d.t())
     assert_bit_equal(out.numpy(), np.ascontiguousarray(x.T))
     assert thc.last_kernel().startswith("tiled")
+
+
+# ------------------------------------------------------------------ reductions --
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_oracle_typed_reductions_match_numpy(oracle, kind):
+    rng = np.random.default_rng(11)
+    dt = np_of(oracle, kind)
+    for shape, dim in (((5, 40), 1), ((30, 6), 0), ((3, 17, 4), 1)):
+        geom = random_geometry(rng, shape)
+        st = rand_storage(rng, kind, geom[0], oracle)
+        v = oracle.View(st, *geom[1:])
+        x = v.numpy()
+        if kind == "double":
+            np.testing.assert_allclose(oracle.typed_reduce_dim("sum", v, dim).numpy(), x.sum(axis=dim, keepdims=True),
+                                       rtol=1e-13, atol=1e-13)
+            np.testing.assert_allclose(oracle.typed_reduce_dim("mean", v, dim).numpy(), x.mean(axis=dim, keepdims=True),
+                                       rtol=1e-13, atol=1e-13)
+            import math
+            assert abs(oracle.typed_reduce_all("sum", v) - math.fsum(x.ravel())) <= 1e-13 * np.abs(x).sum()
+        else:
+            with np.errstate(over="ignore"):
+                want = x.astype(np.int64).sum(axis=dim, keepdims=True)           # wraps in 64 bits
+                assert_bit_equal(oracle.typed_reduce_dim("sum", v, dim).numpy(), want.astype(dt), "sum")
+                wantp = np.multiply.reduce(x.astype(np.int64), axis=dim, keepdims=True)
+                assert_bit_equal(oracle.typed_reduce_dim("prod", v, dim).numpy(), wantp.astype(dt), "prod")
+                assert oracle.typed_reduce_all("sum", v) == int(x.astype(np.int64).sum())
+                s_t = want.astype(dt).astype(np.int64)
+                n_t = int(np.array(shape[dim]).astype(dt))
+                q = np.sign(s_t) * (np.abs(s_t) // n_t)                            # C division truncates
+                assert_bit_equal(oracle.typed_reduce_dim("mean", v, dim).numpy(), q.astype(dt), "mean")
+        assert_bit_equal(oracle.typed_reduce_dim("max", v, dim).numpy(), x.max(axis=dim, keepdims=True))
+        assert_bit_equal(oracle.typed_reduce_dim("min", v, dim).numpy(), x.min(axis=dim, keepdims=True))
+        xs = v.numpy()
+        small = oracle.View.of((xs % 5).astype(dt) if kind != "double" else np.round(xs))   # many ties
+        for which, f in (("max", np.argmax), ("min", np.argmin)):
+            vals, idx = oracle.typed_minmax_dim(which, small, dim)
+            assert np.array_equal(idx.numpy(), np.expand_dims(f(small.numpy(), axis=dim), dim) + 1)
+            assert_bit_equal(vals.numpy(), getattr(small.numpy(), which)(axis=dim, keepdims=True))
+        assert oracle.typed_reduce_all("max", v) == x.max() and oracle.typed_reduce_all("min", v) == x.min()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_gpu_typed_reductions(thc, oracle, kind):
+    rng = np.random.default_rng(106)
+    dt = np_of(oracle, kind)
+    shapes = [((7, 1024), 1), ((300, 64), 1), ((64, 512), 0), ((6, 300, 40), 1), ((3, 1 << 17), 1),
+              ((2, 8192, 96), 1), ((5, 3), 0), ((1000, 17), 1), ((4097,), 0)]
+    for trial, (shape, dim) in enumerate(shapes):
+        geom = contiguous_geometry(shape) if trial < 6 else random_geometry(rng, shape)
+        dev, ref = dev_ref(thc, oracle, rng, kind, geom)
+        for op in ("sum", "prod", "mean"):
+            if op == "mean" and kind != "double" and int(np.array(shape[dim]).astype(dt)) == 0:
+                continue
+            if op == "prod" and kind == "double":
+                st = rng.uniform(0.9, 1.1, geom[0])
+                dev2, ref2 = thc.Tensor.from_storage(st, *geom[1:], kind=kind), oracle.View(st.copy(), *geom[1:])
+            else:
+                dev2, ref2 = dev, ref
+            got = getattr(thc.Tensor(kind), op)(dev2, dim).numpy()
+            want = oracle.typed_reduce_dim(op, ref2, dim).numpy()
+            if kind == "double":
+                mass = np.abs(ref2.numpy()).sum(axis=dim, keepdims=True) if op != "prod" else np.abs(want)
+                if op == "mean":
+                    mass = mass / shape[dim]
+                assert np.all(np.abs(got - want) <= 1e-13 * np.maximum(mass, 1e-300)), (kind, op, shape)
+            else:
+                assert_bit_equal(got, want, "%s %s %s" % (kind, op, shape))
+        for which in ("max", "min"):
+            small = (ref.numpy() % 7).astype(dt) if kind != "double" else np.round(ref.numpy())
+            ds, rs = thc.Tensor.from_numpy(small), oracle.View.of(small)
+            vals, idx = thc.Tensor(kind), thc.Tensor("long")
+            getattr(vals, which)(idx, ds, dim)
+            wv, wi = oracle.typed_minmax_dim(which, rs, dim)
+            assert_bit_equal(vals.numpy(), wv.numpy(), "%s %s values %s" % (kind, which, shape))
+            assert np.array_equal(idx.numpy(), wi.numpy()), (kind, which, shape)
+            vals, idx = thc.Tensor(kind), thc.Tensor("long")
+            getattr(vals, which)(idx, dev, dim)                  # full-range values
+            wv, wi = oracle.typed_minmax_dim(which, ref, dim)
+            assert_bit_equal(vals.numpy(), wv.numpy())
+            assert np.array_equal(idx.numpy(), wi.numpy())
+        if kind == "double":
+            assert abs(dev.sumall() - oracle.typed_reduce_all("sum", ref)) <= 1e-13 * np.abs(ref.numpy()).sum()
+            assert abs(dev.meanall() - oracle.typed_reduce_all("mean", ref)) <= 1e-13 * np.abs(ref.numpy()).mean()
+        else:
+            assert dev.sumall() == oracle.typed_reduce_all("sum", ref)
+            assert dev.prodall() == oracle.typed_reduce_all("prod", ref)
+            assert dev.meanall() == oracle.typed_reduce_all("mean", ref)
+        assert dev.maxall() == oracle.typed_reduce_all("max", ref)
+        assert dev.minall() == oracle.typed_reduce_all("min", ref)
+        assert dev.equal(dev.clone())
+        other = dev.clone()
+        other.add(other, 1)
+        assert not dev.equal(other)
+
+
+@pytest.mark.gpu
+def test_gpu_logicalall_any(thc):
+    rng = np.random.default_rng(107)
+    for n in (1, 1000, 1 << 20):
+        x = np.ones(n, np.uint8) * 3
+        t = thc.Tensor.from_numpy(x)
+        assert t.logicalall() == 1 and t.logicalany() == 1
+        x[int(rng.integers(0, n))] = 0
+        t = thc.Tensor.from_numpy(x)
+        assert t.logicalall() == 0 and t.logicalany() == (1 if n > 1 else 0)
+        z = thc.Tensor.from_numpy(np.zeros(n, np.uint8))
+        assert z.logicalall() == 0 and z.logicalany() == 0
+    # the usual use: any(a > b)
+    a = thc.Tensor.from_numpy(rng.standard_normal((50, 70)).astype(np.float32))
+    m = thc.Tensor("byte").compare_value("gt", a, 10.0)
+    assert m.logicalany() == 0
+    m = thc.Tensor("byte").compare_value("lt", a, 10.0)
+    assert m.logicalall() == 1
+
+
+@pytest.mark.gpu
+def test_gpu_double_norm_var_std_dist(thc, oracle):
+    rng = np.random.default_rng(108)
+    x = rng.uniform(-2, 2, (40, 300, 24))
+    y = rng.uniform(-2, 2, (40, 300, 24))
+    d, e = thc.Tensor.from_numpy(x), thc.Tensor.from_numpy(y)
+    for dim in (0, 1, 2):
+        np.testing.assert_allclose(thc.Tensor("double").norm(d, 2.0, dim).numpy(),
+                                   np.sqrt((x * x).sum(axis=dim, keepdims=True)), rtol=1e-13)
+        np.testing.assert_allclose(thc.Tensor("double").norm(d, 3.0, dim).numpy(),
+                                   (np.abs(x) ** 3).sum(axis=dim, keepdims=True) ** (1 / 3.0), rtol=1e-12)
+        np.testing.assert_allclose(thc.Tensor("double").var(d, dim).numpy(), x.var(axis=dim, ddof=1, keepdims=True),
+                                   rtol=1e-12)
+        np.testing.assert_allclose(thc.Tensor("double").std(d, dim, biased=1).numpy(),
+                                   x.std(axis=dim, keepdims=True), rtol=1e-12)
+    assert abs(d.normall(2.0) - np.sqrt((x * x).sum())) <= 1e-12 * np.sqrt((x * x).sum())
+    assert abs(d.varall() - x.var(ddof=1)) <= 1e-12
+    assert abs(d.stdall(1) - x.std()) <= 1e-12
+    assert abs(d.dist(e, 2.0) - np.sqrt(((x - y) ** 2).sum())) <= 1e-11
