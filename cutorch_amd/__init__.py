@@ -448,6 +448,9 @@ class Tensor(object):
     def cumprod(self, src, dim):
         return self._call("cumprod", self.h, src.h, dim)
 
+    def renorm(self, src, p, dim, maxnorm):
+        return self._call("renorm", self.h, src.h, self._real(p), dim, self._real(maxnorm))
+
     def var(self, src, dim, biased=0, keepdim=1):
         return self._call("var", self.h, src.h, dim, biased, keepdim)
 

@@ -119,6 +119,10 @@ __device__ __forceinline__ float math1(int fn, float x, float v, float w) {
     case (int)MathFn::MinValue: return x < v ? x : v;
     case (int)MathFn::FmodValue: return fmodf(x, v);
     case (int)MathFn::RemainderValue: return v == 0.f ? NAN : x - v * floorf(x / v);
+    case (int)MathFn::RenormFactor: {
+      const float n = powf(x, w);
+      return n > v ? v / (n + 1e-7f) : 1.0f;
+    }
     default: return x;
   }
 }

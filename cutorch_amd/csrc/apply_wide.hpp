@@ -144,6 +144,10 @@ __device__ __forceinline__ double dmath1(int fn, double x, double v, double w) {
     case (int)MathFn::RemainderValue: return v == 0.0 ? (double)NAN : x - v * floor(x / v);
     case (int)MathFn::LShiftValue: return x * pow(2.0, v);   // THCTensorMathPairwise.cu:436-462
     case (int)MathFn::RShiftValue: return x / pow(2.0, v);
+    case (int)MathFn::RenormFactor: {
+      const double n = pow(x, w);
+      return n > v ? v / (n + 1e-7) : 1.0;
+    }
     default: return x;
   }
 }

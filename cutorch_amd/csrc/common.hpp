@@ -235,7 +235,10 @@ enum class MathFn : int {
   SqDiff,     // (a - b)^2
   // shifts and bitwise ops (THCTensorMathPairwise.cu:408-560, THCTensorMathPointwise.cuh:462-620)
   LShiftValue, RShiftValue, BitAndValue, BitOrValue, BitXorValue,   // x (op) v
-  CLShift, CRShift, CBitAnd, CBitOr, CBitXor                        // a (op) b
+  CLShift, CRShift, CBitAnd, CBitOr, CBitXor,                       // a (op) b
+  // x = sum |e|^p of a slice, v = maxnorm, w = 1/p: the factor renorm scales the slice by,
+  // n = x^w; n > v ? v / (n + 1e-7) : 1   (THCTensorMathReduce.cuh:160-176)
+  RenormFactor
 };
 int point_op_inputs(PointOp op);
 

@@ -174,6 +174,45 @@ float var_all(THCState* s, DType dt, AnyTensor* self, int biased) {
   return all_or_throw(s, dt, ReduceOp::SqDev, mean, self) / (n - (biased ? 0.f : 1.f));
 }
 
+// renorm (generic/THCTensorMathReduce.cu:46-74): every slice src[.., i, ..] along
+// `dim` whose p-norm exceeds maxnorm is scaled to norm maxnorm. The reference
+// clones a transposed copy and runs one 32-thread block per slice; here the
+// slice sums of |x|^p come from the reduce engine (all other dims reduced one
+// after the other, the first pass being the only one that reads the whole
+// tensor), the factors from one tiny pointwise launch, and the scaling is a
+// cmul against the factors broadcast with stride 0: no transposed copy.
+void renorm(THCState* s, DType dt, AnyTensor* self, AnyTensor* src, double p, long dim,
+            double maxnorm) {
+  same_gpu(s, {self, src});
+  THC_ARG_CHECK(dim >= 0 && dim < src->nDimension, 3, "invalid dimension");
+  THC_ARG_CHECK(p > 0, 2, "non-positive-norm not supported");
+  THC_ARG_CHECK(src->nDimension > 1, 1, "need at least 2 dimensions");
+  TensorRef sums(s, tensor_new(s));
+  AnyTensor* cur = src;
+  bool first = true;
+  for (int d = 0; d < src->nDimension; ++d) {
+    if (d == dim) continue;
+    ReduceOp op = ReduceOp::Sum;
+    if (first) op = p == 1.0 ? ReduceOp::Norm1 : (p == 2.0 ? ReduceOp::Norm2 : ReduceOp::NormP);
+    if (!reduce_dim(s, dt, op, Epilogue::None, p, sums.t, cur, d, 1))
+      raise_arg_error(2, "%s", kDimWarning);
+    cur = sums.t;
+    first = false;
+  }
+  // sums has size 1 everywhere except at `dim`: turn it into the factors
+  const ApplyDesc fd{dt, dt, PointOp::Math1, (int)MathFn::RenormFactor, scalar_of(maxnorm),
+                     scalar_of(1.0 / p), false};
+  if (!pointwise_apply(s, fd, sums.t, sums.t, nullptr, nullptr)) raise_arg_error(2, "%s", kDimWarning);
+  TensorRef wide(s, tensor_new_with_tensor(s, sums.t, dt));  // factors viewed with src's shape
+  for (int d = 0; d < src->nDimension; ++d) {
+    if (d == dim) continue;
+    wide.t->size[d] = src->size[d];
+    wide.t->stride[d] = 0;
+  }
+  if (self != src) tensor_resize_as(s, self, src, dt);
+  apply_or_throw(s, dt, PointOp::Mul, 0.f, self, src, wide.t);
+}
+
 // dist(a, b, p) = (sum |a - b|^p)^(1/p)  (generic/THCTensorMathReduce.cu:234-259)
 float dist_all(THCState* s, DType dt, AnyTensor* a, AnyTensor* b, float p) {
   same_gpu(s, {a, b});
@@ -409,6 +448,10 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
   THC_API float Tensor##_stdall(THCState* s, Tensor* self, int biased) {                           \
     THC_GUARD_RET(0.f, return sqrtf(var_all(s, DT, TN(self), biased)))                             \
   }                                                                                                \
+  THC_API void Tensor##_renorm(THCState* s, Tensor* self, Tensor* src, real p, long dim,           \
+                               real maxnorm) {                                                     \
+    THC_GUARD_VOID(renorm(s, DT, TN(self), TN(src), to_float(p), dim, to_float(maxnorm)))          \
+  }                                                                                                \
   THC_API float Tensor##_dist(THCState* s, Tensor* self, Tensor* src, real p) {                    \
     THC_GUARD_RET(0.f, return dist_all(s, DT, TN(self), TN(src), to_float(p)))                     \
   }                                                                                                \
@@ -556,6 +599,18 @@ double dist_all_d(THCState* s, AnyTensor* a, AnyTensor* b, double p) {
   }                                                                                                \
   THC_API int Tensor##_equal(THCState* s, Tensor* self, Tensor* src) {                             \
     THC_GUARD_RET(0, return tensors_equal(s, DT, TN(self), TN(src)))                               \
+  }                                                                                                \
+  THC_API void Tensor##_cumsum(THCState* s, Tensor* self, Tensor* src, long dim) {                 \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {self, src});                                                                    \
+      scan_dim(s, DT, false, TN(self), TN(src), (int)dim);                                         \
+    })                                                                                             \
+  }                                                                                                \
+  THC_API void Tensor##_cumprod(THCState* s, Tensor* self, Tensor* src, long dim) {                \
+    THC_GUARD_VOID({                                                                               \
+      same_gpu(s, {self, src});                                                                    \
+      scan_dim(s, DT, true, TN(self), TN(src), (int)dim);                                          \
+    })                                                                                             \
   }
 
 THC_AMD_DEFINE_WIDE_REDUCE_API(THCudaByteTensor, unsigned char, long, DType::U8, 0, 255)
@@ -585,6 +640,10 @@ THC_API void THCudaDoubleTensor_var(THCState* s, THCudaDoubleTensor* self, THCud
 THC_API void THCudaDoubleTensor_std(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
                                     long dim, int biased, int keepdim) {
   THC_GUARD_VOID(var_dim(s, DType::F64, true, TN(self), TN(src), dim, biased, keepdim))
+}
+THC_API void THCudaDoubleTensor_renorm(THCState* s, THCudaDoubleTensor* self, THCudaDoubleTensor* src,
+                                       double p, long dim, double maxnorm) {
+  THC_GUARD_VOID(renorm(s, DType::F64, TN(self), TN(src), p, dim, maxnorm))
 }
 THC_API double THCudaDoubleTensor_normall(THCState* s, THCudaDoubleTensor* self, double p) {
   THC_GUARD_RET(0.0, return norm_all_d(s, TN(self), p))

@@ -64,10 +64,18 @@ bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTe
   if (out->nDimension > kMaxDims || in->nDimension > kMaxDims) return false;  // THCReduce.cuh:278-281
   if (in->nDimension == 0) return true;                                        // :283-286
   THC_ARG_CHECK(dim >= 0 && dim < in->nDimension, 3, "dimension out of range");
-  TensorRef hold(s, nullptr);
-  if (out == in) {  // the output is resized before the input is read
-    hold.t = tensor_new_with_tensor(s, in, dt);
-    in = hold.t;
+  // An output on the input's own storage (x:sum(x, dim), or a view of it) would
+  // be written while other workgroups still read the input: reduce into a
+  // fresh tensor and copy. (A centred reduction reads its centres from `out`,
+  // which never is the input.)
+  if (out->storage && out->storage == in->storage) {
+    TensorRef tmp(s, tensor_new(s));
+    if (!reduce_dim(s, dt, op, ep, p, tmp.t, in, dim, 1)) return false;
+    TensorRef hold(s, tensor_new_with_tensor(s, in, dt));  // keeps `in` alive if out == in
+    resize_reduced(s, out, hold.t, dim, dt);
+    copy_tensor(s, dt, out, tmp.t, false);
+    if (!keepdim) tensor_squeeze1d(s, out, nullptr, dim, dt);
+    return true;
   }
   resize_reduced(s, out, in, dim, dt);
   ReduceGeom g = make_geom(in, out, nullptr, dim);
@@ -96,10 +104,17 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
                       AnyTensor* in, int dim, int keepdim) {
   THC_ARG_CHECK(dim >= 0 && dim < in->nDimension, 3, "dimension out of range");
   if (in->nDimension > kMaxDims) raise_arg_error(2, "%s", kDimWarning);
-  TensorRef hold(s, nullptr);
-  if (values == in) {
-    hold.t = tensor_new_with_tensor(s, in, dt);
-    in = hold.t;
+  if (values->storage && values->storage == in->storage) {  // see reduce_dim
+    TensorRef tmp(s, tensor_new(s));
+    reduce_dim_index(s, dt, isMax, tmp.t, indices, in, dim, 1);
+    TensorRef hold(s, tensor_new_with_tensor(s, in, dt));
+    resize_reduced(s, values, hold.t, dim, dt);
+    copy_tensor(s, dt, values, tmp.t, false);
+    if (!keepdim) {
+      tensor_squeeze1d(s, values, nullptr, dim, dt);
+      tensor_squeeze1d(s, indices, nullptr, dim, DType::I64);
+    }
+    return;
   }
   resize_reduced(s, values, in, dim, dt);
   resize_reduced(s, indices, in, dim, DType::I64);

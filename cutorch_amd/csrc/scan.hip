@@ -10,20 +10,89 @@
 //   inner  > 1  lanes run along the unit-stride inner dim (coalesced), thread
 //               rows split the scanned dim into register-resident segments
 //               and exchange segment totals through LDS.
-// Accumulation is fp32 (also for half tensors, rounded per output element).
+// Accumulation is fp32 for float and half (rounded per output element), double
+// for double, wrapping 64-bit for the integer types.
+#include <type_traits>
+
 #include "common.hpp"
 #include "device_util.hpp"
 
 namespace thc {
 namespace {
 
-struct ScanAdd {
-  static __device__ __forceinline__ float id() { return 0.f; }
-  static __device__ __forceinline__ float op(float a, float b) { return a + b; }
+// Accumulator of an element type: float for float and half, double for
+// double, long for the integer types (wrapping).
+template <typename T>
+struct ScanAcc {
+  using type = int64_t;
 };
+template <>
+struct ScanAcc<float> {
+  using type = float;
+};
+template <>
+struct ScanAcc<__half> {
+  using type = float;
+};
+template <>
+struct ScanAcc<double> {
+  using type = double;
+};
+template <typename A, typename T>
+__device__ __forceinline__ A scan_up(T x) {
+  if constexpr (std::is_same<T, __half>::value) return (A)__half2float(x);
+  else return (A)x;
+}
+template <typename T, typename A>
+__device__ __forceinline__ T scan_down(A a) {
+  if constexpr (std::is_same<T, __half>::value) return __float2half_rn((float)a);
+  else return (T)a;
+}
+// Lane exchange; 8-byte values travel as two 32-bit halves.
+template <typename A, typename Fn>
+__device__ __forceinline__ A lane_exchange(A v, Fn&& fn) {
+  if constexpr (sizeof(A) == 8) {
+    uint64_t bits;
+    __builtin_memcpy(&bits, &v, 8);
+    const uint32_t lo = fn((uint32_t)bits);
+    const uint32_t hi = fn((uint32_t)(bits >> 32));
+    bits = ((uint64_t)hi << 32) | lo;
+    A r;
+    __builtin_memcpy(&r, &bits, 8);
+    return r;
+  } else {
+    uint32_t bits;
+    __builtin_memcpy(&bits, &v, 4);
+    bits = fn(bits);
+    A r;
+    __builtin_memcpy(&r, &bits, 4);
+    return r;
+  }
+}
+template <typename A>
+__device__ __forceinline__ A shfl_up_any(A v, uint32_t o) {
+  return lane_exchange(v, [o](uint32_t w) { return __shfl_up(w, o, 64); });
+}
+template <typename A>
+__device__ __forceinline__ A shfl_any(A v, int lane) {
+  return lane_exchange(v, [lane](uint32_t w) { return __shfl(w, lane, 64); });
+}
+
+template <typename A>
+struct ScanAdd {
+  static __device__ __forceinline__ A id() { return (A)0; }
+  static __device__ __forceinline__ A op(A a, A b) {
+    if constexpr (std::is_integral<A>::value) return (A)((uint64_t)a + (uint64_t)b);
+    else return a + b;
+  }
+};
+template <typename A>
 struct ScanMul {
-  static __device__ __forceinline__ float id() { return 1.f; }
-  static __device__ __forceinline__ float op(float a, float b) { return a * b; }
+  static __device__ __forceinline__ A id() { return (A)1; }
+  static __device__ __forceinline__ A op(A a, A b) {
+    if constexpr (std::is_integral<A>::value) return (A)((uint64_t)a * (uint64_t)b);
+    else return a * b;
+  }
 };
 
 // One wave64 per row. A lane owns VEC consecutive elements of each
@@ -33,6 +102,7 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t numRows, uint64_t R) {
   using P = Pack<T, VEC>;
+  using A = typename ScanAcc<T>::type;
   constexpr int U = 4;
   constexpr uint64_t kChunk = 64 * VEC;
   const uint32_t lane = threadIdx.x & 63;
@@ -41,9 +111,9 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
        row += wavesPerGrid) {
     const T* src = in + row * R;
     T* dst = out + row * R;
-    float carry = Op::id();
+    A carry = Op::id();
     for (uint64_t base = 0; base < R; base += U * kChunk) {
-      float x[U][VEC];
+      A x[U][VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint64_t i0 = base + u * kChunk + (uint64_t)lane * VEC;
@@ -52,13 +122,13 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
           if (i0 < R) {
             const P v = load_pack<true>(reinterpret_cast<const P*>(src + i0));
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) x[u][k] = Cvt<T>::up(v.v[k]);
+            for (int k = 0; k < VEC; ++k) x[u][k] = scan_up<A>(v.v[k]);
           } else {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) x[u][k] = Op::id();
           }
         } else {
-          x[u][0] = i0 < R ? Cvt<T>::up(src[i0]) : Op::id();
+          x[u][0] = i0 < R ? scan_up<A>(src[i0]) : Op::id();
         }
       }
 #pragma unroll
@@ -67,26 +137,26 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
 #pragma unroll
         for (int k = 1; k < VEC; ++k) x[u][k] = Op::op(x[u][k - 1], x[u][k]);
         // inclusive scan of the lane totals across the wave
-        float t = x[u][VEC - 1];
+        A t = x[u][VEC - 1];
 #pragma unroll
         for (uint32_t o = 1; o < 64; o <<= 1) {
-          const float y = __shfl_up(t, o, 64);
+          const A y = shfl_up_any(t, o);
           if (lane >= o) t = Op::op(y, t);
         }
-        float before = __shfl_up(t, 1, 64);  // exclusive prefix of this lane
+        A before = shfl_up_any(t, 1);  // exclusive prefix of this lane
         if (lane == 0) before = Op::id();
-        const float offset = Op::op(carry, before);
+        const A offset = Op::op(carry, before);
         if (i0 < R) {
           if (VEC > 1) {
             P v;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) v.v[k] = Cvt<T>::down(Op::op(offset, x[u][k]));
+            for (int k = 0; k < VEC; ++k) v.v[k] = scan_down<T>(Op::op(offset, x[u][k]));
             *reinterpret_cast<P*>(dst + i0) = v;
           } else {
-            dst[i0] = Cvt<T>::down(Op::op(offset, x[u][0]));
+            dst[i0] = scan_down<T>(Op::op(offset, x[u][0]));
           }
         }
-        carry = Op::op(carry, __shfl(t, 63, 64));
+        carry = Op::op(carry, shfl_any(t, 63));
       }
     }
   }
@@ -105,8 +175,9 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
                                                            uint64_t inner, uint32_t TX,
                                                            uint64_t colTiles) {
   using P = Pack<T, VEC>;
+  using A = typename ScanAcc<T>::type;
   constexpr int U = 8;
-  __shared__ float totals[2][kBlock * VEC];
+  __shared__ A totals[2][kBlock * VEC];
   const uint32_t TY = kBlock / TX;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const uint64_t blocks = outer * colTiles;
@@ -116,19 +187,19 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
     const bool live = col < inner;  // inner % VEC == 0 for VEC > 1
     const T* src = in + o * R * inner + col;
     T* dst = out + o * R * inner + col;
-    float carry[VEC];
+    A carry[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) carry[e] = Op::id();
     uint32_t flip = 0;
     for (uint64_t seg = 0; seg < R; seg += (uint64_t)TY * U, flip ^= 1) {
       const uint64_t r0 = seg + (uint64_t)ty * U;
-      float x[U][VEC];
+      A x[U][VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (live && r0 + u < R) {
           const P v = load_pack<true>(reinterpret_cast<const P*>(src + (r0 + u) * inner));
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) x[u][e] = Cvt<T>::up(v.v[e]);
+          for (int e = 0; e < VEC; ++e) x[u][e] = scan_up<A>(v.v[e]);
         } else {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) x[u][e] = Op::id();
@@ -142,7 +213,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
 #pragma unroll
       for (int e = 0; e < VEC; ++e) totals[flip][(ty * TX + tx) * VEC + e] = x[U - 1][e];
       __syncthreads();  // the other buffer is free again after the next barrier
-      float offset[VEC], running[VEC];
+      A offset[VEC], running[VEC];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         running[e] = Op::id();
@@ -162,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
         if (live && r0 + u < R) {
           P v;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) v.v[e] = Cvt<T>::down(Op::op(offset[e], x[u][e]));
+          for (int e = 0; e < VEC; ++e) v.v[e] = scan_down<T>(Op::op(offset[e], x[u][e]));
           *reinterpret_cast<P*>(dst + (r0 + u) * inner) = v;
         }
       }
@@ -181,7 +252,11 @@ uint32_t pow2_at_least(uint64_t x) {
 
 template <typename T, typename Op>
 void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int64_t inner) {
-  constexpr int VEC = 16 / sizeof(T);
+  // Packs are capped so that a lane's segment stays in registers when the
+  // accumulator (8 bytes for the integer types) is wider than the element.
+  constexpr int kFull = 16 / sizeof(T);
+  constexpr int VEC = kFull > 8 ? 8 : kFull;     // rows kernel
+  constexpr int VECC = (sizeof(typename ScanAcc<T>::type) == 4 || kFull <= 4) ? kFull : 4;  // column kernel
   hipStream_t st = current_stream(s);
   const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
   if (inner == 1) {
@@ -196,8 +271,8 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
                          (uint64_t)outer, (uint64_t)R);
     note_kernel("scan-rows");
   } else {
-    const bool vec = aligned && inner % VEC == 0;
-    const int64_t pack = vec ? VEC : 1;
+    const bool vec = aligned && inner % VECC == 0;
+    const int64_t pack = vec ? VECC : 1;
     const int64_t packs = (inner + pack - 1) / pack;
     // 16..64 lanes along the unit-stride dim: narrower tiles when that is what
     // gives every CU a workgroup
@@ -207,7 +282,7 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t colTiles = (packs + TX - 1) / TX;
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * colTiles, 1 << 30));
     if (vec)
-      hipLaunchKernelGGL((scan_cols_kernel<T, Op, VEC>), dim3(grid), dim3(kBlock), 0, st, out, in,
+      hipLaunchKernelGGL((scan_cols_kernel<T, Op, VECC>), dim3(grid), dim3(kBlock), 0, st, out, in,
                          (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles);
     else
       hipLaunchKernelGGL((scan_cols_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
@@ -235,14 +310,21 @@ void scan_dim(THCState* s, DType dt, bool product, AnyTensor* self, AnyTensor* s
   const int64_t R = src->size[dim];
   void* o = tensor_data(dst.t, dt);
   const void* i = tensor_data(in.t, dt);
-  if (dt == DType::F32) {
-    if (product) launch_scan<float, ScanMul>(s, (float*)o, (const float*)i, outer, R, inner);
-    else launch_scan<float, ScanAdd>(s, (float*)o, (const float*)i, outer, R, inner);
-  } else if (dt == DType::F16) {
-    if (product) launch_scan<__half, ScanMul>(s, (__half*)o, (const __half*)i, outer, R, inner);
-    else launch_scan<__half, ScanAdd>(s, (__half*)o, (const __half*)i, outer, R, inner);
-  } else {
-    raise_error("scan not available for this element type");
+  auto go = [&](auto tag) {
+    using T = decltype(tag);
+    using A = typename ScanAcc<T>::type;
+    if (product) launch_scan<T, ScanMul<A>>(s, (T*)o, (const T*)i, outer, R, inner);
+    else launch_scan<T, ScanAdd<A>>(s, (T*)o, (const T*)i, outer, R, inner);
+  };
+  switch (dt) {
+    case DType::U8: go(uint8_t{}); break;
+    case DType::I8: go(int8_t{}); break;
+    case DType::I16: go(int16_t{}); break;
+    case DType::I32: go(int32_t{}); break;
+    case DType::I64: go(int64_t{}); break;
+    case DType::F16: go(__half{}); break;
+    case DType::F32: go(float{}); break;
+    case DType::F64: go(double{}); break;
   }
   THC_CHECK(hipGetLastError());
   if (dst.t != self) copy_tensor(s, dt, self, dst.t, false);

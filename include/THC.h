@@ -288,6 +288,7 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
 /*   fill / zero        : generic/THCTensorMath.h:5-6                         */
 /* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
 /* Scans: generic/THCTensorMathScan.h (cumsum, cumprod)                       */
+/* renorm: generic/THCTensorMathReduce.h:7                                    */
 /* ------------------------------------------------------------------------ */
 #define THC_AMD_DECLARE_MATH_API(Tensor, real, accreal)                        \
   THC_API void Tensor##_add(THCState *, Tensor *self, Tensor *src, real v);    \
@@ -379,6 +380,8 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
                             int biased, int keepdim);                          \
   THC_API accreal Tensor##_varall(THCState *, Tensor *self, int biased);       \
   THC_API accreal Tensor##_stdall(THCState *, Tensor *self, int biased);       \
+  THC_API void Tensor##_renorm(THCState *, Tensor *self, Tensor *src,          \
+                               real p, long dim, real maxnorm);                \
   THC_API accreal Tensor##_dist(THCState *, Tensor *self, Tensor *src,         \
                                 real p);                                       \
   THC_API void Tensor##_cumsum(THCState *, Tensor *self, Tensor *src,          \
@@ -538,7 +541,11 @@ THC_API void THCudaDoubleTensor_lerp(THCState *, THCudaDoubleTensor *self, THCud
   THC_API accreal Tensor##_meanall(THCState *, Tensor *self);                  \
   THC_API real Tensor##_minall(THCState *, Tensor *self);                      \
   THC_API real Tensor##_maxall(THCState *, Tensor *self);                      \
-  THC_API int Tensor##_equal(THCState *, Tensor *self, Tensor *src);
+  THC_API int Tensor##_equal(THCState *, Tensor *self, Tensor *src);           \
+  THC_API void Tensor##_cumsum(THCState *, Tensor *self, Tensor *src,          \
+                               long dim);                                      \
+  THC_API void Tensor##_cumprod(THCState *, Tensor *self, Tensor *src,         \
+                                long dim);
 THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaByteTensor, unsigned char, long)
 THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaCharTensor, char, long)
 THC_AMD_DECLARE_WIDE_REDUCE_API(THCudaShortTensor, short, long)
@@ -552,6 +559,7 @@ THC_API int THCudaByteTensor_logicalany(THCState *, THCudaByteTensor *self);
 THC_API void THCudaDoubleTensor_norm(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, double p, long dim, int keepdim);
 THC_API void THCudaDoubleTensor_var(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, long dim, int biased, int keepdim);
 THC_API void THCudaDoubleTensor_std(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, long dim, int biased, int keepdim);
+THC_API void THCudaDoubleTensor_renorm(THCState *, THCudaDoubleTensor *self, THCudaDoubleTensor *src, double p, long dim, double maxnorm);
 THC_API double THCudaDoubleTensor_normall(THCState *, THCudaDoubleTensor *self, double p);
 THC_API double THCudaDoubleTensor_varall(THCState *, THCudaDoubleTensor *self, int biased);
 THC_API double THCudaDoubleTensor_stdall(THCState *, THCudaDoubleTensor *self, int biased);

@@ -80,6 +80,8 @@ def lib():
         l.th_typed_minmax_dim.argtypes = [C.c_int, C.c_int, VP, VP, VP, C.c_int]
         l.th_typed_reduce_all.argtypes = [C.c_int, C.c_int, VP, C.POINTER(C.c_long)]
         l.th_typed_reduce_all.restype = C.c_double
+        l.th_typed_scan_dim.argtypes = [C.c_int, C.c_int, VP, VP, C.c_int]
+        l.th_renorm.argtypes = [C.c_int, VP, VP, C.c_double, C.c_int, C.c_double]
         l.th_half2float.argtypes = [C.c_uint16]
         l.th_half2float.restype = C.c_float
         l.th_float2half.argtypes = [C.c_float]
@@ -220,6 +222,22 @@ def typed_minmax_dim(which, src, dim):
                                  _ptr(src), dim):
         raise ValueError("shape mismatch")
     return values, indices
+
+
+def typed_scan_dim(src, dim, product=False):
+    out = View.empty(src.size, src.storage.dtype)
+    if lib().th_typed_scan_dim(DTYPES[src.kind], 1 if product else 0, _ptr(out), _ptr(src), dim):
+        raise ValueError("shape mismatch")
+    return out
+
+
+def renorm(src, p, dim, maxnorm, out=None):
+    """float / half / double views."""
+    if out is None:
+        out = View.empty(src.size, src.storage.dtype)
+    if lib().th_renorm(DTYPES[src.kind], _ptr(out), _ptr(src), float(p), dim, float(maxnorm)):
+        raise ValueError("shape mismatch")
+    return out
 
 
 def typed_reduce_all(kind, src):

@@ -544,3 +544,83 @@ double th_typed_reduce_all(int t, int kind, const th_view *in, long *ri_out) {
   *ri_out = r;
   return (double)r;
 }
+
+/* ------------------------------------------------------------------ scans -- */
+/* Inclusive prefix sum / product along dim for the integer types (64-bit
+ * wrapping accumulator, stored wrapped to the element type) and double
+ * (sequential long double accumulator, rounded per element). Entry semantics
+ * as lib/THC/generic/THCTensorMathScan.cu:76-126. */
+int th_typed_scan_dim(int t, int product, const th_view *out, const th_view *in, int dim) {
+  if (in->nd == 0) return 0;
+  if (out->nd != in->nd || dim < 0 || dim >= in->nd) return 1;
+  long osz[TH_MAX_DIMS];
+  for (int d = 0; d < in->nd; ++d) {
+    if (out->size[d] != in->size[d]) return 1;
+    osz[d] = d == dim ? 1 : in->size[d];
+  }
+  th_view il = *in, ol = *out;
+  il.size = osz;
+  ol.size = osz;
+  const long lines = numel(&il), n = in->size[dim];
+  odo oi, oo;
+  odo_start(&oi);
+  odo_start(&oo);
+  for (long l = 0; l < lines; ++l) {
+    long double facc = product ? 1.0L : 0.0L;
+    uint64_t iacc = product ? 1 : 0;
+    for (long i = 0; i < n; ++i) {
+      const long src = oi.off + i * in->stride[dim], dst = oo.off + i * out->stride[dim];
+      if (t == T_F64) {
+        const double x = ((const double *)in->data)[src];
+        facc = product ? facc * x : facc + x;
+        ((double *)out->data)[dst] = (double)facc;
+      } else {
+        const uint64_t x = (uint64_t)load_i(t, in->data, src);
+        iacc = product ? iacc * x : iacc + x;
+        store_i(t, out->data, dst, (int64_t)iacc);
+      }
+    }
+    odo_next(&oi, &il);
+    odo_next(&oo, &ol);
+  }
+  return 0;
+}
+
+/* ----------------------------------------------------------------- renorm -- */
+/* out = in with every slice along `dim` whose p-norm exceeds maxnorm scaled by
+ * maxnorm / (norm + 1e-7) (lib/THC/THCTensorMathReduce.cuh:132-178,
+ * generic/THCTensorMathReduce.cu:46-74). float, half or double views; the norm
+ * and the factor are computed in (long) double, each output rounded once. */
+int th_renorm(int t, const th_view *out, const th_view *in, double p, int dim, double maxnorm) {
+  if (in->nd < 2 || out->nd != in->nd || dim < 0 || dim >= in->nd) return 1;
+  long ssz[TH_MAX_DIMS];
+  for (int d = 0; d < in->nd; ++d) {
+    if (out->size[d] != in->size[d]) return 1;
+    ssz[d] = d == dim ? 1 : in->size[d];
+  }
+  for (long i = 0; i < in->size[dim]; ++i) {
+    th_view is = *in, os = *out;
+    is.size = ssz;
+    os.size = ssz;
+    const long ibase = i * in->stride[dim], obase = i * out->stride[dim];
+    const long n = numel(&is);
+    odo o1;
+    odo_start(&o1);
+    long double acc = 0;
+    for (long k = 0; k < n; ++k) {
+      acc += powl(fabsl((long double)load_f(t, in->data, ibase + o1.off)), (long double)p);
+      odo_next(&o1, &is);
+    }
+    const double norm = (double)powl(acc, 1.0L / (long double)p);
+    const double factor = norm > maxnorm ? maxnorm / (norm + 1e-7) : 1.0;
+    odo oi, oo;
+    odo_start(&oi);
+    odo_start(&oo);
+    for (long k = 0; k < n; ++k) {
+      store_f(t, out->data, obase + oo.off, load_f(t, in->data, ibase + oi.off) * factor);
+      odo_next(&oi, &is);
+      odo_next(&oo, &os);
+    }
+  }
+  return 0;
+}

@@ -528,3 +528,93 @@ def test_gpu_double_norm_var_std_dist(thc, oracle):
     assert abs(d.varall() - x.var(ddof=1)) <= 1e-12
     assert abs(d.stdall(1) - x.std()) <= 1e-12
     assert abs(d.dist(e, 2.0) - np.sqrt(((x - y) ** 2).sum())) <= 1e-11
+
+
+# ------------------------------------------------------------ scans and renorm --
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_oracle_typed_scan_matches_numpy(oracle, kind):
+    rng = np.random.default_rng(12)
+    dt = np_of(oracle, kind)
+    for shape, dim in (((4, 50), 1), ((30, 5), 0), ((3, 9, 4), 1)):
+        geom = random_geometry(rng, shape)
+        v = oracle.View(rand_storage(rng, kind, geom[0], oracle, small=True), *geom[1:])
+        x = v.numpy()
+        if kind == "double":
+            np.testing.assert_allclose(oracle.typed_scan_dim(v, dim).numpy(), np.cumsum(x, axis=dim), rtol=1e-14, atol=1e-14)
+            np.testing.assert_allclose(oracle.typed_scan_dim(v, dim, True).numpy(), np.cumprod(x, axis=dim), rtol=1e-13)
+        else:
+            with np.errstate(over="ignore"):
+                assert_bit_equal(oracle.typed_scan_dim(v, dim).numpy(), np.cumsum(x.astype(np.int64), axis=dim).astype(dt))
+                assert_bit_equal(oracle.typed_scan_dim(v, dim, True).numpy(),
+                                 np.cumprod(x.astype(np.int64), axis=dim).astype(dt))
+
+
+@pytest.mark.parametrize("kind", ["float", "double", "half"])
+def test_oracle_renorm_matches_numpy(oracle, kind):
+    rng = np.random.default_rng(13)
+    dt = np_of(oracle, kind)
+    x = rng.uniform(-2, 2, (6, 7, 5)).astype(dt)
+    for dim, p in ((0, 2.0), (1, 1.0), (2, 3.0)):
+        xd = x.astype(np.float64)
+        other = tuple(d for d in range(3) if d != dim)
+        norm = (np.abs(xd) ** p).sum(axis=other, keepdims=True) ** (1 / p)
+        srt = np.sort(norm.ravel())
+        maxnorm = float(srt[len(srt) // 2 - 1] + srt[len(srt) // 2]) / 2     # strictly between two norms
+        got = oracle.renorm(oracle.View.of(x), p, dim, maxnorm).numpy().astype(np.float64)
+        want = xd * np.where(norm > maxnorm, maxnorm / (norm + 1e-7), 1.0)
+        assert (norm > maxnorm).any() and (norm <= maxnorm).any()
+        np.testing.assert_allclose(got, want, rtol={"float": 1e-6, "double": 1e-14, "half": 1e-3}[kind])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", WIDE_KINDS)
+def test_gpu_typed_scans(thc, oracle, kind):
+    rng = np.random.default_rng(109)
+    for shape, dim in (((7, 1000), 1), ((300, 5), 1), ((50, 64), 0), ((4, 33, 20), 1), ((9000,), 0),
+                       ((2, 1000, 24), 1), ((3, 300, 7), 1), ((5, 2049), 1)):
+        geom = random_geometry(rng, shape) if len(shape) == 3 else contiguous_geometry(shape)
+        dev, ref = dev_ref(thc, oracle, rng, kind, geom, small=(kind != "double"))
+        got = thc.Tensor(kind).cumsum(dev, dim).numpy()
+        want = oracle.typed_scan_dim(ref, dim).numpy()
+        if kind == "double":
+            mass = np.cumsum(np.abs(ref.numpy()), axis=dim)
+            assert np.all(np.abs(got - want) <= 1e-13 * mass), (shape, dim)
+            st = rng.uniform(0.95, 1.05, geom[0])
+            dp, rp = thc.Tensor.from_storage(st, *geom[1:], kind=kind), oracle.View(st.copy(), *geom[1:])
+            np.testing.assert_allclose(thc.Tensor(kind).cumprod(dp, dim).numpy(),
+                                       oracle.typed_scan_dim(rp, dim, True).numpy(), rtol=1e-12)
+        else:
+            assert_bit_equal(got, want, "%s cumsum %s" % (kind, shape))
+            assert_bit_equal(thc.Tensor(kind).cumprod(dev, dim).numpy(), oracle.typed_scan_dim(ref, dim, True).numpy(),
+                             "%s cumprod %s" % (kind, shape))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "double", "half"])
+def test_gpu_renorm(thc, oracle, kind):
+    rng = np.random.default_rng(110)
+    dt = np_of(oracle, kind)
+    tol = {"float": 1e-5, "double": 1e-12, "half": 2e-3}[kind]
+    for shape in ((6, 70, 5), (40, 33), (3, 4, 5, 6)):
+        geom = random_geometry(rng, shape)
+        st = rng.uniform(-2, 2, geom[0]).astype(dt)
+        dev = thc.Tensor.from_storage(st, *geom[1:], kind=kind)
+        ref = oracle.View(st.copy(), *geom[1:])
+        for dim in range(len(shape)):
+            for p in (1.0, 2.0, 3.0):
+                x = ref.numpy().astype(np.float64)
+                other = tuple(d for d in range(len(shape)) if d != dim)
+                norms = np.sort((np.abs(x) ** p).sum(axis=other) ** (1 / p))
+                k = len(norms) // 2                            # about half of the slices are scaled;
+                maxnorm = float(norms[k - 1] + norms[k]) / 2   # never a tie with a slice's own norm
+                got = thc.Tensor(kind).renorm(dev, p, dim, maxnorm)
+                assert got.shape == tuple(shape)
+                want = oracle.renorm(ref, p, dim, maxnorm).numpy().astype(np.float64)
+                np.testing.assert_allclose(got.numpy().astype(np.float64), want, rtol=tol, atol=tol * 1e-3)
+    t = thc.Tensor.from_numpy(np.ones((4, 4), dt))
+    t.renorm(t, 2.0, 0, 1.0)                                  # in place
+    np.testing.assert_allclose(t.numpy().astype(np.float64), np.full((4, 4), 0.5), rtol=2e-3)
+    with pytest.raises(thc.THCError, match="at least 2 dimensions"):
+        thc.Tensor(kind).renorm(thc.Tensor.from_numpy(np.ones(4, dt)), 2.0, 0, 1.0)
+    with pytest.raises(thc.THCError, match="invalid dimension"):
+        thc.Tensor(kind).renorm(thc.Tensor.from_numpy(np.ones((4, 4), dt)), 2.0, 2, 1.0)
