@@ -85,7 +85,8 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
   const DType dt = d.dt;
   const bool floatFamilyFn =
       (d.op != PointOp::Math1 && d.op != PointOp::Math2) || d.fn <= (int)MathFn::SqDiff ||
-      d.fn == (int)MathFn::RenormFactor;
+      d.fn == (int)MathFn::RenormFactor || d.fn == (int)MathFn::LShiftValue ||
+      d.fn == (int)MathFn::RShiftValue || d.fn == (int)MathFn::CLShift || d.fn == (int)MathFn::CRShift;
   if (d.op == PointOp::Copy) {
     switch (dtype_size(dt)) {
       case 1: apply_copy<uint8_t>(s, pl, sameShape); break;

@@ -119,6 +119,8 @@ __device__ __forceinline__ float math1(int fn, float x, float v, float w) {
     case (int)MathFn::MinValue: return x < v ? x : v;
     case (int)MathFn::FmodValue: return fmodf(x, v);
     case (int)MathFn::RemainderValue: return v == 0.f ? NAN : x - v * floorf(x / v);
+    case (int)MathFn::LShiftValue: return x * powf(2.f, v);   // THCTensorMathPairwise.cu:436-462
+    case (int)MathFn::RShiftValue: return x / powf(2.f, v);
     case (int)MathFn::RenormFactor: {
       const float n = powf(x, w);
       return n > v ? v / (n + 1e-7f) : 1.0f;
@@ -137,6 +139,8 @@ __device__ __forceinline__ float math2(int fn, float a, float b) {
     case (int)MathFn::Atan2: return atan2f(a, b);
     case (int)MathFn::Equal: return a == b ? 1.f : 0.f;
     case (int)MathFn::SqDiff: return (a - b) * (a - b);
+    case (int)MathFn::CLShift: return a * powf(2.f, b);       // THCTensorMathPointwise.cuh:462-520
+    case (int)MathFn::CRShift: return a / powf(2.f, b);
     default: return a;
   }
 }

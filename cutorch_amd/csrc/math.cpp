@@ -448,6 +448,18 @@ void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
   THC_API float Tensor##_stdall(THCState* s, Tensor* self, int biased) {                           \
     THC_GUARD_RET(0.f, return sqrtf(var_all(s, DT, TN(self), biased)))                             \
   }                                                                                                \
+  THC_API void Tensor##_lshift(THCState* s, Tensor* self, Tensor* src, real v) {                   \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::LShiftValue, TN(self), TN(src), to_float(v)))         \
+  }                                                                                                \
+  THC_API void Tensor##_rshift(THCState* s, Tensor* self, Tensor* src, real v) {                   \
+    THC_GUARD_VOID(unary_math(s, DT, MathFn::RShiftValue, TN(self), TN(src), to_float(v)))         \
+  }                                                                                                \
+  THC_API void Tensor##_clshift(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {           \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CLShift, TN(self), TN(src1), TN(src2), 3))           \
+  }                                                                                                \
+  THC_API void Tensor##_crshift(THCState* s, Tensor* self, Tensor* src1, Tensor* src2) {           \
+    THC_GUARD_VOID(binary_math(s, DT, MathFn::CRShift, TN(self), TN(src1), TN(src2), 3))           \
+  }                                                                                                \
   THC_API void Tensor##_renorm(THCState* s, Tensor* self, Tensor* src, real p, long dim,           \
                                real maxnorm) {                                                     \
     THC_GUARD_VOID(renorm(s, DT, TN(self), TN(src), to_float(p), dim, to_float(maxnorm)))          \

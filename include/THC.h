@@ -289,6 +289,8 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
 /* Reductions on the reduce engine: generic/THCTensorMathReduce.h:9-36        */
 /* Scans: generic/THCTensorMathScan.h (cumsum, cumprod)                       */
 /* renorm: generic/THCTensorMathReduce.h:7                                    */
+/* lshift rshift clshift crshift (x * 2^v, x / 2^v for the floating types):   */
+/*   generic/THCTensorMathPairwise.h:9-10, generic/THCTensorMathPointwise.h:54-55 */
 /* ------------------------------------------------------------------------ */
 #define THC_AMD_DECLARE_MATH_API(Tensor, real, accreal)                        \
   THC_API void Tensor##_add(THCState *, Tensor *self, Tensor *src, real v);    \
@@ -380,6 +382,12 @@ THC_API void THCudaHalfTensor_copyCuda(THCState *, THCudaHalfTensor *self, THCud
                             int biased, int keepdim);                          \
   THC_API accreal Tensor##_varall(THCState *, Tensor *self, int biased);       \
   THC_API accreal Tensor##_stdall(THCState *, Tensor *self, int biased);       \
+  THC_API void Tensor##_lshift(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_rshift(THCState *, Tensor *self, Tensor *src, real v); \
+  THC_API void Tensor##_clshift(THCState *, Tensor *self, Tensor *src1,        \
+                                Tensor *src2);                                 \
+  THC_API void Tensor##_crshift(THCState *, Tensor *self, Tensor *src1,        \
+                                Tensor *src2);                                 \
   THC_API void Tensor##_renorm(THCState *, Tensor *self, Tensor *src,          \
                                real p, long dim, real maxnorm);                \
   THC_API accreal Tensor##_dist(THCState *, Tensor *self, Tensor *src,         \

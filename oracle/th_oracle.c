@@ -74,7 +74,8 @@ enum {
   TH_FN_NEG, TH_FN_ABS, TH_FN_SIGN, TH_FN_CLAMP, TH_FN_SQDIFFVALUE, TH_FN_POWSCALAR, TH_FN_TPOW, TH_FN_MAXVALUE,
   TH_FN_MINVALUE, TH_FN_FMODVALUE, TH_FN_REMAINDERVALUE,
   TH_FN_CPOW, TH_FN_CMAX, TH_FN_CMIN, TH_FN_CFMOD, TH_FN_CREMAINDER, TH_FN_ATAN2, TH_FN_EQUAL,
-  TH_FN_SQDIFF
+  TH_FN_SQDIFF, TH_FN_LSHIFTVALUE, TH_FN_RSHIFTVALUE, TH_FN_BITANDVALUE, TH_FN_BITORVALUE,
+  TH_FN_BITXORVALUE, TH_FN_CLSHIFT, TH_FN_CRSHIFT
 };
 
 static int g_threads = 1;
@@ -213,6 +214,9 @@ static float math1(int fn, float x, float v, float w) {
     case TH_FN_MINVALUE: return x < v ? x : v;
     case TH_FN_FMODVALUE: return fmodf(x, v);
     case TH_FN_REMAINDERVALUE: { if (v == 0.f) return NAN; float q = x / v; q = floorf(q); q = v * q; return x - q; }
+    /* shifts of floating types scale by a power of two (THCTensorMathPairwise.cu:436-462) */
+    case TH_FN_LSHIFTVALUE: { float t = powf(2.f, v); return x * t; }
+    case TH_FN_RSHIFTVALUE: { float t = powf(2.f, v); return x / t; }
   }
   return x;
 }
@@ -227,6 +231,8 @@ static float math2(int fn, float a, float b) {
     case TH_FN_ATAN2: return atan2f(a, b);
     case TH_FN_EQUAL: return a == b ? 1.f : 0.f;
     case TH_FN_SQDIFF: { float t = a - b; return t * t; }
+    case TH_FN_CLSHIFT: { float t = powf(2.f, b); return a * t; }
+    case TH_FN_CRSHIFT: { float t = powf(2.f, b); return a / t; }
   }
   return a;
 }

@@ -38,12 +38,17 @@ SCALAR = {   # name -> (numpy formula of (x, v), v, exact?)
     "cminValue": [(lambda x, v: np.where(x < F32(v), x, F32(v)), 0.25, True)],
     "fmod": [(lambda x, v: np.fmod(x, F32(v)), 0.75, True)],
     "remainder": [(lambda x, v: x - F32(v) * np.floor(x / F32(v)), 0.75, True)],
+    # shifts of floating types scale by 2^v (THCTensorMathPairwise.cu:436-462)
+    "lshift": [(lambda x, v: x * F32(2.0 ** v), 3.0, True)],
+    "rshift": [(lambda x, v: x / F32(2.0 ** v), 2.0, True)],
 }
 BINARY = {
     "cmax": (lambda a, b: np.where(a > b, a, b), True), "cmin": (lambda a, b: np.where(a < b, a, b), True),
     "cfmod": (np.fmod, True), "cremainder": (lambda a, b: a - b * np.floor(a / b), True),
     "atan2": (lambda a, b: np.arctan2(a.astype(np.float64), b.astype(np.float64)), False),
     "cpow": (lambda a, b: np.power(np.abs(a).astype(np.float64), b.astype(np.float64)), False),
+    "clshift": (lambda a, b: a.astype(np.float64) * np.power(2.0, b.astype(np.float64)), False),
+    "crshift": (lambda a, b: a.astype(np.float64) / np.power(2.0, b.astype(np.float64)), False),
 }
 
 
