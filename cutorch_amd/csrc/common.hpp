@@ -277,6 +277,11 @@ enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 // out[..., 0, ...] = reduce over dim (THC_reduceDim, lib/THC/THCReduce.cuh:263-453)
 bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTensor* out,
                 AnyTensor* in, int dim, int keepdim);
+// var / std along a unit-stride dim in one read of the input, when the rows are
+// short enough to stay in registers; false = not applicable (nothing was
+// launched, `out` may have been resized to the reduced shape).
+bool reduce_var_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
+                     bool wantStd, int keepdim);
 // (value, 1-based index) of the max/min along dim, lowest index on ties
 // (THC_reduceDimIndex, lib/THC/THCTensorMathReduce.cuh:619-661)
 void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyTensor* indices,
@@ -287,6 +292,11 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
 // Any element type; the result arrives as accreal: .f for the floating types,
 // .i for the integer types (long accumulation).
 bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Scalar* result);
+// The same reduction over a - b without materialising the difference. Only
+// for dense operands of a floating type; returns false when it does not apply
+// (the caller then subtracts into a temporary).
+bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a, AnyTensor* b,
+                     Scalar* result);
 
 // Inclusive prefix sum / product along `dim` (THCTensor_(scanDim),
 // lib/THC/generic/THCTensorMathScan.cu:76-110)

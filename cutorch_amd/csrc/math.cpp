@@ -152,8 +152,11 @@ void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* sr
   same_gpu(s, {self, src});
   THC_ARG_CHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
   const long n = src->size[dim];
+  if (reduce_var_rows(s, dt, self, src, (int)dim, biased, wantStd, keepdim)) return;
   TensorRef mean(s, tensor_new(s));
-  if (!reduce_dim(s, dt, ReduceOp::Sum, Epilogue::DivN, 0.f, mean.t, src, (int)dim, 1))
+  // the mean is the accumulator divided by n, rounded once (a half sum of a
+  // long row would overflow if it were rounded before the division)
+  if (!reduce_dim(s, dt, ReduceOp::Sum, Epilogue::DivBy, (double)n, mean.t, src, (int)dim, 1))
     raise_arg_error(2, "%s", kDimWarning);
   // Second sweep: sum of (x - mean)^2 per slice. The kernels take each slice's
   // centre from the output element itself, so the sweep runs in place on the
@@ -218,9 +221,13 @@ float dist_all(THCState* s, DType dt, AnyTensor* a, AnyTensor* b, float p) {
   same_gpu(s, {a, b});
   THC_ARG_CHECK(tensor_numel(a) == tensor_numel(b), 2, "sizes do not match");
   if (a->nDimension == 0) return 0.f;
+  // |d|^1 and |d|^2 without powf (same value up to pow's own rounding)
+  const ReduceOp op = p == 1.f ? ReduceOp::Norm1 : (p == 2.f ? ReduceOp::Norm2 : ReduceOp::NormP);
+  Scalar fused{0.0, 0};
+  if (reduce_all_diff(s, dt, op, p, a, b, &fused)) return powf((float)fused.f, 1.0f / p);
   TensorRef diff(s, tensor_new_with_size(s, a->nDimension, a->size, dt));
   apply_or_throw(s, dt, PointOp::Sub, 0.f, diff.t, a, b);
-  return powf(all_or_throw(s, dt, ReduceOp::NormP, p, diff.t), 1.0f / p);
+  return powf(all_or_throw(s, dt, op, p, diff.t), 1.0f / p);
 }
 
 void fill_tensor(THCState* s, DType dt, AnyTensor* self, float v) {
@@ -550,9 +557,12 @@ double dist_all_d(THCState* s, AnyTensor* a, AnyTensor* b, double p) {
   same_gpu(s, {a, b});
   THC_ARG_CHECK(tensor_numel(a) == tensor_numel(b), 2, "sizes do not match");
   if (a->nDimension == 0) return 0.0;
+  const ReduceOp op = p == 1.0 ? ReduceOp::Norm1 : (p == 2.0 ? ReduceOp::Norm2 : ReduceOp::NormP);
+  Scalar fused{0.0, 0};
+  if (reduce_all_diff(s, DType::F64, op, p, a, b, &fused)) return std::pow(fused.f, 1.0 / p);
   TensorRef diff(s, tensor_new_with_size(s, a->nDimension, a->size, DType::F64));
   apply_or_throw(s, DType::F64, PointOp::Sub, 0.f, diff.t, a, b);
-  return std::pow(all_scalar(s, DType::F64, ReduceOp::NormP, p, diff.t).f, 1.0 / p);
+  return std::pow(all_scalar(s, DType::F64, op, p, diff.t).f, 1.0 / p);
 }
 
 }  // namespace

@@ -100,6 +100,26 @@ bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTe
   return true;
 }
 
+bool reduce_var_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
+                     bool wantStd, int keepdim) {
+  if (!dtype_is_float(dt) || in->nDimension == 0 || in->nDimension > kMaxDims) return false;
+  if (dim < 0 || dim >= in->nDimension || in->stride[dim] != 1) return false;
+  if (out->storage && out->storage == in->storage) return false;
+  const long n = in->size[dim];
+  if (n > 64 * 8 * 8) return false;  // beyond any type's register budget: skip the resize below
+  resize_reduced(s, out, in, dim, dt);
+  ReduceGeom g = make_geom(in, out, nullptr, dim);
+  const double div = (double)(biased ? n : n - 1);
+  bool done = false;
+  const void* ip = tensor_data(in, dt);
+  void* op = tensor_data(out, dt);
+  with_type(dt, [&](auto tag) { done = reduce_var_rows_type<decltype(tag)>(s, g, ip, op, div, wantStd); });
+  if (!done) return false;
+  THC_CHECK(hipGetLastError());
+  if (!keepdim) tensor_squeeze1d(s, out, nullptr, dim, dt);
+  return true;
+}
+
 void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyTensor* indices,
                       AnyTensor* in, int dim, int keepdim) {
   THC_ARG_CHECK(dim >= 0 && dim < in->nDimension, 3, "dimension out of range");
@@ -174,7 +194,28 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Sca
   g.outElems = g.in.numel();
   g.out = g.in;
   const void* src = tensor_data(in, dt);
-  with_type(dt, [&](auto tag) { reduce_all_type<decltype(tag)>(s, g, src, op, p, result); });
+  with_type(dt, [&](auto tag) { reduce_all_type<decltype(tag)>(s, g, src, nullptr, op, p, result); });
+  return true;
+}
+
+bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a, AnyTensor* b,
+                     Scalar* result) {
+  if (!dtype_is_float(dt) || a->nDimension == 0 || a->nDimension > kMaxDims) return false;
+  if (!tensor_is_contiguous(a) || !tensor_is_contiguous(b)) return false;
+  const int64_t n = tensor_numel(a);
+  if (n != tensor_numel(b)) return false;
+  ReduceGeom g{};
+  g.wide = force_64bit_index() || n >= kIndex32Limit;
+  g.R = n;
+  g.sR = 1;
+  g.in.dims = 1;
+  g.in.size[0] = 1;
+  g.in.stride[0] = 0;
+  g.outElems = 1;
+  g.out = g.in;
+  const void* pa = tensor_data(a, dt);
+  const void* pb = tensor_data(b, dt);
+  with_type(dt, [&](auto tag) { reduce_all_type<decltype(tag)>(s, g, pa, pb, op, p, result); });
   return true;
 }
 

@@ -5,5 +5,7 @@ namespace thc {
 template void reduce_dim_type<__half>(THCState*, const ReduceGeom&, const void*, void*, ReduceOp, Epilogue,
                                   double, double);
 template void reduce_index_type<__half>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
-template void reduce_all_type<__half>(THCState*, ReduceGeom, const void*, ReduceOp, double, Scalar*);
+template bool reduce_var_rows_type<__half>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
+template void reduce_all_type<__half>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
+                                  Scalar*);
 }

@@ -437,6 +437,72 @@ __global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T
   }
 }
 
+// var / std along a unit-stride dim whose rows fit the registers of one lane
+// group (R <= 64 lanes x 8 packs): the row is read once, the mean and the sum
+// of squared deviations both come from the registers.
+template <typename T, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void var_rows_kernel(const T* __restrict__ in,
+                                                          T* __restrict__ out, OuterArgs<I> oa,
+                                                          I numRows, I R, uint32_t G,
+                                                          typename Acc<T>::type div, bool wantStd) {
+  using P = Pack<T, VEC>;
+  using A = typename Acc<T>::type;
+  constexpr int U = 8;
+  const uint32_t groups = kBlock / G;
+  const uint32_t lane = threadIdx.x % G;
+  const uint32_t grp = threadIdx.x / G;
+  for (I r0 = (I)blockIdx.x * groups; r0 < numRows; r0 += (I)gridDim.x * groups) {
+    const I row = r0 + grp;
+    const bool active = row < numRows;
+    A x[U][VEC];
+    bool valid[U];
+    I outOff = 0;
+    if (active) {
+      I inOff;
+      oa.offsets(row, inOff, outOff);
+      const T* src = in + inOff;
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const I i = ((I)lane + (I)u * G) * VEC;
+        valid[u] = i < R;
+        if (valid[u]) v[u] = load_pack<true>(reinterpret_cast<const P*>(src + i));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[u][e] = valid[u] ? acc_up<A>(v[u].v[e]) : (A)0;
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        valid[u] = false;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[u][e] = (A)0;
+      }
+    }
+    A sum = (A)0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sum += x[u][e];
+    }
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) sum += shfl_xor_any(sum, o);
+    const A mean = sum / (A)R;
+    A ss = (A)0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const A d = x[u][e] - mean;
+        if (valid[u]) ss += d * d;
+      }
+    }
+    for (uint32_t o = G >> 1; o > 0; o >>= 1) ss += shfl_xor_any(ss, o);
+    if (active && lane == 0) out[outOff] = acc_down<T>(wantStd ? sqrt_any(ss / div) : ss / div);
+  }
+}
+
 // ------------------------------------------------------------------ cols --
 template <typename I>
 struct ColsArgs {
@@ -756,6 +822,68 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
       const A fin = epi.template finish<A>(r);
       *result = fin;
       *hostResult = fin;
+    } else {
+      partial[blockIdx.x] = r;
+    }
+  }
+}
+
+// Whole-tensor reduction of the element-wise difference of two dense runs
+// (dist: sum |a - b|^p without materialising a - b). Partials are folded by
+// reduce_all_kernel.
+template <typename TIn, typename F, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_all_diff_kernel(
+    const TIn* __restrict__ a, const TIn* __restrict__ b, I n, I chunk,
+    typename F::A* __restrict__ partial, typename F::A* result, typename F::A* hostResult, F f) {
+  using P = Pack<TIn, VEC>;
+  using A = typename F::A;
+  __shared__ A red[kBlock / 64];
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+  const I nv = n - n % VEC;
+  const I begin = (I)blockIdx.x * chunk;
+  const I end = min(nv, begin + chunk);
+  constexpr int U = 4;
+  constexpr I step = (I)kBlock * VEC;
+  if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n) {
+    const A x = acc_up<A>(a[nv + threadIdx.x]) - acc_up<A>(b[nv + threadIdx.x]);
+    acc[0] = f.combine(acc[0], f.modify(x, (A)0));
+  }
+  I i = begin + threadIdx.x * VEC;
+  for (; i + (U - 1) * step < end; i += U * step) {
+    P va[U], vb[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      va[u] = load_pack<true>(reinterpret_cast<const P*>(a + i + u * step));
+      vb[u] = load_pack<true>(reinterpret_cast<const P*>(b + i + u * step));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const A x = acc_up<A>(va[u].v[e]) - acc_up<A>(vb[u].v[e]);
+        acc[e] = f.combine(acc[e], f.modify(x, (A)0));
+      }
+    }
+  }
+  for (; i < end; i += step) {
+    const P va = load_pack<true>(reinterpret_cast<const P*>(a + i));
+    const P vb = load_pack<true>(reinterpret_cast<const P*>(b + i));
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const A x = acc_up<A>(va.v[e]) - acc_up<A>(vb.v[e]);
+      acc[e] = f.combine(acc[e], f.modify(x, (A)0));
+    }
+  }
+  A r = acc[0];
+#pragma unroll
+  for (int e = 1; e < VEC; ++e) r = f.combine(r, acc[e]);
+  r = block_fold(r, red, f);
+  if (threadIdx.x == 0) {
+    if (gridDim.x == 1) {
+      *result = r;
+      *hostResult = r;
     } else {
       partial[blockIdx.x] = r;
     }
@@ -1099,6 +1227,41 @@ void reduce_index_type(THCState* s, const ReduceGeom& g, bool isMax, const void*
 }
 
 
+// var / std over rows that fit one lane group's registers. Returns false when
+// the geometry does not qualify (the caller then runs the two-sweep form).
+template <typename T>
+bool reduce_var_rows_type(THCState* s, const ReduceGeom& g, const void* in_, void* out_, double div,
+                          bool wantStd) {
+  using A = typename Acc<T>::type;
+  if constexpr (std::is_integral<A>::value) {
+    return false;
+  } else {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int U = 8;
+    const T* in = (const T*)in_;
+    T* out = (T*)out_;
+    if (g.sR != 1 || !aligned16(in) || g.R % VEC != 0 || g.R > 64 * VEC * U) return false;
+    for (int d = 0; d < g.in.dims; ++d)
+      if (g.in.stride[d] % VEC != 0 && g.in.size[d] != 1) return false;
+    uint32_t G = pow2_ceil((uint64_t)((g.R + VEC * U - 1) / (VEC * U)));
+    G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+    const int64_t groups = kBlock / G;
+    const int grid = capped_grid(s, (g.outElems + groups - 1) / groups, "reduce.rows.blocks_per_cu", 64);
+    hipStream_t st = current_stream(s);
+    if (g.wide) {
+      OuterArgs<uint64_t> oa = make_outer<uint64_t>(g.in, g.out, g.in.dims);
+      hipLaunchKernelGGL((var_rows_kernel<T, uint64_t, VEC>), dim3(grid), dim3(kBlock), 0, st, in, out,
+                         oa, (uint64_t)g.outElems, (uint64_t)g.R, G, (A)div, wantStd);
+    } else {
+      OuterArgs<uint32_t> oa = make_outer<uint32_t>(g.in, g.out, g.in.dims);
+      hipLaunchKernelGGL((var_rows_kernel<T, uint32_t, VEC>), dim3(grid), dim3(kBlock), 0, st, in, out,
+                         oa, (uint32_t)g.outElems, (uint32_t)g.R, G, (A)div, wantStd);
+    }
+    note_kernel("var-rows");
+    return true;
+  }
+}
+
 // ------------------------------------------------------------------- all --
 template <typename A>
 constexpr DType acc_dtype() {
@@ -1108,8 +1271,8 @@ constexpr DType acc_dtype() {
 
 namespace {
 template <typename T, typename F>
-void reduce_all_with(THCState* s, ReduceGeom g, const void* src, F f1, bool sumSecond,
-                     Scalar* result) {
+void reduce_all_with(THCState* s, ReduceGeom g, const void* src, const void* src2, F f1,
+                     bool sumSecond, Scalar* result) {
   using A = typename F::A;
   const int64_t rows = g.outElems;
   const StreamScratch& sc = stream_scratch(s);
@@ -1163,6 +1326,21 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, F f1, bool sumS
     blocks = (g.R + chunk - 1) / chunk;
     hipStream_t st = current_stream(s);
     A* part = (A*)sc.partials;
+    if (src2 != nullptr) {  // sum over f(a - b): one row, both operands dense
+      if (aligned16(src) && aligned16(src2))
+        hipLaunchKernelGGL((reduce_all_diff_kernel<TI, F2, I, V>), dim3((int)blocks), dim3(kBlock),
+                           0, st, (const TI*)src, (const TI*)src2, (I)g.R, (I)chunk, part, devOut,
+                           hostDev, f);
+      else
+        hipLaunchKernelGGL((reduce_all_diff_kernel<TI, F2, I, 1>), dim3((int)blocks), dim3(kBlock),
+                           0, st, (const TI*)src, (const TI*)src2, (I)g.R, (I)chunk, part, devOut,
+                           hostDev, f);
+      if (blocks > 1)
+        hipLaunchKernelGGL((reduce_all_kernel<A, FSum<A>, I, 1, false>), dim3(1), dim3(kBlock), 0,
+                           st, (const A*)part, (I)blocks, (I)blocks, part, devOut, hostDev, none,
+                           FSum<A>{(A)0});
+      return;
+    }
     if (aligned16(src))
       hipLaunchKernelGGL((reduce_all_kernel<TI, F2, I, V, true>), dim3((int)blocks), dim3(kBlock), 0,
                          st, (const TI*)src, (I)g.R, (I)chunk, part, devOut, hostDev, none, f);
@@ -1198,30 +1376,30 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, F f1, bool sumS
 }  // namespace
 
 template <typename T>
-void reduce_all_type(THCState* s, ReduceGeom g, const void* src, ReduceOp op, double p_,
-                     Scalar* result) {
+void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src2, ReduceOp op,
+                     double p_, Scalar* result) {
   using A = typename Acc<T>::type;
   const A p = (A)p_;
   switch (op) {
-    case ReduceOp::Sum: reduce_all_with<T>(s, g, src, FSum<A>{p}, false, result); return;
-    case ReduceOp::Prod: reduce_all_with<T>(s, g, src, FProd<A>{p}, false, result); return;
-    case ReduceOp::Min: reduce_all_with<T>(s, g, src, FMin<A>{p}, false, result); return;
-    case ReduceOp::Max: reduce_all_with<T>(s, g, src, FMax<A>{p}, false, result); return;
+    case ReduceOp::Sum: reduce_all_with<T>(s, g, src, src2, FSum<A>{p}, false, result); return;
+    case ReduceOp::Prod: reduce_all_with<T>(s, g, src, src2, FProd<A>{p}, false, result); return;
+    case ReduceOp::Min: reduce_all_with<T>(s, g, src, src2, FMin<A>{p}, false, result); return;
+    case ReduceOp::Max: reduce_all_with<T>(s, g, src, src2, FMax<A>{p}, false, result); return;
     default: break;
   }
   if constexpr (!std::is_integral<A>::value) {
     switch (op) {
-      case ReduceOp::Norm0: reduce_all_with<T>(s, g, src, FNorm0<A>{p}, true, result); return;
-      case ReduceOp::Norm1: reduce_all_with<T>(s, g, src, FNorm1<A>{p}, true, result); return;
-      case ReduceOp::Norm2: reduce_all_with<T>(s, g, src, FNorm2<A>{p}, true, result); return;
-      case ReduceOp::NormP: reduce_all_with<T>(s, g, src, FNormP<A>{p}, true, result); return;
-      case ReduceOp::SqDev: reduce_all_with<T>(s, g, src, FSqDev<A>{p}, true, result); return;
+      case ReduceOp::Norm0: reduce_all_with<T>(s, g, src, src2, FNorm0<A>{p}, true, result); return;
+      case ReduceOp::Norm1: reduce_all_with<T>(s, g, src, src2, FNorm1<A>{p}, true, result); return;
+      case ReduceOp::Norm2: reduce_all_with<T>(s, g, src, src2, FNorm2<A>{p}, true, result); return;
+      case ReduceOp::NormP: reduce_all_with<T>(s, g, src, src2, FNormP<A>{p}, true, result); return;
+      case ReduceOp::SqDev: reduce_all_with<T>(s, g, src, src2, FSqDev<A>{p}, true, result); return;
       default: break;
     }
   }
   if constexpr (std::is_same<T, uint8_t>::value) {
-    if (op == ReduceOp::All) { reduce_all_with<T>(s, g, src, FAll<A>{p}, false, result); return; }
-    if (op == ReduceOp::Any) { reduce_all_with<T>(s, g, src, FAny<A>{p}, false, result); return; }
+    if (op == ReduceOp::All) { reduce_all_with<T>(s, g, src, src2, FAll<A>{p}, false, result); return; }
+    if (op == ReduceOp::Any) { reduce_all_with<T>(s, g, src, src2, FAny<A>{p}, false, result); return; }
   }
   raise_error("reduction not available for this element type");
 }

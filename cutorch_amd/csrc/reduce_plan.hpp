@@ -22,11 +22,16 @@ void reduce_dim_type(THCState* s, const ReduceGeom& g, const void* in, void* out
 template <typename T>
 void reduce_index_type(THCState* s, const ReduceGeom& g, bool isMax, const void* in, void* outV,
                        long* outI);
+// var / std of rows short enough to stay in registers (one read of the input).
+template <typename T>
+bool reduce_var_rows_type(THCState* s, const ReduceGeom& g, const void* in, void* out, double div,
+                          bool wantStd);
 // Whole-tensor reduction of a tensor whose innermost collapsed dim has unit
 // stride (`g.R` long, `g.in` = the remaining dims = rows). Blocks until the
-// scalar is on the host.
+// scalar is on the host. With `src2` (then the tensor is one dense row) the
+// reduction runs over src - src2.
 template <typename T>
-void reduce_all_type(THCState* s, ReduceGeom g, const void* src, ReduceOp op, double p,
-                     Scalar* result);
+void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src2, ReduceOp op,
+                     double p, Scalar* result);
 
 }  // namespace thc

@@ -74,3 +74,28 @@ def test_gpu_varall_stdall_dist(thc, oracle):
     e = thc.Tensor("float")
     with pytest.raises(thc.THCError, match="empty Tensor"):
         e.varall()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_gpu_var_rows_single_read_and_fallback(thc, oracle, kind):
+    """Rows that fit a lane group's registers take the one-read kernel; longer
+    rows, ragged lengths and offsets that break 16-byte alignment take the
+    two-sweep form. Both must agree with the oracle."""
+    rng = np.random.default_rng(8)
+    tol = 1e-5 if kind == "float" else 2e-3
+    dtype = np.float32 if kind == "float" else np.float16
+    vec = 4 if kind == "float" else 8
+    for shape, expect in (((300, 1024), "var-rows"), ((7, 64 * vec * 8), "var-rows"), ((5, 8), "var-rows"),
+                          ((3, 64 * vec * 8 + vec), "rows"), ((50, 1023), "rows-scalar"), ((2, 40000), None)):
+        x = (rng.standard_normal(shape) * 2 + 3).astype(dtype)
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        for name, okind in (("var", "var"), ("std", "std")):
+            for biased in (0, 1):
+                out = getattr(thc.Tensor(kind), name)(dev, 1, biased=biased)
+                if expect:
+                    assert thc.last_kernel() == expect, (shape, thc.last_kernel())
+                want = oracle.reduce_dim(okind + ("_biased" if biased else ""), ref, 1).numpy().astype(np.float64)
+                np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol, atol=tol * 1e-2)
+    out = thc.Tensor(kind).var(thc.Tensor.from_numpy(np.ones((4, 16), dtype)), 1, keepdim=0)
+    assert out.shape == (4,) and np.all(out.numpy() == 0)
