@@ -181,7 +181,9 @@ def build_configs(thc, hip, which, only=None):
 
     # Neighbours of the hot path on the same engines (same operands where possible).
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
-                      "N-cumsum-cols", "N-dist", "N-varall") if (only and n in only) or (not only and which == "all")]
+                      "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
+                      "N-double-sum", "N-renorm")
+          if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
         e_src = T.from_numpy(rng.uniform(-1, 1, ne).astype(np.float32))
@@ -207,6 +209,24 @@ def build_configs(thc, hip, which, only=None):
             "N-dist": ("dist(a, b, 2) over 2^26 fp32", 8 * ne, ne, lambda i: e_src.dist(e_dst, 2.0)),
             "N-varall": ("varall over 2^26 fp32 (input counted once)", 4 * ne, ne, lambda i: e_src.varall()),
         }
+        if set(nx) & {"N-int-add", "N-lt-byte", "N-cvt-half", "N-double-sum", "N-renorm"}:
+            ia = T.from_numpy(rng.integers(-1000, 1000, ne).astype(np.int32))
+            ib = T.from_numpy(rng.integers(-1000, 1000, ne).astype(np.int32))
+            ic = T("int").resize((ne,))
+            mask = T("byte").resize((ne,))
+            hdst = T("half").resize((ne,))
+            dsrc = T.from_numpy(rng.uniform(-1, 1, (8192, 4096)))
+            dout = T("double").resize((8192, 1))
+            table.update({
+                "N-int-add": ("c = a + b, 2^26 int32 contiguous", 12 * ne, ne, lambda i: ic.cadd(ia, 1, ib)),
+                "N-lt-byte": ("mask = x < 0 into a Byte tensor, 2^26 fp32", 5 * ne, ne,
+                              lambda i: mask.compare_value("lt", e_src, 0.0)),
+                "N-cvt-half": ("half <- float converting copy, 2^26", 6 * ne, ne, lambda i: hdst.copy_from(e_src)),
+                "N-double-sum": ("sum over last dim of 8192x4096 fp64", 8 * 8192 * 4096 + 8 * 8192, 8192 * 4096,
+                                 lambda i: dout.sum(dsrc, 1)),
+                "N-renorm": ("renorm(p=2, dim 0, maxnorm 1) of 8192x8192 fp32 (read + write counted once)",
+                             8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.renorm(sq, 2.0, 0, 1.0)),
+            })
         if "N-fill" in nx and xa.numel() != big:
             table["N-fill"] = ("fill of 2^26 fp32", 4 * ne, ne, lambda i: e_dst.fill(0.5))
         for n in nx:
