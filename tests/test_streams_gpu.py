@@ -1,0 +1,75 @@
+"""The engine launches on the caller's current stream (thread-local, as
+THCState_getCurrentStream / setStream in lib/THC/THCGeneral.c:516-546) and
+keeps its scratch per stream (THCGeneral.c:677-712)."""
+import ctypes as C
+import threading
+
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def streams(thc):
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    made = []
+    for _ in range(2):
+        s = C.c_void_p()
+        assert hip.hipStreamCreate(C.byref(s)) == 0          # default priority
+        made.append(s)
+    yield hip, made
+    thc.lib().THCState_setCurrentStream(thc.state(), None)
+    thc.synchronize()
+    for s in made:
+        hip.hipStreamDestroy(s)
+
+
+def test_ops_follow_the_current_stream(thc, oracle, streams):
+    hip, (s1, s2) = streams
+    lib, st = thc.lib(), thc.state()
+    rng = np.random.default_rng(61)
+    a = rng.standard_normal((512, 384)).astype(np.float32)
+    b = rng.standard_normal((384, 512)).astype(np.float32)
+    big = rng.integers(-8, 9, (3, 1 << 18)).astype(np.float32)      # split reduction: uses the stream's scratch
+    da, db, dbig = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b), thc.Tensor.from_numpy(big)
+    thc.synchronize()
+    want_mul = a * b.T
+    want_sum = big.astype(np.int64).sum(axis=1, keepdims=True).astype(np.float32)
+    for stream in (s1, s2, None, s1):
+        lib.THCState_setCurrentStream(st, stream)
+        assert lib.THCState_getCurrentStream(st) == (stream.value if stream else None)
+        out = thc.Tensor("float").cmul(da, db.t())
+        sums = thc.Tensor("float").sum(dbig, 1)
+        assert thc.last_kernel() == "rows-split"
+        total = dbig.sumall()                                        # waits on the current stream itself
+        assert total == float(big.astype(np.int64).sum())
+        if stream:
+            assert hip.hipStreamSynchronize(stream) == 0
+        else:
+            thc.synchronize()
+        assert_bit_equal(out.numpy(), want_mul)
+        assert_bit_equal(sums.numpy(), want_sum)
+
+
+def test_current_stream_is_per_thread(thc, streams):
+    hip, (s1, _) = streams
+    lib, st = thc.lib(), thc.state()
+    lib.THCState_setCurrentStream(st, s1)
+    seen = {}
+
+    def worker():
+        seen["stream"] = lib.THCState_getCurrentStream(st)           # a fresh thread starts on the default stream
+        x = thc.Tensor.from_numpy(np.arange(1000, dtype=np.float32))
+        seen["sum"] = x.sumall()
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert seen["stream"] is None and seen["sum"] == 499500.0
+    assert lib.THCState_getCurrentStream(st) == s1.value
