@@ -96,7 +96,64 @@ for f in [1.0, 65504.0, 65520.0, 65519.0, 5.9604645e-08, 2.9802322e-08, 2.980232
     half.append({"f32_bits": int(np.float32(f).view(np.uint32)),
                  "f16_bits": int(np.float32(f).astype(np.float16).view(np.uint16))})
 
-out = {"pointwise": pointwise, "argmax": argmax, "sum": sums, "half": half}
+# Hand-checked known answers for the integer types, double, comparisons, conversions and scans
+# (C semantics on the element type: wrap-around, truncating division, fmod = sign of the dividend,
+# remainder = sign of the divisor; conversions truncate toward zero).
+typed = [
+    {"kind": "byte", "op": "add", "a": [250, 1, 255], "b": [10, 2, 1], "expect": [4, 3, 0]},
+    {"kind": "byte", "op": "sub", "a": [3, 0], "b": [5, 1], "expect": [254, 255]},
+    {"kind": "byte", "op": "mul", "a": [16, 200], "b": [16, 2], "expect": [0, 144]},
+    {"kind": "char", "op": "add", "a": [127, -128], "b": [1, -1], "expect": [-128, 127]},
+    {"kind": "short", "op": "mul", "a": [300, -300], "b": [300, 300], "expect": [24464, -24464]},
+    {"kind": "int", "op": "div", "a": [7, -7, 7, -7], "b": [2, 2, -2, -2], "expect": [3, -3, -3, 3]},
+    {"kind": "int", "op": "fn:cfmod", "a": [7, -7, 7, -7], "b": [3, 3, -3, -3], "expect": [1, -1, 1, -1]},
+    {"kind": "int", "op": "fn:cremainder", "a": [7, -7, 7, -7], "b": [3, 3, -3, -3], "expect": [1, 2, -2, -1]},
+    {"kind": "int", "op": "add", "a": [2147483647], "b": [1], "expect": [-2147483648]},
+    {"kind": "long", "op": "mul", "a": [4294967296, 3037000500], "b": [4294967296, 3037000500],
+     "expect": [0, -9223372036709301616]},
+    {"kind": "long", "op": "fn:cpow", "a": [3, -2, 2], "b": [4, 3, 62], "expect": [81, -8, 4611686018427387904]},
+    {"kind": "short", "op": "fn:cbitand", "a": [0x0ff0, -1], "b": [0x00ff, 0x1234], "expect": [0x00f0, 0x1234]},
+    {"kind": "byte", "op": "fn:clshift", "a": [1, 0x81], "b": [7, 1], "expect": [128, 2]},
+    {"kind": "char", "op": "fn:crshift", "a": [-128, 64], "b": [2, 3], "expect": [-32, 8]},
+    {"kind": "double", "op": "add", "a": [0.1, 1e308], "b": [0.2, 1e308], "expect": [0.30000000000000004, float("inf")]},
+    {"kind": "double", "op": "div", "a": [1.0, -1.0], "b": [3.0, 0.0], "expect": [0.3333333333333333, float("-inf")]},
+]
+compare = [
+    {"kind": "float", "cmp": "lt", "a": [1.0, 2.0, float("nan"), -0.0], "b": [2.0, 2.0, 1.0, 0.0], "expect": [1, 0, 0, 0]},
+    {"kind": "float", "cmp": "ne", "a": [1.0, float("nan"), -0.0], "b": [1.0, float("nan"), 0.0], "expect": [0, 1, 0]},
+    {"kind": "byte", "cmp": "gt", "a": [200, 5], "b": [100, 5], "expect": [1, 0]},       # unsigned: 200 > 100
+    {"kind": "char", "cmp": "gt", "a": [-56, 5], "b": [100, 5], "expect": [0, 0]},       # signed: -56 < 100
+    {"kind": "long", "cmp": "ge", "a": [9007199254740993, -1], "b": [9007199254740992, 0], "expect": [1, 0]},
+    {"kind": "half", "cmp": "eq", "a": [1.0, 0.5], "b": [1.0, 0.25], "expect": [1, 0]},
+]
+convert = [
+    {"src": "float", "dst": "int", "x": [2.9, -2.9, 0.5, -0.5, 1e9], "expect": [2, -2, 0, 0, 1000000000]},
+    {"src": "double", "dst": "byte", "x": [0.99, 255.0, 128.5], "expect": [0, 255, 128]},
+    {"src": "int", "dst": "byte", "x": [256, 257, -1, 511], "expect": [0, 1, 255, 255]},
+    {"src": "long", "dst": "int", "x": [4294967297, -4294967295], "expect": [1, 1]},
+    {"src": "char", "dst": "byte", "x": [-1, -128, 127], "expect": [255, 128, 127]},
+    {"src": "byte", "dst": "char", "x": [255, 128, 127], "expect": [-1, -128, 127]},
+    {"src": "int", "dst": "float", "x": [16777217, -16777219], "expect": [16777216.0, -16777220.0]},
+    {"src": "long", "dst": "double", "x": [9007199254740993], "expect": [9007199254740992.0]},
+    {"src": "float", "dst": "half", "x": [65519.0, 65520.0, 1.0009766], "expect": [65504.0, float("inf"), 1.0009765625]},
+    {"src": "double", "dst": "float", "x": [0.1, 1e40], "expect": [0.10000000149011612, float("inf")]},
+    {"src": "half", "dst": "long", "x": [2.5, -3.5, 2048.0], "expect": [2, -3, 2048]},
+]
+typed_reduce = [
+    {"kind": "byte", "op": "sum", "shape": [2, 3], "dim": 1, "x": [100, 100, 100, 255, 1, 0], "expect": [44, 0]},
+    {"kind": "byte", "op": "sumall", "shape": [2, 3], "x": [100, 100, 100, 255, 1, 0], "expect": 556},
+    {"kind": "char", "op": "prod", "shape": [1, 3], "dim": 1, "x": [16, 16, 2], "expect": [0]},
+    {"kind": "int", "op": "mean", "shape": [1, 4], "dim": 1, "x": [-1, -2, -3, -1], "expect": [-1]},   # -7 / 4 truncates
+    {"kind": "long", "op": "max", "shape": [1, 4], "dim": 1, "x": [-5, 7, 7, 1], "expect": [7], "index": [2]},
+    {"kind": "short", "op": "min", "shape": [3, 1], "dim": 0, "x": [4, -9, -9], "expect": [-9], "index": [2]},
+    {"kind": "int", "op": "cumsum", "shape": [1, 4], "dim": 1, "x": [2147483647, 1, 1, -3],
+     "expect": [2147483647, -2147483648, -2147483647, 2147483646]},
+    {"kind": "byte", "op": "cumprod", "shape": [1, 4], "dim": 1, "x": [3, 5, 20, 2], "expect": [3, 15, 44, 88]},
+    {"kind": "double", "op": "sum", "shape": [1, 3], "dim": 1, "x": [1e16, 1.0, -1e16], "expect": [1.0]},  # needs > 53 bits
+]
+
+out = {"pointwise": pointwise, "argmax": argmax, "sum": sums, "half": half, "typed": typed, "compare": compare,
+       "convert": convert, "typed_reduce": typed_reduce}
 path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fixtures.json")
 with open(path, "w") as f:
     json.dump(out, f)
