@@ -359,7 +359,10 @@ def main():
     traffic = None   # HBM bytes per launch from the committed rocprofv3 --pmc summary, if any
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            traffic = json.load(f).get(cfgs[0].name, {}).get("traffic_bytes")
+            measured = json.load(f)
+        traffic = measured.get(cfgs[0].name, {}).get("traffic_bytes")
+        for r in results:
+            r["traffic_bytes"] = measured.get(r["name"], {}).get("traffic_bytes")
     except (OSError, ValueError):
         pass
     line = {
