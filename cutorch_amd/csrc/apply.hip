@@ -68,6 +68,32 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     return true;
   }
 
+  // Ops that stay off the LDS-tiled kernels (the six wider element types and
+  // the comparisons) would read a transposed input with one useful element per
+  // sector. Such an input is first brought into the output's memory order by
+  // the same-type copy, which does own a tiled kernel for every element size:
+  // two extra coalesced passes instead of one uncoalesced one.
+  TensorRef dense[kMaxOps] = {{s, nullptr}, {s, nullptr}, {s, nullptr}, {s, nullptr}};
+  const bool offTiled = d.op != PointOp::Copy &&
+                        (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor ||
+                         !(d.dt == DType::F32 || d.dt == DType::F16));
+  if (offTiled && n >= 4096 && tensor_is_contiguous(out)) {
+    for (int k = 1; k < nops; ++k) {
+      const AnyTensor* in = t[k];
+      if (in == out || in->nDimension != out->nDimension || in->nDimension < 2) continue;
+      bool same = true, unitElsewhere = false;
+      for (int dd = 0; dd < in->nDimension; ++dd) {
+        same = same && in->size[dd] == out->size[dd];
+        if (dd < in->nDimension - 1 && in->stride[dd] == 1 && in->size[dd] >= 8) unitElsewhere = true;
+      }
+      const int last = in->nDimension - 1;
+      if (same && unitElsewhere && in->size[last] >= 8 && in->stride[last] != 1) {
+        dense[k].t = tensor_new_contiguous(s, t[k], d.dt);
+        t[k] = dense[k].t;
+      }
+    }
+  }
+
   Plan pl{};
   pl.nops = nops;
   pl.numel = n;

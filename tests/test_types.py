@@ -618,3 +618,29 @@ def test_gpu_renorm(thc, oracle, kind):
         thc.Tensor(kind).renorm(thc.Tensor.from_numpy(np.ones(4, dt)), 2.0, 0, 1.0)
     with pytest.raises(thc.THCError, match="invalid dimension"):
         thc.Tensor(kind).renorm(thc.Tensor.from_numpy(np.ones((4, 4), dt)), 2.0, 2, 1.0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["int", "byte", "double"])
+def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
+    """The wider types have no LDS-tiled arithmetic kernels: a transposed input
+    is brought into the output's order by the (tiled) same-type copy first."""
+    rng = np.random.default_rng(111)
+    dt = np_of(oracle, kind)
+    a = rand_storage(rng, kind, 200 * 136, oracle).reshape(200, 136)
+    b = rand_storage(rng, kind, 200 * 136, oracle).reshape(136, 200)
+    da, db = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
+    out = thc.Tensor(kind).cadd(da.t(), 1, db)
+    assert thc.last_kernel() == "contig"
+    ra = oracle.View(a.reshape(-1).copy(), 0, (136, 200), (1, 136))
+    want = oracle.typed_pointwise("add", oracle.View.empty((136, 200), dt), ra, oracle.View.of(b))
+    assert_bit_equal(out.numpy(), want.numpy())
+    m = thc.Tensor("byte").compare_tensor("lt", da.t(), db)
+    assert thc.last_kernel() == "contig"
+    wm = oracle.typed_compare("lt", oracle.View.empty((136, 200), np.uint8), ra, oracle.View.of(b))
+    assert_bit_equal(m.numpy(), wm.numpy())
+    f = thc.Tensor.from_numpy(rng.standard_normal((200, 136)).astype(np.float32))
+    g = thc.Tensor.from_numpy(rng.standard_normal((136, 200)).astype(np.float32))
+    m = thc.Tensor("byte").compare_tensor("ge", f.t(), g)
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(m.numpy(), (f.numpy().T >= g.numpy()).astype(np.uint8))
