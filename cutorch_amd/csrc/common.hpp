@@ -277,10 +277,11 @@ enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 // out[..., 0, ...] = reduce over dim (THC_reduceDim, lib/THC/THCReduce.cuh:263-453)
 bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTensor* out,
                 AnyTensor* in, int dim, int keepdim);
-// var / std along a unit-stride dim in one read of the input, when the rows are
-// short enough to stay in registers; false = not applicable (nothing was
-// launched, `out` may have been resized to the reduced shape).
-bool reduce_var_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
+// var / std in one read of the input: rows along a unit-stride dim that are
+// short enough to stay in registers, or a strided dim next to a unit-stride
+// one (Welford). false = not applicable (nothing was launched, `out` may have
+// been resized to the reduced shape).
+bool reduce_var_fast(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
                      bool wantStd, int keepdim);
 // (value, 1-based index) of the max/min along dim, lowest index on ties
 // (THC_reduceDimIndex, lib/THC/THCTensorMathReduce.cuh:619-661)

@@ -144,15 +144,16 @@ float norm_all(THCState* s, DType dt, float p, AnyTensor* self) {
   return powf(all_or_throw(s, dt, ReduceOp::NormP, p, self), 1.0f / p);
 }
 
-// var / std along a dim (generic/THCTensorMathReduce.cu:70-120), two sweeps
-// for accuracy in fp32: m = mean over dim; self = sum((src - m)^2) /
-// (n - !biased) [sqrt for std].
+// var / std along a dim (generic/THCTensorMathReduce.cu:70-120). The common
+// geometries take a one-read kernel (register-resident rows, or Welford along a
+// strided dim); anything else runs two sweeps: m = mean over dim; self =
+// sum((src - m)^2) / (n - !biased) [sqrt for std].
 void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* src, long dim,
              int biased, int keepdim) {
   same_gpu(s, {self, src});
   THC_ARG_CHECK(dim >= 0 && dim < src->nDimension, 3, "dimension out of range");
   const long n = src->size[dim];
-  if (reduce_var_rows(s, dt, self, src, (int)dim, biased, wantStd, keepdim)) return;
+  if (reduce_var_fast(s, dt, self, src, (int)dim, biased, wantStd, keepdim)) return;
   TensorRef mean(s, tensor_new(s));
   // the mean is the accumulator divided by n, rounded once (a half sum of a
   // long row would overflow if it were rounded before the division)

@@ -100,20 +100,23 @@ bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTe
   return true;
 }
 
-bool reduce_var_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
+bool reduce_var_fast(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int dim, int biased,
                      bool wantStd, int keepdim) {
   if (!dtype_is_float(dt) || in->nDimension == 0 || in->nDimension > kMaxDims) return false;
-  if (dim < 0 || dim >= in->nDimension || in->stride[dim] != 1) return false;
+  if (dim < 0 || dim >= in->nDimension) return false;
   if (out->storage && out->storage == in->storage) return false;
   const long n = in->size[dim];
-  if (n > 64 * 8 * 8) return false;  // beyond any type's register budget: skip the resize below
   resize_reduced(s, out, in, dim, dt);
   ReduceGeom g = make_geom(in, out, nullptr, dim);
   const double div = (double)(biased ? n : n - 1);
   bool done = false;
   const void* ip = tensor_data(in, dt);
   void* op = tensor_data(out, dt);
-  with_type(dt, [&](auto tag) { done = reduce_var_rows_type<decltype(tag)>(s, g, ip, op, div, wantStd); });
+  with_type(dt, [&](auto tag) {
+    using T = decltype(tag);
+    done = reduce_var_rows_type<T>(s, g, ip, op, div, wantStd) ||
+           reduce_var_cols_type<T>(s, g, ip, op, div, wantStd);
+  });
   if (!done) return false;
   THC_CHECK(hipGetLastError());
   if (!keepdim) tensor_squeeze1d(s, out, nullptr, dim, dt);

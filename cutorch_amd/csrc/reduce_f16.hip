@@ -6,6 +6,7 @@ template void reduce_dim_type<__half>(THCState*, const ReduceGeom&, const void*,
                                   double, double);
 template void reduce_index_type<__half>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
 template bool reduce_var_rows_type<__half>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
+template bool reduce_var_cols_type<__half>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
 template void reduce_all_type<__half>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
                                   Scalar*);
 }

@@ -631,6 +631,145 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const TIn* __restri
   }
 }
 
+// var / std along a strided dim in ONE read of the input: every thread keeps a
+// running (count, mean, M2) per column (Welford), thread rows and, for split
+// reductions, workgroup partials are merged with the pairwise update of Chan,
+// Golub & LeVeque. Same geometry as reduce_cols_kernel. Partial planes hold
+// (mean, M2) per output: partial[(s * 2 + {0, 1}) * outElems + out].
+template <typename A>
+__device__ __forceinline__ void moments_merge(A& na, A& ma, A& sa, A nb, A mb, A sb) {
+  const A n = na + nb;
+  if (n > (A)0) {
+    const A delta = mb - ma;
+    const A w = nb / n;
+    ma += delta * w;
+    sa += sb + delta * delta * na * w;
+  }
+  na = n;
+}
+
+template <typename T, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void var_cols_kernel(const T* __restrict__ in,
+                                                          T* __restrict__ out,
+                                                          typename Acc<T>::type* __restrict__ partial,
+                                                          ColsArgs<I> a, I totalBlocks,
+                                                          typename Acc<T>::type div, bool wantStd,
+                                                          bool foldPass) {
+  using P = Pack<T, VEC>;
+  using A = typename Acc<T>::type;
+  __shared__ A smean[kBlock * VEC];
+  __shared__ A sm2[kBlock * VEC];
+  __shared__ A scnt[kBlock];
+  const uint32_t TX = a.TX, TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  for (I b = blockIdx.x; b < totalBlocks; b += gridDim.x) {
+    I group = b, s = 0, rest, ct;
+    if (!foldPass) a.S.divmod(b, group, s);
+    a.colTiles.divmod(group, rest, ct);
+    I inOff, outOff;
+    a.oa.offsets(rest, inOff, outOff);
+    const I col = (ct * TX + tx) * VEC;
+    A cnt = (A)0, mean[VEC], m2[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      mean[e] = (A)0;
+      m2[e] = (A)0;
+    }
+    if (foldPass) {
+      if (col < a.C) {
+        const A* plane = partial + rest * a.C + col;
+        for (I sp = ty; sp < a.S.d; sp += TY) {
+          const I begin = sp * a.chunkR;
+          const A nb = (A)(min(a.R, begin + a.chunkR) - begin);
+          A n = cnt;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            n = cnt;
+            moments_merge(n, mean[e], m2[e], nb, plane[(sp * 2) * a.outElems + e],
+                          plane[(sp * 2 + 1) * a.outElems + e]);
+          }
+          cnt = n;
+        }
+      }
+    } else if (col < a.C) {
+      const I begin = s * a.chunkR;
+      const I end = min(a.R, begin + a.chunkR);
+      const T* src = in + inOff + col;
+      constexpr int U = 8;
+      I r = begin + ty;
+      for (; r + (U - 1) * TY < end; r += U * TY) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (r + u * TY) * a.sR));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          cnt += (A)1;
+          const A inv = (A)1 / cnt;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            const A delta = x - mean[e];
+            mean[e] += delta * inv;
+            m2[e] += delta * (x - mean[e]);
+          }
+        }
+      }
+      for (; r < end; r += TY) {
+        const P v = load_pack<true>(reinterpret_cast<const P*>(src + r * a.sR));
+        cnt += (A)1;
+        const A inv = (A)1 / cnt;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const A x = acc_up<A>(v.v[e]);
+          const A delta = x - mean[e];
+          mean[e] += delta * inv;
+          m2[e] += delta * (x - mean[e]);
+        }
+      }
+    }
+    // fold the TY thread rows in a fixed tree
+    scnt[ty * TX + tx] = cnt;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      smean[(ty * TX + tx) * VEC + e] = mean[e];
+      sm2[(ty * TX + tx) * VEC + e] = m2[e];
+    }
+    __syncthreads();
+    for (uint32_t h = TY >> 1; h > 0; h >>= 1) {
+      if (ty < h) {
+        const uint32_t i = ty * TX + tx, j = i + h * TX;
+        const A na = scnt[i], nb = scnt[j];
+        A n = na;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          n = na;
+          moments_merge(n, smean[i * VEC + e], sm2[i * VEC + e], nb, smean[j * VEC + e], sm2[j * VEC + e]);
+        }
+        scnt[i] = n;
+      }
+      __syncthreads();
+    }
+    if (ty == 0 && col < a.C) {
+      if (foldPass || a.S.d == 1) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          const A v = sm2[tx * VEC + e] / div;
+          out[outOff + (col + e) * a.outInner] = acc_down<T>(wantStd ? sqrt_any(v) : v);
+        }
+      } else {
+        A* plane = partial + rest * a.C + col;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          plane[(s * 2) * a.outElems + e] = smean[tx * VEC + e];
+          plane[(s * 2 + 1) * a.outElems + e] = sm2[tx * VEC + e];
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
 template <typename T, typename I, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
     const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
@@ -1258,6 +1397,45 @@ bool reduce_var_rows_type(THCState* s, const ReduceGeom& g, const void* in_, voi
                          oa, (uint32_t)g.outElems, (uint32_t)g.R, G, (A)div, wantStd);
     }
     note_kernel("var-rows");
+    return true;
+  }
+}
+
+// var / std along a strided dim next to a unit-stride one, in one read
+// (Welford + pairwise merges). Returns false when the geometry is not the
+// column shape.
+template <typename T>
+bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in_, void* out_, double div,
+                          bool wantStd) {
+  using A = typename Acc<T>::type;
+  if constexpr (std::is_integral<A>::value) {
+    return false;
+  } else {
+    constexpr int VEC = 16 / sizeof(T);
+    const int nd = g.in.dims;
+    if (g.sR == 1 || nd < 1 || g.in.stride[nd - 1] != 1 || g.in.size[nd - 1] <= 1) return false;
+    auto go = [&](auto idxTag) {
+      using I = decltype(idxTag);
+      ColsPlan<I> p = plan_cols<T, I>(s, g, in_, 2 * sizeof(A));
+      const bool split = p.a.S.d > 1;
+      A* scratch = split ? (A*)scratch_space(s, nullptr) : nullptr;
+      const int grid = (int)std::min<int64_t>(p.totalBlocks, 1 << 30);
+      const int64_t groups = p.totalBlocks / (int64_t)p.a.S.d;
+      hipStream_t st = current_stream(s);
+      for (int pass = 0; pass < (split ? 2 : 1); ++pass) {
+        const bool fold = pass == 1;
+        const int gr = fold ? (int)groups : grid;
+        const I tb = fold ? (I)groups : (I)p.totalBlocks;
+        if (p.vec)
+          hipLaunchKernelGGL((var_cols_kernel<T, I, VEC>), dim3(gr), dim3(kBlock), 0, st, (const T*)in_,
+                             (T*)out_, scratch, p.a, tb, (A)div, wantStd, fold);
+        else
+          hipLaunchKernelGGL((var_cols_kernel<T, I, 1>), dim3(gr), dim3(kBlock), 0, st, (const T*)in_,
+                             (T*)out_, scratch, p.a, tb, (A)div, wantStd, fold);
+      }
+      note_kernel(split ? "var-cols-split" : "var-cols");
+    };
+    if (g.wide) go(uint64_t{}); else go(uint32_t{});
     return true;
   }
 }

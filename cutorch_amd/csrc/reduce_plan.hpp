@@ -26,6 +26,10 @@ void reduce_index_type(THCState* s, const ReduceGeom& g, bool isMax, const void*
 template <typename T>
 bool reduce_var_rows_type(THCState* s, const ReduceGeom& g, const void* in, void* out, double div,
                           bool wantStd);
+// var / std along a strided dim whose neighbour has unit stride (one read).
+template <typename T>
+bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in, void* out, double div,
+                          bool wantStd);
 // Whole-tensor reduction of a tensor whose innermost collapsed dim has unit
 // stride (`g.R` long, `g.in` = the remaining dims = rows). Blocks until the
 // scalar is on the host. With `src2` (then the tensor is one dense row) the

@@ -6,6 +6,7 @@ template void reduce_dim_type<double>(THCState*, const ReduceGeom&, const void*,
                                   double, double);
 template void reduce_index_type<double>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
 template bool reduce_var_rows_type<double>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
+template bool reduce_var_cols_type<double>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
 template void reduce_all_type<double>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
                                   Scalar*);
 }

@@ -6,6 +6,7 @@ template void reduce_dim_type<int16_t>(THCState*, const ReduceGeom&, const void*
                                   double, double);
 template void reduce_index_type<int16_t>(THCState*, const ReduceGeom&, bool, const void*, void*, long*);
 template bool reduce_var_rows_type<int16_t>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
+template bool reduce_var_cols_type<int16_t>(THCState*, const ReduceGeom&, const void*, void*, double, bool);
 template void reduce_all_type<int16_t>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
                                   Scalar*);
 }

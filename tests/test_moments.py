@@ -99,3 +99,26 @@ def test_gpu_var_rows_single_read_and_fallback(thc, oracle, kind):
                 np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol, atol=tol * 1e-2)
     out = thc.Tensor(kind).var(thc.Tensor.from_numpy(np.ones((4, 16), dtype)), 1, keepdim=0)
     assert out.shape == (4,) and np.all(out.numpy() == 0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
+    """Welford along a strided dim: the large common offset (mean 1000 x the
+    spread for float) must not cost accuracy, split and unsplit shapes."""
+    rng = np.random.default_rng(9)
+    tol = 1e-5 if kind == "float" else 2e-3
+    dtype = np.float32 if kind == "float" else np.float16
+    offset = 100.0 if kind == "float" else 4.0
+    for shape, dim, expect in (((64, 512), 0, "var-cols"), ((6, 300, 40), 1, "var-cols"),
+                               ((2, 8192, 96), 1, "var-cols-split"), ((129, 7), 0, "var-cols-scalar"),
+                               ((3, 50, 8, 24), 1, "var-cols")):
+        x = (rng.standard_normal(shape) * 0.1 + offset).astype(dtype)
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        for name in ("var", "std"):
+            for biased in (0, 1):
+                out = getattr(thc.Tensor(kind), name)(dev, dim, biased=biased)
+                assert thc.last_kernel().startswith(expect.replace("-scalar", "")), (shape, thc.last_kernel())
+                want = oracle.reduce_dim(name + ("_biased" if biased else ""), ref, dim).numpy().astype(np.float64)
+                np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol * (8 if kind == "float" else 1),
+                                           atol=0, err_msg="%s %s %s" % (shape, name, kind))
