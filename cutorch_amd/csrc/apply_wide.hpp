@@ -218,82 +218,154 @@ __device__ __forceinline__ C imath2(int fn, C a, C b) {
   }
 }
 
+// out = op(a, b, c) in the compute type; with constant `op` / `fn` the switches fold away.
+template <typename T>
+__device__ __forceinline__ typename Num<T>::C wide_arith(int op, int fn, typename Num<T>::C v,
+                                                          typename Num<T>::C w, typename Num<T>::C a,
+                                                          typename Num<T>::C b, typename Num<T>::C c) {
+  using C = typename Num<T>::C;
+  if constexpr (Num<T>::kFloat) {
+    switch (op) {
+      case (int)PointOp::Fill: return v;
+      case (int)PointOp::AddC: return a + v;
+      case (int)PointOp::SubC: return a - v;
+      case (int)PointOp::MulC: return a * v;
+      case (int)PointOp::DivC: return a / v;
+      case (int)PointOp::Add: return a + b;
+      case (int)PointOp::Sub: return a - b;
+      case (int)PointOp::Mul: return a * b;
+      case (int)PointOp::Div: return a / b;
+      case (int)PointOp::CAdd: return a + v * b;
+      case (int)PointOp::Lerp: return a + v * (b - a);
+      case (int)PointOp::AddCMul: return a + v * (b * c);
+      case (int)PointOp::AddCDiv: return a + v * (b / c);
+      case (int)PointOp::Math1: return (C)dmath1(fn, a, v, w);
+      case (int)PointOp::Math2: return (C)dmath2(fn, a, b);
+      default: return a;
+    }
+  } else {
+    switch (op) {
+      case (int)PointOp::Fill: return v;
+      case (int)PointOp::AddC: return wrap_add(a, v);
+      case (int)PointOp::SubC: return wrap_sub(a, v);
+      case (int)PointOp::MulC: return wrap_mul(a, v);
+      case (int)PointOp::DivC: return int_div(a, v);
+      case (int)PointOp::Add: return wrap_add(a, b);
+      case (int)PointOp::Sub: return wrap_sub(a, b);
+      case (int)PointOp::Mul: return wrap_mul(a, b);
+      case (int)PointOp::Div: return int_div(a, b);
+      case (int)PointOp::CAdd: return wrap_add(a, wrap_mul(v, b));
+      case (int)PointOp::AddCMul: return wrap_add(a, wrap_mul(v, wrap_mul(b, c)));
+      case (int)PointOp::AddCDiv: return wrap_add(a, wrap_mul(v, int_div(b, c)));
+      case (int)PointOp::Math1: return imath1<T, C>(fn, a, v, w);
+      case (int)PointOp::Math2: return imath2<T, C>(fn, a, b);
+      default: return a;
+    }
+  }
+}
+
+constexpr int kNumPointOp = (int)PointOp::CmpTensor + 1;
+constexpr int wide_op_inputs(int op) {
+  return op == (int)PointOp::Fill ? 0
+       : (op == (int)PointOp::AddC || op == (int)PointOp::SubC || op == (int)PointOp::MulC ||
+          op == (int)PointOp::DivC || op == (int)PointOp::Math1) ? 1
+       : (op == (int)PointOp::Add || op == (int)PointOp::Sub || op == (int)PointOp::Mul ||
+          op == (int)PointOp::Div || op == (int)PointOp::CAdd || op == (int)PointOp::Lerp ||
+          op == (int)PointOp::Math2) ? 2
+       : (op == (int)PointOp::AddCMul || op == (int)PointOp::AddCDiv) ? 3 : -1;
+}
+
+template <typename T, int NIN_, int OP, int FN>
+struct WideFixed {
+  static constexpr int NIN = NIN_;
+  using C = typename Num<T>::C;
+  C v, w;
+  __device__ __forceinline__ T operator()(T a, T b, T c) const {
+    return Num<T>::down(wide_arith<T>(OP, FN, v, w, Num<T>::up(a), Num<T>::up(b), Num<T>::up(c)));
+  }
+};
+
 // One functor per arity; `op` is a PointOp, `fn` a MathFn.
 template <typename T, int NIN_>
 struct WideOp {
   static constexpr int NIN = NIN_;
+  using Dispatched = void;
   using C = typename Num<T>::C;
   int op, fn;
   C v, w;
-
-  __device__ __forceinline__ C arith(C a, C b, C c) const {
-    if constexpr (Num<T>::kFloat) {
-      switch (op) {
-        case (int)PointOp::Fill: return v;
-        case (int)PointOp::AddC: return a + v;
-        case (int)PointOp::SubC: return a - v;
-        case (int)PointOp::MulC: return a * v;
-        case (int)PointOp::DivC: return a / v;
-        case (int)PointOp::Add: return a + b;
-        case (int)PointOp::Sub: return a - b;
-        case (int)PointOp::Mul: return a * b;
-        case (int)PointOp::Div: return a / b;
-        case (int)PointOp::CAdd: return a + v * b;
-        case (int)PointOp::Lerp: return a + v * (b - a);
-        case (int)PointOp::AddCMul: return a + v * (b * c);
-        case (int)PointOp::AddCDiv: return a + v * (b / c);
-        case (int)PointOp::Math1: return (C)dmath1(fn, a, v, w);
-        case (int)PointOp::Math2: return (C)dmath2(fn, a, b);
-        default: return a;
-      }
-    } else {
-      switch (op) {
-        case (int)PointOp::Fill: return v;
-        case (int)PointOp::AddC: return wrap_add(a, v);
-        case (int)PointOp::SubC: return wrap_sub(a, v);
-        case (int)PointOp::MulC: return wrap_mul(a, v);
-        case (int)PointOp::DivC: return int_div(a, v);
-        case (int)PointOp::Add: return wrap_add(a, b);
-        case (int)PointOp::Sub: return wrap_sub(a, b);
-        case (int)PointOp::Mul: return wrap_mul(a, b);
-        case (int)PointOp::Div: return int_div(a, b);
-        case (int)PointOp::CAdd: return wrap_add(a, wrap_mul(v, b));
-        case (int)PointOp::AddCMul: return wrap_add(a, wrap_mul(v, wrap_mul(b, c)));
-        case (int)PointOp::AddCDiv: return wrap_add(a, wrap_mul(v, int_div(b, c)));
-        case (int)PointOp::Math1: return imath1<T, C>(fn, a, v, w);
-        case (int)PointOp::Math2: return imath2<T, C>(fn, a, b);
-        default: return a;
-      }
-    }
-  }
   __device__ __forceinline__ T operator()(T a, T b, T c) const {
-    return Num<T>::down(arith(Num<T>::up(a), Num<T>::up(b), Num<T>::up(c)));
+    return Num<T>::down(wide_arith<T>(op, fn, v, w, Num<T>::up(a), Num<T>::up(b), Num<T>::up(c)));
+  }
+  template <typename Body>
+  __device__ __forceinline__ void dispatch(Body&& body) const {
+    const C v_ = v, w_ = w;
+    const int fn_ = fn;
+    for_code<0, kNumPointOp>(op, [&](auto oc) {
+      constexpr int OP = decltype(oc)::value;
+      if constexpr (wide_op_inputs(OP) == NIN_) {
+        if constexpr (OP == (int)PointOp::Math1) {
+          for_code<0, (int)MathFn::CPow>(fn_, [&](auto fc) {
+            body(WideFixed<T, NIN_, OP, decltype(fc)::value>{v_, w_});
+          });
+          for_code<(int)MathFn::LShiftValue, (int)MathFn::CLShift>(fn_, [&](auto fc) {
+            body(WideFixed<T, NIN_, OP, decltype(fc)::value>{v_, w_});
+          });
+          if (fn_ == (int)MathFn::RenormFactor) body(WideFixed<T, NIN_, OP, (int)MathFn::RenormFactor>{v_, w_});
+        } else if constexpr (OP == (int)PointOp::Math2) {
+          for_code<(int)MathFn::CPow, (int)MathFn::LShiftValue>(fn_, [&](auto fc) {
+            body(WideFixed<T, NIN_, OP, decltype(fc)::value>{v_, w_});
+          });
+          for_code<(int)MathFn::CLShift, (int)MathFn::RenormFactor>(fn_, [&](auto fc) {
+            body(WideFixed<T, NIN_, OP, decltype(fc)::value>{v_, w_});
+          });
+        } else {
+          body(WideFixed<T, NIN_, OP, 0>{v_, w_});
+        }
+      }
+    });
   }
 };
 
 // Comparisons: result 0/1 in TOut (a Byte tensor or the input's own type).
 template <typename T, typename TOut, int NIN_>
+__device__ __forceinline__ TOut compare_values(int fn, typename Num<T>::C a, typename Num<T>::C b) {
+  bool r;
+  switch (fn) {
+    case (int)CmpFn::LT: r = a < b; break;
+    case (int)CmpFn::GT: r = a > b; break;
+    case (int)CmpFn::LE: r = a <= b; break;
+    case (int)CmpFn::GE: r = a >= b; break;
+    case (int)CmpFn::EQ: r = a == b; break;
+    default: r = a != b; break;
+  }
+  if constexpr (std::is_same<TOut, __half>::value)
+    return __float2half_rn(r ? 1.f : 0.f);
+  else
+    return (TOut)(r ? 1 : 0);
+}
+template <typename T, typename TOut, int NIN_, int FN>
+struct CmpFixed {
+  static constexpr int NIN = NIN_;
+  using C = typename Num<T>::C;
+  C v;
+  __device__ __forceinline__ TOut operator()(T a_, T b_, T) const {
+    return compare_values<T, TOut, NIN_>(FN, Num<T>::up(a_), NIN_ == 1 ? v : Num<T>::up(b_));
+  }
+};
+template <typename T, typename TOut, int NIN_>
 struct CmpOp {
   static constexpr int NIN = NIN_;
+  using Dispatched = void;
   using C = typename Num<T>::C;
   int fn;
   C v;
   __device__ __forceinline__ TOut operator()(T a_, T b_, T) const {
-    const C a = Num<T>::up(a_);
-    const C b = NIN_ == 1 ? v : Num<T>::up(b_);
-    bool r;
-    switch (fn) {
-      case (int)CmpFn::LT: r = a < b; break;
-      case (int)CmpFn::GT: r = a > b; break;
-      case (int)CmpFn::LE: r = a <= b; break;
-      case (int)CmpFn::GE: r = a >= b; break;
-      case (int)CmpFn::EQ: r = a == b; break;
-      default: r = a != b; break;
-    }
-    if constexpr (std::is_same<TOut, __half>::value)
-      return __float2half_rn(r ? 1.f : 0.f);
-    else
-      return (TOut)(r ? 1 : 0);
+    return compare_values<T, TOut, NIN_>(fn, Num<T>::up(a_), NIN_ == 1 ? v : Num<T>::up(b_));
+  }
+  template <typename Body>
+  __device__ __forceinline__ void dispatch(Body&& body) const {
+    const C v_ = v;
+    for_code<0, 6>(fn, [&](auto fc) { body(CmpFixed<T, TOut, NIN_, decltype(fc)::value>{v_}); });
   }
 };
 
