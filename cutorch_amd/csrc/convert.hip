@@ -30,20 +30,33 @@ __device__ __forceinline__ D convert_value(S x) {
   }
 }
 
-// N consecutive elements per lane as one load and one store.
-template <typename D, typename S, int N>
+// N consecutive elements per lane as one load and one store; N is chosen so
+// that the wider of the two packs is 16 bytes. U packs per lane are loaded
+// (streaming hint) before the first is converted.
+template <typename D, typename S, int N, int U>
 __global__ __launch_bounds__(kBlock) void convert_kernel(D* __restrict__ dst,
                                                          const S* __restrict__ src, uint64_t n) {
   using PS = Pack<S, N>;
   using PD = Pack<D, N>;
   const uint64_t packs = n / N;
-  const uint64_t step = (uint64_t)gridDim.x * kBlock;
-  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < packs; i += step) {
-    const PS v = reinterpret_cast<const PS*>(src)[i];
-    PD r;
+  const uint64_t step = (uint64_t)gridDim.x * (kBlock * U);
+  for (uint64_t base = (uint64_t)blockIdx.x * (kBlock * U) + threadIdx.x; base < packs; base += step) {
+    PS v[U];
 #pragma unroll
-    for (int e = 0; e < N; ++e) r.v[e] = convert_value<D, S>(v.v[e]);
-    reinterpret_cast<PD*>(dst)[i] = r;
+    for (int u = 0; u < U; ++u) {
+      const uint64_t i = base + (uint64_t)u * kBlock;
+      if (i < packs) v[u] = load_pack<true>(reinterpret_cast<const PS*>(src) + i);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint64_t i = base + (uint64_t)u * kBlock;
+      if (i < packs) {
+        PD r;
+#pragma unroll
+        for (int e = 0; e < N; ++e) r.v[e] = convert_value<D, S>(v[u].v[e]);
+        reinterpret_cast<PD*>(dst)[i] = r;
+      }
+    }
   }
   const uint64_t tail = packs * N + (uint64_t)blockIdx.x * kBlock + threadIdx.x;
   if (N > 1 && tail < n) dst[tail] = convert_value<D, S>(src[tail]);
@@ -51,17 +64,18 @@ __global__ __launch_bounds__(kBlock) void convert_kernel(D* __restrict__ dst,
 
 template <typename D, typename S>
 void launch_convert(THCState* s, void* dst, const void* src, int64_t n) {
-  constexpr int N = 8;
+  constexpr int N = 16 / (sizeof(S) > sizeof(D) ? sizeof(S) : sizeof(D));
+  constexpr int U = 4;
   const bool vec = (reinterpret_cast<uintptr_t>(dst) % (N * sizeof(D)) == 0) &&
                    (reinterpret_cast<uintptr_t>(src) % (N * sizeof(S)) == 0);
-  const int64_t items = vec ? n / N + 1 : n;
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((items + kBlock - 1) / kBlock, 1 << 20));
+  const int64_t items = vec ? (n / N + U - 1) / U + 1 : n;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((items + kBlock - 1) / kBlock, 1 << 22));
   hipStream_t st = current_stream(s);
   if (vec)
-    hipLaunchKernelGGL((convert_kernel<D, S, N>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
+    hipLaunchKernelGGL((convert_kernel<D, S, N, U>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
                        (const S*)src, (uint64_t)n);
   else
-    hipLaunchKernelGGL((convert_kernel<D, S, 1>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
+    hipLaunchKernelGGL((convert_kernel<D, S, 1, 1>), dim3(grid), dim3(kBlock), 0, st, (D*)dst,
                        (const S*)src, (uint64_t)n);
 }
 
