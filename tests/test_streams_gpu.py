@@ -73,3 +73,51 @@ def test_current_stream_is_per_thread(thc, streams):
     t.join()
     assert seen["stream"] is None and seen["sum"] == 499500.0
     assert lib.THCState_getCurrentStream(st) == s1.value
+
+
+def test_concurrent_host_threads_on_their_own_streams(thc, streams):
+    """Four host threads, each on its own stream (two created here, two more
+    below), run pointwise ops, split reductions, *all reductions and temporaries
+    (caching allocator) at the same time; every result must be exact."""
+    hip, (s1, s2) = streams
+    lib, st = thc.lib(), thc.state()
+    extra = []
+    for _ in range(2):
+        s = C.c_void_p()
+        assert hip.hipStreamCreate(C.byref(s)) == 0
+        extra.append(s)
+    errors = []
+
+    def worker(idx, stream):
+        try:
+            lib.THCState_setCurrentStream(st, stream)
+            rng = np.random.default_rng(700 + idx)
+            for it in range(25):
+                a = rng.integers(-8, 9, (64, 333)).astype(np.float32)
+                b = rng.integers(-8, 9, (333, 64)).astype(np.float32)
+                big = rng.integers(-4, 5, (2, 1 << 17)).astype(np.float32)
+                da, db, dbig = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b), thc.Tensor.from_numpy(big)
+                out = thc.Tensor("float").addcmul(da, 2.0, da, db.t())       # tiled kernel
+                sums = thc.Tensor("float").sum(dbig, 1)                        # split reduction (stream scratch)
+                mx, ix = thc.Tensor("float"), thc.Tensor("long")
+                mx.max(ix, out, 1)
+                total = dbig.sumall()                                          # blocks on this stream only
+                cont = db.t().contiguous()                                     # temporary through the allocator
+                want = a + 2.0 * (a * b.T)
+                assert np.array_equal(out.numpy(), want), (idx, it, "addcmul")
+                assert np.array_equal(sums.numpy().ravel(), big.astype(np.int64).sum(axis=1).astype(np.float32))
+                assert total == float(big.astype(np.int64).sum()), (idx, it, "sumall")
+                assert np.array_equal(ix.numpy().ravel(), want.argmax(axis=1) + 1), (idx, it, "argmax")
+                assert np.array_equal(cont.numpy(), b.T)
+        except Exception as e:                                                  # noqa: BLE001
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=worker, args=(i, s)) for i, s in enumerate([s1, s2] + extra)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    thc.synchronize()
+    for s in extra:
+        hip.hipStreamDestroy(s)
+    assert not errors, errors

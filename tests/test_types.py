@@ -644,3 +644,38 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
     m = thc.Tensor("byte").compare_tensor("ge", f.t(), g)
     assert thc.last_kernel() == "contig"
     assert_bit_equal(m.numpy(), (f.numpy().T >= g.numpy()).astype(np.uint8))
+
+
+@pytest.mark.gpu
+def test_gpu_error_paths_of_the_wider_types(thc):
+    a = thc.Tensor.from_numpy(np.arange(6, dtype=np.int32).reshape(2, 3))
+    b = thc.Tensor.from_numpy(np.arange(8, dtype=np.int32).reshape(2, 4))
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("int").cadd(a, 1, b)
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("int").binary("cmax", a, b)
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("int").addcmul(a, 1, a, b)
+    with pytest.raises(thc.THCError, match="divide by zero"):
+        thc.Tensor("int").div(a, 0)
+    with pytest.raises(thc.THCError, match="dimension out of range"):
+        thc.Tensor("int").sum(a, 2)
+    with pytest.raises(thc.THCError, match="out of range"):
+        thc.Tensor("int").cumsum(a, -1)
+    with pytest.raises(thc.THCError, match="sizes do not match"):
+        thc.Tensor("long").resize((5,)).copy_from(a)
+    with pytest.raises(thc.THCError, match="empty Tensor"):
+        thc.Tensor("double").meanall()
+    e = thc.Tensor("short")
+    assert e.sumall() == 0 and e.prodall() == 1 and e.maxall() == -32768 and e.minall() == 32767
+    assert thc.Tensor("byte").logicalall() == 1 and thc.Tensor("byte").logicalany() == 0
+    out = thc.Tensor("int").cadd(thc.Tensor("int"), 1, thc.Tensor("int"))       # empty operands: no-op
+    assert out.shape == ()
+    # in place on a view with holes: untouched storage stays untouched
+    st = np.arange(40, dtype=np.int16)
+    t = thc.Tensor.from_storage(st, 2, (3, 4), (12, 2), kind="short")
+    t.mul(t, 3)
+    want = st.copy()
+    v = np.lib.stride_tricks.as_strided(want[2:], (3, 4), (24, 4))
+    v *= 3
+    assert_bit_equal(t.storage_numpy(), want)
