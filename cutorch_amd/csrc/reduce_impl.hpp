@@ -1143,7 +1143,8 @@ struct ColsPlan {
 
 // cols: reduced dim strided, innermost joint dim has unit input stride.
 template <typename T, typename I>
-ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t partialElemBytes) {
+ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t partialElemBytes,
+                      const char* perCuKey = "reduce.cols.blocks_per_cu", int perCuDefault = 1) {
   constexpr int VEC = 16 / sizeof(T);
   ColsPlan<I> p{};
   const int nd = g.in.dims;
@@ -1151,7 +1152,7 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   bool vec = aligned16(in) && C % VEC == 0 && g.sR % VEC == 0;
   for (int d = 0; d < nd - 1 && vec; ++d) vec = g.in.stride[d] % VEC == 0;
   const int pack = vec ? VEC : 1;
-  const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning("reduce.cols.blocks_per_cu", 1));
+  const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning(perCuKey, perCuDefault));
   const int64_t outer = g.outElems / C;
   // Lanes along the unit-stride dim: a full wave if the dim is long enough, but
   // narrower column tiles (down to 256-byte rows) are preferred over splitting
@@ -1164,9 +1165,28 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   const int64_t colTiles = tiles_for(TX);
   const int64_t base = outer * colTiles;
   const int64_t minRows = (int64_t)TY * tuning("reduce.cols.min_rows_per_thread", 8);
+  // Split the reduced dim over S workgroups when the output alone gives too few
+  // blocks, or a block count that is neither a multiple of the CU count nor
+  // large: then some CUs carry twice the work of others (320 blocks on 256 CUs
+  // ran at 4.5 TB/s, cut into 4-8x as many at 5.4-5.7). S is searched for the
+  // least imbalance, with a small bias towards fewer, longer chunks.
   int64_t S = 1;
-  if (base < target && g.R >= 2 * minRows) {
-    S = std::min<int64_t>((target + base - 1) / base, g.R / minRows);
+  const int64_t cus = num_compute_units(s);
+  const int64_t maxS = g.R / minRows;
+  if ((base < target || (base % cus != 0 && base < 8 * cus)) && maxS >= 2) {
+    const int64_t minS = std::min<int64_t>(maxS, std::max<int64_t>(1, (target + base - 1) / base));
+    const int64_t hiS = std::min<int64_t>(maxS, std::max<int64_t>(minS * 8, 8));
+    double best = 1e30;
+    for (int64_t c = minS; c <= hiS; ++c) {
+      const int64_t blocks = base * c;
+      const double imbalance = (double)((blocks + cus - 1) / cus * cus) / (double)blocks;
+      const double cost = imbalance + 0.01 * (double)c / (double)minS;
+      if (cost < best) {
+        best = cost;
+        S = c;
+      }
+    }
+    S = std::min<int64_t>(S, maxS);
     size_t scratchBytes = 0;
     scratch_space(s, &scratchBytes);
     S = std::min<int64_t>(S, (int64_t)(scratchBytes / partialElemBytes) / std::max<int64_t>(g.outElems, 1));
@@ -1295,7 +1315,9 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
     return;
   }
   {
-    ColsPlan<I> p = plan_cols<T, I>(s, g, in, 16);
+    // the (value, index) kernel does several ALU steps per element: two workgroups
+    // per CU hide them (6.5 TB/s against 4.4 with one), the plain reductions want one
+    ColsPlan<I> p = plan_cols<T, I>(s, g, in, 16, "reduce.cols.index_blocks_per_cu", 2);
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
     const I idxInner = (I)g.idx.stride[nd - 1];
     const bool split = p.a.S.d > 1;
