@@ -6,6 +6,7 @@
 // (lib/THC/THCTensorCopy.cu:24-122).
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include "apply_plan.hpp"
 #include "common.hpp"
 #include "device_util.hpp"
@@ -68,27 +69,46 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     return true;
   }
 
-  // Ops that stay off the LDS-tiled kernels (the six wider element types and
-  // the comparisons) would read a transposed input with one useful element per
-  // sector. Such an input is first brought into the output's memory order by
+  // Ops that stay off the LDS-tiled kernels (the six wider element types, the
+  // comparisons, the two-input math family and the one-input family on half)
+  // would read a transposed input with one useful element per sector. Such an input is first brought into the output's memory order by
   // the same-type copy, which does own a tiled kernel for every element size:
   // two extra coalesced passes instead of one uncoalesced one.
   TensorRef dense[kMaxOps] = {{s, nullptr}, {s, nullptr}, {s, nullptr}, {s, nullptr}};
   const bool offTiled = d.op != PointOp::Copy &&
                         (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor ||
+                         d.op == PointOp::Math2 || (d.op == PointOp::Math1 && d.dt == DType::F16) ||
                          !(d.dt == DType::F32 || d.dt == DType::F16));
-  if (offTiled && n >= 4096 && tensor_is_contiguous(out)) {
+  // The output's fastest-running dim (smallest stride among dims longer than 1).
+  int po = -1;
+  for (int dd = out->nDimension - 1; dd >= 0; --dd)
+    if (out->size[dd] > 1 && (po < 0 || out->stride[dd] < out->stride[po])) po = dd;
+  if (offTiled && n >= 4096 && po >= 0 && out->stride[po] == 1 && out->size[po] >= 8) {
     for (int k = 1; k < nops; ++k) {
       const AnyTensor* in = t[k];
       if (in == out || in->nDimension != out->nDimension || in->nDimension < 2) continue;
       bool same = true, unitElsewhere = false;
       for (int dd = 0; dd < in->nDimension; ++dd) {
         same = same && in->size[dd] == out->size[dd];
-        if (dd < in->nDimension - 1 && in->stride[dd] == 1 && in->size[dd] >= 8) unitElsewhere = true;
+        if (dd != po && in->stride[dd] == 1 && in->size[dd] >= 8) unitElsewhere = true;
       }
-      const int last = in->nDimension - 1;
-      if (same && unitElsewhere && in->size[last] >= 8 && in->stride[last] != 1) {
-        dense[k].t = tensor_new_contiguous(s, t[k], d.dt);
+      if (same && unitElsewhere && in->stride[po] != 1) {
+        // a dense tensor whose dims nest in the order of the output's strides
+        const int nd = out->nDimension;
+        int order[kMaxDims];
+        for (int dd = 0; dd < nd; ++dd) order[dd] = nd - 1 - dd;
+        std::stable_sort(order, order + nd, [&](int a, int b) {
+          const long sa = out->size[a] > 1 ? out->stride[a] : 0, sb = out->size[b] > 1 ? out->stride[b] : 0;
+          return sa < sb;
+        });
+        long stride[kMaxDims], run = 1;
+        for (int j = 0; j < nd; ++j) {
+          stride[order[j]] = run;
+          run *= out->size[order[j]];
+        }
+        dense[k].t = tensor_new(s);
+        tensor_resize_nd(s, dense[k].t, nd, out->size, stride, d.dt);
+        copy_tensor(s, d.dt, dense[k].t, t[k], /*ignoreOverlap=*/true);
         t[k] = dense[k].t;
       }
     }

@@ -830,12 +830,19 @@ void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
 template <typename T, int GROUP>
 void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
                           float w) {
+  // The code-dispatched families keep the switch inside the LDS-tiled kernels'
+  // unrolled passes (hoisting it there spills far more). That costs little for
+  // the one-input family on float (5.2-5.7 TB/s on a transposed 8192^2 input)
+  // but the half variant (8 elements a pack) ran at 1.5 TB/s and the two-input
+  // family spilled 400 bytes a lane: those stay off the tiled kernels, and the
+  // front end brings a transposed input into the output's order first.
   if (op == PointOp::Math1) {
-    if constexpr (GROUP == 0) run_plan<T>(s, pl, sameShape, OpMath1{v, w, (int)fn});
+    if constexpr (GROUP == 0)
+      run_plan<T, OpMath1, T, std::is_same<T, float>::value>(s, pl, sameShape, OpMath1{v, w, (int)fn});
     return;
   }
   if (op == PointOp::Math2) {
-    if constexpr (GROUP == 1) run_plan<T>(s, pl, sameShape, OpMath2{(int)fn});
+    if constexpr (GROUP == 1) run_plan<T, OpMath2, T, false>(s, pl, sameShape, OpMath2{(int)fn});
     return;
   }
   switch (op) {

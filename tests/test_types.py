@@ -647,6 +647,52 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
 
 
 @pytest.mark.gpu
+def test_gpu_transposed_output_and_math_family_are_densified(thc, oracle):
+    """The same route when it is the output that is transposed (its memory
+    order decides), for a wider type and for the code-dispatched float math,
+    which owns no tiled kernels either; 3-D permutations included."""
+    rng = np.random.default_rng(112)
+    a = rng.integers(-1000, 1000, (136, 200)).astype(np.int32)
+    b = rng.integers(-1000, 1000, (136, 200)).astype(np.int32)
+    da, db = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
+    base = thc.Tensor.from_numpy(np.zeros((200, 136), np.int32))
+    base.t().cadd(da, 3, db)
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(base.numpy(), (a + 3 * b).T)
+
+    x = rng.standard_normal((136, 200)).astype(np.float32)
+    y = rng.standard_normal((200, 136)).astype(np.float32)
+    dx, dy = thc.Tensor.from_numpy(x), thc.Tensor.from_numpy(y)
+    fbase = thc.Tensor.from_numpy(np.zeros((200, 136), np.float32))
+    fbase.t().unary("exp", dx)          # one-input float math owns tiled kernels
+    assert thc.last_kernel().startswith("tiled")
+    want = oracle.pointwise("fn:exp", oracle.View.empty((136, 200)), oracle.View.of(x))
+    np.testing.assert_allclose(fbase.numpy().T, want.numpy(), rtol=2e-6)
+    out = thc.Tensor("float").binary("cmax", dx, dy.t())
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(out.numpy(), np.maximum(x, y.T))
+    fbase.t().binary("cmin", dx, dy.t())   # y is already in the output's order
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(fbase.numpy().T, np.minimum(x, y.T))
+    hx = x.astype(np.float16)
+    hbase = thc.Tensor.from_numpy(np.zeros((200, 136), np.float16))
+    hbase.t().unary("abs", thc.Tensor.from_numpy(hx))
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(hbase.numpy().T, np.abs(hx))
+    out = thc.Tensor("half").unary("neg", thc.Tensor.from_numpy(hx).t())
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(out.numpy(), -hx.T)
+
+    z = rng.standard_normal((24, 40, 56)).astype(np.float32)
+    dz = thc.Tensor.from_numpy(z)
+    out = thc.Tensor("float").unary("neg", dz.t(0, 2))
+    assert_bit_equal(out.numpy(), -z.transpose(2, 1, 0))
+    zbase = thc.Tensor.from_numpy(np.zeros((56, 40, 24), np.float32))
+    zbase.t(0, 2).unary("neg", dz)
+    assert_bit_equal(zbase.numpy(), -z.transpose(2, 1, 0))
+
+
+@pytest.mark.gpu
 def test_gpu_error_paths_of_the_wider_types(thc):
     a = thc.Tensor.from_numpy(np.arange(6, dtype=np.int32).reshape(2, 3))
     b = thc.Tensor.from_numpy(np.arange(8, dtype=np.int32).reshape(2, 4))
