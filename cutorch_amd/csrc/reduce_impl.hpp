@@ -1144,7 +1144,8 @@ struct ColsPlan {
 // cols: reduced dim strided, innermost joint dim has unit input stride.
 template <typename T, typename I>
 ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t partialElemBytes,
-                      const char* perCuKey = "reduce.cols.blocks_per_cu", int perCuDefault = 1) {
+                      const char* perCuKey = "reduce.cols.blocks_per_cu", int perCuDefault = 1,
+                      const char* rowBytesKey = "reduce.cols.min_row_bytes", int rowBytesDefault = 1024) {
   constexpr int VEC = 16 / sizeof(T);
   ColsPlan<I> p{};
   const int nd = g.in.dims;
@@ -1154,11 +1155,24 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   const int pack = vec ? VEC : 1;
   const int64_t target = tuning("reduce.cols.target_blocks", (int64_t)num_compute_units(s) * tuning(perCuKey, perCuDefault));
   const int64_t outer = g.outElems / C;
-  // Lanes along the unit-stride dim: a full wave if the dim is long enough, but
-  // narrower column tiles (down to 256-byte rows) are preferred over splitting
-  // the reduced dim when they already give every CU a workgroup.
-  uint32_t TX = std::min<uint32_t>(64, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
-  const uint32_t minTX = (uint32_t)tuning("reduce.cols.min_tx", 16);
+  // Lanes along the unit-stride dim: up to 1 KiB of a row per workgroup, halved
+  // while the output gives too few workgroups, but not below `rowBytes`: 256
+  // when every row starts on a 128-byte line; otherwise a segment shares its
+  // first and last line with the neighbouring tile and narrow segments pay
+  // for that (256-byte segments of a 16400-byte-stride matrix summed at
+  // 4.1 TB/s, 1 KiB ones at 5.2), so the floor is 1 KiB (512 bytes for the
+  // value+index kernel, which prefers more workgroups). The
+  // scalar path (rows not 16-byte aligned) counts bytes the same way: with 16
+  // lanes of 4 bytes it ran at half the bandwidth of the pack path.
+  const uint32_t laneBytes = (uint32_t)(pack * sizeof(T));
+  const uint32_t maxTX = std::min<uint32_t>(kBlock, std::max<uint32_t>(64, 1024 / laneBytes));
+  uint32_t TX = std::min<uint32_t>(maxTX, pow2_ceil((uint64_t)((C + pack - 1) / pack)));
+  bool lineAligned = reinterpret_cast<uintptr_t>(in) % 128 == 0 && (g.sR * (int64_t)sizeof(T)) % 128 == 0;
+  for (int d = 0; d < nd - 1 && lineAligned; ++d)
+    lineAligned = (g.in.stride[d] * (int64_t)sizeof(T)) % 128 == 0 || g.in.size[d] == 1;
+  const uint32_t rowBytes = lineAligned ? 256u : (uint32_t)tuning(rowBytesKey, rowBytesDefault);
+  const uint32_t minTX = std::min<uint32_t>(
+      maxTX, std::max<uint32_t>((uint32_t)tuning("reduce.cols.min_tx", 16), rowBytes / laneBytes));
   auto tiles_for = [&](uint32_t tx) { return (C + (int64_t)tx * pack - 1) / ((int64_t)tx * pack); };
   while (TX > minTX && outer * tiles_for(TX) < target) TX >>= 1;
   const uint32_t TY = kBlock / TX;
@@ -1187,13 +1201,16 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
       }
     }
     S = std::min<int64_t>(S, maxS);
+  }
+  const int64_t forced = tuning("reduce.cols.force_split", 0);
+  if (forced > 0) S = std::min<int64_t>(forced, g.R);
+  if (S > 1) {
+    // the partial planes must fit the scratch buffer, whoever chose S
     size_t scratchBytes = 0;
     scratch_space(s, &scratchBytes);
     S = std::min<int64_t>(S, (int64_t)(scratchBytes / partialElemBytes) / std::max<int64_t>(g.outElems, 1));
     if (S < 2) S = 1;
   }
-  const int64_t forced = tuning("reduce.cols.force_split", 0);
-  if (forced > 0) S = std::min<int64_t>(forced, g.R);
   int64_t chunk = (g.R + S - 1) / S;
   S = (g.R + chunk - 1) / chunk;
   p.vec = vec;
@@ -1317,7 +1334,8 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
   {
     // the (value, index) kernel does several ALU steps per element: two workgroups
     // per CU hide them (6.5 TB/s against 4.4 with one), the plain reductions want one
-    ColsPlan<I> p = plan_cols<T, I>(s, g, in, 16, "reduce.cols.index_blocks_per_cu", 2);
+    ColsPlan<I> p = plan_cols<T, I>(s, g, in, 16, "reduce.cols.index_blocks_per_cu", 2,
+                                    "reduce.cols.index_min_row_bytes", 512);
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
     const I idxInner = (I)g.idx.stride[nd - 1];
     const bool split = p.a.S.d > 1;

@@ -360,3 +360,22 @@ def test_minmax_of_few_long_rows_is_split(thc, oracle, kind):
         assert run_minmax(thc, oracle, "max", dev, ref, 1) == "rows-index-split"
     finally:
         thc.force_64bit_index(False)
+
+
+def test_forced_split_is_capped_by_the_scratch_buffer(thc, oracle):
+    """The split knob is a request: the partial planes of a column reduction
+    must fit the per-stream scratch buffer whatever it asks for."""
+    rng = np.random.default_rng(53)
+    x = rng.integers(-50, 50, (600, 70000)).astype(np.float32)
+    dev = thc.Tensor.from_numpy(x)
+    thc.set_tuning("reduce.cols.force_split", 512)   # 512 x 70000 (value, index) pairs do not fit
+    try:
+        vals, idx = thc.Tensor("float"), thc.Tensor("long")
+        vals.max(idx, dev, 0)
+        sums = thc.Tensor("float").sum(dev, 0)
+    finally:
+        thc.set_tuning("reduce.cols.force_split", 0)
+    wv, wi = oracle.minmax_dim("max", oracle.View.of(x), 0)
+    assert_bit_equal(vals.numpy(), wv.numpy())
+    np.testing.assert_array_equal(idx.numpy(), wi.numpy())
+    assert_bit_equal(sums.numpy(), x.sum(axis=0, dtype=np.float64).astype(np.float32).reshape(1, -1))
