@@ -355,6 +355,11 @@ struct TiledArgs {
   I bstride[kMaxOps][kMaxDims];
   Divisor<uint32_t> tilesP, tilesQ;
   uint32_t totalTiles;
+  // Tiles per XCD when workgroup b (dispatched to XCD b % 8) takes tile
+  // (b % 8) * xcdPer + b / 8, so that neighbouring tiles, which share partly
+  // read and partly written lines when rows do not start on 128-byte lines,
+  // run on one XCD's L2; 0 = identity mapping.
+  uint32_t xcdPer;
 };
 
 // A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
@@ -418,7 +423,10 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
   }
   const bool fused = args.nq > 1;
 
-  for (uint32_t tile = blockIdx.x; tile < args.totalTiles; tile += gridDim.x) {
+  const uint32_t slots = args.xcdPer ? args.xcdPer * 8 : args.totalTiles;
+  for (uint32_t b = blockIdx.x; b < slots; b += gridDim.x) {
+    const uint32_t tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
+    if (tile >= args.totalTiles) continue;  // uniform over the workgroup
     uint32_t rest, tq, tp;
     args.tilesQ.divmod(tile, rest, tq);
     args.tilesP.divmod(rest, rest, tp);
@@ -528,6 +536,167 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
       body(std::true_type{});
     else
       body(std::false_type{});
+    __syncthreads();  // the slabs are reused by the next tile
+  }
+}
+
+// The tiled kernel for rows that do not start on 16-byte boundaries (odd
+// sizes, views at odd offsets). Every global access is still an aligned
+// 16-byte pack: a lane row covers a window of LX*VEC elements that starts at
+// the aligned address at or below the row's first tile element, so the
+// window's element j sits at tile coordinate j - m, with m < VEC the row's own
+// misalignment. A tile therefore spans VEC fewer elements than the window in
+// both dims. Packs that straddle a tile or tensor edge are loaded whole (they
+// hold at least one element of the row, so the access stays inside a 16-byte
+// unit the tensor owns part of) and stored element by element. The host
+// guarantees that all direct operands share the output's misalignment on
+// every row. The element-wise staging through LDS absorbs the shifts for free.
+template <typename T, typename Op, typename I, int VEC, int LXP, int LXQ, int MASK>
+__global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const T* in0,
+                                                                   const T* in1, const T* in2,
+                                                                   TiledArgs<I> args, Op op) {
+  constexpr int NOPS = Op::NIN + 1;
+  constexpr int TP = LXP * VEC - VEC, TQ = LXQ * VEC - VEC;
+  constexpr int ROWS_P = kBlock / LXP, PASSES_P = (TQ + ROWS_P - 1) / ROWS_P;
+  constexpr int ROWS_Q = kBlock / LXQ, PASSES_Q = (TP + ROWS_Q - 1) / ROWS_Q;
+  constexpr int PITCH = TP | 1;
+  using P = Pack<T, VEC>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  auto misalignment = [](const T* row) {
+    return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(T)) & (uintptr_t)(VEC - 1));
+  };
+
+  const T* ptr[kMaxOps] = {out, in0, in1, in2};
+  const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
+  const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  bool staged[kMaxOps];
+  int slot[kMaxOps];
+  {
+    int s = 0;
+    staged[0] = false;
+    slot[0] = -1;
+#pragma unroll
+    for (int k = 1; k < NOPS; ++k) {
+      staged[k] = ((MASK >> (k - 1)) & 1) != 0;
+      slot[k] = staged[k] ? s++ : -1;
+    }
+  }
+  uint32_t vo[kMaxOps];     // lane's row offset (elements) inside a tile
+  size_t rowStep[kMaxOps];  // uniform distance between two passes
+#pragma unroll
+  for (int k = 0; k < NOPS; ++k) {
+    if (staged[k]) {
+      vo[k] = lyp * (uint32_t)args.strideQ[k];
+      rowStep[k] = (size_t)ROWS_P * (size_t)args.strideQ[k];
+    } else {
+      vo[k] = lyq * (uint32_t)args.strideP[k];
+      rowStep[k] = (size_t)ROWS_Q * (size_t)args.strideP[k];
+    }
+  }
+
+  const uint32_t slots = args.xcdPer ? args.xcdPer * 8 : args.totalTiles;
+  for (uint32_t b = blockIdx.x; b < slots; b += gridDim.x) {
+    const uint32_t tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
+    if (tile >= args.totalTiles) continue;  // uniform over the workgroup
+    uint32_t rest, tq, tp;
+    args.tilesQ.divmod(tile, rest, tq);
+    args.tilesP.divmod(rest, rest, tp);
+    I base[kMaxOps] = {0, 0, 0, 0};
+    for (int j = 0; j < args.nbatch; ++j) {
+      uint32_t r;
+      args.bsize[j].divmod(rest, rest, r);
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) base[k] += (I)r * args.bstride[k][j];
+    }
+    const uint32_t p0 = tp * TP, q0 = tq * TQ;
+    const int pn = (int)min((uint32_t)TP, args.sizeP - p0);
+    const int qn = (int)min((uint32_t)TQ, args.sizeQ - q0);
+    const T* tbase[kMaxOps];
+#pragma unroll
+    for (int k = 0; k < NOPS; ++k)
+      tbase[k] = ptr[k] + (base[k] + (I)p0 * args.strideP[k] + (I)q0 * args.strideQ[k]);
+
+    // phase 1: staged inputs, lanes along p, into lds[slot][q][p]
+#pragma unroll
+    for (int k = 1; k < NOPS; ++k) {
+      if (!staged[k]) continue;
+      T* slab = lds + slot[k] * (TQ * PITCH);
+      P v[PASSES_P];
+      int first[PASSES_P];  // tile coordinate (along p) of the pack's element 0
+#pragma unroll
+      for (int r = 0; r < PASSES_P; ++r) {
+        const int qi = (int)lyp + r * ROWS_P;
+        const T* row = tbase[k] + r * rowStep[k] + vo[k];
+        first[r] = (int)(lxp * VEC) - misalignment(row);
+        if (qi < qn && first[r] < pn) v[r] = load_pack<true>(reinterpret_cast<const P*>(row + first[r]));
+      }
+#pragma unroll
+      for (int r = 0; r < PASSES_P; ++r) {
+        const int qi = (int)lyp + r * ROWS_P;
+        if (qi < qn && first[r] < pn) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const int pi = first[r] + e;
+            if (pi >= 0 && pi < pn) slab[qi * PITCH + pi] = v[r].v[e];
+          }
+        }
+      }
+    }
+    __syncthreads();
+
+    // phase 2: compute with lanes along q
+    P din[3][PASSES_Q];
+    int first[PASSES_Q];  // tile coordinate (along q) of the pack's element 0
+#pragma unroll
+    for (int r = 0; r < PASSES_Q; ++r) {
+      const int pi = (int)lyq + r * ROWS_Q;
+      first[r] = (int)(lxq * VEC) - misalignment(tbase[0] + r * rowStep[0] + vo[0]);
+      if (!(pi < pn && first[r] < qn)) first[r] = qn;  // marks an idle pass
+    }
+#pragma unroll
+    for (int k = 1; k < NOPS; ++k) {
+      if (staged[k]) continue;
+#pragma unroll
+      for (int r = 0; r < PASSES_Q; ++r) {
+        if (first[r] < qn)
+          din[k - 1][r] = load_pack<true>(
+              reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k] + first[r]));
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < PASSES_Q; ++r) {
+      const int pi = (int)lyq + r * ROWS_Q;
+      if (first[r] < qn) {
+        P in[3] = {};
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k) {
+          if (staged[k]) {
+            const T* slab = lds + slot[k] * (TQ * PITCH);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const int qi = min(max(first[r] + e, 0), TQ - 1);
+              in[k - 1].v[e] = slab[qi * PITCH + pi];
+            }
+          } else {
+            in[k - 1] = din[k - 1][r];
+          }
+        }
+        P res;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) res.v[e] = op(in[0].v[e], in[1].v[e], in[2].v[e]);
+        T* orow = const_cast<T*>(tbase[0]) + r * rowStep[0] + vo[0];
+        if (first[r] >= 0 && first[r] + VEC <= qn) {
+          store_pack<false>(reinterpret_cast<P*>(orow + first[r]), res);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const int qi = first[r] + e;
+            if (qi >= 0 && qi < qn) orow[qi] = res.v[e];
+          }
+        }
+      }
+    }
     __syncthreads();  // the slabs are reused by the next tile
   }
 }
@@ -700,9 +869,30 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
   }
   const size_t ldsV = nstaged * tqV * (tpV + 1) * sizeof(T);
   const size_t ldsS = nstaged * tS * (tS + 1) * sizeof(T);
+  const size_t ldsH = nstaged * (tqV - VEC) * ((tpV - VEC) | 1) * sizeof(T);
   if (vec && ldsV > 64 * 1024) vec = false;
-  if (!vec && ldsS > 64 * 1024) return false;
-  const int64_t tileP = vec ? tpV : tS, tileQ = vec ? tqV : tS;
+  // Misaligned rows: the shifted-window variant keeps 16-byte accesses when
+  // every operand has unit stride along its fast dim and the direct operands
+  // share the output's misalignment on every row (equal base offsets and
+  // strides modulo the pack width); otherwise the element-wise variant runs.
+  bool shift = !vec && ldsH <= 64 * 1024 && tuning("apply.tiled.shift", 1);
+  if (shift) {
+    auto mod = [](int64_t x) { return ((x % VEC) + VEC) % VEC; };
+    auto base_mod = [&](int k) {
+      return (int64_t)((reinterpret_cast<uintptr_t>(pl.ptr[k]) / sizeof(T)) % VEC);
+    };
+    for (int k = 0; k < pl.nops && shift; ++k) {
+      shift = pl.lay[k].stride[staged[k] ? p : q] == 1 &&
+              reinterpret_cast<uintptr_t>(pl.ptr[k]) % sizeof(T) == 0;
+      if (!shift || staged[k] || k == 0) continue;
+      shift = base_mod(k) == base_mod(0);
+      for (int d = 0; d < nd && shift; ++d)
+        if (d != q) shift = mod(pl.lay[k].stride[d]) == mod(pl.lay[0].stride[d]);
+    }
+  }
+  if (!vec && !shift && ldsS > 64 * 1024) return false;
+  const int64_t tileP = vec ? tpV : (shift ? tpV - VEC : tS);
+  const int64_t tileQ = vec ? tqV : (shift ? tqV - VEC : tS);
 
   TiledArgs<I> args{};
   for (int k = 0; k < pl.nops; ++k) {
@@ -754,7 +944,20 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
   const int64_t outSpan = (int64_t)tileP * pl.lay[0].stride[p] * (int64_t)sizeof(T);
   const int64_t ntKnob = tuning("apply.tiled.nt_store", -1);
   const bool nts = ntKnob >= 0 ? ntKnob != 0 : outSpan >= (int64_t(32) << 20);
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, tuning("apply.tiled.max_grid", 1 << 22)));
+  bool lineAligned = true;  // every row of every operand starts on a 128-byte line
+  for (int k = 0; k < pl.nops; ++k) {
+    lineAligned = lineAligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % 128 == 0;
+    for (int d = 0; d < nd; ++d)
+      if (pl.lay[k].stride[d] != 1 && pl.lay[k].size[d] > 1)
+        lineAligned = lineAligned && (pl.lay[k].stride[d] * (int64_t)sizeof(T)) % 128 == 0;
+  }
+  const int64_t swz = tuning("apply.tiled.xcd_swizzle", 1);
+  // (not with fused q: there the direct operands are one long aligned run and
+  // the remap cost 2% on a permuted 2048 x 2048 x 520 operand)
+  if ((swz == 2 || (swz == 1 && !lineAligned && args.nq == 1)) && total >= 64 && total < (int64_t(1) << 28))
+    args.xcdPer = (uint32_t)((total + 7) / 8);
+  const int64_t slots = args.xcdPer ? (int64_t)args.xcdPer * 8 : total;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(slots, tuning("apply.tiled.max_grid", 1 << 22)));
   T* out = (T*)pl.ptr[0];
   const T* i0 = (const T*)pl.ptr[1];
   const T* i1 = (const T*)pl.ptr[2];
@@ -768,7 +971,10 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
   case M:                                                                                         \
     if ((M) < (1 << Op::NIN)) {                                                                   \
       constexpr int MM = (M) < (1 << Op::NIN) ? (M) : 1;                                          \
-      if (!vec)                                                                                   \
+      if (shift)                                                                                  \
+        hipLaunchKernelGGL((apply_tiled_shift_kernel<T, Op, I, VEC, LXP, LXQ, MM>), dim3(grid),   \
+                           dim3(kBlock), ldsH, st, out, i0, i1, i2, args, op);                    \
+      else if (!vec)                                                                              \
         hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, 1, 64, 64, MM, false>), dim3(grid),      \
                            dim3(kBlock), ldsS, st, out, i0, i1, i2, args, op);                    \
       else if (nts)                                                                               \
@@ -785,7 +991,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op) {
     default: return false;
   }
 #undef THC_TILED_CASE
-  note_kernel(vec ? (args.nq > 1 ? "tiled-fused" : "tiled") : "tiled-scalar");
+  note_kernel(vec ? (args.nq > 1 ? "tiled-fused" : "tiled") : (shift ? "tiled-shift" : "tiled-scalar"));
   return true;
 }
 

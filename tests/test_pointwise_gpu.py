@@ -81,13 +81,17 @@ def test_random_strided_geometries(thc, oracle, seed):
     run_binary(thc, oracle, name, geoms, rng, inplace=(seed % 5 == 0))
 
 
+@pytest.mark.parametrize("shift", [1, 0])
 @pytest.mark.parametrize("force64", [False, True])
 @pytest.mark.parametrize("shape", [(64, 64), (70, 131), (257, 33), (8, 8), (5, 300, 7), (3, 40, 50),
                                    (128, 4, 96), (1, 200, 200), (2, 3, 65, 67)])
-def test_transposed_operand_uses_tiles(thc, oracle, shape, force64):
+def test_transposed_operand_uses_tiles(thc, oracle, shape, force64, shift):
     """One operand's unit-stride dim is the first logical dim (a:t(), or a
-    permute(3,2,1) view); out and b are contiguous."""
+    permute(3,2,1) view); out and b are contiguous. Rows that are not 16-byte
+    aligned run on the shifted-window variant, or, with it switched off, on
+    the element-wise one."""
     rng = np.random.default_rng(sum(shape))
+    thc.set_tuning("apply.tiled.shift", shift)
     nd = len(shape)
     st, run = [0] * nd, 1
     for d in range(nd):            # dim 0 innermost in memory
@@ -102,11 +106,61 @@ def test_transposed_operand_uses_tiles(thc, oracle, shape, force64):
         k3 = run_binary(thc, oracle, "cdiv", [ga, gc, gc], rng)   # transposed OUTPUT
     finally:
         thc.force_64bit_index(False)
+        thc.set_tuning("apply.tiled.shift", 1)
     dims = [s for s in shape if s != 1]
     if dims[0] >= 8 and dims[-1] >= 8:      # tiny tile dims fall back to the strided kernel
         assert k.startswith("tiled") and k2.startswith("tiled") and k3.startswith("tiled"), (k, k2, k3)
+        if dims[0] % 4 or dims[-1] % 4:
+            assert k == ("tiled-shift" if shift else "tiled-scalar"), k
     else:
         assert k.startswith("strided"), (k, k2, k3)
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_shifted_window_tiles_at_every_misalignment(thc, oracle, kind):
+    """Sizes around the window edges (a tile spans 4 elements fewer than its
+    window; 8 for half), views that start 1..3 elements into their storage,
+    rows with gaps, and operands whose misalignments differ (those fall back
+    to the element-wise variant). Whole storages are compared, so a store
+    outside the tensor's own elements fails the test."""
+    rng = np.random.default_rng(77)
+    for rows, cols in ((60, 124), (61, 125), (59, 123), (121, 249), (333, 515), (1001, 67)):
+        for off in (0, 1, 3):
+            ga = (rows * cols + off, off, (rows, cols), (1, rows))          # a:t()
+            gc = (rows * cols + off, off, (rows, cols), (cols, 1))
+            k = run_binary(thc, oracle, "cadd1", [gc, ga, gc], rng, kind=kind)
+            vec = 8 if kind == "half" else 4
+            aligned = rows % vec == 0 and cols % vec == 0 and off == 0
+            assert k == ("tiled" if aligned else "tiled-shift"), (rows, cols, off, k)
+            k = run_binary(thc, oracle, "cmul", [ga, gc, gc], rng, kind=kind)   # transposed output
+            assert k.startswith("tiled"), k
+    # rows with gaps (a narrowed view of a wider matrix), transposed partner at another offset
+    gout = (200 * 131 + 2, 2, (200, 127), (131, 1))
+    ga = (127 * 203 + 1, 1, (200, 127), (1, 203))
+    gb = (200 * 131 + 2, 2, (200, 127), (131, 1))
+    assert run_binary(thc, oracle, "cadd", [gout, ga, gb], rng, kind=kind) == "tiled-shift"
+    # b starts one element later than out: no common window
+    gb = (200 * 131 + 3, 3, (200, 127), (131, 1))
+    assert run_binary(thc, oracle, "cadd", [gout, ga, gb], rng, kind=kind) == "tiled-scalar"
+    # b's rows drift against out's (row strides differ modulo the pack width)
+    gb = (200 * 130 + 2, 2, (200, 127), (130, 1))
+    assert run_binary(thc, oracle, "cadd", [gout, ga, gb], rng, kind=kind) == "tiled-scalar"
+
+
+def test_shifted_window_tiles_with_two_staged_inputs(thc, oracle):
+    rng = np.random.default_rng(78)
+    x = rng.standard_normal((203, 331)).astype(np.float32)
+    y = rng.standard_normal((203, 331)).astype(np.float32)
+    z = rng.standard_normal((331, 203)).astype(np.float32)
+    dx, dy, dz = (thc.Tensor.from_numpy(v) for v in (x, y, z))
+    out = thc.Tensor("float").addcmul(dz, 0.5, dx.t(), dy.t())
+    assert thc.last_kernel() == "tiled-shift"
+    want = oracle.pointwise("addcmul", oracle.View.empty((331, 203)), oracle.View.of(z),
+                            oracle.View(x.reshape(-1).copy(), 0, (331, 203), (1, 331)),
+                            oracle.View(y.reshape(-1).copy(), 0, (331, 203), (1, 331)), value=0.5)
+    assert_bit_equal(out.numpy(), want.numpy())
+    out = thc.Tensor("float").cadd(dx.t(), 2.0, dy.t())      # both inputs staged, nothing direct but out
+    assert_bit_equal(out.numpy(), (x.T + np.float32(2.0) * y.T).astype(np.float32))
 
 
 def test_all_operands_transposed_alike_is_flat(thc, oracle):
