@@ -437,6 +437,130 @@ __global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T
   }
 }
 
+// Short rows that lie back to back in memory (row r starts at in + r * R).
+// A lane group per row reads 64-byte pieces at the rows' own, mostly
+// misaligned, addresses (100-element fp32 rows summed at 2.8 TB/s, 10-element
+// ones at 1.9). Here a workgroup streams its run of rows into LDS as one flat
+// sequence of aligned 16-byte packs (the first pack starts at the aligned
+// address at or below the run's first element, so it and the last pack may
+// hold a few elements of the neighbouring runs) and the lane groups reduce
+// out of LDS, where alignment is free.
+template <typename TIn, int U>
+__device__ __forceinline__ uint32_t stage_rows_to_lds(const TIn* first, uint32_t count, TIn* lds) {
+  constexpr int VEC = 16 / sizeof(TIn);
+  using P = Pack<TIn, VEC>;
+  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(first) / sizeof(TIn)) & (uintptr_t)(VEC - 1));
+  const P* src = reinterpret_cast<const P*>(first - mis);
+  const uint32_t npacks = (mis + count + VEC - 1) / VEC;
+  for (uint32_t i0 = threadIdx.x; i0 < npacks; i0 += U * kBlock) {
+    P v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + u * kBlock < npacks) v[u] = load_pack<true>(src + i0 + u * kBlock);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + u * kBlock < npacks) reinterpret_cast<P*>(lds)[i0 + u * kBlock] = v[u];
+  }
+  return mis;  // element 0 of the run sits at lds[mis]
+}
+
+template <typename TIn, typename TOut, typename F, typename I>
+__global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __restrict__ in,
+                                                                 TOut* __restrict__ out,
+                                                                 OuterArgs<I> oa, I numRows, I R,
+                                                                 uint32_t rowsPerBlock, uint32_t G,
+                                                                 Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  TIn* lds = reinterpret_cast<TIn*>(lds_raw);
+  const uint32_t lane = threadIdx.x % G, grp = threadIdx.x / G, groups = kBlock / G;
+  const I numBlocks = (numRows + rowsPerBlock - 1) / rowsPerBlock;
+  for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const I row0 = blk * rowsPerBlock;
+    const uint32_t nrows = (uint32_t)min((I)rowsPerBlock, numRows - row0);
+    const uint32_t mis = stage_rows_to_lds<TIn, 8>(in + row0 * R, nrows * (uint32_t)R, lds);
+    __syncthreads();
+    // lanes of one group share r, so they leave the loop together
+    for (uint32_t r = grp; r < nrows; r += groups) {
+      const TIn* row = lds + mis + r * (uint32_t)R;
+      I inOff, outOff;
+      oa.offsets(row0 + r, inOff, outOff);
+      A c = (A)0;
+      if constexpr (F::kCentred) c = acc_up<A>(out[outOff]);
+      A acc = f.init();
+      for (uint32_t j = lane; j < (uint32_t)R; j += G) acc = f.combine(acc, f.modify(acc_up<A>(row[j]), c));
+      for (uint32_t o = G >> 1; o > 0; o >>= 1) acc = f.combine(acc, shfl_xor_any(acc, o));
+      if (lane == 0) out[outOff] = epi.template finish<TOut>(acc);
+    }
+    __syncthreads();  // the buffer is refilled by the next run
+  }
+}
+
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
+    const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI, OuterArgs<I> oa,
+    OuterArgs<I> oaIdx, I numRows, I R, uint32_t rowsPerBlock, uint32_t G) {
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  const uint32_t lane = threadIdx.x % G, grp = threadIdx.x / G, groups = kBlock / G;
+  const I numBlocks = (numRows + rowsPerBlock - 1) / rowsPerBlock;
+  for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const I row0 = blk * rowsPerBlock;
+    const uint32_t nrows = (uint32_t)min((I)rowsPerBlock, numRows - row0);
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + row0 * R, nrows * (uint32_t)R, lds);
+    __syncthreads();
+    for (uint32_t r = grp; r < nrows; r += groups) {
+      const T* row = lds + mis + r * (uint32_t)R;
+      // two independent candidate chains per lane (elements j and j + G of
+      // each step), merged with the lowest-index rule
+      A bv = O::worst(), bv1 = O::worst();
+      uint32_t bi = ~0u, bi1 = ~0u;
+      uint32_t j = lane;
+      for (; j + G < (uint32_t)R; j += 2 * G) {
+        const A x = acc_up<A>(row[j]), x1 = acc_up<A>(row[j + G]);
+        if (O::better_later(x, bv)) {
+          bv = x;
+          bi = j;
+        }
+        if (O::better_later(x1, bv1)) {
+          bv1 = x1;
+          bi1 = j + G;
+        }
+      }
+      if (j < (uint32_t)R) {
+        const A x = acc_up<A>(row[j]);
+        if (O::better_later(x, bv)) {
+          bv = x;
+          bi = j;
+        }
+      }
+      if (O::better(bv1, bi1, bv, bi)) {
+        bv = bv1;
+        bi = bi1;
+      }
+      for (uint32_t o = G >> 1; o > 0; o >>= 1) {
+        const A ov = shfl_xor_any(bv, o);
+        const uint32_t oi = __shfl_xor(bi, o, 64);
+        if (O::better(ov, oi, bv, bi)) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (lane == 0) {
+        I unusedA, unusedB, outOff, idxOff;
+        oa.offsets(row0 + r, unusedA, outOff);
+        oaIdx.offsets(row0 + r, unusedB, idxOff);
+        if (bi == ~0u) bi = 0;  // nothing beat the start value: first element
+        outV[outOff] = acc_down<T>(bv);
+        outI[idxOff] = (long)bi + 1;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // var / std along a unit-stride dim whose rows fit the registers of one lane
 // group (R <= 64 lanes x 8 packs): the row is read once, the mean and the sum
 // of squared deviations both come from the registers.
@@ -1088,6 +1212,39 @@ void launch_rows_pass(THCState* s, const TIn* in, TOut* out, typename F::A* part
                        st, in, out, partial, oa, (I)numRows, (I)R, (I)sR, Sd, (I)chunk, G, epi, f);
 }
 
+// Short rows lying back to back: geometry of the LDS-staged kernels. Rows
+// below 512 bytes when they could also be read as aligned packs (from there
+// on the lane-group kernel is faster: 6.4 against 5.5 TB/s on 128-element
+// fp32 rows, 3.5 against 5.5 on 64-element ones), up to 8 KiB otherwise.
+template <typename T>
+bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPerBlock, uint32_t& G,
+                   size_t& ldsBytes) {
+  if (!tuning("reduce.rows.lds", 1) || g.sR != 1) return false;
+  int64_t run = g.R;
+  for (int d = g.in.dims - 1; d >= 0; --d) {
+    if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
+    run *= g.in.size[d];
+  }
+  const int64_t rowBytes = g.R * (int64_t)sizeof(T);
+  const int64_t limit = vec ? tuning("reduce.rows.lds_max_vec_bytes", 511) : tuning("reduce.rows.lds_max_bytes", 8192);
+  if (rowBytes > limit) return false;
+  // about four runs per CU, each between 4 and 32 KiB (32 KiB = one batch of
+  // eight 16-byte loads per lane)
+  int64_t chunk = g.outElems * rowBytes / ((int64_t)num_compute_units(s) * 4);
+  chunk = std::min<int64_t>(32768, std::max<int64_t>(4096, chunk));
+  rowsPerBlock = (uint32_t)std::max<int64_t>(1, chunk / rowBytes);
+  // about 16 elements per lane: the group's shuffle tree and the per-row
+  // bookkeeping are a dependent chain, so wide groups on short rows are
+  // latency bound (33-element fp32 rows summed at 0.9 TB/s with a lane per
+  // element, 3.0 with 2 elements per lane, 5.7 with 16; 64 and more lose again)
+  const uint64_t perLane = (uint64_t)tuning("reduce.rows.lds_elems_per_lane", 16);
+  G = pow2_ceil((uint64_t)g.R / perLane + 1);
+  if (G > 1 && (uint64_t)G * perLane > (uint64_t)g.R) G >>= 1;
+  G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+  ldsBytes = (((size_t)rowsPerBlock * (size_t)g.R + 2 * (16 / sizeof(T))) * sizeof(T) + 15) & ~size_t(15);
+  return true;
+}
+
 // rows: a group of lanes per output. Packs when the reduced dim has unit stride
 // and everything is 16-byte aligned, scalar strided loads otherwise.
 template <typename T, typename F, typename I>
@@ -1112,6 +1269,16 @@ void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typenam
     chunk = (g.R + S - 1) / S;
     chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
     S = (g.R + chunk - 1) / chunk;
+  }
+  uint32_t ldsRows = 0, ldsG = 0;
+  size_t ldsBytes = 0;
+  if (S == 1 && plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
+    const int64_t blocks = (rows + ldsRows - 1) / ldsRows;
+    const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+    hipLaunchKernelGGL((reduce_rows_lds_kernel<T, T, F, I>), dim3(grid), dim3(kBlock), ldsBytes,
+                       current_stream(s), in, out, oa, (I)rows, (I)g.R, ldsRows, ldsG, epi, f);
+    note_kernel("rows-lds");
+    return;
   }
   if (S == 1) {
     launch_rows_pass<T, T, F, I, true>(s, in, out, nullptr, oa, rows, g.R, g.sR, 1, g.R, vec, epi, f);
@@ -1284,6 +1451,17 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
     OuterArgs<I> oa = make_outer<I>(g.in, g.out, nd);
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
     const int64_t rows = g.outElems;
+    {
+      uint32_t ldsRows = 0, ldsG = 0;
+      size_t ldsBytes = 0;
+      if (plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
+        const int grid = capped_grid(s, (rows + ldsRows - 1) / ldsRows, "reduce.rows.blocks_per_cu", 64);
+        hipLaunchKernelGGL((reduce_rows_index_lds_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock),
+                           ldsBytes, st, in, outV, outI, oa, oaIdx, (I)rows, (I)g.R, ldsRows, ldsG);
+        note_kernel("rows-index-lds");
+        return;
+      }
+    }
     // Few long rows: cut them as run_rows does.
     const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
     const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);

@@ -87,7 +87,7 @@ def test_gpu_var_rows_single_read_and_fallback(thc, oracle, kind):
     dtype = np.float32 if kind == "float" else np.float16
     vec = 4 if kind == "float" else 8
     for shape, expect in (((300, 1024), "var-rows"), ((7, 64 * vec * 8), "var-rows"), ((5, 8), "var-rows"),
-                          ((3, 64 * vec * 8 + vec), "rows"), ((50, 1023), "rows-scalar"), ((2, 40000), None)):
+                          ((3, 64 * vec * 8 + vec), "rows"), ((50, 1023), "rows-lds"), ((2, 40000), None)):
         x = (rng.standard_normal(shape) * 2 + 3).astype(dtype)
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
         for name, okind in (("var", "var"), ("std", "std")):

@@ -379,3 +379,70 @@ def test_forced_split_is_capped_by_the_scratch_buffer(thc, oracle):
     assert_bit_equal(vals.numpy(), wv.numpy())
     np.testing.assert_array_equal(idx.numpy(), wi.numpy())
     assert_bit_equal(sums.numpy(), x.sum(axis=0, dtype=np.float64).astype(np.float32).reshape(1, -1))
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_short_dense_rows_are_staged_through_lds(thc, oracle, kind):
+    """Rows that lie back to back are streamed into LDS as one flat run of
+    aligned packs, whatever the rows' own alignment: every row length from 1
+    to 40, lengths around the limits, storage offsets 0..3, row counts that
+    leave a ragged last run; same results with the kernel switched off."""
+    rng = np.random.default_rng(54)
+    shapes = [(37, r) for r in range(1, 41)] + [(5000, 10), (777, 70), (300, 100), (41, 1001), (3, 2048),
+                                               (2, 3, 250), (9, 511)]
+    for shape in shapes:
+        n = int(np.prod(shape))
+        for off in (0, 1, 3) if shape[-1] in (10, 70, 100) else (0,):
+            st = [1] * len(shape)
+            for d in range(len(shape) - 2, -1, -1):
+                st[d] = st[d + 1] * shape[d + 1]
+            dev, ref = dev_and_ref(thc, oracle, rng, (n + off, off, shape, tuple(st)), kind, "ints")
+            dim = len(shape) - 1
+            rowbytes = shape[-1] * (4 if kind == "float" else 2)
+            vec = 4 if kind == "float" else 8
+            packs = shape[-1] % vec == 0 and off % vec == 0
+            expect = "rows-lds" if rowbytes <= (511 if packs else 8192) else "rows"
+            for name in ("sum", "norm2", "mean"):
+                k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
+                assert k == expect, (shape, off, name, k)
+            for which in ("max", "min"):
+                k = run_minmax(thc, oracle, which, dev, ref, dim, kind)
+                assert k == expect.replace("rows", "rows-index"), (shape, off, which, k)
+    thc.set_tuning("reduce.rows.lds", 0)
+    try:
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((777, 70)), kind, "ints")
+        assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind) == "rows-scalar"
+        assert run_minmax(thc, oracle, "max", dev, ref, 1, kind) == "rows-index-scalar"
+    finally:
+        thc.set_tuning("reduce.rows.lds", 1)
+
+
+def test_short_dense_rows_special_cases(thc, oracle):
+    x = np.full((300, 33), -np.inf, np.float32)        # nothing beats the start value
+    x[7, 20] = np.nan
+    x[8, :] = 2.5                                      # all tied: first index
+    x[9, 5] = x[9, 31] = 7.0
+    vals, idx = thc.Tensor("float"), thc.Tensor("long")
+    vals.max(idx, thc.Tensor.from_numpy(x), 1)
+    assert thc.last_kernel() == "rows-index-lds"
+    i = idx.numpy().ravel()
+    assert i[0] == 1 and i[7] == 21 and i[8] == 1 and i[9] == 6
+    v = vals.numpy().ravel()
+    assert v[0] == -np.inf and np.isnan(v[7]) and v[8] == 2.5 and v[9] == 7.0
+    # rows dense in the input, outputs strided (a column of a wider matrix)
+    rng = np.random.default_rng(55)
+    y = rng.integers(-9, 9, (500, 21)).astype(np.float32)
+    wide = thc.Tensor.from_numpy(np.zeros((500, 3), np.float32))
+    col = wide.narrow(1, 1, 1)
+    col.sum(thc.Tensor.from_numpy(y), 1)
+    assert thc.last_kernel() == "rows-lds"
+    got = wide.numpy()
+    assert_bit_equal(got[:, 1], y.sum(axis=1).astype(np.float32))
+    assert not got[:, 0].any() and not got[:, 2].any()
+    thc.force_64bit_index(True)
+    try:
+        out = thc.Tensor("float").sum(thc.Tensor.from_numpy(y), 1)
+        assert thc.last_kernel() == "rows-lds"
+        assert_bit_equal(out.numpy().ravel(), y.sum(axis=1).astype(np.float32))
+    finally:
+        thc.force_64bit_index(False)
