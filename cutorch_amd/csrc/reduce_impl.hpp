@@ -561,6 +561,157 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
   }
 }
 
+// Small slices: the input is a dense [O][R][C] array reduced over R, and one
+// R x C slice is a few KiB at most. The column kernels give every slice (and
+// column tile) a workgroup of its own, which for an 8 x 16 slice means 256
+// threads per 512 bytes (0.3 TB/s). Here a workgroup streams a run of whole
+// slices into LDS (as stage_rows_to_lds does for short rows) and its threads
+// take one output each: consecutive lanes take consecutive columns, so the
+// LDS reads of a step are consecutive words. When a run holds fewer outputs
+// than the workgroup has threads, P threads share an output (thread p takes
+// rows p, p + P, ...) and their partials meet in LDS.
+template <typename I>
+struct SlabArgs {
+  OuterArgs<I> oa;        // outer dims: slice index -> output offset
+  I O, R, C;              // slices, reduced length, columns
+  I outInner, idxInner;   // output strides along the columns
+  Divisor<uint32_t> cdiv; // division by C
+  uint32_t slicesPerBlock;
+  uint32_t dataElems;     // LDS elements reserved for the staged run
+};
+
+template <typename TIn, typename TOut, typename F, typename I>
+__global__ __launch_bounds__(kBlock) void reduce_slab_kernel(const TIn* __restrict__ in,
+                                                             TOut* __restrict__ out, SlabArgs<I> a,
+                                                             Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  TIn* lds = reinterpret_cast<TIn*>(lds_raw);
+  A* part = reinterpret_cast<A*>(lds_raw + (((size_t)a.dataElems * sizeof(TIn) + 15) & ~size_t(15)));
+  const uint32_t R = (uint32_t)a.R, C = (uint32_t)a.C, slice = R * C;
+  const I numBlocks = (a.O + a.slicesPerBlock - 1) / a.slicesPerBlock;
+  for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const I o0 = blk * a.slicesPerBlock;
+    const uint32_t ns = (uint32_t)min((I)a.slicesPerBlock, a.O - o0);
+    const uint32_t mis = stage_rows_to_lds<TIn, 8>(in + o0 * (I)slice, ns * slice, lds);
+    __syncthreads();
+    const uint32_t nOut = ns * C;
+    const uint32_t P = nOut >= kBlock ? 1u : min(R, kBlock / nOut);  // uniform over the workgroup
+    auto reduce_one = [&](uint32_t o, uint32_t c, uint32_t first, uint32_t step, I& outOff) {
+      I inOff;
+      a.oa.offsets(o0 + o, inOff, outOff);
+      outOff += (I)c * a.outInner;
+      A ctr = (A)0;
+      if constexpr (F::kCentred) ctr = acc_up<A>(out[outOff]);
+      const TIn* col = lds + mis + o * slice + c;
+      A acc = f.init();
+      for (uint32_t r = first; r < R; r += step) acc = f.combine(acc, f.modify(acc_up<A>(col[r * C]), ctr));
+      return acc;
+    };
+    if (P == 1) {
+      for (uint32_t t = threadIdx.x; t < nOut; t += kBlock) {
+        uint32_t o, c;
+        a.cdiv.divmod(t, o, c);
+        I outOff;
+        const A acc = reduce_one(o, c, 0, 1, outOff);
+        out[outOff] = epi.template finish<TOut>(acc);
+      }
+    } else {
+      const uint32_t p = threadIdx.x / nOut, t = threadIdx.x - p * nOut;
+      uint32_t o, c;
+      a.cdiv.divmod(t, o, c);
+      I outOff = 0;
+      if (p < P) part[p * nOut + t] = reduce_one(o, c, p, P, outOff);
+      __syncthreads();
+      if (p == 0) {
+        A acc = part[t];
+        for (uint32_t q = 1; q < P; ++q) acc = f.combine(acc, part[q * nOut + t]);
+        out[outOff] = epi.template finish<TOut>(acc);
+      }
+    }
+    __syncthreads();  // the buffers are reused by the next run
+  }
+}
+
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_slab_index_kernel(const T* __restrict__ in,
+                                                                   T* __restrict__ outV,
+                                                                   long* __restrict__ outI,
+                                                                   SlabArgs<I> a, OuterArgs<I> oaIdx) {
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  A* partV = reinterpret_cast<A*>(lds_raw + (((size_t)a.dataElems * sizeof(T) + 15) & ~size_t(15)));
+  uint32_t* partI = reinterpret_cast<uint32_t*>(partV + kBlock);
+  const uint32_t R = (uint32_t)a.R, C = (uint32_t)a.C, slice = R * C;
+  const I numBlocks = (a.O + a.slicesPerBlock - 1) / a.slicesPerBlock;
+  for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const I o0 = blk * a.slicesPerBlock;
+    const uint32_t ns = (uint32_t)min((I)a.slicesPerBlock, a.O - o0);
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + o0 * (I)slice, ns * slice, lds);
+    __syncthreads();
+    const uint32_t nOut = ns * C;
+    const uint32_t P = nOut >= kBlock ? 1u : min(R, kBlock / nOut);
+    auto scan_one = [&](uint32_t o, uint32_t c, uint32_t first, uint32_t step, A& bv, uint32_t& bi) {
+      const T* col = lds + mis + o * slice + c;
+      bv = O::worst();
+      bi = ~0u;
+      for (uint32_t r = first; r < R; r += step) {
+        const A x = acc_up<A>(col[r * C]);
+        if (O::better_later(x, bv)) {
+          bv = x;
+          bi = r;
+        }
+      }
+    };
+    auto publish = [&](uint32_t o, uint32_t c, A bv, uint32_t bi) {
+      I unusedA, unusedB, outOff, idxOff;
+      a.oa.offsets(o0 + o, unusedA, outOff);
+      oaIdx.offsets(o0 + o, unusedB, idxOff);
+      if (bi == ~0u) bi = 0;  // nothing beat the start value: first element
+      outV[outOff + (I)c * a.outInner] = acc_down<T>(bv);
+      outI[idxOff + (I)c * a.idxInner] = (long)bi + 1;
+    };
+    if (P == 1) {
+      for (uint32_t t = threadIdx.x; t < nOut; t += kBlock) {
+        uint32_t o, c;
+        a.cdiv.divmod(t, o, c);
+        A bv;
+        uint32_t bi;
+        scan_one(o, c, 0, 1, bv, bi);
+        publish(o, c, bv, bi);
+      }
+    } else {
+      const uint32_t p = threadIdx.x / nOut, t = threadIdx.x - p * nOut;
+      uint32_t o, c;
+      a.cdiv.divmod(t, o, c);
+      if (p < P) {
+        A bv;
+        uint32_t bi;
+        scan_one(o, c, p, P, bv, bi);
+        partV[p * nOut + t] = bv;
+        partI[p * nOut + t] = bi;
+      }
+      __syncthreads();
+      if (p == 0) {
+        A bv = partV[t];
+        uint32_t bi = partI[t];
+        for (uint32_t q = 1; q < P; ++q) {
+          const A v = partV[q * nOut + t];
+          const uint32_t ix = partI[q * nOut + t];
+          if (O::better(v, ix, bv, bi)) {
+            bv = v;
+            bi = ix;
+          }
+        }
+        publish(o, c, bv, bi);
+      }
+    }
+    __syncthreads();
+  }
+}
+
 // var / std along a unit-stride dim whose rows fit the registers of one lane
 // group (R <= 64 lanes x 8 packs): the row is read once, the mean and the sum
 // of squared deviations both come from the registers.
@@ -1395,10 +1546,58 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
   return p;
 }
 
+// Small dense slices (see reduce_slab_kernel): [O][R][C] with rows of a slice
+// and the slices themselves back to back, a slice of at most 16 KiB.
+template <typename T, typename I>
+bool plan_slab(THCState* s, const ReduceGeom& g, SlabArgs<I>& a, int64_t& blocks) {
+  const int nd = g.in.dims;
+  if (!tuning("reduce.slab", 1) || nd < 1) return false;
+  const int64_t C = g.in.size[nd - 1];
+  if (g.in.stride[nd - 1] != 1 || g.sR != C) return false;
+  const int64_t slice = g.R * C;
+  int64_t run = slice;
+  for (int d = nd - 2; d >= 0; --d) {
+    if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
+    run *= g.in.size[d];
+  }
+  const int64_t sliceBytes = slice * (int64_t)sizeof(T);
+  if (sliceBytes > tuning("reduce.slab.max_slice_bytes", 16384)) return false;
+  const int64_t O = g.outElems / C;
+  int64_t chunk = O * sliceBytes / ((int64_t)num_compute_units(s) * 4);
+  chunk = std::min<int64_t>(32768, std::max<int64_t>(4096, chunk));
+  const int64_t spb = std::max<int64_t>(1, chunk / sliceBytes);
+  a.oa = make_outer<I>(g.in, g.out, nd - 1);
+  a.O = (I)O;
+  a.R = (I)g.R;
+  a.C = (I)C;
+  a.outInner = (I)g.out.stride[nd - 1];
+  a.idxInner = (I)g.idx.stride[nd - 1];
+  a.cdiv.set((uint64_t)C);
+  a.slicesPerBlock = (uint32_t)spb;
+  a.dataElems = (uint32_t)(spb * slice + 2 * (16 / sizeof(T)));
+  blocks = (O + spb - 1) / spb;
+  return true;
+}
+template <typename T, typename I>
+size_t slab_data_bytes(const SlabArgs<I>& a) {
+  return ((size_t)a.dataElems * sizeof(T) + 15) & ~size_t(15);
+}
+
 template <typename T, typename F, typename I>
 void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi, F f) {
   using A = typename F::A;
   constexpr int VEC = 16 / sizeof(T);
+  {
+    SlabArgs<I> sa{};
+    int64_t blocks = 0;
+    if (plan_slab<T, I>(s, g, sa, blocks)) {
+      const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+      hipLaunchKernelGGL((reduce_slab_kernel<T, T, F, I>), dim3(grid), dim3(kBlock),
+                         slab_data_bytes<T>(sa) + kBlock * sizeof(A), current_stream(s), in, out, sa, epi, f);
+      note_kernel("slab");
+      return;
+    }
+  }
   ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(A));
   const bool split = p.a.S.d > 1;
   A* scratch = split ? (A*)scratch_space(s, nullptr) : nullptr;
@@ -1508,6 +1707,19 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
     else
       note_kernel(vec ? "rows-index" : (g.sR == 1 ? "rows-index-scalar" : "rows-index-strided"));
     return;
+  }
+  {
+    SlabArgs<I> sa{};
+    int64_t blocks = 0;
+    if (plan_slab<T, I>(s, g, sa, blocks)) {
+      const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+      OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd - 1);
+      hipLaunchKernelGGL((reduce_slab_index_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock),
+                         slab_data_bytes<T>(sa) + kBlock * (sizeof(A) + sizeof(uint32_t)), st, in, outV,
+                         outI, sa, oaIdx);
+      note_kernel("slab-index");
+      return;
+    }
   }
   {
     // the (value, index) kernel does several ALU steps per element: two workgroups
@@ -1632,6 +1844,12 @@ bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in_, voi
     constexpr int VEC = 16 / sizeof(T);
     const int nd = g.in.dims;
     if (g.sR == 1 || nd < 1 || g.in.stride[nd - 1] != 1 || g.in.size[nd - 1] <= 1) return false;
+    {
+      // small dense slices: two sweeps of the slab kernel beat one of this one
+      SlabArgs<uint64_t> sa{};
+      int64_t blocks = 0;
+      if (plan_slab<T, uint64_t>(s, g, sa, blocks)) return false;
+    }
     auto go = [&](auto idxTag) {
       using I = decltype(idxTag);
       ColsPlan<I> p = plan_cols<T, I>(s, g, in_, 2 * sizeof(A));

@@ -111,7 +111,7 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
     dtype = np.float32 if kind == "float" else np.float16
     offset = 100.0 if kind == "float" else 4.0
     for shape, dim, expect in (((64, 512), 0, "var-cols"), ((6, 300, 40), 1, "var-cols"),
-                               ((2, 8192, 96), 1, "var-cols-split"), ((129, 7), 0, "var-cols-scalar"),
+                               ((2, 8192, 96), 1, "var-cols-split"), ((129, 7), 0, "slab"),
                                ((3, 50, 8, 24), 1, "var-cols")):
         x = (rng.standard_normal(shape) * 0.1 + offset).astype(dtype)
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)

@@ -82,7 +82,7 @@ def test_non_innermost_dim(thc, oracle, name, kind):
                        ((3, 50, 8, 24), 1), ((2, 2000, 3), 1), ((16, 33, 1), 1)):
         dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "uniform")
         k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
-        assert k.startswith("cols") or shape[-1] == 1, k
+        assert k.startswith("cols") or k == "slab" or shape[-1] == 1, k
 
 
 def test_split_reduction_is_used_and_correct(thc, oracle):
@@ -446,3 +446,69 @@ def test_short_dense_rows_special_cases(thc, oracle):
         assert_bit_equal(out.numpy().ravel(), y.sum(axis=1).astype(np.float32))
     finally:
         thc.force_64bit_index(False)
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_small_dense_slices_are_staged_through_lds(thc, oracle, kind):
+    """[O][R][C] inputs whose R x C slice is a few KiB: a workgroup stages a
+    run of whole slices and a thread (or P threads, when outputs are few)
+    takes each output. Ragged last runs, storage offsets, R = 1, one slice."""
+    rng = np.random.default_rng(56)
+    cases = [((1000, 8, 16), 1), ((500, 33, 2), 1), ((129, 7), 0), ((50, 100, 10), 1), ((3, 2, 5, 7), 1),
+             ((3, 2, 5, 7), 2), ((77, 1, 9), 1), ((4100, 2, 3), 1), ((2, 200, 5), 1), ((1, 1000, 4), 1),
+             ((300, 3, 130), 1)]
+    for shape, dim in cases:
+        n = int(np.prod(shape))
+        for off in (0, 1, 3) if shape == (500, 33, 2) else (0,):
+            st = [1] * len(shape)
+            for d in range(len(shape) - 2, -1, -1):
+                st[d] = st[d + 1] * shape[d + 1]
+            dev, ref = dev_and_ref(thc, oracle, rng, (n + off, off, shape, tuple(st)), kind, "ints")
+            # a reduced dim of length 1 counts as unit stride: the short-rows kernel takes it
+            ek, eki = ("slab", "slab-index") if shape[dim] > 1 else ("rows-lds", "rows-index-lds")
+            for name in ("sum", "norm2", "mean"):
+                assert run_reduce(thc, oracle, name, dev, ref, dim, kind) == ek, (shape, dim, name)
+            for which in ("max", "min"):
+                assert run_minmax(thc, oracle, which, dev, ref, dim, kind) == eki, (shape, dim)
+    thc.set_tuning("reduce.slab", 0)
+    try:
+        dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((500, 33, 2)), kind, "ints")
+        assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
+        assert run_minmax(thc, oracle, "max", dev, ref, 1, kind).startswith("cols-index")
+    finally:
+        thc.set_tuning("reduce.slab", 1)
+
+
+def test_small_dense_slices_special_cases(thc, oracle):
+    x = np.full((40, 6, 5), np.inf, np.float32)          # nothing beats min's start value
+    x[3, 4, 2] = np.nan
+    x[4, :, 1] = -1.0                                    # all tied: first index
+    x[5, 2, 0] = x[5, 5, 0] = -3.0
+    vals, idx = thc.Tensor("float"), thc.Tensor("long")
+    vals.min(idx, thc.Tensor.from_numpy(x), 1)
+    assert thc.last_kernel() == "slab-index"
+    i, v = idx.numpy()[:, 0, :], vals.numpy()[:, 0, :]
+    assert i[0, 0] == 1 and i[3, 2] == 5 and i[4, 1] == 1 and i[5, 0] == 3
+    assert v[0, 0] == np.inf and np.isnan(v[3, 2]) and v[4, 1] == -1.0 and v[5, 0] == -3.0
+    # outputs strided: a plane of a wider tensor
+    rng = np.random.default_rng(57)
+    y = rng.integers(-9, 9, (200, 9, 4)).astype(np.float32)
+    wide = thc.Tensor.from_numpy(np.zeros((200, 3, 4), np.float32))
+    plane = wide.narrow(1, 1, 1)
+    plane.sum(thc.Tensor.from_numpy(y), 1)
+    assert thc.last_kernel() == "slab"
+    got = wide.numpy()
+    assert_bit_equal(got[:, 1, :], y.sum(axis=1).astype(np.float32))
+    assert not got[:, 0, :].any() and not got[:, 2, :].any()
+    thc.force_64bit_index(True)
+    try:
+        out = thc.Tensor("float").sum(thc.Tensor.from_numpy(y), 1)
+        assert thc.last_kernel() == "slab"
+        assert_bit_equal(out.numpy()[:, 0, :], y.sum(axis=1).astype(np.float32))
+    finally:
+        thc.force_64bit_index(False)
+    # var / std of small slices: two sweeps of the slab kernel
+    z = (rng.standard_normal((300, 12, 6)) * 2 + 5).astype(np.float32)
+    out = thc.Tensor("float").var(thc.Tensor.from_numpy(z), 1)
+    assert thc.last_kernel() == "slab"
+    np.testing.assert_allclose(out.numpy()[:, 0, :], z.astype(np.float64).var(axis=1, ddof=1), rtol=1e-5)
