@@ -111,4 +111,31 @@ struct Divisor<uint64_t> {
   }
 };
 
+// Streams `count` elements starting at `first` (any alignment) into LDS as
+// aligned 16-byte packs, U loads in flight per lane: the first pack starts at
+// the aligned address at or below `first`, so it and the last pack may hold a
+// few neighbouring elements (each pack holds at least one element of the run,
+// so the access stays inside a 16-byte unit the run owns part of). Returns m
+// such that element i of the run is lds[m + i]; `lds` needs room for
+// count + 2 * (16 / sizeof(TIn)) elements. The caller synchronises.
+template <typename TIn, int U>
+__device__ __forceinline__ uint32_t stage_rows_to_lds(const TIn* first, uint32_t count, TIn* lds) {
+  constexpr int VEC = 16 / sizeof(TIn);
+  using P = Pack<TIn, VEC>;
+  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(first) / sizeof(TIn)) & (uintptr_t)(VEC - 1));
+  const P* src = reinterpret_cast<const P*>(first - mis);
+  const uint32_t npacks = (mis + count + VEC - 1) / VEC;
+  for (uint32_t i0 = threadIdx.x; i0 < npacks; i0 += U * kBlock) {
+    P v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + u * kBlock < npacks) v[u] = load_pack<true>(src + i0 + u * kBlock);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + u * kBlock < npacks) reinterpret_cast<P*>(lds)[i0 + u * kBlock] = v[u];
+  }
+  return mis;  // element 0 of the run sits at lds[mis]
+}
+
+
 }  // namespace thc

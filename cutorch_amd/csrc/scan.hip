@@ -12,6 +12,7 @@
 //               and exchange segment totals through LDS.
 // Accumulation is fp32 for float and half (rounded per output element), double
 // for double, wrapping 64-bit for the integer types.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -244,6 +245,60 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
   }
 }
 
+// Small slices of the dense [outer][R][inner] block (short rows when
+// inner == 1): a wave per row, or a workgroup per slice and column tile,
+// leaves most lanes idle (10-element rows scanned at 0.24 TB/s, 8 x 16 slices
+// at 0.5). Here a workgroup streams a run of whole slices into LDS, a thread
+// per (slice, column) scans its R elements in place, and the run goes back
+// out as aligned packs of the OUTPUT's alignment (edge packs element-wise).
+template <typename T, typename Op>
+__global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
+                                                           const T* __restrict__ in,
+                                                           uint64_t outer, uint32_t R,
+                                                           uint32_t inner, uint32_t slicesPerBlock) {
+  constexpr int VEC = 16 / sizeof(T);
+  using P = Pack<T, VEC>;
+  using A = typename ScanAcc<T>::type;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  const uint32_t slice = R * inner;
+  const uint64_t numBlocks = (outer + slicesPerBlock - 1) / slicesPerBlock;
+  for (uint64_t blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const uint64_t o0 = blk * slicesPerBlock;
+    const uint32_t ns = (uint32_t)min((uint64_t)slicesPerBlock, outer - o0);
+    const uint32_t count = ns * slice;
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + o0 * slice, count, lds);
+    __syncthreads();
+    for (uint32_t t = threadIdx.x; t < ns * inner; t += kBlock) {
+      const uint32_t o = t / inner, c = t - o * inner;
+      T* col = lds + mis + o * slice + c;
+      A acc = Op::id();
+      for (uint32_t r = 0; r < R; ++r) {
+        acc = Op::op(acc, scan_up<A>(col[r * inner]));
+        col[r * inner] = scan_down<T>(acc);
+      }
+    }
+    __syncthreads();
+    T* dst = out + o0 * slice;
+    const int mo = (int)((reinterpret_cast<uintptr_t>(dst) / sizeof(T)) & (uintptr_t)(VEC - 1));
+    const uint32_t npacks = ((uint32_t)mo + count + VEC - 1) / VEC;
+    for (uint32_t k = threadIdx.x; k < npacks; k += kBlock) {
+      const int first = (int)(k * VEC) - mo;  // run index of the pack's element 0
+      if (first >= 0 && first + VEC <= (int)count) {
+        P v;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v.v[e] = lds[mis + first + e];
+        *reinterpret_cast<P*>(dst + first) = v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+          if (first + e >= 0 && first + e < (int)count) dst[first + e] = lds[mis + first + e];
+      }
+    }
+    __syncthreads();  // the buffer is refilled by the next run
+  }
+}
+
 uint32_t pow2_at_least(uint64_t x) {
   uint32_t p = 1;
   while (p < x && p < 64) p <<= 1;
@@ -259,6 +314,20 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
   constexpr int VECC = (sizeof(typename ScanAcc<T>::type) == 4 || kFull <= 4) ? kFull : 4;  // column kernel
   hipStream_t st = current_stream(s);
   const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
+  // small slices: rows below 2 KiB, or R x inner slices up to 16 KiB
+  const int64_t sliceBytes = R * inner * (int64_t)sizeof(T);
+  if (tuning("scan.slab", 1) && sliceBytes <= (inner == 1 ? 2047 : 16384) && R > 0 && inner > 0) {
+    int64_t chunk = outer * sliceBytes / ((int64_t)num_compute_units(s) * 4);
+    chunk = std::min<int64_t>(32768, std::max<int64_t>(4096, chunk));
+    const int64_t spb = std::max<int64_t>(1, chunk / sliceBytes);
+    const int64_t blocks = (outer + spb - 1) / spb;
+    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)num_compute_units(s) * 64));
+    const size_t lds = (((size_t)(spb * R * inner) + 2 * kFull) * sizeof(T) + 15) & ~size_t(15);
+    hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds, st, out, in,
+                       (uint64_t)outer, (uint32_t)R, (uint32_t)inner, (uint32_t)spb);
+    note_kernel("scan-slab");
+    return;
+  }
   if (inner == 1) {
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
     const int64_t blocks = (outer + (kBlock / 64) - 1) / (kBlock / 64);

@@ -27,7 +27,49 @@ def test_oracle_scan_matches_numpy(oracle, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["float", "half"])
-def test_gpu_scan(thc, oracle, kind):
+def test_gpu_scan_of_small_slices_goes_through_lds(thc, oracle, kind):
+    """Short rows and small R x inner slices are scanned in LDS by a thread per
+    column; input and output runs may sit at different misalignments."""
+    rng = np.random.default_rng(18)
+    dtype = np.float32 if kind == "float" else np.float16
+    for shape, dim in (((5000, 10), 1), ((777, 33), 1), ((300, 8, 16), 1), ((1000, 33, 2), 1), ((41, 7), 0),
+                       ((2, 3, 5, 7), 2), ((3, 500), 1), ((9, 1, 4), 1), ((1, 60, 60), 1)):
+        n = int(np.prod(shape))
+        for off in (0, 1, 3):
+            st = [1] * len(shape)
+            for d in range(len(shape) - 2, -1, -1):
+                st[d] = st[d + 1] * shape[d + 1]
+            x = rng.integers(-4, 5, n + off).astype(dtype)
+            dev = thc.Tensor.from_storage(x, off, shape, tuple(st), kind=kind)
+            got = thc.Tensor(kind).cumsum(dev, dim)
+            assert thc.last_kernel() == "scan-slab", (shape, dim, thc.last_kernel())
+            want = np.cumsum(x[off:].reshape(shape).astype(np.int64), axis=dim).astype(dtype)   # exact: small integers
+            assert_bit_equal(got.numpy(), want, "%s %d off %d" % (shape, dim, off))
+            dev.cumsum(dev, dim)                                         # in place, misaligned output
+            assert_bit_equal(dev.numpy(), want)
+            assert_bit_equal(dev.storage_numpy()[:off], x[:off])       # nothing written before the run
+    thc.set_tuning("scan.slab", 0)
+    try:
+        x = rng.integers(-4, 5, (777, 33)).astype(dtype)
+        got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), 1)
+        assert thc.last_kernel() == "scan-rows"
+        assert_bit_equal(got.numpy(), np.cumsum(x.astype(np.int64), axis=1).astype(dtype))
+    finally:
+        thc.set_tuning("scan.slab", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("slab", [1, 0])
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_gpu_scan(thc, oracle, kind, slab):
+    thc.set_tuning("scan.slab", slab)
+    try:
+        _gpu_scan_cases(thc, oracle, kind)
+    finally:
+        thc.set_tuning("scan.slab", 1)
+
+
+def _gpu_scan_cases(thc, oracle, kind):
     rng = np.random.default_rng(17)
     dtype = np.float32 if kind == "float" else np.float16
     tol = 1e-5 if kind == "float" else 2e-3
