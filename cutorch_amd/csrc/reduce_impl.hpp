@@ -559,6 +559,23 @@ struct SlabArgs {
   Divisor<uint32_t> cdiv; // division by C
   uint32_t slicesPerBlock;
   uint32_t dataElems;     // LDS elements reserved for the staged run
+  // Chunk mode (S > 1), for slices too long for LDS but narrow (few columns):
+  // workgroup b takes rows [s * chunkRows, ...) of slice o, (o, s) = divmod(b, S),
+  // and writes its C partial results densely at out[(o * S + s) * C + c]; the
+  // next level reduces that dense [O][S][C] array over S.
+  I S;
+  uint32_t chunkRows;
+};
+
+// The functor of the later levels of a chunked reduction: partials only combine.
+template <typename F>
+struct FoldOnly {
+  using A = typename F::A;
+  static constexpr bool kCentred = false;
+  F f;
+  __host__ __device__ __forceinline__ A init() const { return f.init(); }
+  __device__ __forceinline__ A modify(A x, A) const { return x; }
+  __device__ __forceinline__ A combine(A a, A b) const { return f.combine(a, b); }
 };
 
 template <typename TIn, typename TOut, typename F, typename I>
@@ -569,19 +586,35 @@ __global__ __launch_bounds__(kBlock) void reduce_slab_kernel(const TIn* __restri
   extern __shared__ __align__(16) unsigned char lds_raw[];
   TIn* lds = reinterpret_cast<TIn*>(lds_raw);
   A* part = reinterpret_cast<A*>(lds_raw + (((size_t)a.dataElems * sizeof(TIn) + 15) & ~size_t(15)));
-  const uint32_t R = (uint32_t)a.R, C = (uint32_t)a.C, slice = R * C;
-  const I numBlocks = (a.O + a.slicesPerBlock - 1) / a.slicesPerBlock;
+  const uint32_t C = (uint32_t)a.C;
+  const bool chunked = a.S > 1;
+  const I numBlocks = chunked ? a.O * a.S : (a.O + a.slicesPerBlock - 1) / a.slicesPerBlock;
   for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
-    const I o0 = blk * a.slicesPerBlock;
-    const uint32_t ns = (uint32_t)min((I)a.slicesPerBlock, a.O - o0);
-    const uint32_t mis = stage_rows_to_lds<TIn, 8>(in + o0 * (I)slice, ns * slice, lds);
+    I o0 = blk * a.slicesPerBlock;
+    uint32_t ns = 1, R = (uint32_t)a.R;
+    const TIn* runStart = nullptr;
+    if (chunked) {
+      o0 = blk / a.S;
+      const I r0 = (blk - o0 * a.S) * a.chunkRows;
+      R = (uint32_t)min((I)a.chunkRows, a.R - r0);
+      runStart = in + (o0 * a.R + r0) * a.C;
+    } else {
+      ns = (uint32_t)min((I)a.slicesPerBlock, a.O - o0);
+      runStart = in + o0 * a.R * a.C;
+    }
+    const uint32_t slice = R * C;
+    const uint32_t mis = stage_rows_to_lds<TIn, 8>(runStart, ns * slice, lds);
     __syncthreads();
     const uint32_t nOut = ns * C;
     const uint32_t P = nOut >= kBlock ? 1u : min(R, kBlock / nOut);  // uniform over the workgroup
     auto reduce_one = [&](uint32_t o, uint32_t c, uint32_t first, uint32_t step, I& outOff) {
-      I inOff;
-      a.oa.offsets(o0 + o, inOff, outOff);
-      outOff += (I)c * a.outInner;
+      if (chunked) {
+        outOff = blk * a.C + c;
+      } else {
+        I inOff;
+        a.oa.offsets(o0 + o, inOff, outOff);
+        outOff += (I)c * a.outInner;
+      }
       A ctr = (A)0;
       if constexpr (F::kCentred) ctr = acc_up<A>(out[outOff]);
       const TIn* col = lds + mis + o * slice + c;
@@ -1572,6 +1605,98 @@ size_t slab_data_bytes(const SlabArgs<I>& a) {
   return ((size_t)a.dataElems * sizeof(T) + 15) & ~size_t(15);
 }
 
+// Long narrow slices ([O][R][C] dense, a row of C elements shorter than a
+// couple of cache lines, R too long for LDS): the column kernels read such
+// rows with most lanes idle when the rows are not 16-byte aligned and the
+// reduced dim must be split (2.1 TB/s on 8M x 10). Instead every 32 KiB run
+// of rows is reduced by the slab kernel in chunk mode into a dense
+// [O][S][C] array of partials, which is reduced the same way until a level
+// fits whole slices; two halves of the scratch buffer alternate.
+template <typename TIn, typename TOut, typename F, typename I>
+void launch_slab_level(THCState* s, const TIn* in, TOut* out, SlabArgs<I> a, int64_t blocks,
+                       Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  const size_t lds = (((size_t)a.dataElems * sizeof(TIn) + 15) & ~size_t(15)) + kBlock * sizeof(A);
+  const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+  hipLaunchKernelGGL((reduce_slab_kernel<TIn, TOut, F, I>), dim3(grid), dim3(kBlock), lds,
+                     current_stream(s), in, out, a, epi, f);
+}
+
+template <typename T, typename F, typename I>
+bool run_slab_chunked(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi, F f) {
+  using A = typename F::A;
+  const int nd = g.in.dims;
+  if (F::kCentred || !tuning("reduce.slab.chunked", 1) || nd < 1) return false;
+  const int64_t C = g.in.size[nd - 1];
+  if (g.in.stride[nd - 1] != 1 || g.sR != C) return false;
+  if (C * (int64_t)sizeof(T) > tuning("reduce.slab.chunked_max_row_bytes", 512)) return false;
+  int64_t run = g.R * C;
+  for (int d = nd - 2; d >= 0; --d) {
+    if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
+    run *= g.in.size[d];
+  }
+  const int64_t O = g.outElems / C;
+  // Where the column kernel reads aligned packs, or has a workgroup's worth of
+  // slices per CU without splitting the reduced dim, it is the faster one
+  // (6.3-6.8 against 5.8-6.0 TB/s on 16..64-column fp32 slices, 6.1 against
+  // 3.9 on 4096 slices of 4096 x 3).
+  constexpr int64_t VEC = 16 / sizeof(T);
+  if (aligned16(in) && C % VEC == 0) return false;
+  if (O >= (int64_t)num_compute_units(s)) return false;
+  // bytes staged per workgroup (tunable so that tests reach many levels)
+  const int64_t kRun = std::min<int64_t>(32768, std::max<int64_t>(256, tuning("reduce.slab.run_bytes", 32768)));
+  const int64_t rows1 = std::max<int64_t>(1, kRun / (C * (int64_t)sizeof(T)));
+  const int64_t S1 = (g.R + rows1 - 1) / rows1;
+  if (S1 < 2) return false;
+  size_t scratchBytes = 0;
+  char* scratch = (char*)scratch_space(s, &scratchBytes);
+  const size_t half = (scratchBytes / 2) & ~size_t(255);
+  if ((size_t)(O * S1 * C) * sizeof(A) > half) return false;
+  A* buf[2] = {(A*)scratch, (A*)(scratch + half)};
+
+  auto level_args = [&](int64_t R, int64_t rows, int64_t S, size_t elemBytes) {
+    SlabArgs<I> a{};
+    a.O = (I)O;
+    a.R = (I)R;
+    a.C = (I)C;
+    a.cdiv.set((uint64_t)C);
+    a.slicesPerBlock = 1;
+    a.S = (I)S;
+    a.chunkRows = (uint32_t)rows;
+    a.dataElems = (uint32_t)(rows * C + 2 * (16 / elemBytes));
+    return a;
+  };
+  const Epi<A> none{(int)Epilogue::None, (A)0};
+  launch_slab_level<T, A, F, I>(s, in, buf[0], level_args(g.R, rows1, S1, sizeof(T)), O * S1, none, f);
+  const FoldOnly<F> fold{f};
+  int64_t R = S1;
+  int cur = 0;
+  const int64_t rowsA = std::max<int64_t>(1, kRun / (C * (int64_t)sizeof(A)));
+  while (R > rowsA) {
+    const int64_t S = (R + rowsA - 1) / rowsA;
+    launch_slab_level<A, A, FoldOnly<F>, I>(s, buf[cur], buf[cur ^ 1], level_args(R, rowsA, S, sizeof(A)), O * S,
+                                            none, fold);
+    R = S;
+    cur ^= 1;
+  }
+  // last level: whole slices of R x C partials, results to the real output
+  SlabArgs<I> a{};
+  const int64_t sliceBytes = R * C * (int64_t)sizeof(A);
+  int64_t chunk = std::min<int64_t>(kRun, std::max<int64_t>(4096, O * sliceBytes / ((int64_t)num_compute_units(s) * 4)));
+  const int64_t spb = std::max<int64_t>(1, chunk / sliceBytes);
+  a.oa = make_outer<I>(g.in, g.out, nd - 1);
+  a.O = (I)O;
+  a.R = (I)R;
+  a.C = (I)C;
+  a.outInner = (I)g.out.stride[nd - 1];
+  a.cdiv.set((uint64_t)C);
+  a.slicesPerBlock = (uint32_t)spb;
+  a.dataElems = (uint32_t)(spb * R * C + 2 * (16 / sizeof(A)));
+  launch_slab_level<A, T, FoldOnly<F>, I>(s, buf[cur], out, a, (O + spb - 1) / spb, epi, fold);
+  note_kernel("slab-chunked");
+  return true;
+}
+
 template <typename T, typename F, typename I>
 void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typename F::A> epi, F f) {
   using A = typename F::A;
@@ -1587,6 +1712,7 @@ void run_cols(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typenam
       return;
     }
   }
+  if (run_slab_chunked<T, F, I>(s, g, in, out, epi, f)) return;
   ColsPlan<I> p = plan_cols<T, I>(s, g, in, sizeof(A));
   const bool split = p.a.S.d > 1;
   A* scratch = split ? (A*)scratch_space(s, nullptr) : nullptr;

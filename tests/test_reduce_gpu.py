@@ -512,3 +512,46 @@ def test_small_dense_slices_special_cases(thc, oracle):
     out = thc.Tensor("float").var(thc.Tensor.from_numpy(z), 1)
     assert thc.last_kernel() == "slab"
     np.testing.assert_allclose(out.numpy()[:, 0, :], z.astype(np.float64).var(axis=1, ddof=1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_long_narrow_slices_reduce_in_chunks(thc, oracle, kind):
+    """Few slices, each long and only a few (misaligned) columns wide: 32 KiB
+    runs of rows are reduced to dense partials level by level (also with tiny
+    runs, which takes four levels); ragged last chunks; the sum family."""
+    rng = np.random.default_rng(58)
+    dtype = np.float32 if kind == "float" else np.float16
+    x = ((rng.integers(0, 40, (100003, 3)) == 0) * rng.integers(-2, 3, (100003, 3))).astype(dtype)  # fits half
+    thc.set_tuning("reduce.slab.run_bytes", 512)
+    try:
+        out = thc.Tensor(kind).norm(thc.Tensor.from_numpy(x), 1, 0)
+        assert thc.last_kernel() == "slab-chunked"
+    finally:
+        thc.set_tuning("reduce.slab.run_bytes", 32768)
+    want = np.abs(x.astype(np.int64)).sum(axis=0, keepdims=True)
+    if kind == "float":
+        assert_bit_equal(out.numpy(), want.astype(dtype))
+    else:
+        np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=2e-3)
+    for shape, dim in (((700001, 3), 0), ((3, 50001, 7), 1), ((120000, 10), 0), ((2, 9000, 33), 1)):
+        x = ((rng.integers(0, 40, shape) == 0) * rng.integers(-2, 3, shape)).astype(dtype)   # sums fit half
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        for name in ("sum", "norm1", "norm2", "mean"):
+            k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
+            assert k == "slab-chunked", (shape, name, k)
+        out = thc.Tensor(kind).sum(dev, dim)                       # exact: small integers
+        want = x.astype(np.int64).sum(axis=dim, keepdims=True)
+        if np.abs(want).max() < (2048 if kind == "half" else 1 << 24):
+            assert_bit_equal(out.numpy(), want.astype(dtype))
+    # max / min without indices ride the same engine
+    x = rng.standard_normal((90000, 5)).astype(np.float32)
+    x[77777, 2] = np.nan
+    vals, idx = thc.Tensor("float"), thc.Tensor("long")
+    vals.max(idx, thc.Tensor.from_numpy(x), 0)                     # the indexed form keeps its own kernel
+    assert thc.last_kernel().startswith("cols-index")
+    assert np.isnan(vals.numpy()[0, 2]) and idx.numpy()[0, 2] == 77778
+    # aligned packs, or many slices: the column kernels stay
+    dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((3, 50000, 8)), kind, "ints")
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
+    dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((300, 5000, 3)), kind, "ints")
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
