@@ -251,35 +251,65 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
 // at 0.5). Here a workgroup streams a run of whole slices into LDS, a thread
 // per (slice, column) scans its R elements in place, and the run goes back
 // out as aligned packs of the OUTPUT's alignment (edge packs element-wise).
+// Chunk mode (S > 1) serves long scans with too few columns to occupy the
+// chip: workgroup b takes rows [s * chunkRows, ...) of slice o, (o, s) =
+// divmod(b, S), and starts every column from carryIn[(o * S + s - 1) * inner + c]
+// (the inclusive scan of the chunk totals; the identity for s == 0).
 template <typename T, typename Op>
 __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
-                                                           uint64_t outer, uint32_t R,
-                                                           uint32_t inner, uint32_t slicesPerBlock) {
+                                                           const typename ScanAcc<T>::type* __restrict__ carryIn,
+                                                           uint64_t outer, uint64_t R, uint32_t inner,
+                                                           uint32_t slicesPerBlock, uint64_t S,
+                                                           uint32_t chunkRows) {
   constexpr int VEC = 16 / sizeof(T);
   using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
-  const uint32_t slice = R * inner;
-  const uint64_t numBlocks = (outer + slicesPerBlock - 1) / slicesPerBlock;
+  const bool chunked = S > 1;
+  const uint64_t numBlocks = chunked ? outer * S : (outer + slicesPerBlock - 1) / slicesPerBlock;
   for (uint64_t blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
-    const uint64_t o0 = blk * slicesPerBlock;
-    const uint32_t ns = (uint32_t)min((uint64_t)slicesPerBlock, outer - o0);
-    const uint32_t count = ns * slice;
-    const uint32_t mis = stage_rows_to_lds<T, 8>(in + o0 * slice, count, lds);
+    uint64_t start;  // element offset of the run in the dense block
+    uint32_t ns = 1, rows = (uint32_t)R;
+    if (chunked) {
+      const uint64_t o = blk / S, r0 = (blk - o * S) * chunkRows;
+      rows = (uint32_t)min((uint64_t)chunkRows, R - r0);
+      start = (o * R + r0) * inner;
+    } else {
+      const uint64_t o0 = blk * slicesPerBlock;
+      ns = (uint32_t)min((uint64_t)slicesPerBlock, outer - o0);
+      start = o0 * R * inner;
+    }
+    const uint32_t slice = rows * inner, count = ns * slice;
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + start, count, lds);
     __syncthreads();
     for (uint32_t t = threadIdx.x; t < ns * inner; t += kBlock) {
       const uint32_t o = t / inner, c = t - o * inner;
       T* col = lds + mis + o * slice + c;
       A acc = Op::id();
-      for (uint32_t r = 0; r < R; ++r) {
+      if (chunked && blk % S != 0) acc = carryIn[(blk - 1) * inner + c];
+      // batches of 8 rows: the loads of a batch are independent of its stores,
+      // so one LDS round trip is paid per batch instead of per element
+      constexpr uint32_t B = 8;
+      uint32_t r = 0;
+      for (; r + B <= rows; r += B) {
+        T x[B];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) {
+          acc = Op::op(acc, scan_up<A>(x[u]));
+          col[(r + u) * inner] = scan_down<T>(acc);
+        }
+      }
+      for (; r < rows; ++r) {
         acc = Op::op(acc, scan_up<A>(col[r * inner]));
         col[r * inner] = scan_down<T>(acc);
       }
     }
     __syncthreads();
-    T* dst = out + o0 * slice;
+    T* dst = out + start;
     const int mo = (int)((reinterpret_cast<uintptr_t>(dst) / sizeof(T)) & (uintptr_t)(VEC - 1));
     const uint32_t npacks = ((uint32_t)mo + count + VEC - 1) / VEC;
     for (uint32_t k = threadIdx.x; k < npacks; k += kBlock) {
@@ -299,14 +329,60 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
   }
 }
 
+// Totals of every chunk of rows, per column: totals[(o * S + s) * inner + c].
+// P threads share a column (thread p takes rows p, p + P, ...) when the
+// columns are fewer than the threads; their partials meet in LDS.
+template <typename T, typename Op>
+__global__ __launch_bounds__(kBlock) void scan_chunk_totals_kernel(
+    typename ScanAcc<T>::type* __restrict__ totals, const T* __restrict__ in, uint64_t outer, uint64_t R,
+    uint32_t inner, uint64_t S, uint32_t chunkRows, uint32_t dataElems) {
+  using A = typename ScanAcc<T>::type;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  A* part = reinterpret_cast<A*>(lds_raw + (((size_t)dataElems * sizeof(T) + 15) & ~size_t(15)));
+  for (uint64_t blk = blockIdx.x; blk < outer * S; blk += gridDim.x) {
+    const uint64_t o = blk / S, r0 = (blk - o * S) * chunkRows;
+    const uint32_t rows = (uint32_t)min((uint64_t)chunkRows, R - r0);
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + (o * R + r0) * inner, rows * inner, lds);
+    __syncthreads();
+    const uint32_t P = inner >= kBlock ? 1u : min(rows, kBlock / inner);
+    if (P == 1) {
+      for (uint32_t c = threadIdx.x; c < inner; c += kBlock) {
+        A acc = Op::id();
+        for (uint32_t r = 0; r < rows; ++r) acc = Op::op(acc, scan_up<A>(lds[mis + r * inner + c]));
+        totals[blk * inner + c] = acc;
+      }
+    } else {
+      const uint32_t p = threadIdx.x / inner, c = threadIdx.x - p * inner;
+      if (p < P) {
+        // a contiguous band of rows per thread keeps the combine order that of the scan
+        const uint32_t band = (rows + P - 1) / P, rb = p * band, re = min(rows, rb + band);
+        A acc = Op::id();
+        for (uint32_t r = rb; r < re; ++r) acc = Op::op(acc, scan_up<A>(lds[mis + r * inner + c]));
+        part[p * inner + c] = acc;
+      }
+      __syncthreads();
+      if (p == 0) {
+        A acc = part[c];
+        for (uint32_t q = 1; q < P; ++q) acc = Op::op(acc, part[q * inner + c]);
+        totals[blk * inner + c] = acc;
+      }
+    }
+    __syncthreads();
+  }
+}
+
 uint32_t pow2_at_least(uint64_t x) {
   uint32_t p = 1;
   while (p < x && p < 64) p <<= 1;
   return p;
 }
 
+// `scratch` is device memory this level (and the levels below it, for the
+// chunk totals of long scans) may use; nullptr = the stream's scratch buffer.
 template <typename T, typename Op>
-void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int64_t inner) {
+void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int64_t inner,
+                 char* scratch = nullptr, size_t scratchBytes = 0) {
   // Packs are capped so that a lane's segment stays in registers when the
   // accumulator (8 bytes for the integer types) is wider than the element.
   constexpr int kFull = 16 / sizeof(T);
@@ -323,10 +399,42 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t blocks = (outer + spb - 1) / spb;
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)num_compute_units(s) * 64));
     const size_t lds = (((size_t)(spb * R * inner) + 2 * kFull) * sizeof(T) + 15) & ~size_t(15);
-    hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds, st, out, in,
-                       (uint64_t)outer, (uint32_t)R, (uint32_t)inner, (uint32_t)spb);
+    hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds, st, out, in, nullptr,
+                       (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint32_t)spb, (uint64_t)1, 0u);
     note_kernel("scan-slab");
     return;
+  }
+  // Long scans that give the row / column kernels fewer workgroups than CUs
+  // (an 8M x 10 matrix scanned along dim 0 is ONE workgroup there: 6 GB/s):
+  // totals of 32 KiB chunks of rows, their scan (this function again, on the
+  // accumulator type), then every chunk scans from its carry. The input is
+  // read twice, which still is 500x faster.
+  {
+    using A = typename ScanAcc<T>::type;
+    const int64_t rowBytes = inner * (int64_t)sizeof(T);
+    const int64_t run = std::min<int64_t>(32768, std::max<int64_t>(256, tuning("scan.chunk_bytes", 32768)));
+    const int64_t chunkRows = std::max<int64_t>(1, run / rowBytes);
+    const int64_t S = (R + chunkRows - 1) / chunkRows;
+    const int64_t packsPerRow = (inner + kFull - 1) / kFull;
+    const int64_t plainBlocks = inner == 1 ? (outer + 3) / 4 : outer * ((packsPerRow + 15) / 16);
+    if (!scratch) scratch = (char*)scratch_space(s, &scratchBytes);
+    const size_t need = (((size_t)(outer * S * inner) * sizeof(A)) + 255) & ~size_t(255);
+    if (tuning("scan.chunked", 1) && rowBytes <= 32768 && S >= 4 && plainBlocks < (int64_t)num_compute_units(s) &&
+        2 * need <= scratchBytes) {
+      A* totals = (A*)scratch;
+      A* carries = (A*)(scratch + need);
+      const uint32_t dataElems = (uint32_t)(chunkRows * inner + 2 * kFull);
+      const size_t ldsData = ((size_t)dataElems * sizeof(T) + 15) & ~size_t(15);
+      const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * S, (int64_t)num_compute_units(s) * 64));
+      hipLaunchKernelGGL((scan_chunk_totals_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsData + kBlock * sizeof(A),
+                         st, totals, in, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint64_t)S,
+                         (uint32_t)chunkRows, dataElems);
+      launch_scan<A, Op>(s, carries, totals, outer, S, inner, scratch + 2 * need, scratchBytes - 2 * need);
+      hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsData, st, out, in, carries,
+                         (uint64_t)outer, (uint64_t)R, (uint32_t)inner, 1u, (uint64_t)S, (uint32_t)chunkRows);
+      note_kernel("scan-chunked");
+      return;
+    }
   }
   if (inner == 1) {
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
