@@ -182,7 +182,8 @@ def build_configs(thc, hip, which, only=None):
     # Neighbours of the hot path on the same engines (same operands where possible).
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
-                      "N-double-sum", "N-renorm")
+                      "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
+                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -226,6 +227,36 @@ def build_configs(thc, hip, which, only=None):
                                  lambda i: dout.sum(dsrc, 1)),
                 "N-renorm": ("renorm(p=2, dim 0, maxnorm 1) of 8192x8192 fp32 (read + write counted once)",
                              8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.renorm(sq, 2.0, 0, 1.0)),
+            })
+        if set(nx) & {"N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall", "N-cumsum-rows10",
+                      "N-cumsum-tall", "N-add-t-odd"}:
+            # shapes off the aligned grid: short / misaligned rows, small slices, tall narrow matrices
+            nr = 1 << 26
+            flat = e_src
+            v33 = flat.view_as_strided(0, ((nr // 33), 33), (33, 1))
+            v10 = flat.view_as_strided(0, ((nr // 10), 10), (10, 1))
+            vslab = flat.view_as_strided(0, (nr // 128, 8, 16), (128, 16, 1))
+            o33, i33 = T("float").resize((nr // 33, 1)), T("long").resize((nr // 33, 1))
+            otall, oslab = T("float").resize((1, 10)), T("float").resize((nr // 128, 1, 16))
+            s10 = T("float").resize((nr // 10, 10))
+            oddT = T.from_numpy(rng.standard_normal((8193, 8191), dtype=np.float32)).t()
+            oddB = T.from_numpy(rng.standard_normal((8191, 8193), dtype=np.float32))
+            oddO = T("float").resize((8191, 8193))
+            n33, n10, nodd = (nr // 33) * 33, (nr // 10) * 10, 8191 * 8193
+            table.update({
+                "N-sum-rows33": ("sum over last dim of 2033601x33 fp32 (misaligned short rows)", 4 * n33 + 4 * (nr // 33),
+                                 n33, lambda i: o33.sum(v33, 1)),
+                "N-max-rows33": ("max+argmax over last dim of 2033601x33 fp32", 4 * n33 + 12 * (nr // 33), n33,
+                                 lambda i: o33.max(i33, v33, 1)),
+                "N-sum-slab": ("sum over middle dim of 524288x8x16 fp32 (512-byte slices)", 4 * nr + 4 * (nr // 8), nr,
+                               lambda i: oslab.sum(vslab, 1)),
+                "N-sum-tall": ("sum over dim 0 of 6710886x10 fp32 (tall, 40-byte rows)", 4 * n10, n10,
+                               lambda i: otall.sum(v10, 0)),
+                "N-cumsum-rows10": ("cumsum over last dim of 6710886x10 fp32", 8 * n10, n10, lambda i: s10.cumsum(v10, 1)),
+                "N-cumsum-tall": ("cumsum over dim 0 of 6710886x10 fp32 (input read twice, counted once)", 8 * n10, n10,
+                                  lambda i: s10.cumsum(v10, 0)),
+                "N-add-t-odd": ("c = a:t() + b, 8191x8193 fp32 (no 16-byte aligned rows)", 12 * nodd, nodd,
+                                lambda i: oddO.cadd(oddT, 1.0, oddB)),
             })
         if "N-fill" in nx and xa.numel() != big:
             table["N-fill"] = ("fill of 2^26 fp32", 4 * ne, ne, lambda i: e_dst.fill(0.5))
