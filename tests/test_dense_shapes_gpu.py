@@ -1,0 +1,78 @@
+"""Dense tensors of many shapes through every reduction / scan kernel family.
+
+Which kernel serves a dense reduction depends on the lengths around the
+reduced dim (short rows, small slices, tall narrow slices, aligned or not), so
+this sweep draws shapes from a grid of awkward lengths and checks sum, max
+(+index), min (+index), mean and cumsum against numpy on small-integer data,
+where every partial sum is exact in the element type: results must match bit
+for bit whatever order the kernel adds in."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [1, 2, 3, 4, 5, 7, 8, 10, 15, 16, 17, 31, 33, 64, 100, 127, 128, 130, 250, 257, 511, 1000, 1025, 4099]
+SEEN = set()      # kernel families the sweep reached
+DTYPES = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64, "byte": np.uint8,
+          "long": np.int64}
+
+
+def draw_shape(rng, budget=300000):
+    nd = int(rng.integers(1, 4))
+    while True:
+        shape = tuple(int(rng.choice(LENGTHS)) for _ in range(nd))
+        if np.prod(shape) <= budget:
+            return shape
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_dense_shapes_against_numpy(thc, seed):
+    rng = np.random.default_rng(9000 + seed)
+    kind = ["float", "half", "int", "double", "byte", "long"][seed % 6]
+    dtype = DTYPES[kind]
+    shape = draw_shape(rng)
+    if seed % 7 == 0:                      # one long dim next to short ones
+        shape = (int(rng.choice([40000, 70001, 131072])),) + tuple(int(rng.choice([1, 3, 10, 16])) for _ in range(1))
+        if seed % 14 == 0:
+            shape = shape[::-1]
+    n = int(np.prod(shape))
+    # sparse small values: |running sums| stay below 2048 (exact in half) and 255 (byte)
+    dense = rng.integers(0, 3, shape) if kind == "byte" else rng.integers(-2, 3, shape)
+    keep = rng.random(shape) < min(1.0, (100.0 if kind == "byte" else 800.0) / max(shape))
+    x = (dense * keep).astype(dtype)
+    off = int(rng.integers(0, 4))
+    storage = np.zeros(n + off, dtype)
+    storage[off:] = x.reshape(-1)
+    strides = [1] * len(shape)
+    for d in range(len(shape) - 2, -1, -1):
+        strides[d] = strides[d + 1] * shape[d + 1]
+    dev = thc.Tensor.from_storage(storage, off, shape, tuple(strides), kind=kind)
+    wide = x.astype(np.int64)
+    for dim in range(len(shape)):
+        what = "%s %s dim %d off %d" % (kind, shape, dim, off)
+        out = thc.Tensor(kind).sum(dev, dim)
+        k = thc.last_kernel()
+        SEEN.add(k)
+        assert_bit_equal(out.numpy(), wide.sum(axis=dim, keepdims=True).astype(dtype), what + " sum " + k)
+        for which, arg, red in (("max", np.argmax, np.max), ("min", np.argmin, np.min)):
+            vals, idx = thc.Tensor(kind), thc.Tensor("long")
+            getattr(vals, which)(idx, dev, dim)
+            k = thc.last_kernel()
+            SEEN.add(k)
+            assert_bit_equal(vals.numpy(), red(x, axis=dim, keepdims=True), what + " " + which + " " + k)
+            assert np.array_equal(idx.numpy(), np.expand_dims(arg(x, axis=dim), dim) + 1), what + " arg" + which + " " + k
+        out = thc.Tensor(kind).cumsum(dev, dim)
+        k = thc.last_kernel()
+        SEEN.add(k)
+        assert_bit_equal(out.numpy(), np.cumsum(wide, axis=dim).astype(dtype), what + " cumsum " + k)
+    assert_bit_equal(dev.storage_numpy(), storage)      # inputs untouched
+
+
+def test_dense_shape_sweep_reached_every_kernel_family():
+    if len(SEEN) == 0:
+        pytest.skip("the sweep did not run in this process")
+    want = {"rows", "rows-lds", "rows-index-lds", "slab", "slab-index", "slab-chunked", "cols", "cols-index",
+            "scan-slab", "scan-chunked", "scan-rows", "scan-cols"}
+    assert want <= SEEN, sorted(want - SEEN)
