@@ -76,3 +76,25 @@ def test_dense_shape_sweep_reached_every_kernel_family():
     want = {"rows", "rows-lds", "rows-index-lds", "slab", "slab-index", "slab-chunked", "cols", "cols-index",
             "scan-slab", "scan-chunked", "scan-rows", "scan-cols"}
     assert want <= SEEN, sorted(want - SEEN)
+
+
+@pytest.mark.parametrize("kind", ["byte", "char", "short", "half", "int", "float", "long", "double"])
+def test_transposed_copies_of_every_element_size_at_odd_shapes(thc, kind):
+    """out:copy(a:t()) for 1-, 2-, 4- and 8-byte elements on shapes that leave no
+    row 16-byte aligned (the shifted-window tiles) and with both tensors 1..3
+    elements into their storages; the whole output storage is compared."""
+    rng = np.random.default_rng(9100)
+    dtype = {"char": np.int8, "short": np.int16}.get(kind) or DTYPES[kind]
+    for rows, cols in ((61, 125), (333, 515), (130, 1001), (17, 9), (250, 64)):
+        for off_in, off_out in ((0, 0), (1, 3), (2, 1)):
+            n = rows * cols
+            src = rng.integers(0, 100, n + off_in).astype(dtype)
+            dst = np.full(n + off_out, 7, dtype)
+            a = thc.Tensor.from_storage(src, off_in, (rows, cols), (1, rows), kind=kind)     # a = b:t()
+            out = thc.Tensor.from_storage(dst, off_out, (rows, cols), (cols, 1), kind=kind)
+            out.copy(a)
+            k = thc.last_kernel()
+            assert k.startswith("tiled"), (kind, rows, cols, k)
+            want = dst.copy()
+            want[off_out:] = src[off_in:].reshape(cols, rows).T.reshape(-1)
+            assert_bit_equal(out.storage_numpy(), want, "%s %dx%d +%d/+%d %s" % (kind, rows, cols, off_in, off_out, k))
