@@ -208,7 +208,7 @@ def build_configs(thc, hip, which, only=None):
                               lambda i: s3.cumsum(x3, 1)),
             "N-cumsum-cols": ("cumsum over middle dim of 64x4096x512 fp32", 8 * n4, n4, lambda i: s4o.cumsum(d4, 1)),
             "N-dist": ("dist(a, b, 2) over 2^26 fp32", 8 * ne, ne, lambda i: e_src.dist(e_dst, 2.0)),
-            "N-varall": ("varall over 2^26 fp32 (input counted once)", 4 * ne, ne, lambda i: e_src.varall()),
+            "N-varall": ("varall over 2^26 fp32 (one read, blocks on the scalar)", 4 * ne, ne, lambda i: e_src.varall()),
         }
         if set(nx) & {"N-int-add", "N-lt-byte", "N-cvt-half", "N-double-sum", "N-renorm"}:
             ia = T.from_numpy(rng.integers(-1000, 1000, ne).astype(np.int32))

@@ -296,6 +296,10 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Sca
 // The same reduction over a - b without materialising the difference. Only
 // for dense operands of a floating type; returns false when it does not apply
 // (the caller then subtracts into a temporary).
+// Sum of squared deviations from the mean over all elements of a contiguous
+// float-typed tensor, in one read; false if the tensor is not one dense run
+// (the caller then takes two sweeps).
+bool reduce_all_moments(THCState* s, DType dt, AnyTensor* in, Scalar* result);
 bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a, AnyTensor* b,
                      Scalar* result);
 

@@ -174,6 +174,11 @@ void var_dim(THCState* s, DType dt, bool wantStd, AnyTensor* self, AnyTensor* sr
 float var_all(THCState* s, DType dt, AnyTensor* self, int biased) {
   THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");
   const float n = (float)tensor_numel(self);
+  // one read when the tensor is a dense run (Welford + pairwise merges), else
+  // the reference's two sweeps: mean, then the squared deviations from it
+  Scalar m2{0.0, 0};
+  same_gpu(s, {self});
+  if (reduce_all_moments(s, dt, self, &m2)) return (float)m2.f / (n - (biased ? 0.f : 1.f));
   const float mean = all_or_throw(s, dt, ReduceOp::Sum, 0.f, self) / n;
   return all_or_throw(s, dt, ReduceOp::SqDev, mean, self) / (n - (biased ? 0.f : 1.f));
 }
@@ -551,6 +556,9 @@ double norm_all_d(THCState* s, AnyTensor* self, double p) {
 double var_all_d(THCState* s, AnyTensor* self, int biased) {
   THC_ARG_CHECK(self->nDimension > 0, 1, "empty Tensor");
   const double n = (double)tensor_numel(self);
+  Scalar m2{0.0, 0};
+  same_gpu(s, {self});
+  if (reduce_all_moments(s, DType::F64, self, &m2)) return m2.f / (n - (biased ? 0.0 : 1.0));
   const double mean = all_scalar(s, DType::F64, ReduceOp::Sum, 0.0, self).f / n;
   return all_scalar(s, DType::F64, ReduceOp::SqDev, mean, self).f / (n - (biased ? 0.0 : 1.0));
 }

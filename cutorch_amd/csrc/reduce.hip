@@ -222,6 +222,18 @@ bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a,
   return true;
 }
 
+bool reduce_all_moments(THCState* s, DType dt, AnyTensor* in, Scalar* result) {
+  if (!dtype_is_float(dt) || in->nDimension == 0 || in->nDimension > kMaxDims) return false;
+  if (!tensor_is_contiguous(in) || !tuning("reduce.all.moments", 1)) return false;
+  const int64_t n = tensor_numel(in);
+  if (n < 1) return false;
+  const void* p = tensor_data(in, dt);
+  if (dt == DType::F32) reduce_all_moments_type<float>(s, n, p, result);
+  else if (dt == DType::F16) reduce_all_moments_type<__half>(s, n, p, result);
+  else reduce_all_moments_type<double>(s, n, p, result);
+  return true;
+}
+
 bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, float* result) {
   Scalar r{0.0, 0};
   const bool ok = reduce_all(s, dt, op, (double)p, in, &r);

@@ -1256,6 +1256,98 @@ __global__ __launch_bounds__(kBlock) void reduce_all_kernel(const TIn* __restric
   }
 }
 
+// Sum of squared deviations from the mean of a dense run in ONE read (varall /
+// stdall): every lane runs Welford's update per pack slot over its share, and
+// (count, mean, M2) triples merge pairwise (Chan et al.) across slots, lanes,
+// waves and, in the second launch, workgroups. partial[3 * b + {0, 1, 2}].
+template <typename A>
+__device__ __forceinline__ void moments_wave_merge(A& n, A& mean, A& m2) {
+  for (uint32_t o = 32; o > 0; o >>= 1) {
+    const A nb = shfl_xor_any(n, o), mb = shfl_xor_any(mean, o), sb = shfl_xor_any(m2, o);
+    moments_merge(n, mean, m2, nb, mb, sb);
+  }
+}
+template <typename A>
+__device__ __forceinline__ void moments_block_merge(A& n, A& mean, A& m2, A (*red)[3]) {
+  moments_wave_merge(n, mean, m2);
+  const uint32_t w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    red[w][0] = n;
+    red[w][1] = mean;
+    red[w][2] = m2;
+  }
+  __syncthreads();
+  n = red[0][0];
+  mean = red[0][1];
+  m2 = red[0][2];
+  for (uint32_t k = 1; k < kBlock / 64; ++k) moments_merge(n, mean, m2, red[k][0], red[k][1], red[k][2]);
+}
+
+template <typename TIn, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void moments_all_kernel(const TIn* __restrict__ in, I n, I chunk,
+                                                             typename Acc<TIn>::type* __restrict__ partial) {
+  using P = Pack<TIn, VEC>;
+  using A = typename Acc<TIn>::type;
+  __shared__ A red[kBlock / 64][3];
+  A cnt = (A)0, mean[VEC], m2[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    mean[e] = (A)0;
+    m2[e] = (A)0;
+  }
+  const I nv = n - n % VEC;
+  const I begin = (I)blockIdx.x * chunk;
+  const I end = min(nv, begin + chunk);
+  constexpr int U = 8;
+  constexpr I step = (I)kBlock * VEC;
+  auto update = [&](const P& v) {
+    cnt += (A)1;
+    const A inv = (A)1 / cnt;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const A x = acc_up<A>(v.v[e]);
+      const A delta = x - mean[e];
+      mean[e] += delta * inv;
+      m2[e] += delta * (x - mean[e]);
+    }
+  };
+  I i = begin + threadIdx.x * VEC;
+  for (; i + (U - 1) * step < end; i += U * step) {
+    P v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const P*>(in + i + u * step));
+#pragma unroll
+    for (int u = 0; u < U; ++u) update(v[u]);
+  }
+  for (; i < end; i += step) update(load_pack<true>(reinterpret_cast<const P*>(in + i)));
+  // the pack slots of a lane have seen `cnt` elements each
+  A nn = cnt, mm = mean[0], ss = m2[0];
+#pragma unroll
+  for (int e = 1; e < VEC; ++e) moments_merge(nn, mm, ss, cnt, mean[e], m2[e]);
+  if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n)  // the last n % VEC elements
+    moments_merge(nn, mm, ss, (A)1, acc_up<A>(in[nv + threadIdx.x]), (A)0);
+  moments_block_merge(nn, mm, ss, red);
+  if (threadIdx.x == 0) {
+    partial[3 * blockIdx.x] = nn;
+    partial[3 * blockIdx.x + 1] = mm;
+    partial[3 * blockIdx.x + 2] = ss;
+  }
+}
+
+template <typename A>
+__global__ __launch_bounds__(kBlock) void moments_fold_kernel(const A* __restrict__ partial, uint32_t blocks,
+                                                              A* result, A* hostResult) {
+  __shared__ A red[kBlock / 64][3];
+  A n = (A)0, mean = (A)0, m2 = (A)0;
+  for (uint32_t b = threadIdx.x; b < blocks; b += kBlock)
+    moments_merge(n, mean, m2, partial[3 * b], partial[3 * b + 1], partial[3 * b + 2]);
+  moments_block_merge(n, mean, m2, red);
+  if (threadIdx.x == 0) {
+    *result = m2;
+    *hostResult = m2;
+  }
+}
+
 // Whole-tensor reduction of the element-wise difference of two dense runs
 // (dist: sum |a - b|^p without materialising a - b). Partials are folded by
 // reduce_all_kernel.
@@ -2103,6 +2195,49 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, const void* src
   result->i = (int64_t)r;
 }
 }  // namespace
+
+// Sum of squared deviations from the mean over a dense run of n elements, one
+// read of the input. Blocks until the scalar is on the host, like the others.
+template <typename T>
+void reduce_all_moments_type(THCState* s, int64_t n, const void* src, Scalar* result) {
+  using A = typename Acc<T>::type;
+  if constexpr (std::is_integral<A>::value) {
+    raise_error("moments of an integer tensor");
+  } else {
+    const StreamScratch& sc = stream_scratch(s);
+    A* devOut = reinterpret_cast<A*>(sc.result);
+    A* hostDev = reinterpret_cast<A*>(sc.hostResultDev);
+    constexpr int V = 16 / sizeof(T);
+    const int64_t batch = (int64_t)kBlock * V * 8;
+    int64_t blocks = std::min<int64_t>((int64_t)num_compute_units(s) * tuning("reduce.all.blocks_per_cu", 2),
+                                       (n + batch - 1) / batch);
+    blocks = std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)(sc.partialBytes / (3 * sizeof(A)))));
+    int64_t chunk = (n + blocks - 1) / blocks;
+    chunk = (chunk + batch - 1) / batch * batch;
+    blocks = (n + chunk - 1) / chunk;
+    hipStream_t st = current_stream(s);
+    A* part = (A*)sc.partials;
+    auto go = [&](auto idxTag) {
+      using I = decltype(idxTag);
+      if (aligned16(src))
+        hipLaunchKernelGGL((moments_all_kernel<T, I, V>), dim3((int)blocks), dim3(kBlock), 0, st, (const T*)src,
+                           (I)n, (I)chunk, part);
+      else
+        hipLaunchKernelGGL((moments_all_kernel<T, I, 1>), dim3((int)blocks), dim3(kBlock), 0, st, (const T*)src,
+                           (I)n, (I)chunk, part);
+    };
+    if (force_64bit_index() || n >= kIndex32Limit) go(uint64_t{});
+    else go(uint32_t{});
+    hipLaunchKernelGGL((moments_fold_kernel<A>), dim3(1), dim3(kBlock), 0, st, (const A*)part, (uint32_t)blocks,
+                       devOut, hostDev);
+    note_kernel("all-moments");
+    THC_CHECK(hipGetLastError());
+    THC_CHECK(hipStreamSynchronize(st));
+    const A r = *reinterpret_cast<const volatile A*>(sc.hostResult);
+    result->f = (double)r;
+    result->i = (int64_t)r;
+  }
+}
 
 template <typename T>
 void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src2, ReduceOp op,

@@ -38,4 +38,9 @@ template <typename T>
 void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src2, ReduceOp op,
                      double p, Scalar* result);
 
+// Sum of squared deviations from the mean of a dense run of n elements in one
+// read (float element types only). Blocks until the scalar is on the host.
+template <typename T>
+void reduce_all_moments_type(THCState* s, int64_t n, const void* src, Scalar* result);
+
 }  // namespace thc

@@ -53,6 +53,44 @@ def test_gpu_var_std(thc, oracle, kind):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double"])
+def test_gpu_varall_of_a_dense_tensor_is_one_read(thc, kind):
+    """Welford per lane plus pairwise merges: sizes around the pack and batch
+    boundaries, a storage offset (scalar loads), a large common offset, and an
+    outlier in front, all against float64 numpy; the two-sweep form, reached
+    with the kernel switched off or through a strided view, agrees."""
+    rng = np.random.default_rng(81)
+    dtype = {"float": np.float32, "half": np.float16, "double": np.float64}[kind]
+    tol = {"float": 2e-5, "half": 2e-3, "double": 1e-12}[kind]
+    for n in (1, 2, 5, 1023, 8192, 8193, 100003, (1 << 21) + 3):
+        for off in (0, 1):
+            x = (rng.standard_normal(n + off) * 0.5 + (3.0 if kind == "half" else 1000.0)).astype(dtype)
+            x[off] = -7.0                                              # outlier first
+            dev = thc.Tensor.from_storage(x, off, (n,), (1,), kind=kind)
+            ref = x[off:].astype(np.float64)
+            for biased in (0, 1):
+                if n == 1 and not biased:
+                    continue
+                want = ref.var(ddof=0 if biased else 1)
+                got = dev.varall(biased)
+                assert thc.last_kernel() == "all-moments"
+                assert abs(got - want) <= tol * max(want, 1e-30), (kind, n, off, biased, got, want)
+    x = (rng.standard_normal((300, 70)) + 5).astype(dtype)
+    dev = thc.Tensor.from_numpy(x)
+    a = dev.varall(0)
+    thc.set_tuning("reduce.all.moments", 0)
+    try:
+        b = dev.varall(0)
+        assert thc.last_kernel() != "all-moments"
+    finally:
+        thc.set_tuning("reduce.all.moments", 1)
+    c = dev.t().varall(0)                                            # not one dense run in logical order
+    want = x.astype(np.float64).var(ddof=1)
+    for v in (a, b, c):
+        assert abs(v - want) <= tol * want
+
+
+@pytest.mark.gpu
 def test_gpu_varall_stdall_dist(thc, oracle):
     rng = np.random.default_rng(8)
     for shape in ((1000,), (257, 129), (1 << 20,)):
