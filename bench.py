@@ -225,7 +225,7 @@ def build_configs(thc, hip, which, only=None):
                 "N-cvt-half": ("half <- float converting copy, 2^26", 6 * ne, ne, lambda i: hdst.copy_from(e_src)),
                 "N-double-sum": ("sum over last dim of 8192x4096 fp64", 8 * 8192 * 4096 + 8 * 8192, 8192 * 4096,
                                  lambda i: dout.sum(dsrc, 1)),
-                "N-renorm": ("renorm(p=2, dim 0, maxnorm 1) of 8192x8192 fp32 (read + write counted once)",
+                "N-renorm": ("renorm(p=2, dim 0, maxnorm 1) of 8192x8192 fp32 (one read, one write)",
                              8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.renorm(sq, 2.0, 0, 1.0)),
             })
         if set(nx) & {"N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall", "N-cumsum-rows10",

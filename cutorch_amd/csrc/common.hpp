@@ -296,6 +296,9 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Sca
 // The same reduction over a - b without materialising the difference. Only
 // for dense operands of a floating type; returns false when it does not apply
 // (the caller then subtracts into a temporary).
+// renorm along dim 0 when src and out are contiguous and a slice fits the
+// staging buffer: one read, one write; false otherwise.
+bool renorm_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* src, double p, double maxnorm);
 // Sum of squared deviations from the mean over all elements of a contiguous
 // float-typed tensor, in one read; false if the tensor is not one dense run
 // (the caller then takes two sweeps).

@@ -138,4 +138,29 @@ __device__ __forceinline__ uint32_t stage_rows_to_lds(const TIn* first, uint32_t
 }
 
 
+// The way back: `count` elements held in LDS (element i at run[i], any
+// alignment) go to `dst` as 16-byte packs aligned on dst; the packs that
+// straddle the run's ends are stored element by element, so nothing outside
+// [dst, dst + count) is written.
+template <typename T>
+__device__ __forceinline__ void write_run_from_lds(T* dst, const T* run, uint32_t count) {
+  constexpr int VEC = 16 / sizeof(T);
+  using P = Pack<T, VEC>;
+  const int mo = (int)((reinterpret_cast<uintptr_t>(dst) / sizeof(T)) & (uintptr_t)(VEC - 1));
+  const uint32_t npacks = ((uint32_t)mo + count + VEC - 1) / VEC;
+  for (uint32_t k = threadIdx.x; k < npacks; k += kBlock) {
+    const int first = (int)(k * VEC) - mo;  // run index of the pack's element 0
+    if (first >= 0 && first + VEC <= (int)count) {
+      P v;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v.v[e] = run[first + e];
+      *reinterpret_cast<P*>(dst + first) = v;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        if (first + e >= 0 && first + e < (int)count) dst[first + e] = run[first + e];
+    }
+  }
+}
+
 }  // namespace thc

@@ -196,6 +196,11 @@ void renorm(THCState* s, DType dt, AnyTensor* self, AnyTensor* src, double p, lo
   THC_ARG_CHECK(dim >= 0 && dim < src->nDimension, 3, "invalid dimension");
   THC_ARG_CHECK(p > 0, 2, "non-positive-norm not supported");
   THC_ARG_CHECK(src->nDimension > 1, 1, "need at least 2 dimensions");
+  // dim 0 of a dense tensor (rows of an embedding table): one fused pass
+  if (dim == 0) {
+    if (self != src) tensor_resize_as(s, self, src, dt);
+    if (renorm_rows(s, dt, self, src, p, maxnorm)) return;
+  }
   TensorRef sums(s, tensor_new(s));
   AnyTensor* cur = src;
   bool first = true;

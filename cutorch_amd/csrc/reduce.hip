@@ -222,6 +222,18 @@ bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a,
   return true;
 }
 
+bool renorm_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* src, double p, double maxnorm) {
+  if (!dtype_is_float(dt) || src->nDimension < 2 || !tuning("renorm.rows", 1)) return false;
+  if (!tensor_is_contiguous(src) || !tensor_is_contiguous(out) || tensor_numel(out) != tensor_numel(src)) return false;
+  const int64_t rows = src->size[0], R = tensor_numel(src) / std::max<int64_t>(rows, 1);
+  if (rows < 1 || R < 1) return false;
+  const void* ip = tensor_data(src, dt);
+  void* op = tensor_data(out, dt);
+  if (dt == DType::F32) return renorm_rows_type<float>(s, rows, R, ip, op, p, maxnorm);
+  if (dt == DType::F16) return renorm_rows_type<__half>(s, rows, R, ip, op, p, maxnorm);
+  return renorm_rows_type<double>(s, rows, R, ip, op, p, maxnorm);
+}
+
 bool reduce_all_moments(THCState* s, DType dt, AnyTensor* in, Scalar* result) {
   if (!dtype_is_float(dt) || in->nDimension == 0 || in->nDimension > kMaxDims) return false;
   if (!tensor_is_contiguous(in) || !tuning("reduce.all.moments", 1)) return false;

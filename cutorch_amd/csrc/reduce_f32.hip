@@ -10,4 +10,5 @@ template bool reduce_var_cols_type<float>(THCState*, const ReduceGeom&, const vo
 template void reduce_all_type<float>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
                                   Scalar*);
 template void reduce_all_moments_type<float>(THCState*, int64_t, const void*, Scalar*);
+template bool renorm_rows_type<float>(THCState*, int64_t, int64_t, const void*, void*, double, double);
 }

@@ -726,6 +726,70 @@ __global__ __launch_bounds__(kBlock) void reduce_slab_index_kernel(const T* __re
   }
 }
 
+// renorm along dim 0 of a dense tensor in one read and one write: the slices
+// are rows lying back to back, so a workgroup stages a run of whole rows in
+// LDS (at most 32 KiB, one row or many), a lane group per row sums |x|^p,
+// forms the factor (maxnorm / (norm + 1e-7) where norm > maxnorm, else 1;
+// generic/THCTensorMathReduce.cu:46-74 with THCTensorMathReduce.cuh:253-306)
+// rounded to the element type as a multiplication of two tensors would see
+// it, scales the row in LDS, and the run goes back out as aligned packs.
+// PK: 1 or 2 = that power without powf, 0 = general p.
+template <typename T, typename I, int PK>
+__global__ __launch_bounds__(kBlock) void renorm_rows_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                                             I numRows, I R, uint32_t rowsPerBlock,
+                                                             uint32_t G, typename Acc<T>::type p,
+                                                             typename Acc<T>::type maxnorm) {
+  using A = typename Acc<T>::type;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ A waveSum[kBlock / 64];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  const uint32_t lane = threadIdx.x % G, grp = threadIdx.x / G, groups = kBlock / G;
+  const I numBlocks = (numRows + rowsPerBlock - 1) / rowsPerBlock;
+  for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+    const I row0 = blk * rowsPerBlock;
+    const uint32_t nrows = (uint32_t)min((I)rowsPerBlock, numRows - row0);
+    const uint32_t mis = stage_rows_to_lds<T, 8>(in + row0 * R, nrows * (uint32_t)R, lds);
+    __syncthreads();
+    auto power = [&](T v) {
+      const A x = abs_any(acc_up<A>(v));
+      return PK == 1 ? x : (PK == 2 ? x * x : pow_any(x, p));
+    };
+    auto scale = [&](T* row, A sum, uint32_t first, uint32_t step) {
+      const A norm = PK == 1 ? sum : (PK == 2 ? sqrt_any(sum) : pow_any(sum, (A)1 / p));
+      if (norm > maxnorm) {
+        const A factor = acc_up<A>(acc_down<T>(maxnorm / (norm + (A)1e-7)));
+        for (uint32_t j = first; j < (uint32_t)R; j += step) row[j] = acc_down<T>(acc_up<A>(row[j]) * factor);
+      }
+    };
+    if (rowsPerBlock < kBlock / 64) {
+      // long rows, fewer than one per wave: the whole workgroup takes each row
+      for (uint32_t r = 0; r < nrows; ++r) {
+        T* row = lds + mis + r * (uint32_t)R;
+        A acc = (A)0;
+        for (uint32_t j = threadIdx.x; j < (uint32_t)R; j += kBlock) acc += power(row[j]);
+        for (uint32_t o = 32; o > 0; o >>= 1) acc += shfl_xor_any(acc, o);
+        if ((threadIdx.x & 63) == 0) waveSum[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        A sum = waveSum[0];
+        for (uint32_t w = 1; w < kBlock / 64; ++w) sum += waveSum[w];
+        scale(row, sum, threadIdx.x, kBlock);
+        __syncthreads();  // waveSum is reused by the next row
+      }
+    } else {
+      for (uint32_t r = grp; r < nrows; r += groups) {  // lanes of a group share r
+        T* row = lds + mis + r * (uint32_t)R;
+        A acc = (A)0;
+        for (uint32_t j = lane; j < (uint32_t)R; j += G) acc += power(row[j]);
+        for (uint32_t o = G >> 1; o > 0; o >>= 1) acc += shfl_xor_any(acc, o);
+        scale(row, acc, lane, G);
+      }
+    }
+    __syncthreads();
+    write_run_from_lds<T>(out + row0 * R, lds + mis, nrows * (uint32_t)R);
+    __syncthreads();  // the buffer is refilled by the next run
+  }
+}
+
 // var / std along a unit-stride dim whose rows fit the registers of one lane
 // group (R <= 64 lanes x 8 packs): the row is read once, the mean and the sum
 // of squared deviations both come from the registers.
@@ -2195,6 +2259,42 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, const void* src
   result->i = (int64_t)r;
 }
 }  // namespace
+
+// renorm over dim 0 of a dense [rows][R] block whose rows are at most 32 KiB.
+template <typename T>
+bool renorm_rows_type(THCState* s, int64_t rows, int64_t R, const void* in, void* out, double p, double maxnorm) {
+  using A = typename Acc<T>::type;
+  if constexpr (std::is_integral<A>::value) {
+    return false;
+  } else {
+    const int64_t rowBytes = R * (int64_t)sizeof(T);
+    if (rowBytes > 32768 || rows < 1 || R < 1) return false;
+    int64_t chunk = rows * rowBytes / ((int64_t)num_compute_units(s) * 4);
+    chunk = std::min<int64_t>(32768, std::max<int64_t>(std::max<int64_t>(4096, rowBytes), chunk));
+    const uint32_t rpb = (uint32_t)std::max<int64_t>(1, chunk / rowBytes);
+    uint32_t G = pow2_ceil((uint64_t)R / 16 + 1);
+    if (G > 1 && (uint64_t)G * 16 > (uint64_t)R) G >>= 1;
+    G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+    const size_t lds = (((size_t)rpb * (size_t)R + 2 * (16 / sizeof(T))) * sizeof(T) + 15) & ~size_t(15);
+    const int grid = capped_grid(s, (rows + rpb - 1) / rpb, "reduce.rows.blocks_per_cu", 64);
+    hipStream_t st = current_stream(s);
+    auto go = [&](auto idxTag, auto pk) {
+      using I = decltype(idxTag);
+      hipLaunchKernelGGL((renorm_rows_kernel<T, I, decltype(pk)::value>), dim3(grid), dim3(kBlock), lds, st,
+                         (const T*)in, (T*)out, (I)rows, (I)R, rpb, G, (A)p, (A)maxnorm);
+    };
+    auto pick = [&](auto idxTag) {
+      if (p == 1.0) go(idxTag, std::integral_constant<int, 1>{});
+      else if (p == 2.0) go(idxTag, std::integral_constant<int, 2>{});
+      else go(idxTag, std::integral_constant<int, 0>{});
+    };
+    if (force_64bit_index() || rows * R >= kIndex32Limit) pick(uint64_t{});
+    else pick(uint32_t{});
+    note_kernel("renorm-rows");
+    THC_CHECK(hipGetLastError());
+    return true;
+  }
+}
 
 // Sum of squared deviations from the mean over a dense run of n elements, one
 // read of the input. Blocks until the scalar is on the host, like the others.

@@ -43,4 +43,9 @@ void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src
 template <typename T>
 void reduce_all_moments_type(THCState* s, int64_t n, const void* src, Scalar* result);
 
+// renorm over dim 0 of a dense [rows][R] block in one read and one write;
+// false when a row does not fit the staging buffer (or the type is integral).
+template <typename T>
+bool renorm_rows_type(THCState* s, int64_t rows, int64_t R, const void* in, void* out, double p, double maxnorm);
+
 }  // namespace thc

@@ -10,4 +10,5 @@ template bool reduce_var_cols_type<double>(THCState*, const ReduceGeom&, const v
 template void reduce_all_type<double>(THCState*, ReduceGeom, const void*, const void*, ReduceOp, double,
                                   Scalar*);
 template void reduce_all_moments_type<double>(THCState*, int64_t, const void*, Scalar*);
+template bool renorm_rows_type<double>(THCState*, int64_t, int64_t, const void*, void*, double, double);
 }

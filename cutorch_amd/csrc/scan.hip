@@ -262,8 +262,6 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
                                                            uint64_t outer, uint64_t R, uint32_t inner,
                                                            uint32_t slicesPerBlock, uint64_t S,
                                                            uint32_t chunkRows) {
-  constexpr int VEC = 16 / sizeof(T);
-  using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
@@ -309,22 +307,7 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
       }
     }
     __syncthreads();
-    T* dst = out + start;
-    const int mo = (int)((reinterpret_cast<uintptr_t>(dst) / sizeof(T)) & (uintptr_t)(VEC - 1));
-    const uint32_t npacks = ((uint32_t)mo + count + VEC - 1) / VEC;
-    for (uint32_t k = threadIdx.x; k < npacks; k += kBlock) {
-      const int first = (int)(k * VEC) - mo;  // run index of the pack's element 0
-      if (first >= 0 && first + VEC <= (int)count) {
-        P v;
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) v.v[e] = lds[mis + first + e];
-        *reinterpret_cast<P*>(dst + first) = v;
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e)
-          if (first + e >= 0 && first + e < (int)count) dst[first + e] = lds[mis + first + e];
-      }
-    }
+    write_run_from_lds<T>(out + start, lds + mis, count);
     __syncthreads();  // the buffer is refilled by the next run
   }
 }

@@ -621,6 +621,52 @@ def test_gpu_renorm(thc, oracle, kind):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "double", "half"])
+def test_gpu_renorm_of_dense_rows_is_one_pass(thc, oracle, kind):
+    """renorm over dim 0 of a contiguous tensor (the rows of an embedding
+    table): norm, factor and scaling in one kernel that stages runs of rows in
+    LDS. Short and long rows, a misaligned storage offset, in place, and a row
+    too long for the staging buffer (which takes the general route)."""
+    rng = np.random.default_rng(113)
+    dt = np_of(oracle, kind)
+    tol = {"float": 1e-5, "double": 1e-12, "half": 2e-3}[kind]
+    for shape, fused in (((1000, 33), True), ((300, 128), True), ((50, 1000), True), ((7, 4096), True),
+                         ((5, 3, 11), True), ((3, 1), True), ((2, 20000), False)):
+        n = int(np.prod(shape))
+        for off in (0, 1):
+            st = rng.uniform(-2, 2, n + off).astype(dt)
+            strides = [1] * len(shape)
+            for d in range(len(shape) - 2, -1, -1):
+                strides[d] = strides[d + 1] * shape[d + 1]
+            dev = thc.Tensor.from_storage(st, off, shape, tuple(strides), kind=kind)
+            ref = oracle.View(st.copy(), off, shape, tuple(strides))
+            x = ref.numpy().astype(np.float64).reshape(shape[0], -1)
+            for p in (1.0, 2.0, 3.0):
+                norms = np.sort((np.abs(x) ** p).sum(axis=1) ** (1 / p))
+                k = len(norms) // 2
+                maxnorm = float(norms[k - 1] + norms[k]) / 2
+                got = thc.Tensor(kind).renorm(dev, p, 0, maxnorm)
+                assert (thc.last_kernel() == "renorm-rows") == fused, (shape, thc.last_kernel())
+                want = oracle.renorm(ref, p, 0, maxnorm).numpy().astype(np.float64)
+                np.testing.assert_allclose(got.numpy().astype(np.float64), want, rtol=tol, atol=tol * 1e-3)
+            before = dev.storage_numpy().copy()
+            dev.renorm(dev, 2.0, 0, 1e9)                         # nothing exceeds: bit-identical
+            assert thc.last_kernel() == ("renorm-rows" if fused else thc.last_kernel())
+            assert_bit_equal(dev.storage_numpy(), before)
+            dev.renorm(dev, 2.0, 0, 0.5)                          # in place
+            got = dev.numpy().astype(np.float64).reshape(shape[0], -1)
+            np.testing.assert_allclose(np.minimum(np.sqrt((got ** 2).sum(axis=1)), 0.5),
+                                       np.minimum(np.sqrt((x ** 2).sum(axis=1)), 0.5), rtol=max(tol, 1e-6) * 4)
+            assert_bit_equal(dev.storage_numpy()[:off], before[:off])
+    thc.set_tuning("renorm.rows", 0)
+    try:
+        thc.Tensor(kind).renorm(thc.Tensor.from_numpy(np.ones((8, 8), dt)), 2.0, 0, 1.0)
+        assert thc.last_kernel() != "renorm-rows"
+    finally:
+        thc.set_tuning("renorm.rows", 1)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["int", "byte", "double"])
 def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
     """The wider types have no LDS-tiled arithmetic kernels: a transposed input
