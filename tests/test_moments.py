@@ -125,7 +125,7 @@ def test_gpu_var_rows_single_read_and_fallback(thc, oracle, kind):
     dtype = np.float32 if kind == "float" else np.float16
     vec = 4 if kind == "float" else 8
     for shape, expect in (((300, 1024), "var-rows"), ((7, 64 * vec * 8), "var-rows"), ((5, 8), "var-rows"),
-                          ((3, 64 * vec * 8 + vec), "rows"), ((50, 1023), "rows-lds"), ((2, 40000), None)):
+                          ((3, 64 * vec * 8 + vec), "rows"), ((50, 1023), "var-rows-lds"), ((2, 40000), None)):
         x = (rng.standard_normal(shape) * 2 + 3).astype(dtype)
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
         for name, okind in (("var", "var"), ("std", "std")):
@@ -149,7 +149,7 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
     dtype = np.float32 if kind == "float" else np.float16
     offset = 100.0 if kind == "float" else 4.0
     for shape, dim, expect in (((64, 512), 0, "var-cols"), ((6, 300, 40), 1, "var-cols"),
-                               ((2, 8192, 96), 1, "var-cols-split"), ((129, 7), 0, "slab"),
+                               ((2, 8192, 96), 1, "var-cols-split"), ((129, 7), 0, "var-slab"),
                                ((3, 50, 8, 24), 1, "var-cols")):
         x = (rng.standard_normal(shape) * 0.1 + offset).astype(dtype)
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
@@ -160,3 +160,39 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
                 want = oracle.reduce_dim(name + ("_biased" if biased else ""), ref, dim).numpy().astype(np.float64)
                 np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol * (8 if kind == "float" else 1),
                                            atol=0, err_msg="%s %s %s" % (shape, name, kind))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double"])
+def test_gpu_var_of_short_rows_and_small_slices_is_one_read(thc, kind):
+    """Dense short rows and small R x C slices are staged in LDS and swept
+    there twice (mean, squared deviations): row lengths around the group
+    sizes, misaligned storage offsets, a common offset of 40 sigma, against float64
+    numpy."""
+    rng = np.random.default_rng(82)
+    dtype = {"float": np.float32, "half": np.float16, "double": np.float64}[kind]
+    tol = {"float": 2e-5, "half": 4e-3, "double": 1e-12}[kind]
+    centre = 3.0 if kind == "half" else 20.0
+    atol = {"float": 1e-6, "half": 2e-3, "double": 1e-14}[kind]    # rounding of the mean, squared-deviation scale
+    cases = [((1000, 2), 1), ((777, 10), 1), ((300, 33), 1), ((64, 100), 1), ((9, 1001), 1), ((4, 5, 70), 2),
+             ((500, 8, 16), 1), ((300, 33, 2), 1), ((129, 7), 0), ((40, 100, 10), 1), ((3, 2, 5, 7), 2)]
+    for shape, dim in cases:
+        n = int(np.prod(shape))
+        for off in (0, 1, 3):
+            x = (rng.standard_normal(n + off) * 0.5 + centre).astype(dtype)
+            strides = [1] * len(shape)
+            for d in range(len(shape) - 2, -1, -1):
+                strides[d] = strides[d + 1] * shape[d + 1]
+            dev = thc.Tensor.from_storage(x, off, shape, tuple(strides), kind=kind)
+            ref = x[off:].reshape(shape).astype(np.float64)
+            # rows that are whole aligned packs keep the register kernel
+            expect = ("var-rows-lds", "var-rows") if dim == len(shape) - 1 else ("var-slab",)
+            if shape == (300, 33) or (off % 2 and dim == len(shape) - 1):
+                expect = ("var-rows-lds",)
+            for name, fn in (("var", np.var), ("std", np.std)):
+                for biased in (0, 1):
+                    out = getattr(thc.Tensor(kind), name)(dev, dim, biased=biased)
+                    assert thc.last_kernel() in expect, (shape, dim, off, thc.last_kernel())
+                    want = fn(ref, axis=dim, ddof=0 if biased else 1, keepdims=True)
+                    np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol, atol=atol,
+                                               err_msg="%s %s %s off %d" % (kind, name, shape, off))

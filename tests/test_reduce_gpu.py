@@ -507,10 +507,10 @@ def test_small_dense_slices_special_cases(thc, oracle):
         assert_bit_equal(out.numpy()[:, 0, :], y.sum(axis=1).astype(np.float32))
     finally:
         thc.force_64bit_index(False)
-    # var / std of small slices: two sweeps of the slab kernel
+    # var / std of small slices: staged once, swept twice in LDS
     z = (rng.standard_normal((300, 12, 6)) * 2 + 5).astype(np.float32)
     out = thc.Tensor("float").var(thc.Tensor.from_numpy(z), 1)
-    assert thc.last_kernel() == "slab"
+    assert thc.last_kernel() == "var-slab"
     np.testing.assert_allclose(out.numpy()[:, 0, :], z.astype(np.float64).var(axis=1, ddof=1), rtol=1e-5)
 
 
