@@ -1614,7 +1614,7 @@ void launch_rows_pass(THCState* s, const TIn* in, TOut* out, typename F::A* part
 template <typename T>
 bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPerBlock, uint32_t& G,
                    size_t& ldsBytes) {
-  if (!tuning("reduce.rows.lds", 1) || g.sR != 1) return false;
+  if (!tuning("reduce.rows.lds", 1) || g.sR != 1 || g.R < 1 || g.outElems < 1) return false;
   int64_t run = g.R;
   for (int d = g.in.dims - 1; d >= 0; --d) {
     if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
@@ -1803,7 +1803,7 @@ ColsPlan<I> plan_cols(THCState* s, const ReduceGeom& g, const void* in, size_t p
 template <typename T, typename I>
 bool plan_slab(THCState* s, const ReduceGeom& g, SlabArgs<I>& a, int64_t& blocks) {
   const int nd = g.in.dims;
-  if (!tuning("reduce.slab", 1) || nd < 1) return false;
+  if (!tuning("reduce.slab", 1) || nd < 1 || g.R < 1 || g.outElems < 1) return false;
   const int64_t C = g.in.size[nd - 1];
   if (g.in.stride[nd - 1] != 1 || g.sR != C) return false;
   const int64_t slice = g.R * C;

@@ -98,3 +98,22 @@ def test_transposed_copies_of_every_element_size_at_odd_shapes(thc, kind):
             want = dst.copy()
             want[off_out:] = src[off_in:].reshape(cols, rows).T.reshape(-1)
             assert_bit_equal(out.storage_numpy(), want, "%s %dx%d +%d/+%d %s" % (kind, rows, cols, off_in, off_out, k))
+
+
+def test_reductions_and_scans_are_reproducible_run_to_run(thc):
+    """No atomics, fixed fold orders: the same call on the same data returns
+    the same bits, on every kernel family (split ones included)."""
+    rng = np.random.default_rng(9200)
+    for shape, dim in (((3, 1 << 18), 1), ((2, 8192, 96), 1), ((65536, 33), 1), ((4096, 8, 16), 1),
+                       ((300001, 3), 0), ((8191, 513), 0), ((1024, 1024), 1), ((200000, 10), 0)):
+        x = thc.Tensor.from_numpy(rng.standard_normal(shape).astype(np.float32))
+        first = {}
+        for rep in range(3):
+            got = {"sum": thc.Tensor("float").sum(x, dim).numpy(), "norm": thc.Tensor("float").norm(x, 2.0, dim).numpy(),
+                   "std": thc.Tensor("float").std(x, dim).numpy(), "cumsum": thc.Tensor("float").cumsum(x, dim).numpy(),
+                   "sumall": np.float32(x.sumall()), "varall": np.float32(x.varall())}
+            for k, v in got.items():
+                if rep == 0:
+                    first[k] = v
+                else:
+                    assert_bit_equal(np.asarray(v), np.asarray(first[k]), "%s %s rep %d" % (k, shape, rep))
