@@ -183,7 +183,7 @@ def build_configs(thc, hip, which, only=None):
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
-                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd")
+                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -229,7 +229,7 @@ def build_configs(thc, hip, which, only=None):
                              8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.renorm(sq, 2.0, 0, 1.0)),
             })
         if set(nx) & {"N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall", "N-cumsum-rows10",
-                      "N-cumsum-tall", "N-add-t-odd"}:
+                      "N-cumsum-tall", "N-add-t-odd", "N-bias-odd"}:
             # shapes off the aligned grid: short / misaligned rows, small slices, tall narrow matrices
             nr = 1 << 26
             flat = e_src
@@ -243,7 +243,10 @@ def build_configs(thc, hip, which, only=None):
             oddB = T.from_numpy(rng.standard_normal((8191, 8193), dtype=np.float32))
             oddO = T("float").resize((8191, 8193))
             n33, n10, nodd = (nr // 33) * 33, (nr // 10) * 10, 8191 * 8193
+            bias = T.from_numpy(rng.standard_normal(8193, dtype=np.float32)).view_as_strided(0, (8191, 8193), (0, 1))
             table.update({
+                "N-bias-odd": ("c = x + bias (stride-0 row bias), 8191x8193 fp32 (no 16-byte aligned rows)", 8 * nodd,
+                               nodd, lambda i: oddO.cadd(oddB, 1.0, bias)),
                 "N-sum-rows33": ("sum over last dim of 2033601x33 fp32 (misaligned short rows)", 4 * n33 + 4 * (nr // 33),
                                  n33, lambda i: o33.sum(v33, 1)),
                 "N-max-rows33": ("max+argmax over last dim of 2033601x33 fp32", 4 * n33 + 12 * (nr // 33), n33,

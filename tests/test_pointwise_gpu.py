@@ -342,3 +342,63 @@ def test_config5_full_size_64bit_index_path(thc):
     for jj in (0, 2047):
         want = ba[(k * 2048 * 2048 + jj * 2048 + i) % L] + bb[(i * 2048 * 520 + jj * 520 + k) % L]
         assert_bit_equal(c.select(1, jj).numpy(), want, "plane j=%d" % jj)
+
+
+@pytest.mark.parametrize("kind", ["float", "half"])
+def test_broadcast_operands_on_rows_that_are_not_pack_aligned(thc, kind):
+    """x + bias where bias is a stride-0 view (row bias, column bias, a scalar, a
+    middle-dim bias) and the rows of x are not 16-byte aligned: the dense
+    operands stream as flat aligned packs, the broadcast one is gathered element
+    by element. Aligned shapes keep the strided / tiled pack kernels; a
+    permuted operand of full size never takes this route."""
+    rng = np.random.default_rng(90)
+    dtype = np.float32 if kind == "float" else np.float16
+    for shape in ((333, 515), (61, 1001), (7, 9, 131), (1001,), (2, 3, 5, 67)):
+        n = int(np.prod(shape))
+        nd = len(shape)
+        x = rng.integers(-8, 9, shape).astype(dtype)
+        dx = thc.Tensor.from_numpy(x)
+        for d in range(nd):
+            bias = rng.integers(-8, 9, shape[d]).astype(dtype)
+            strides = tuple(1 if k == d else 0 for k in range(nd))
+            db = thc.Tensor.from_numpy(bias).view_as_strided(0, shape, strides)
+            view = bias.reshape([shape[d] if k == d else 1 for k in range(nd)])
+            if nd == 1:
+                continue                                   # a 1-D "bias" is just a dense operand
+            out = thc.Tensor(kind).cadd(dx, 1.0, db)
+            assert thc.last_kernel() == "flat-gather", (shape, d, thc.last_kernel())
+            assert_bit_equal(out.numpy(), (x + view).astype(dtype))
+            out = thc.Tensor(kind).cmul(db, dx)             # broadcast operand first
+            assert thc.last_kernel() == "flat-gather"
+            assert_bit_equal(out.numpy(), (x * view).astype(dtype))
+            if nd == 2:
+                both = thc.Tensor(kind).addcmul(dx, 1.0, db, db)       # two gathered inputs
+                assert thc.last_kernel() == "flat-gather"
+                assert_bit_equal(both.numpy(), (x + view * view).astype(dtype))
+        scalar = thc.Tensor.from_numpy(np.array([3], dtype)).view_as_strided(0, shape, (0,) * nd)
+        acc = thc.Tensor.from_numpy(x.copy())
+        acc.cadd(acc, 2.0, scalar)                          # in place on the dense operand
+        assert thc.last_kernel() == "flat-gather"
+        assert_bit_equal(acc.numpy(), (x + dtype(6)).astype(dtype))
+    # aligned rows: the strided pack kernel is the faster one and stays
+    x = rng.integers(-8, 9, (64, 256)).astype(dtype)
+    bias = rng.integers(-8, 9, 256).astype(dtype)
+    db = thc.Tensor.from_numpy(bias).view_as_strided(0, (64, 256), (0, 1))
+    out = thc.Tensor(kind).cadd(thc.Tensor.from_numpy(x), 1.0, db)
+    assert thc.last_kernel() == "strided"
+    assert_bit_equal(out.numpy(), (x + bias).astype(dtype))
+    # a transposed operand of the output's own size is not a broadcast
+    y = rng.integers(-8, 9, (515, 333)).astype(dtype)
+    out = thc.Tensor(kind).cadd(thc.Tensor.from_numpy(y).t(), 1.0, thc.Tensor.from_numpy(y.T.copy()))
+    assert thc.last_kernel().startswith("tiled")
+    assert_bit_equal(out.numpy(), (y.T + y.T).astype(dtype))
+    thc.set_tuning("apply.flatmix", 0)
+    try:
+        x = rng.integers(-8, 9, (333, 515)).astype(dtype)
+        bias = rng.integers(-8, 9, 515).astype(dtype)
+        db = thc.Tensor.from_numpy(bias).view_as_strided(0, (333, 515), (0, 1))
+        out = thc.Tensor(kind).cadd(thc.Tensor.from_numpy(x), 1.0, db)
+        assert thc.last_kernel() == "strided-scalar"
+        assert_bit_equal(out.numpy(), (x + bias).astype(dtype))
+    finally:
+        thc.set_tuning("apply.flatmix", 1)
