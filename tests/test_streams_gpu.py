@@ -77,8 +77,9 @@ def test_current_stream_is_per_thread(thc, streams):
 
 def test_concurrent_host_threads_on_their_own_streams(thc, streams):
     """Four host threads, each on its own stream (two created here, two more
-    below), run pointwise ops, split reductions, *all reductions and temporaries
-    (caching allocator) at the same time; every result must be exact."""
+    below), run pointwise ops, split and chunked reductions and scans, *all reductions
+    and temporaries (caching allocator) at the same time; every result must be
+    exact."""
     hip, (s1, s2) = streams
     lib, st = thc.lib(), thc.state()
     extra = []
@@ -103,6 +104,16 @@ def test_concurrent_host_threads_on_their_own_streams(thc, streams):
                 mx.max(ix, out, 1)
                 total = dbig.sumall()                                          # blocks on this stream only
                 cont = db.t().contiguous()                                     # temporary through the allocator
+                tall = rng.integers(-2, 3, (40000, 3)).astype(np.float32)      # chunked kernels: partials and carries
+                dtall = thc.Tensor.from_numpy(tall)                            # live in this stream's scratch
+                colsum = thc.Tensor("float").sum(dtall, 0)
+                assert thc.last_kernel() == "slab-chunked"
+                run = thc.Tensor("float").cumsum(dtall, 0)
+                assert thc.last_kernel() == "scan-chunked"
+                var = dtall.varall()
+                assert np.array_equal(colsum.numpy().ravel(), tall.astype(np.int64).sum(axis=0).astype(np.float32))
+                assert np.array_equal(run.numpy(), np.cumsum(tall.astype(np.int64), axis=0).astype(np.float32))
+                assert abs(var - tall.astype(np.float64).var(ddof=1)) <= 1e-5 * var, (idx, it, "varall")
                 want = a + 2.0 * (a * b.T)
                 assert np.array_equal(out.numpy(), want), (idx, it, "addcmul")
                 assert np.array_equal(sums.numpy().ravel(), big.astype(np.int64).sum(axis=1).astype(np.float32))
