@@ -216,7 +216,8 @@ def _longs(seq):
 
 
 def _half_bits(v):
-    return int(np.array(v, dtype=np.float16).view(np.uint16))
+    with np.errstate(over="ignore"):          # a scalar beyond half's range is +-inf, as in C
+        return int(np.array(v, dtype=np.float16).view(np.uint16))
 
 
 class Tensor(object):
