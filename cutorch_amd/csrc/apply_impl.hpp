@@ -449,6 +449,10 @@ struct TiledArgs {
   // read and partly written lines when rows do not start on 128-byte lines,
   // run on one XCD's L2; 0 = identity mapping.
   uint32_t xcdPer;
+  // Shifted-window variant: tiles are walked in bands of groupP tiles along p
+  // (p fastest inside a band, then q), so that tiles whose staged windows
+  // share cache lines run back to back; 1 = q fastest throughout.
+  uint32_t groupP;
 };
 
 // A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
@@ -689,8 +693,19 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
     const uint32_t tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
     if (tile >= args.totalTiles) continue;  // uniform over the workgroup
     uint32_t rest, tq, tp;
-    args.tilesQ.divmod(tile, rest, tq);
-    args.tilesP.divmod(rest, rest, tp);
+    if (args.groupP > 1) {
+      const uint32_t perBatch = args.tilesP.d * args.tilesQ.d;
+      rest = tile / perBatch;
+      const uint32_t t = tile - rest * perBatch;
+      const uint32_t band = t / (args.groupP * args.tilesQ.d);
+      const uint32_t r = t - band * (args.groupP * args.tilesQ.d);
+      const uint32_t gp = min(args.groupP, args.tilesP.d - band * args.groupP);  // ragged last band
+      tq = r / gp;
+      tp = band * args.groupP + (r - tq * gp);
+    } else {
+      args.tilesQ.divmod(tile, rest, tq);
+      args.tilesP.divmod(rest, rest, tp);
+    }
     I base[kMaxOps] = {0, 0, 0, 0};
     for (int j = 0; j < args.nbatch; ++j) {
       uint32_t r;
@@ -1046,6 +1061,11 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
       if (pl.lay[k].stride[d] != 1 && pl.lay[k].size[d] > 1)
         lineAligned = lineAligned && (pl.lay[k].stride[d] * (int64_t)sizeof(T)) % 128 == 0;
   }
+  // bands of 8 tiles along p: the staged windows of neighbours in p share cache
+  // lines (8191 x 8193: add 4.5 -> 4.7 TB/s, copy 5.1 -> 5.6); only where a
+  // band is a small part of p, since p-fastest order as a whole is the slow one
+  args.groupP = shift ? (uint32_t)std::max<int64_t>(1, tuning("apply.tiled.group_p", 8)) : 1;
+  if ((int64_t)args.groupP * 2 > tp) args.groupP = 1;
   const int64_t swz = tuning("apply.tiled.xcd_swizzle", 1);
   // (not with fused q: there the direct operands are one long aligned run and
   // the remap cost 2% on a permuted 2048 x 2048 x 520 operand)

@@ -402,3 +402,22 @@ def test_broadcast_operands_on_rows_that_are_not_pack_aligned(thc, kind):
         assert_bit_equal(out.numpy(), (x + bias).astype(dtype))
     finally:
         thc.set_tuning("apply.flatmix", 1)
+
+
+@pytest.mark.parametrize("band", [1, 2, 3, 8])
+def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band):
+    """The shifted-window variant walks its tiles in bands of `band` tiles along
+    p (p fastest inside a band): whole bands, a ragged last band, and shapes
+    too short in p for banding must all cover every tile exactly once."""
+    rng = np.random.default_rng(91)
+    thc.set_tuning("apply.tiled.group_p", band)
+    try:
+        for rows, cols in ((333, 515), (400, 130), (1001, 67), (61, 125), (977, 251)):
+            ga = (rows * cols + 1, 1, (rows, cols), (1, rows))           # a:t(), one element into its storage
+            gc = contiguous_geometry((rows, cols))
+            assert run_binary(thc, oracle, "cadd", [gc, ga, gc], rng) == "tiled-shift"
+        g3 = (7 * 130 * 401, 0, (7, 401, 130), (130 * 401, 1, 401))      # batch dim in front, p = 401
+        assert run_binary(thc, oracle, "cmul", [contiguous_geometry((7, 401, 130)), g3,
+                                                contiguous_geometry((7, 401, 130))], rng) == "tiled-shift"
+    finally:
+        thc.set_tuning("apply.tiled.group_p", 8)
