@@ -18,6 +18,19 @@
 //          workgroup partials in a fixed order (bit-reproducible).
 //   generic  anything else: one thread per output walks the reduced dim.
 //
+// Shapes off that grid get LDS-staged forms, all built on one idea: a
+// workgroup streams a contiguous run of the input into LDS as aligned 16-byte
+// packs, whatever the alignment and length of the rows inside it, and reduces
+// out of LDS:
+//   rows-lds  short rows lying back to back (also ragged or misaligned ones);
+//   slab      dense [O][R][C] with an R x C slice of a few KiB: a run of whole
+//             slices per workgroup, a thread per output; in chunk mode, long
+//             narrow misaligned slices are reduced level by level through
+//             dense partials;
+//   var-*-lds / var-slab, renorm-rows  the same staging for var / std and for
+//             renorm along dim 0 (one read, one write);
+//   moments   whole-tensor variance in one read (Welford + pairwise merges).
+//
 // Accumulation is fp32 for float and half input (accreal = float,
 // THCGenerateFloatType.h:5-8, THCGenerateHalfType.h:9-10); results are rounded
 // once on store. max/min carry (value, index) pairs whose combine step prefers

@@ -9,7 +9,12 @@
 //               chunks of a long row;
 //   inner  > 1  lanes run along the unit-stride inner dim (coalesced), thread
 //               rows split the scanned dim into register-resident segments
-//               and exchange segment totals through LDS.
+//               and exchange segment totals through LDS;
+//   small slices (short rows, or R x inner of a few KiB)  a workgroup stages a
+//               run of whole slices in LDS, a thread per column scans in
+//               place, the run goes back out as aligned packs;
+//   long scans with few columns  chunk totals, their scan (this code again on
+//               the accumulator type), then every chunk scans from its carry.
 // Accumulation is fp32 for float and half (rounded per output element), double
 // for double, wrapping 64-bit for the integer types.
 #include <algorithm>
