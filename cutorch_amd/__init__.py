@@ -209,6 +209,8 @@ def _declare(l):
     l.THCudaByteTensor_logicalall.argtypes = [P, TP]
     l.THCudaByteTensor_logicalany.argtypes = [P, TP]
     l.THCudaHalfTensor_copyCuda.argtypes = [P, TP, TP]
+    l.THCudaTensor_sumallNoAlloc.argtypes = [P, TP, P]
+    l.THCudaTensor_sumallNoAlloc.restype = None
 
 
 def _longs(seq):
@@ -482,6 +484,13 @@ class Tensor(object):
 
     def sumall(self):
         return self._scalar("sumall")
+
+    def sumall_no_alloc(self, result):
+        """Launches the sum of all elements into result[0] (a float device tensor);
+        does not wait for the stream (THCudaTensor_sumallNoAlloc)."""
+        lib().THCudaTensor_sumallNoAlloc(self._st, self.h, C.c_void_p(result.data_ptr()))
+        _check()
+        return result
 
     def prodall(self):
         return self._scalar("prodall")

@@ -19,7 +19,7 @@ LIB = os.path.join(HERE, "libTHC.so")
 SOURCES = ["general.cpp", "tensor.cpp", "math.cpp", "math_wide.cpp", "caching_allocator.cpp", "apply.hip", "apply_f32_0.hip", "apply_f32_1.hip",
            "apply_f32_2.hip", "apply_f16_0.hip", "apply_f16_1.hip", "apply_f16_2.hip", "apply_raw.hip",
            "reduce.hip", "reduce_f32.hip", "reduce_f16.hip", "reduce_w_u8.hip", "reduce_w_i8.hip",
-           "reduce_w_i16.hip", "reduce_w_i32.hip", "reduce_w_i64.hip", "reduce_w_f64.hip", "scan.hip", "convert.hip", "apply_cmp_f.hip", "apply_w_u8.hip",
+           "reduce_w_i16.hip", "reduce_w_i32.hip", "reduce_w_i64.hip", "reduce_w_f64.hip", "scan.hip", "no_alloc.hip", "convert.hip", "apply_cmp_f.hip", "apply_w_u8.hip",
            "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip"]
 HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", "apply_plan.hpp", "apply_impl.hpp", "apply_wide.hpp", "reduce_plan.hpp", "reduce_impl.hpp",
            os.path.join("..", "..", "include", "THC.h")]

@@ -142,6 +142,9 @@ const StreamScratch& stream_scratch(THCState* state);
 void* scratch_space(THCState* state, size_t* bytes);
 void check_same_gpu(THCState* state, int n, const AnyTensor* const* ts);
 void note_kernel(const char* name);  // for THCAmd_lastKernel
+// Looks up, for the current device, the address of the fixed partials array
+// of THCudaTensor_sumallNoAlloc (so that the entry point itself finds it ready).
+void no_alloc_setup();
 long tuning(const char* key, long fallback);
 bool force_64bit_index();
 

@@ -199,6 +199,7 @@ THC_API void THCudaInit(THCState* state) {
     // largest shapes); the reference keeps 128 KiB (THCGeneral.c:12-17)
     // because its pass 1 is capped at 1024 partials.
     state->scratchBytes = size_t(16) << 20;
+    no_alloc_setup();
     state->initialised = true;
   })
 }

@@ -576,4 +576,20 @@ THC_API double THCudaDoubleTensor_dist(THCState *, THCudaDoubleTensor *self, THC
 THC_AMD_DECLARE_MATH_API(THCudaTensor, float, float)
 THC_AMD_DECLARE_MATH_API(THCudaHalfTensor, THHalf, float)
 
+/* No counterpart in the reference. For callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc. The sum of all elements of `self`, as
+ * THCudaTensor_sumall computes it (same launches, same bits), except that
+ *   - `self` must be contiguous (or empty) and hold at most 2^32 elements;
+ *     anything else is an argument error and nothing is launched;
+ *   - the scalar is written to `*result`, a device-accessible pointer the
+ *     caller owns (4 bytes), by the second launch on the current stream; the
+ *     call does not wait for the stream and returns nothing;
+ *   - no device memory is allocated or freed: the per-workgroup partials go
+ *     to a fixed 4 KiB array that every GPU the library runs on holds until
+ *     the process ends. All calls on one GPU share that array, so calls that
+ *     overlap on one GPU (several streams or host threads) race: serialise
+ *     them. */
+THC_API void THCudaTensor_sumallNoAlloc(THCState *state, THCudaTensor *self, float *result);
+
 #endif /* THC_AMD_THC_H */
