@@ -5,17 +5,30 @@
 
 A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM. The headline line is quoted on the strided apply3
-configuration (out = a:t() * b + d on 8192 x 8192 fp32, a viewed transposed);
-the other benchmark configurations are measured in the same run and reported
-under "all_configs". Prints ONE JSON line.
+configuration (out = a:t() * b + d on 8192 x 8192 fp32, a viewed transposed,
+out and d rotating over three buffer sets so that the Infinity Cache cannot
+absorb the rewrites of one output buffer); every other benchmark configuration
+is measured in the same run and reported, compactly, under "roofline.configs"
+(fraction of peak, microseconds per launch, parity flag), with a plain
+1-read-1-write calibration stream ("CAL-copy") that tells a slow box from a
+regression. Prints ONE JSON line.
 
   value               algorithmic bytes * steps / wall time of the timed region
   roofline.achieved   algorithmic bytes / average launch duration, from two
                       HIP events that bracket the K launches of the timed
                       region on the stream the engine launches on
+  roofline.configs    the same per configuration; "parity" is a check of the
+                      configuration's own output, outside the timed region,
+                      against a closed form computed with numpy on the host
+                      copy of the inputs (bit-exact for add/mul/addcmul and
+                      max+argmax, 1e-5 / 2e-3 relative for sums and norms)
   cpu_baseline        the CPU restatement (oracle/) timed on this box's host
-                      cores on the same workload, single thread; the all-core
-                      figure is reported beside it
+                      cores: the headline workload single-threaded is the
+                      value; all-core figures and the reduction path (row sums
+                      of 65536 x 1024, middle-dim sums of 64 x 4096 x 512) are
+                      reported beside it under "configs"
+  --configs all       adds the neighbours of the hot path (N-* lines) and the
+                      full per-configuration detail under "all_configs"
 """
 import argparse
 import ctypes as C
@@ -86,78 +99,136 @@ def device_fill_from_block(hip, thc, shape, block):
 
 class Config(object):
     """One benchmark configuration: `sets` rotating operand sets, a `run(i)`
-    that launches the op on set i, and its algorithmic byte count."""
+    that launches the op on set i, its algorithmic byte count, and `check()`,
+    which runs the op once more outside the timed region and compares its
+    output with a closed form computed by numpy from the host inputs."""
 
     def __init__(self, name, desc, nbytes, elements, sets, run, check=None, kernel=None):
         self.name, self.desc, self.nbytes, self.elements = name, desc, nbytes, elements
         self.sets, self.run, self.check, self.kernel = sets, run, check, kernel
+        self.note = None
+
+
+def bit_equal(got, want):
+    got, want = np.ascontiguousarray(got), np.ascontiguousarray(want)
+    u = {2: np.uint16, 4: np.uint32, 8: np.uint64}[got.itemsize]
+    return got.shape == want.shape and bool(np.array_equal(got.view(u), want.view(u)))
+
+
+def sums_close(got, ref64, mass, rel):
+    """|got - ref| <= rel * max(|ref|, mass / 64): the stated relative bound, with a
+    floor of 1/64 of the summed magnitudes for results that cancel."""
+    got = np.asarray(got, np.float64).reshape(-1)
+    ref64 = np.asarray(ref64, np.float64).reshape(-1)
+    mass = np.asarray(mass, np.float64).reshape(-1)
+    return bool(np.all(np.abs(got - ref64) <= rel * np.maximum(np.abs(ref64), mass / 64.0)))
 
 
 def build_configs(thc, hip, which, only=None):
     rng = np.random.default_rng(0xC0FFEE)
     cfgs = []
     T = thc.Tensor
+    host = {}
 
     def want(*names):
         return not only or any(n in only for n in names)
 
-    def c2():
-        n = 8192
-        a = rng.standard_normal((n, n), dtype=np.float32)
-        b = rng.standard_normal((n, n), dtype=np.float32)
-        d = rng.standard_normal((n, n), dtype=np.float32)
-        da, db, dd = T.from_numpy(a), T.from_numpy(b), T.from_numpy(d)
-        at = da.t()
-        out = T("float").resize((n, n))
+    # C2: out = a:t() * b + d. Headline = out and d rotating over three buffer sets.
+    n2 = 8192
+    a2 = rng.standard_normal((n2, n2), dtype=np.float32)
+    b2 = rng.standard_normal((n2, n2), dtype=np.float32)
+    d2 = [rng.standard_normal((n2, n2), dtype=np.float32)]
+    da, db = T.from_numpy(a2), T.from_numpy(b2)
+    at = da.t()
+    dd = [T.from_numpy(d2[0])]
+    out2 = [T("float").resize((n2, n2))]
+    for k in (1, 2):      # the other two d buffers are shifted copies of the first (set up on the host once)
+        d2.append(np.roll(d2[0], k * 1237, axis=1))
+        dd.append(T.from_numpy(d2[k]))
+        out2.append(T("float").resize((n2, n2)))
 
-        def run(i):
-            out.addcmul(dd, 1.0, at, db)
-
+    def c2_check(k):
         def check():
-            got = out.numpy()
-            rows = np.array([0, 1, 63, 64, 4097, 8191])
-            want = (a.T[rows] * b[rows]).astype(np.float32) + d[rows]
-            return bool(np.array_equal(got[rows].view(np.uint32), want.view(np.uint32)))
-        host = (a, b, d)
-        return Config("C2", "out = a:t()*b + d, 8192x8192 fp32, a stride (1,8192) [addcmul]",
-                      16 * n * n, n * n, 1, run, check), host
-
-    primary, host_c2 = c2()
-    cfgs.append(primary)
+            out2[k].fill(0.0)
+            out2[k].addcmul(dd[k], 1.0, at, db)
+            want_ = a2.T * b2
+            want_ += d2[k]
+            return bit_equal(out2[k].numpy(), want_)
+        return check
+    desc2 = "out = a:t()*b + d, 8192x8192 fp32, a stride (1,8192) [addcmul]"
+    cfgs.append(Config("C2", desc2 + ", out and d rotate over 3 buffer sets", 16 * n2 * n2, n2 * n2, 3,
+                       lambda i: out2[i % 3].addcmul(dd[i % 3], 1.0, at, db), c2_check(2)))
+    host["C2"] = (a2, b2, d2[0])
     if which == "primary":
-        return cfgs, host_c2
+        return cfgs, host
+    cfgs.append(Config("C2-fixed", desc2 + ", one buffer set (the output is rewritten in place every step)",
+                       16 * n2 * n2, n2 * n2, 1, lambda i: out2[0].addcmul(dd[0], 1.0, at, db), c2_check(0)))
 
     # C1: contiguous 2^24, three rotating buffer sets (working set < Infinity Cache)
     n1 = 1 << 24
-    sets1 = []
-    for _ in range(3 if want('C1-add', 'C1-mul') else 0):
-        a = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
-        b = T.from_numpy(rng.uniform(-1, 1, n1).astype(np.float32))
-        sets1.append((a, b, T("float").resize((n1,))))
-    cfgs.append(Config("C1-add", "c = a + b, 2^24 fp32 contiguous [cadd]", 12 * n1, n1, 3,
-                       lambda i: sets1[i % 3][2].cadd(sets1[i % 3][0], 1.0, sets1[i % 3][1])))
-    cfgs.append(Config("C1-mul", "c = a * b, 2^24 fp32 contiguous [cmul]", 12 * n1, n1, 3,
-                       lambda i: sets1[i % 3][2].cmul(sets1[i % 3][0], sets1[i % 3][1])))
+    sets1, h1 = [], None
+    for k in range(3 if want('C1-add', 'C1-mul') else 0):
+        ha, hb = rng.uniform(-1, 1, n1).astype(np.float32), rng.uniform(-1, 1, n1).astype(np.float32)
+        if k == 0:
+            h1 = (ha, hb)
+        sets1.append((T.from_numpy(ha), T.from_numpy(hb), T("float").resize((n1,))))
 
-    # C3a/b: 65536 x 1024, last dim
+    def c1_check(op):
+        def check():
+            a, b, c = sets1[0]
+            c.fill(0.0)
+            (c.cadd(a, 1.0, b) if op == "add" else c.cmul(a, b))
+            return bit_equal(c.numpy(), h1[0] + h1[1] if op == "add" else h1[0] * h1[1])
+        return check
+    cfgs.append(Config("C1-add", "c = a + b, 2^24 fp32 contiguous [cadd]", 12 * n1, n1, 3,
+                       lambda i: sets1[i % 3][2].cadd(sets1[i % 3][0], 1.0, sets1[i % 3][1]), c1_check("add")))
+    cfgs.append(Config("C1-mul", "c = a * b, 2^24 fp32 contiguous [cmul]", 12 * n1, n1, 3,
+                       lambda i: sets1[i % 3][2].cmul(sets1[i % 3][0], sets1[i % 3][1]), c1_check("mul")))
+
+    # C3a/b: 65536 x 1024, last dim; ~1 % of every row are copies of other entries of the row,
+    # one of them a copy of the row maximum (so that argmax has a tie to resolve)
     r3, n3 = 65536, 1024
-    sets3 = []
-    for _ in range(3 if want('C3a-sum', 'C3b-max') else 0):
+    sets3, h3 = [], None
+    for k in range(3 if want('C3a-sum', 'C3b-max') else 0):
         x = rng.standard_normal((r3, n3), dtype=np.float32)
+        rows = np.arange(r3)
         dup = rng.integers(0, n3, (r3, 10))
-        x[np.arange(r3)[:, None], dup] = x[np.arange(r3)[:, None], dup[:, ::-1]]
+        x[rows[:, None], dup] = x[rows[:, None], dup[:, ::-1]]
+        x[rows, rng.integers(0, n3, r3)] = x.max(axis=1)
+        if k == 0:
+            h3 = x
         sets3.append((T.from_numpy(x), T("float").resize((r3, 1)), T("long").resize((r3, 1))))
+
+    def c3a_check():
+        x, o, _ = sets3[0]
+        o.fill(0.0)
+        o.sum(x, 1)
+        return sums_close(o.numpy(), h3.sum(axis=1, dtype=np.float64), np.abs(h3).sum(axis=1, dtype=np.float64), 1e-5)
+
+    def c3b_check():
+        x, o, ix = sets3[0]
+        o.fill(0.0)
+        o.max(ix, x, 1)
+        am = h3.argmax(axis=1)                   # numpy returns the first occurrence
+        return (bit_equal(o.numpy().reshape(-1), h3[np.arange(r3), am])
+                and bool(np.array_equal(ix.numpy().reshape(-1), am + 1)))
     cfgs.append(Config("C3a-sum", "sum over last dim of 65536x1024 fp32", 4 * r3 * n3 + 4 * r3, r3 * n3,
-                       3, lambda i: sets3[i % 3][1].sum(sets3[i % 3][0], 1)))
+                       3, lambda i: sets3[i % 3][1].sum(sets3[i % 3][0], 1), c3a_check))
     cfgs.append(Config("C3b-max", "max+argmax over last dim of 65536x1024 fp32",
                        4 * r3 * n3 + 12 * r3, r3 * n3, 3,
-                       lambda i: sets3[i % 3][1].max(sets3[i % 3][2], sets3[i % 3][0], 1)))
+                       lambda i: sets3[i % 3][1].max(sets3[i % 3][2], sets3[i % 3][0], 1), c3b_check))
+    host["C3a-sum"] = h3
 
     # C3c: reduceAll over 2^28
     n3c = 1 << 28
-    xa = T.from_numpy(rng.random(n3c if want('C3c-sumall', 'N-fill') else 4, dtype=np.float32))
+    h3c = rng.random(n3c if want('C3c-sumall', 'N-fill') else 4, dtype=np.float32)
+    xa = T.from_numpy(h3c)
+    ref3c = float(h3c.sum(dtype=np.float64))
+
+    def c3c_check():
+        return sums_close([xa.sumall()], [ref3c], [ref3c], 1e-5)      # all summands are positive: mass = sum
     cfgs.append(Config("C3c-sumall", "sumall over 2^28 fp32 (blocks on a 4-byte D2H copy)",
-                       4 * n3c + 4, n3c, 1, lambda i: xa.sumall()))
+                       4 * n3c + 4, n3c, 1, lambda i: xa.sumall(), c3c_check))
 
     # C4: 64 x 4096 x 512, middle dim; fp32 and fp16
     s4 = (64, 4096, 512) if want('C4-sum-f32', 'C4-norm-f32', 'C4-sum-f16', 'C4-norm-f16', 'N-std-cols', 'N-cumsum-cols') else (1, 4, 8)
@@ -165,20 +236,56 @@ def build_configs(thc, hip, which, only=None):
     d4 = T.from_numpy(x4)
     o4 = T("float").resize((s4[0], 1, s4[2]))
     n4 = int(np.prod(s4))
+
+    def c4_check(kind, half):
+        def check():
+            if half:
+                x, o = sets4h[0]
+                hx = h4h.astype(np.float32)
+            else:
+                x, o, hx = d4, o4, x4
+            o.fill(0.0)
+            (o.sum(x, 1) if kind == "sum" else o.norm(x, 2.0, 1))
+            got = o.numpy().astype(np.float64)
+            if kind == "sum":
+                ref, mass = hx.sum(axis=1, dtype=np.float64), np.abs(hx).sum(axis=1, dtype=np.float64)
+            else:
+                ref = np.sqrt(np.square(hx.astype(np.float64)).sum(axis=1))
+                mass = ref
+            return sums_close(got, ref, mass, 2e-3 if half else 1e-5)
+        return check
     cfgs.append(Config("C4-sum-f32", "sum over middle dim of 64x4096x512 fp32", 4 * n4 + 4 * s4[0] * s4[2],
-                       n4, 1, lambda i: o4.sum(d4, 1)))
+                       n4, 1, lambda i: o4.sum(d4, 1), c4_check("sum", False)))
     cfgs.append(Config("C4-norm-f32", "L2 norm over middle dim of 64x4096x512 fp32",
-                       4 * n4 + 4 * s4[0] * s4[2], n4, 1, lambda i: o4.norm(d4, 2.0, 1)))
-    sets4h = []
-    for _ in range(3):
-        h = T.from_numpy((x4 * np.float32(rng.uniform(0.5, 1.0))).astype(np.float16))
-        sets4h.append((h, T("half").resize((s4[0], 1, s4[2]))))
+                       4 * n4 + 4 * s4[0] * s4[2], n4, 1, lambda i: o4.norm(d4, 2.0, 1), c4_check("norm", False)))
+    sets4h, h4h = [], None
+    for k in range(3):
+        hh = (x4 * np.float32(rng.uniform(0.5, 1.0))).astype(np.float16)
+        if k == 0:
+            h4h = hh
+        sets4h.append((T.from_numpy(hh), T("half").resize((s4[0], 1, s4[2]))))
     cfgs.append(Config("C4-sum-f16", "sum over middle dim of 64x4096x512 fp16, fp32 accumulate",
-                       2 * n4 + 2 * s4[0] * s4[2], n4, 3, lambda i: sets4h[i % 3][1].sum(sets4h[i % 3][0], 1)))
+                       2 * n4 + 2 * s4[0] * s4[2], n4, 3, lambda i: sets4h[i % 3][1].sum(sets4h[i % 3][0], 1),
+                       c4_check("sum", True)))
     cfgs.append(Config("C4-norm-f16", "L2 norm over middle dim of 64x4096x512 fp16, fp32 accumulate",
                        2 * n4 + 2 * s4[0] * s4[2], n4, 3,
-                       lambda i: sets4h[i % 3][1].norm(sets4h[i % 3][0], 2.0, 1)))
+                       lambda i: sets4h[i % 3][1].norm(sets4h[i % 3][0], 2.0, 1), c4_check("norm", True)))
+    host["C4-sum-f32"] = x4
 
+    # A plain 1-read-1-write stream of known size: out = src + 0 on 2^26 contiguous fp32 (reads 256 MiB,
+    # writes 256 MiB). About 0.88-0.90 of peak on a healthy box; a box that runs write-heavy kernels slowly
+    # shows here first.
+    nc = 1 << 26
+    if want("CAL-copy"):
+        hcal = rng.uniform(-1, 1, nc).astype(np.float32)
+        csrc, cdst = T.from_numpy(hcal), T("float").resize((nc,))
+
+        def cal_check():
+            cdst.fill(1.0)
+            cdst.add(csrc, 0.0)
+            return bit_equal(cdst.numpy(), hcal + np.float32(0.0))
+        cfgs.append(Config("CAL-copy", "out = src + 0, 2^26 fp32 contiguous (1 read + 1 write of 256 MiB each)",
+                           8 * nc, nc, 1, lambda i: cdst.add(csrc, 0.0), cal_check))
     # Neighbours of the hot path on the same engines (same operands where possible).
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
@@ -189,8 +296,7 @@ def build_configs(thc, hip, which, only=None):
         ne = 1 << 26
         e_src = T.from_numpy(rng.uniform(-1, 1, ne).astype(np.float32))
         e_dst = T("float").resize((ne,))
-        sq = T.from_numpy(rng.standard_normal((8192, 8192), dtype=np.float32))
-        sq_t, sq_out = sq.t(), T("float").resize((8192, 8192))
+        sq, sq_t, sq_out = da, at, out2[0]
         x3 = sets3[0][0] if sets3 else T.from_numpy(rng.standard_normal((r3, n3), dtype=np.float32))
         o3 = T("float").resize((r3, 1))
         s3 = T("float").resize((r3, n3))
@@ -267,18 +373,32 @@ def build_configs(thc, hip, which, only=None):
             d, nb, el, fn = table[n]
             cfgs.append(Config(n, d, nb, el, 1, fn))
 
-    # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path
+    # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path. The 8.7 GB operands repeat
+    # a 2^24-element block of normal(0,1) values (the element at storage offset o is block[o % 2^24]).
     if not want('C5'):
-        return [c for c in cfgs if c is cfgs[0] or want(c.name)], host_c2
-    block = rng.standard_normal(1 << 24, dtype=np.float32)
+        return [c for c in cfgs if c is cfgs[0] or want(c.name)], host
+    nb = 1 << 24
+    block = rng.standard_normal(nb, dtype=np.float32)
+    rblock = block[::-1].copy()
     a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
-    b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), block[::-1].copy())
+    b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), rblock)
     c5 = T("float").resize((2048, 2048, 520))
     a5v = a5.view_as_strided(0, (2048, 2048, 520), (1, 2048, 2048 * 2048))
     n5 = 2048 * 2048 * 520
+
+    def c5_check():
+        ok = True
+        j, k = np.arange(2048, dtype=np.int64)[:, None], np.arange(520, dtype=np.int64)[None, :]
+        for i in (0, 1, 1023, 2047):             # whole [j][k] planes of the output, first to last
+            got = c5.select(0, i).numpy()
+            wa = block[(i + 2048 * j + 2048 * 2048 * k) % nb]
+            wb = rblock[((i * 2048 + j) * 520 + k) % nb]
+            ok = ok and bit_equal(got, wa + wb)
+        return ok
     cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
-                       12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5)))
-    return cfgs, host_c2
+                       12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5), c5_check))
+    cfgs[-1].note = "parity on 4 of the 2048 output planes"
+    return [c for c in cfgs if c is cfgs[0] or want(c.name)], host
 
 
 def time_config(hip, thc, cfg, steps, warmup, stream):
@@ -311,29 +431,41 @@ def time_config(hip, thc, cfg, steps, warmup, stream):
     return wall, region_ms, ms
 
 
-def cpu_baseline(host, nbytes, budget_s=24.0):
-    """Times the CPU restatement of out = a:t()*b + d on the full 8192x8192
-    operands: single thread (the reported baseline) and all cores."""
+def cpu_baseline(host, cfg_bytes, budget_s=24.0):
+    """Times the CPU restatement on this box's host cores, single thread and all
+    cores: the headline workload out = a:t()*b + d on the full 8192x8192
+    operands (TH_TENSOR_APPLY path) and, for the reduction path, the row sums
+    of 65536x1024 and the middle-dim sums of 64x4096x512. Every figure is the
+    median of the runs after the first, GB/s on the algorithmic bytes."""
     from oracle import th_oracle as oracle
-    a, b, d = host
-    n = a.shape[0]
-    va = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
-    vb, vd = oracle.View(b.reshape(-1)), oracle.View(d.reshape(-1))
-    vb = oracle.View(vb.storage, 0, (n, n))
-    vd = oracle.View(vd.storage, 0, (n, n))
-    out = oracle.View.empty((n, n))
-    res = {}
     cores = len(os.sched_getaffinity(0))
-    for label, threads in (("single", 1), ("all", cores)):
-        oracle.set_num_threads(threads)
-        times = []
-        t_start = time.perf_counter()
-        while len(times) < 26 and (time.perf_counter() - t_start) < budget_s / 2:   # ~10 s single thread
-            t0 = time.perf_counter()
-            oracle.pointwise("addcmul", out, vd, va, vb, value=1.0)
-            times.append(time.perf_counter() - t0)
-        best = times[1:] if len(times) > 1 else times
-        res[label] = (nbytes / float(np.median(best)) / 1e9, threads, len(times))
+    jobs = []
+    if "C2" in host and "C2" in cfg_bytes:
+        a, b, d = host["C2"]
+        n = a.shape[0]
+        va = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
+        vb, vd = oracle.View(b.reshape(-1), 0, (n, n)), oracle.View(d.reshape(-1), 0, (n, n))
+        out = oracle.View.empty((n, n))
+        jobs.append(("C2", 0.5, lambda: oracle.pointwise("addcmul", out, vd, va, vb, value=1.0)))
+    if host.get("C3a-sum") is not None and "C3a-sum" in cfg_bytes:
+        x = host["C3a-sum"]
+        vx, o3 = oracle.View(x.reshape(-1), 0, x.shape), oracle.View.empty((x.shape[0], 1))
+        jobs.append(("C3a-sum", 0.2, lambda: oracle.reduce_dim("sum", vx, 1, out=o3)))
+    if host.get("C4-sum-f32") is not None and host["C4-sum-f32"].size > 64 and "C4-sum-f32" in cfg_bytes:
+        x4 = host["C4-sum-f32"]
+        v4, o4 = oracle.View(x4.reshape(-1), 0, x4.shape), oracle.View.empty((x4.shape[0], 1, x4.shape[2]))
+        jobs.append(("C4-sum-f32", 0.3, lambda: oracle.reduce_dim("sum", v4, 1, out=o4)))
+    res = {}
+    for name, share, fn in jobs:
+        res[name] = {}
+        for label, threads, part in (("single", 1, 0.7), ("all", cores, 0.3)):
+            oracle.set_num_threads(threads)
+            times, t_start = [], time.perf_counter()
+            while len(times) < 26 and (len(times) < 3 or time.perf_counter() - t_start < budget_s * share * part):
+                t0 = time.perf_counter()
+                fn()
+                times.append(time.perf_counter() - t0)
+            res[name][label] = (cfg_bytes[name] / float(np.median(times[1:])) / 1e9, threads, len(times) - 1)
     oracle.set_num_threads(1)
     return res
 
@@ -343,11 +475,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--configs", default="all", choices=["all", "primary"])
+    ap.add_argument("--configs", default="bar", choices=["bar", "all", "primary"],
+                    help="bar: the benchmark configurations + calibration stream (default); all: also the "
+                         "neighbouring ops (N-*) and full detail; primary: the headline only")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="skip the per-configuration parity checks")
     ap.add_argument("--only", default="", help="comma-separated config names to measure")
-    ap.add_argument("--calibrate", action="store_true",
-                    help="also run a plain 1-read-1-write stream of known size (counter calibration)")
     ap.add_argument("--tune", action="append", default=[], help="engine tuning knob key=value")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -361,21 +494,14 @@ def main():
         k, v = kv.split("=")
         thc.set_tuning(k, int(v))
     only = set(args.only.split(",")) if args.only else None
-    cfgs, host_c2 = build_configs(thc, hip, args.configs, only)
+    cfgs, host = build_configs(thc, hip, args.configs, only)
     if only:
         cfgs = [cfgs[0]] + [c for c in cfgs[1:] if c.name in only]
-    if args.calibrate:
-        # out = src + 0 on 2^26 contiguous fp32: reads 256 MiB, writes 256 MiB.
-        nc = 1 << 26
-        csrc = thc.Tensor.from_numpy(np.ones(nc, np.float32))
-        cdst = thc.Tensor("float").resize((nc,))
-        cfgs.append(Config("CAL-copy", "out = src + 0, 2^26 fp32 contiguous (1 read + 1 write of 256 MiB each)",
-                           8 * nc, nc, 1, lambda i: cdst.add(csrc, 0.0)))
     results = []
     for cfg in cfgs:
         steps = args.steps if cfg.name != "C5" else max(3, args.steps // 5)
         wall, region_ms, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
-        ok = cfg.check() if cfg.check else None
+        ok = None if (args.no_check or cfg.check is None) else bool(cfg.check())
         mean_ms = region_ms / steps
         results.append({
             "name": cfg.name, "desc": cfg.desc, "kernel": cfg.kernel, "steps": steps,
@@ -387,18 +513,27 @@ def main():
             "frac_of_peak": round(cfg.nbytes / mean_ms / 1e6 / PEAK_GBPS, 4),
             "gelem_per_s": round(cfg.elements / mean_ms / 1e6, 2),
             "wall_gbps": round(cfg.nbytes * steps / wall / 1e9, 1),
-            "rotating_sets": cfg.sets, "parity_sample_ok": ok,
+            "rotating_sets": cfg.sets, "parity_ok": ok, "note": cfg.note,
         })
     p = results[0]
-    traffic = None   # HBM bytes per launch from the committed rocprofv3 --pmc summary, if any
+    traffic, traffic_src = None, None   # HBM bytes per launch from the committed rocprofv3 --pmc summary
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             measured = json.load(f)
-        traffic = measured.get(cfgs[0].name, {}).get("traffic_bytes")
+        traffic = measured.get("C2", {}).get("traffic_bytes")
+        traffic_src = "profiles/traffic.json (committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary; not measured in this run)"
         for r in results:
             r["traffic_bytes"] = measured.get(r["name"], {}).get("traffic_bytes")
     except (OSError, ValueError):
         pass
+    compact = {}
+    for r in results:
+        compact[r["name"]] = {"frac": r["frac_of_peak"], "us": round(1e3 * r["ms_mean"], 2),
+                              "us_min": round(1e3 * r["ms_min"], 2), "gbps": r["gbps_mean"],
+                              "gelem_s": r["gelem_per_s"], "parity": r["parity_ok"], "kernel": r["kernel"],
+                              "sets": r["rotating_sets"]}
+        if r["note"]:
+            compact[r["name"]]["note"] = r["note"]
     line = {
         "metric": METRIC, "value": p["wall_gbps"], "unit": "GB/s", "n_gpus": 1,
         "steps": p["steps"], "warmup": args.warmup,
@@ -406,19 +541,26 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (fixed-seed host generator, copied to HBM before timing)",
         "config": {"workload": p["desc"], "elements": cfgs[0].elements, "kernel": p["kernel"],
-                   "parity_sample_ok": p["parity_sample_ok"]},
+                   "parity_ok": p["parity_ok"]},
         "roofline": {"bound": "hbm", "achieved": p["gbps_mean"], "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": p["frac_of_peak"], "traffic": traffic},
-        "all_configs": results,
+                     "frac": p["frac_of_peak"], "traffic": traffic, "traffic_source": traffic_src,
+                     "configs": compact},
     }
     if not args.no_cpu:
-        cb = cpu_baseline(host_c2, cfgs[0].nbytes)
+        cb = cpu_baseline(host, {c.name: c.nbytes for c in cfgs})
+        per = {}
+        for name, r in cb.items():
+            per[name] = {"single_gbps": round(r["single"][0], 2), "all_cores_gbps": round(r["all"][0], 2),
+                         "cores": r["all"][1], "runs": [r["single"][2], r["all"][2]]}
+        head = cb.get("C2")
         line["cpu_baseline"] = {
-            "value": round(cb["single"][0], 2), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "full workload (8192x8192 addcmul with transposed operand), median of %d runs"
-                      % max(1, cb["single"][2] - 1)}
-        line["cpu_baseline_all_cores"] = {"value": round(cb["all"][0], 2), "unit": "GB/s",
-                                          "cores": cb["all"][1], "kind": "port"}
+            "value": round(head["single"][0], 2) if head else None, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "full workload (8192x8192 addcmul with transposed operand), median of %d runs; "
+                      "\"configs\" holds the same for the reduction path (C3a row sums, C4 middle-dim sums), "
+                      "single thread and all cores" % (head["single"][2] if head else 0),
+            "configs": per}
+    if args.configs == "all":
+        line["all_configs"] = results
     print(json.dumps(line))
 
 
