@@ -45,9 +45,16 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+# headers only some sources include (touching one rebuilds only those)
+EXTRA_DEPS = {"caching_allocator.cpp": ["caching_pool.hpp", "stream_guard.hpp"],
+              "general.cpp": ["stream_guard.hpp"], "tensor.cpp": ["stream_guard.hpp"],
+              "apply.hip": ["stream_guard.hpp"], "reduce.hip": ["stream_guard.hpp"],
+              "scan.hip": ["stream_guard.hpp"], "convert.hip": ["stream_guard.hpp"]}
+
+
 def _compile(src, force):
     obj = os.path.join(BUILD, src + ".o")
-    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS]
+    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS + EXTRA_DEPS.get(src, [])]
     if not force and not _stale(obj, deps):
         return obj
     cmd = [_hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS

@@ -9,6 +9,7 @@
 #include <algorithm>
 #include "apply_plan.hpp"
 #include "common.hpp"
+#include "stream_guard.hpp"
 #include "device_util.hpp"
 
 namespace thc {
@@ -57,6 +58,7 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     if (t[k]->nDimension > kMaxDims) return false;      // :441-445
   }
   if (out->nDimension == 0) return true;                // :447-450
+  note_stream_use(s, {out, in0, in1, in2});
 
   // An output that addresses one element through several indices is computed
   // into a dense temporary and copied back, last writer wins (:472-489).
@@ -174,6 +176,7 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
   const ptrdiff_t n = tensor_numel(dst);
   THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
   if (dst->nDimension == 0) return;
+  note_stream_use(s, {dst, src});
   if ((tensor_is_contiguous(dst) && tensor_is_contiguous(src)) || n == 1) {
     THC_CHECK(hipMemcpyAsync(tensor_data(dst, dt), tensor_data(src, dt), (size_t)n * dtype_size(dt),
                              hipMemcpyDeviceToDevice, current_stream(s)));

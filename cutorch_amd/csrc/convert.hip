@@ -12,6 +12,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "stream_guard.hpp"
 #include "device_util.hpp"
 
 namespace thc {
@@ -103,6 +104,7 @@ void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor
   const ptrdiff_t n = tensor_numel(dst);
   THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
   if (n == 0) return;
+  note_stream_use(s, {dst, src});
   // The flat kernel pairs elements by logical linear index, which is what a
   // dense tensor's memory order is.
   TensorRef cs(s, tensor_new_contiguous(s, src, srcT));

@@ -12,6 +12,7 @@
 #include <string>
 
 #include "common.hpp"
+#include "stream_guard.hpp"
 
 struct THCState {
   bool initialised = false;
@@ -36,6 +37,9 @@ thread_local std::string t_last_error;
 thread_local const char* t_last_kernel = "";
 thread_local hipStream_t t_stream = nullptr;
 int g_force64 = 0;
+// Set once a stream other than the default one has been made current: from then
+// on operands are reported to the caching allocator on every launch.
+std::atomic<bool> g_multi_stream{false};
 
 // Tuning knobs: a small append-only table, read without locks on every launch.
 struct Knob {
@@ -142,6 +146,15 @@ void check_same_gpu(THCState* s, int n, const AnyTensor* const* ts) {
   }
 }
 
+void note_stream_use(THCState* s, std::initializer_list<const AnyTensor*> ts) {
+  if (!g_multi_stream.load(std::memory_order_relaxed)) return;
+  const THCDeviceAllocator* caching = THCCachingAllocator_get();
+  hipStream_t st = current_stream(s);
+  for (const AnyTensor* t : ts)
+    if (t && t->storage && t->storage->data && t->storage->allocator == caching)
+      caching_record_stream(t->storage->data, st);
+}
+
 void note_kernel(const char* name) { t_last_kernel = name; }
 bool force_64bit_index() { return g_force64 != 0; }
 
@@ -223,6 +236,7 @@ THC_API hipStream_t_ THCState_getCurrentStream(THCState* state) {
   return (hipStream_t_)current_stream(state);
 }
 THC_API void THCState_setCurrentStream(THCState*, hipStream_t_ stream) {
+  if (stream != nullptr) g_multi_stream.store(true, std::memory_order_relaxed);
   t_stream = (hipStream_t)stream;
 }
 THC_API void* THCState_getCurrentDeviceScratchSpace(THCState* state) {

@@ -9,6 +9,7 @@
 #include <limits>
 
 #include "reduce_plan.hpp"
+#include "stream_guard.hpp"
 
 namespace thc {
 
@@ -78,6 +79,7 @@ bool reduce_dim(THCState* s, DType dt, ReduceOp op, Epilogue ep, double p, AnyTe
     return true;
   }
   resize_reduced(s, out, in, dim, dt);
+  note_stream_use(s, {out, in});
   ReduceGeom g = make_geom(in, out, nullptr, dim);
   double epArg = 0.0;
   if (ep == Epilogue::PowInv) epArg = dt == DType::F64 ? 1.0 / p : (double)(1.0f / (float)p);
@@ -107,6 +109,7 @@ bool reduce_var_fast(THCState* s, DType dt, AnyTensor* out, AnyTensor* in, int d
   if (out->storage && out->storage == in->storage) return false;
   const long n = in->size[dim];
   resize_reduced(s, out, in, dim, dt);
+  note_stream_use(s, {out, in});
   ReduceGeom g = make_geom(in, out, nullptr, dim);
   const double div = (double)(biased ? n : n - 1);
   bool done = false;
@@ -141,6 +144,7 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
   }
   resize_reduced(s, values, in, dim, dt);
   resize_reduced(s, indices, in, dim, DType::I64);
+  note_stream_use(s, {values, indices, in});
   ReduceGeom g = make_geom(in, values, indices, dim);
   const void* ip = tensor_data(in, dt);
   void* vp = tensor_data(values, dt);
@@ -168,6 +172,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Sca
     *result = init;
     return true;
   }
+  note_stream_use(s, {in});
   // View the tensor as rows of its innermost collapsed dim; a tensor whose
   // innermost dim is strided is densified first.
   Layout l = tensor_layout(in);
@@ -207,6 +212,7 @@ bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a,
   if (!tensor_is_contiguous(a) || !tensor_is_contiguous(b)) return false;
   const int64_t n = tensor_numel(a);
   if (n != tensor_numel(b)) return false;
+  note_stream_use(s, {a, b});
   ReduceGeom g{};
   g.wide = force_64bit_index() || n >= kIndex32Limit;
   g.R = n;
@@ -227,6 +233,7 @@ bool renorm_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* src, double p
   if (!tensor_is_contiguous(src) || !tensor_is_contiguous(out) || tensor_numel(out) != tensor_numel(src)) return false;
   const int64_t rows = src->size[0], R = tensor_numel(src) / std::max<int64_t>(rows, 1);
   if (rows < 1 || R < 1) return false;
+  note_stream_use(s, {out, src});
   const void* ip = tensor_data(src, dt);
   void* op = tensor_data(out, dt);
   if (dt == DType::F32) return renorm_rows_type<float>(s, rows, R, ip, op, p, maxnorm);
@@ -239,6 +246,7 @@ bool reduce_all_moments(THCState* s, DType dt, AnyTensor* in, Scalar* result) {
   if (!tensor_is_contiguous(in) || !tuning("reduce.all.moments", 1)) return false;
   const int64_t n = tensor_numel(in);
   if (n < 1) return false;
+  note_stream_use(s, {in});
   const void* p = tensor_data(in, dt);
   if (dt == DType::F32) reduce_all_moments_type<float>(s, n, p, result);
   else if (dt == DType::F16) reduce_all_moments_type<__half>(s, n, p, result);

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "stream_guard.hpp"
 
 struct THCState;
 
@@ -71,7 +72,11 @@ void storage_resize(THCState* s, AnyStorage* st, ptrdiff_t size, DType dt) {
     }
   }
   if (st->data) {
-    // hipFree waits for outstanding work, so the copy above has landed.
+    // The copy above is still in flight on the current stream. Plain hipFree waits
+    // for the device; the caching allocator parks the block for the stream it was
+    // allocated on, so a copy on any other stream is reported to it first (the
+    // block is then held back behind an event on that stream).
+    caching_record_stream(st->data, current_stream(s));
     THC_CHECK((hipError_t)st->allocator->free(st->allocatorContext, st->data));
   }
   st->data = fresh;
@@ -296,6 +301,10 @@ static void tensor_copy_from_host(THCState* s, AnyTensor* self, const void* src,
   const ptrdiff_t n = tensor_numel(self);
   if (n == 0) return;
   const size_t bytes = (size_t)n * dtype_size(dt);
+  // The copies below run on the null stream: work queued on the current stream
+  // (a non-blocking one does not order itself against the null stream) may still
+  // read the destination, or the block a fresh temporary was recycled from.
+  THC_CHECK(hipStreamSynchronize(current_stream(s)));
   if (tensor_is_contiguous(self)) {
     THC_CHECK(hipMemcpy(tensor_data(self, dt), src, bytes, hipMemcpyHostToDevice));
     return;

@@ -78,6 +78,16 @@ THC_API int THCState_isCachingAllocatorEnabled(THCState *state);
 THC_API struct _THCDeviceAllocator *THCCachingAllocator_get(void);
 THC_API int THCudaMemGetInfoCached(THCState *state, size_t *freeBytes, size_t *totalBytes,
                                    size_t *largestBlock);
+/* `ptr` (the start of a block handed out by the caching allocator) is used by
+ * work queued on `stream`, which is not the stream it was allocated for: when
+ * the block is freed it is held back until that work has completed
+ * (lib/THC/THCCachingAllocator.h:13, THCCachingAllocator.cpp:221-240; the
+ * stream is a raw HIP stream here, as for THCState_setCurrentStream). The
+ * engine's own entry points report their operands themselves; a host calls
+ * this for work it launches on its own streams. Other pointers are ignored. */
+THC_API void THCCachingAllocator_recordStream(void *ptr, hipStream_t_ stream);
+/* Blocks freed but still held back behind such events (diagnostic). */
+THC_API size_t THCAmd_cachingAllocatorPendingBlocks(void);
 
 /* Diagnostics with no counterpart in the reference. */
 THC_API int THCAmd_getNumComputeUnits(THCState *state);

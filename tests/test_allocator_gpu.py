@@ -53,3 +53,115 @@ def test_plain_allocator_can_be_selected(thc):
     lib.THCudaTensor_free(st, t)
     lib.THCudaShutdown(st)
     lib.THCState_free(st)
+
+
+@pytest.fixture()
+def nonblocking_streams(thc):
+    """Two streams that do not synchronise with the default stream."""
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamCreateWithFlags.argtypes = [C.POINTER(C.c_void_p), C.c_uint]
+    hip.hipStreamDestroy.argtypes = [C.c_void_p]
+    hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+    made = []
+    for _ in range(2):
+        s = C.c_void_p()
+        assert hip.hipStreamCreateWithFlags(C.byref(s), 1) == 0      # hipStreamNonBlocking, default priority
+        made.append(s)
+    yield hip, made
+    for s in made:
+        assert hip.hipStreamSynchronize(s) == 0
+    thc.lib().THCState_setCurrentStream(thc.state(), None)
+    thc.synchronize()
+    for s in made:
+        hip.hipStreamDestroy(s)
+
+
+def _busy(thc, w, launches):
+    """Queues `launches` passes over the 1 GiB tensor w on the current stream (a few ms of work)."""
+    for _ in range(launches):
+        w.add(w, 1.0)
+
+
+def test_block_used_on_another_stream_is_held_back(thc, nonblocking_streams):
+    """Allocated under stream A, read by work queued on stream B, freed: the block may not serve a new
+    request on A (which would overwrite it at once) until B's work has completed."""
+    hip, (sa, sb) = nonblocking_streams
+    lib, st = thc.lib(), thc.state()
+    lib.THCAmd_cachingAllocatorPendingBlocks.restype = C.c_size_t
+    n = (1 << 24) + 12345
+    lib.THCState_setCurrentStream(st, sa)
+    x = thc.Tensor("float").resize((n,)).fill(1.0)
+    px = x.data_ptr()
+    assert hip.hipStreamSynchronize(sa) == 0
+    lib.THCState_setCurrentStream(st, sb)
+    w = thc.Tensor("float").resize((1 << 28,)).fill(0.0)
+    r = thc.Tensor("float").resize((n,))
+    _busy(thc, w, 40)                                  # stream B is busy for a while ...
+    r.copy(x)                                          # ... and only then reads x
+    del x                                              # freed while B's copy has not even started
+    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 1
+    lib.THCState_setCurrentStream(st, sa)
+    z = thc.Tensor("float").resize((n,))
+    assert z.data_ptr() != px                          # not handed out while B may still read it
+    z.fill(7.0)                                        # runs on A at once, concurrently with B
+    assert hip.hipStreamSynchronize(sa) == 0 and hip.hipStreamSynchronize(sb) == 0
+    assert np.all(r.numpy() == 1.0)
+    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 0
+    z2 = thc.Tensor("float").resize((n,))             # B has caught up: the block is back in A's pool
+    assert z2.data_ptr() == px
+    assert w.narrow(0, 12345, 4).numpy().tolist() == [40.0] * 4
+
+
+def test_record_stream_entry_point_and_resize_on_another_stream(thc, nonblocking_streams):
+    hip, (sa, sb) = nonblocking_streams
+    lib, st = thc.lib(), thc.state()
+    lib.THCAmd_cachingAllocatorPendingBlocks.restype = C.c_size_t
+    lib.THCCachingAllocator_recordStream.argtypes = [C.c_void_p, C.c_void_p]
+    lib.THCState_setCurrentStream(st, sb)
+    w = thc.Tensor("float").resize((1 << 28,)).fill(0.0)
+    # a host that launches its own work on B reports the use itself
+    lib.THCState_setCurrentStream(st, sa)
+    y = thc.Tensor("float").resize((1 << 22,)).fill(2.0)
+    py = y.data_ptr()
+    lib.THCState_setCurrentStream(st, sb)
+    _busy(thc, w, 20)
+    lib.THCCachingAllocator_recordStream(C.c_void_p(py), sb)
+    lib.THCState_setCurrentStream(st, sa)
+    del y
+    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 1
+    assert thc.Tensor("float").resize((1 << 22,)).data_ptr() != py
+    assert hip.hipStreamSynchronize(sb) == 0
+    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 0
+    # resize on a stream other than the block's own: the old block is copied from on B, then freed
+    lib.THCState_setCurrentStream(st, sa)
+    t = thc.Tensor.from_numpy(np.arange(1 << 20, dtype=np.float32))
+    pt = t.data_ptr()
+    assert hip.hipStreamSynchronize(sa) == 0
+    lib.THCState_setCurrentStream(st, sb)
+    _busy(thc, w, 20)
+    t.resize((1 << 21,))                               # storage grows: copy of the old contents queued on B
+    assert t.data_ptr() != pt
+    lib.THCState_setCurrentStream(st, sa)
+    q = thc.Tensor("float").resize((1 << 20,))
+    assert q.data_ptr() != pt                          # the source of B's pending copy is not recycled on A
+    q.fill(-1.0)
+    assert hip.hipStreamSynchronize(sa) == 0 and hip.hipStreamSynchronize(sb) == 0
+    assert np.array_equal(t.numpy()[:1 << 20], np.arange(1 << 20, dtype=np.float32))
+
+
+def test_host_copy_waits_for_a_nonblocking_stream(thc, nonblocking_streams):
+    """copyFromHost runs on the null stream; it must not overtake work queued on a non-blocking current stream."""
+    hip, (sa, _) = nonblocking_streams
+    lib, st = thc.lib(), thc.state()
+    lib.THCState_setCurrentStream(st, sa)
+    w = thc.Tensor("float").resize((1 << 28,)).fill(0.0)
+    t = thc.Tensor("float").resize((1 << 20,)).fill(0.0)
+    tv = thc.Tensor("float").resize((1024, 2048)).fill(0.0).t()     # a strided destination (staged through a temporary)
+    _busy(thc, w, 20)
+    t.add(t, 1.0)
+    tv.add(tv, 1.0)
+    fives = np.full(1 << 20, 5.0, np.float32)
+    t._fn("copyFromHost")(t._st, t.h, fives.ctypes.data_as(C.c_void_p))
+    tv._fn("copyFromHost")(tv._st, tv.h, np.full((2048, 1024), 5.0, np.float32).ctypes.data_as(C.c_void_p))
+    assert hip.hipStreamSynchronize(sa) == 0
+    assert np.all(t.numpy() == 5.0) and np.all(tv.numpy() == 5.0)
