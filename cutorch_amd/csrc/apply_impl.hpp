@@ -225,7 +225,7 @@ struct OpMath2 {
 // ------------------------------------------------------------------------
 // TOut differs from T only for ops that change the element type (comparisons
 // into a Byte tensor); the output pack then has VEC elements of TOut.
-template <typename T, typename Op, int VEC, int UNROLL, bool NT, typename TOut = T>
+template <typename T, typename Op, int VEC, int UNROLL, bool NT, typename TOut = T, bool NTS = false>
 __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T* in0, const T* in1,
                                                               const T* in2, uint64_t n, Op op) {
   using P = Pack<T, VEC>;
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T
           PO r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = f(a[u].v[e], b[u].v[e], c[u].v[e]);
-          store_pack<false>(reinterpret_cast<PO*>(out) + i, r);
+          store_pack<NTS>(reinterpret_cast<PO*>(out) + i, r);
         }
       }
     }
@@ -278,6 +278,7 @@ struct IndexedArgs {
   int dims[kMaxOps];                  // JOINT: only dims[0] is used
   Divisor<I> size[kMaxOps][kMaxDims]; // JOINT: only size[0][*] is used
   I stride[kMaxOps][kMaxDims];        // in elements; pre-multiplied by VEC in the packed dim
+  int ntStore;                        // packs of the output go out with the streaming hint
 };
 
 // JOINT = all operands share sizes (one division chain); VEC packs along the
@@ -324,7 +325,8 @@ __global__ __launch_bounds__(kBlock) void apply_indexed_kernel(TOut* out, const 
       PO r;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) r.v[e] = f(a.v[e], b.v[e], c.v[e]);
-      store_pack<false>(reinterpret_cast<PO*>(out + off[0]), r);
+      if (args.ntStore) store_pack<true>(reinterpret_cast<PO*>(out + off[0]), r);
+      else store_pack<false>(reinterpret_cast<PO*>(out + off[0]), r);
     });
   }
 }
@@ -408,7 +410,8 @@ __global__ __launch_bounds__(kBlock) void apply_flatmix_kernel(TOut* out, const 
 #pragma unroll
       for (int e = 0; e < VEC; ++e) r.v[e] = f(in[0].v[e], in[1].v[e], in[2].v[e]);
       if (cnt == VEC) {
-        store_pack<false>(reinterpret_cast<PO*>(out + i0), r);
+        if (args.ntStore) store_pack<true>(reinterpret_cast<PO*>(out + i0), r);
+        else store_pack<false>(reinterpret_cast<PO*>(out + i0), r);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; ++e)
@@ -453,6 +456,7 @@ struct TiledArgs {
   // (p fastest inside a band, then q), so that tiles whose staged windows
   // share cache lines run back to back; 1 = q fastest throughout.
   uint32_t groupP;
+  uint32_t ntStore;  // shifted-window variant: whole packs of the output go out with the streaming hint
 };
 
 // A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
@@ -791,7 +795,8 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
         for (int e = 0; e < VEC; ++e) res.v[e] = op(in[0].v[e], in[1].v[e], in[2].v[e]);
         T* orow = const_cast<T*>(tbase[0]) + r * rowStep[0] + vo[0];
         if (first[r] >= 0 && first[r] + VEC <= qn) {
-          store_pack<false>(reinterpret_cast<P*>(orow + first[r]), res);
+          if (args.ntStore) store_pack<true>(reinterpret_cast<P*>(orow + first[r]), res);
+          else store_pack<false>(reinterpret_cast<P*>(orow + first[r]), res);
         } else {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
@@ -820,6 +825,20 @@ inline bool pack_aligned(const Plan& pl, int k) {
   return (reinterpret_cast<uintptr_t>(pl.ptr[k]) & (bytes - 1)) == 0;
 }
 
+// Whether an output of `bytes` goes out with the streaming (nontemporal) hint.
+// Plain stores leave the output in the L2s and the 256 MiB memory-side cache,
+// where a consumer launched next finds it; the dirty lines are written back
+// when the kernel ends. Measured with producer -> consumer pairs of flat fp32
+// kernels over rotating buffers: outputs up to 32 MiB are 3-8 % faster with
+// plain stores, 64 MiB is even, from 128 MiB on the streaming hint wins by
+// 6-8 % (and by 9 % on a transposed 256 MiB addcmul). A timing loop that
+// rewrites ONE output buffer that fits the memory-side cache flatters plain
+// stores (the writes never reach HBM).
+inline bool streaming_store(const char* knob, int64_t bytes) {
+  const int64_t k = tuning(knob, -1);
+  return k >= 0 ? k != 0 : bytes >= (int64_t(64) << 20);
+}
+
 inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* key, int default_per_cu) {
   const int64_t blocks = (work_items + per_block - 1) / per_block;
   const int64_t cap = (int64_t)num_compute_units(s) * tuning(key, default_per_cu);
@@ -843,12 +862,17 @@ void launch_contig(THCState* s, const Plan& pl, Op op) {
   const int64_t packs = vec ? (int64_t)(n / VEC) + 1 : (int64_t)n;
   // Streaming hint only when the operands cannot stay cache resident anyway.
   const bool nt = (int64_t)n * (int64_t)sizeof(T) * pl.nops >= tuning("apply.contig.nt_bytes", 8 << 20);
+  // (a pure write stream, fill, is not helped by the hint: 1 GiB 176 us plain, 186 us streaming)
+  const bool nts = Op::NIN > 0 && streaming_store("apply.contig.nt_store", (int64_t)n * (int64_t)sizeof(TOut));
   const int64_t unroll = tuning("apply.contig.unroll", 2);
   auto launch = [&](auto uTag) {
     constexpr int UU = decltype(uTag)::value;
     const int64_t blk = (packs + kBlock * UU - 1) / (kBlock * UU);
     const int gr = (int)std::max<int64_t>(1, std::min<int64_t>(blk, tuning("apply.contig.max_grid", 1 << 20)));
-    if (vec && nt)
+    if (vec && nt && nts)
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut, true>), dim3(gr), dim3(kBlock),
+                         0, st, out, i0, i1, i2, n, op);
+    else if (vec && nt)
       hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut>), dim3(gr), dim3(kBlock),
                          0, st, out, i0, i1, i2, n, op);
     else if (vec)
@@ -905,6 +929,7 @@ void launch_indexed(THCState* s, const Plan& pl, Op op) {
       args.stride[k][d] = (I)sd;
     }
   }
+  args.ntStore = vec && streaming_store("apply.indexed.nt_store", pl.numel * (int64_t)sizeof(TOut)) ? 1 : 0;
   const int64_t total = pl.numel / pack;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((total + kBlock - 1) / kBlock,
                                                                tuning("apply.indexed.max_grid", 1 << 22)));
@@ -1053,7 +1078,9 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   // distance covered by the output rows of one tile
   const int64_t outSpan = (int64_t)tileP * pl.lay[0].stride[p] * (int64_t)sizeof(T);
   const int64_t ntKnob = tuning("apply.tiled.nt_store", -1);
-  const bool nts = ntKnob >= 0 ? ntKnob != 0 : outSpan >= (int64_t(32) << 20);
+  const bool nts = ntKnob >= 0 ? ntKnob != 0
+                               : (outSpan >= (int64_t(32) << 20) || pl.numel * (int64_t)sizeof(T) >= (int64_t(64) << 20));
+  args.ntStore = nts ? 1u : 0u;
   bool lineAligned = true;  // every row of every operand starts on a 128-byte line
   for (int k = 0; k < pl.nops; ++k) {
     lineAligned = lineAligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % 128 == 0;
@@ -1156,6 +1183,7 @@ bool launch_flatmix(THCState* s, const Plan& pl, Op op) {
       args.stride[k][d] = (I)pl.lay[k].stride[d];
     }
   }
+  args.ntStore = streaming_store("apply.indexed.nt_store", pl.numel * (int64_t)sizeof(TOut)) ? 1 : 0;
   const int64_t packs = pl.numel / VEC + 1;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((packs + kBlock - 1) / kBlock,
                                                                tuning("apply.indexed.max_grid", 1 << 22)));

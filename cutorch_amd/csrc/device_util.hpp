@@ -40,12 +40,11 @@ struct RawBits<1> {
   typedef uint8_t type;
 };
 
-// Streaming access: every byte of these kernels is touched once. Measured on
-// MI355X with a flat 3-read-1-write fp32 stream over 1 GiB: plain loads and
-// stores 5.7 TB/s, nontemporal loads AND stores 6.5 TB/s, nontemporal loads
-// with plain (write-back cached) stores 7.1 TB/s. So inputs are loaded with
-// the nontemporal hint and outputs are stored normally, except where a kernel
-// says otherwise.
+// Streaming access: every byte of these kernels is touched once, so inputs
+// are loaded with the nontemporal hint (a flat 3-read-1-write fp32 stream over
+// 1 GiB: plain loads 5.7 TB/s, nontemporal loads 6.5-7.1). Stores take the
+// hint only for large outputs (the launch code decides, see streaming_store):
+// small outputs are better left in the caches for the next kernel.
 template <bool NT, typename P>
 __device__ __forceinline__ P load_pack(const P* p) {
   if (NT) {

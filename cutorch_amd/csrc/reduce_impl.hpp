@@ -198,6 +198,19 @@ struct PairOrder {
     if (an || bn) return an && (!bn || ai < bi);
     return (IS_MAX ? av > bv : av < bv) || (av == bv && ai < bi);
   }
+  // The larger (smaller) of two values; a NaN operand gives NaN. On gfx950 the
+  // floating forms fold pairwise into three-input instructions.
+  static __device__ __forceinline__ V extreme(V a, V b) {
+    if constexpr (std::is_integral<V>::value) return IS_MAX ? (a > b ? a : b) : (a < b ? a : b);
+    else return IS_MAX ? __builtin_elementwise_maximum(a, b) : __builtin_elementwise_minimum(a, b);
+  }
+  // false for the values that `extreme` does not order the way a sequential
+  // scan does: NaN (the first one must win) and zero (-0 == +0, the first one
+  // must keep its sign).
+  static __device__ __forceinline__ bool plain(V m) {
+    if constexpr (std::is_integral<V>::value) return true;
+    else return m == m && m != (V)0;
+  }
   // Same decision when `a` is known to come after `b` in index order (a lane
   // scanning its elements front to back): ties never replace, a NaN replaces
   // only a non-NaN.
@@ -344,14 +357,38 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u)
           v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
+        // The batch's extreme value first (one three-input instruction per two
+        // elements, NaN propagating), then, only in lanes whose batch beats
+        // their running best, the first slot that holds it. A compare-select
+        // chain over every element costs about six instructions per element
+        // and made this kernel issue bound.
+        A m = O::worst();
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) {
-            const A x = acc_up<A>(v[u].v[e]);
-            if (O::better_later(x, bv)) {
-              bv = x;
-              bi = i + u * step + e;
+          for (int e = 0; e < VEC; ++e) m = O::extreme(m, acc_up<A>(v[u].v[e]));
+        }
+        if (O::plain(m)) {
+          if (O::better_later(m, bv)) {
+            uint32_t slot = 0;
+#pragma unroll
+            for (int q = U * VEC - 1; q >= 0; --q)
+              slot = acc_up<A>(v[q / VEC].v[q % VEC]) == m ? (uint32_t)q : slot;
+            bv = m;
+            bi = i + (I)(slot / VEC) * step + (I)(slot % VEC);
+          }
+        } else {
+          // a NaN or a zero is the batch's extreme: element by element, so that the
+          // first NaN wins and a zero keeps the sign of its first occurrence
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const A x = acc_up<A>(v[u].v[e]);
+              if (O::better_later(x, bv)) {
+                bv = x;
+                bi = i + u * step + e;
+              }
             }
           }
         }

@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "stream_guard.hpp"
 #include "device_util.hpp"
 
 namespace thc {
@@ -106,7 +107,7 @@ struct ScanMul {
 template <typename T, typename Op, int VEC>
 __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
-                                                           uint64_t numRows, uint64_t R) {
+                                                           uint64_t numRows, uint64_t R, int nts) {
   using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   constexpr int U = 4;
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
             P v;
 #pragma unroll
             for (int k = 0; k < VEC; ++k) v.v[k] = scan_down<T>(Op::op(offset, x[u][k]));
-            *reinterpret_cast<P*>(dst + i0) = v;
+            if (nts) store_pack<true>(reinterpret_cast<P*>(dst + i0), v);
+            else store_pack<false>(reinterpret_cast<P*>(dst + i0), v);
           } else {
             dst[i0] = scan_down<T>(Op::op(offset, x[u][0]));
           }
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t outer, uint64_t R,
                                                            uint64_t inner, uint32_t TX,
-                                                           uint64_t colTiles) {
+                                                           uint64_t colTiles, int nts) {
   using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   constexpr int U = 8;
@@ -240,7 +242,8 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
           P v;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) v.v[e] = scan_down<T>(Op::op(offset[e], x[u][e]));
-          *reinterpret_cast<P*>(dst + (r0 + u) * inner) = v;
+          if (nts) store_pack<true>(reinterpret_cast<P*>(dst + (r0 + u) * inner), v);
+          else store_pack<false>(reinterpret_cast<P*>(dst + (r0 + u) * inner), v);
         }
       }
 #pragma unroll
@@ -266,10 +269,11 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
                                                            const typename ScanAcc<T>::type* __restrict__ carryIn,
                                                            uint64_t outer, uint64_t R, uint32_t inner,
                                                            uint32_t slicesPerBlock, uint64_t S,
-                                                           uint32_t chunkRows) {
+                                                           uint32_t chunkRows, uint32_t dataBytes) {
   using A = typename ScanAcc<T>::type;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
+  A* part = reinterpret_cast<A*>(lds_raw + dataBytes);  // kBlock band totals behind the staged run
   const bool chunked = S > 1;
   const uint64_t numBlocks = chunked ? outer * S : (outer + slicesPerBlock - 1) / slicesPerBlock;
   for (uint64_t blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
@@ -287,28 +291,77 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
     const uint32_t slice = rows * inner, count = ns * slice;
     const uint32_t mis = stage_rows_to_lds<T, 8>(in + start, count, lds);
     __syncthreads();
-    for (uint32_t t = threadIdx.x; t < ns * inner; t += kBlock) {
-      const uint32_t o = t / inner, c = t - o * inner;
-      T* col = lds + mis + o * slice + c;
-      A acc = Op::id();
-      if (chunked && blk % S != 0) acc = carryIn[(blk - 1) * inner + c];
-      // batches of 8 rows: the loads of a batch are independent of its stores,
-      // so one LDS round trip is paid per batch instead of per element
-      constexpr uint32_t B = 8;
-      uint32_t r = 0;
-      for (; r + B <= rows; r += B) {
-        T x[B];
+    // `cols` independent columns in this run. With fewer columns than threads,
+    // P threads share a column: each takes a contiguous band of rows, the band
+    // totals meet in LDS, and every band scans from the totals before it (an
+    // 8M x 10 matrix scanned along dim 0 kept 10 of 256 threads busy otherwise).
+    const uint32_t cols = ns * inner;
+    const uint32_t P = cols >= kBlock ? 1u : min(rows, kBlock / cols);
+    if (P == 1) {
+      for (uint32_t t = threadIdx.x; t < cols; t += kBlock) {
+        const uint32_t o = t / inner, c = t - o * inner;
+        T* col = lds + mis + o * slice + c;
+        A acc = Op::id();
+        if (chunked && blk % S != 0) acc = carryIn[(blk - 1) * inner + c];
+        // batches of 8 rows: the loads of a batch are independent of its stores,
+        // so one LDS round trip is paid per batch instead of per element
+        constexpr uint32_t B = 8;
+        uint32_t r = 0;
+        for (; r + B <= rows; r += B) {
+          T x[B];
 #pragma unroll
-        for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+          for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
 #pragma unroll
-        for (uint32_t u = 0; u < B; ++u) {
-          acc = Op::op(acc, scan_up<A>(x[u]));
-          col[(r + u) * inner] = scan_down<T>(acc);
+          for (uint32_t u = 0; u < B; ++u) {
+            acc = Op::op(acc, scan_up<A>(x[u]));
+            col[(r + u) * inner] = scan_down<T>(acc);
+          }
+        }
+        for (; r < rows; ++r) {
+          acc = Op::op(acc, scan_up<A>(col[r * inner]));
+          col[r * inner] = scan_down<T>(acc);
         }
       }
-      for (; r < rows; ++r) {
-        acc = Op::op(acc, scan_up<A>(col[r * inner]));
-        col[r * inner] = scan_down<T>(acc);
+    } else {
+      const uint32_t p = threadIdx.x / cols, t = threadIdx.x - p * cols;
+      const uint32_t o = t / inner, c = t - o * inner;
+      const uint32_t band = (rows + P - 1) / P;
+      const uint32_t rb = min(rows, p * band), re = min(rows, rb + band);
+      T* col = lds + mis + o * slice + c;
+      constexpr uint32_t B = 8;
+      if (p < P) {
+        A acc = Op::id();
+        uint32_t r = rb;
+        for (; r + B <= re; r += B) {
+          T x[B];
+#pragma unroll
+          for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+#pragma unroll
+          for (uint32_t u = 0; u < B; ++u) acc = Op::op(acc, scan_up<A>(x[u]));
+        }
+        for (; r < re; ++r) acc = Op::op(acc, scan_up<A>(col[r * inner]));
+        part[p * cols + t] = acc;
+      }
+      __syncthreads();
+      if (p < P) {
+        A acc = Op::id();
+        if (chunked && blk % S != 0) acc = carryIn[(blk - 1) * inner + c];
+        for (uint32_t q = 0; q < p; ++q) acc = Op::op(acc, part[q * cols + t]);  // bands before this one, in order
+        uint32_t r = rb;
+        for (; r + B <= re; r += B) {
+          T x[B];
+#pragma unroll
+          for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+#pragma unroll
+          for (uint32_t u = 0; u < B; ++u) {
+            acc = Op::op(acc, scan_up<A>(x[u]));
+            col[(r + u) * inner] = scan_down<T>(acc);
+          }
+        }
+        for (; r < re; ++r) {
+          acc = Op::op(acc, scan_up<A>(col[r * inner]));
+          col[r * inner] = scan_down<T>(acc);
+        }
       }
     }
     __syncthreads();
@@ -387,8 +440,9 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t blocks = (outer + spb - 1) / spb;
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, (int64_t)num_compute_units(s) * 64));
     const size_t lds = (((size_t)(spb * R * inner) + 2 * kFull) * sizeof(T) + 15) & ~size_t(15);
-    hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds, st, out, in, nullptr,
-                       (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint32_t)spb, (uint64_t)1, 0u);
+    hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds + kBlock * sizeof(typename ScanAcc<T>::type),
+                       st, out, in, nullptr, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint32_t)spb, (uint64_t)1, 0u,
+                       (uint32_t)lds);
     note_kernel("scan-slab");
     return;
   }
@@ -418,22 +472,26 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
                          st, totals, in, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint64_t)S,
                          (uint32_t)chunkRows, dataElems);
       launch_scan<A, Op>(s, carries, totals, outer, S, inner, scratch + 2 * need, scratchBytes - 2 * need);
-      hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsData, st, out, in, carries,
-                         (uint64_t)outer, (uint64_t)R, (uint32_t)inner, 1u, (uint64_t)S, (uint32_t)chunkRows);
+      hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsData + kBlock * sizeof(A), st, out, in,
+                         carries, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, 1u, (uint64_t)S, (uint32_t)chunkRows,
+                         (uint32_t)ldsData);
       note_kernel("scan-chunked");
       return;
     }
   }
+  // large outputs go out with the streaming hint (they cannot stay cache resident for a consumer)
+  const int64_t ntsKnob = tuning("scan.nt_store", -1);
+  const int nts = (ntsKnob >= 0 ? ntsKnob != 0 : outer * R * inner * (int64_t)sizeof(T) >= (int64_t(64) << 20)) ? 1 : 0;
   if (inner == 1) {
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
     const int64_t blocks = (outer + (kBlock / 64) - 1) / (kBlock / 64);
     const int grid = (int)std::max<int64_t>(1, std::min(blocks, cap));
     if (aligned && R % VEC == 0)
       hipLaunchKernelGGL((scan_rows_kernel<T, Op, VEC>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R);
+                         (uint64_t)outer, (uint64_t)R, nts);
     else
       hipLaunchKernelGGL((scan_rows_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R);
+                         (uint64_t)outer, (uint64_t)R, nts);
     note_kernel("scan-rows");
   } else {
     const bool vec = aligned && inner % VECC == 0;
@@ -448,10 +506,10 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * colTiles, 1 << 30));
     if (vec)
       hipLaunchKernelGGL((scan_cols_kernel<T, Op, VECC>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles);
+                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts);
     else
       hipLaunchKernelGGL((scan_cols_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles);
+                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts);
     note_kernel("scan-cols");
   }
 }
@@ -467,8 +525,17 @@ void scan_dim(THCState* s, DType dt, bool product, AnyTensor* self, AnyTensor* s
   if (dim < 0 || dim >= nd)
     raise_arg_error(3, "dimension %d out of range", dim + 1);  // generic/THCTensorMathScan.cu:83-84
   tensor_resize_as(s, self, src, dt);
-  TensorRef dst(s, tensor_new_contiguous(s, self, dt));
+  note_stream_use(s, {self, src});
+  // a non-contiguous destination gets a fresh dense temporary (its contents are
+  // overwritten anyway, so nothing is copied in), then a strided copy back
   TensorRef in(s, tensor_new_contiguous(s, src, dt));
+  TensorRef dst(s, nullptr);
+  if (tensor_is_contiguous(self)) {
+    tensor_retain(self);
+    dst.t = self;
+  } else {
+    dst.t = tensor_new_with_size(s, nd, src->size, dt);
+  }
   int64_t outer = 1, inner = 1;
   for (int d = 0; d < dim; ++d) outer *= src->size[d];
   for (int d = dim + 1; d < nd; ++d) inner *= src->size[d];
