@@ -315,6 +315,33 @@ def test_large_transposed_roundtrip_property(thc):
     assert_bit_equal(back.numpy(), x)
 
 
+def test_config2_full_size_against_the_oracle(thc, oracle):
+    """The headline workload itself: out = a:t() * b + d (addcmul, value 1) on
+    8192 x 8192 fp32 with the benchmark's seed, a viewed transposed; the whole
+    output storage bit for bit against the CPU oracle (8 threads, ~0.1 s)."""
+    n = 8192
+    rng = np.random.default_rng(0xC0FFEE)
+    a = rng.standard_normal((n, n), dtype=np.float32)
+    b = rng.standard_normal((n, n), dtype=np.float32)
+    d = rng.standard_normal((n, n), dtype=np.float32)
+    out = thc.Tensor("float").addcmul(thc.Tensor.from_numpy(d), 1.0, thc.Tensor.from_numpy(a).t(),
+                                      thc.Tensor.from_numpy(b))
+    assert thc.last_kernel() == "tiled" and out.shape == (n, n)
+    va = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
+    ref = oracle.View.empty((n, n))
+    oracle.set_num_threads(8)
+    try:
+        oracle.pointwise("addcmul", ref, oracle.View(d.reshape(-1), 0, (n, n)), va,
+                         oracle.View(b.reshape(-1), 0, (n, n)), value=1.0)
+    finally:
+        oracle.set_num_threads(1)
+    assert_bit_equal(out.storage_numpy(), ref.storage, "config 2 at full size")
+    # in place on d, as cutorch's addcmul(self == t) runs it
+    dd = thc.Tensor.from_numpy(d)
+    dd.addcmul(dd, 1.0, thc.Tensor.from_numpy(a).t(), thc.Tensor.from_numpy(b))
+    assert_bit_equal(dd.storage_numpy(), ref.storage, "config 2 in place")
+
+
 def test_config5_full_size_64bit_index_path(thc):
     """c = a + b on 2048 x 2048 x 520 fp32 (2.18e9 elements, 26 GB), a being a
     permute(3,2,1) view of a dense 520 x 2048 x 2048 tensor. The operands repeat

@@ -76,3 +76,59 @@ def device_fill_from_block(thc, shape, block):
         assert hip.hipMemcpy(base + 4 * done, blk.data_ptr(), 4 * m, 3) == 0
         done += m
     return t
+
+
+def holed_geometry(rng, shape, holes=True, swaps=10, inflate=(4, 15)):
+    """(storage_len, offset, size, stride) of a view with the logical `shape`,
+    built the way cutorch's suite builds its hardest operands
+    (createHoledTensorWithSizes + randomlyTranspose, test/test.lua:81-98,647-661):
+    a dense allocation in which up to three dims are inflated by 4..15 elements,
+    narrowed back to size at a random start (holes on both sides of the view),
+    seen through `swaps` random transpositions. The transpositions are applied
+    to the allocation's dim order so that the view comes out with `shape`."""
+    nd = len(shape)
+    perm = list(range(nd))                      # perm[k] = logical dim stored at allocation position k
+    for _ in range(swaps):
+        a, b = int(rng.integers(0, nd)), int(rng.integers(0, nd))
+        perm[a], perm[b] = perm[b], perm[a]
+    alloc = [int(shape[d]) for d in perm]
+    start = [0] * nd
+    if holes:
+        for _ in range(3):
+            k = int(rng.integers(0, nd))
+            alloc[k] += int(rng.integers(inflate[0], inflate[1] + 1))
+        for k in range(nd):
+            start[k] = int(rng.integers(0, alloc[k] - int(shape[perm[k]]) + 1))
+    astride, run = [0] * nd, 1
+    for k in reversed(range(nd)):
+        astride[k] = run
+        run *= alloc[k]
+    offset = sum(s * st for s, st in zip(start, astride))
+    stride = [0] * nd
+    for k, d in enumerate(perm):
+        stride[d] = astride[k]
+    return run, offset, tuple(int(s) for s in shape), tuple(stride)
+
+
+def refactorised_shape(rng, shape, moves=10):
+    """A shape with the same element count: `moves` times a prime factor of a
+    random dim becomes a new dim or is multiplied into another dim
+    (constructOutput of copyRandomizedTest, test/test.lua:584-622)."""
+    out = [int(s) for s in shape]
+    for _ in range(moves):
+        d = int(rng.integers(0, len(out)))
+        n, f, factors = out[d], 2, []
+        while n > 1:
+            while n % f == 0:
+                factors.append(f)
+                n //= f
+            f += 1
+        if not factors:
+            continue
+        f = factors[int(rng.integers(0, len(factors)))]
+        out[d] //= f
+        if rng.random() < 0.5 and len(out) < 25:
+            out.insert(int(rng.integers(0, len(out) + 1)), f)
+        else:
+            out[int(rng.integers(0, len(out)))] *= f
+    return tuple(out)
