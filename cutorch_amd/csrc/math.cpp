@@ -65,10 +65,21 @@ void binary_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, AnyT
 
 // self = t + v * (src1 (op) src2). The reference copies t into self and then
 // runs an in-place apply3 (generic/THCTensorMathPointwise.cu:586-590); here
-// t is read directly as a fourth operand, which saves a full pass.
+// t is read directly as a fourth operand, which saves a full pass. The two
+// differ when self (not being t) lies on the storage of src1 or src2: after the
+// reference's copy those operands hold t's values. That case keeps the
+// reference's two steps.
 void ternary_op(THCState* s, DType dt, PointOp op, float v, AnyTensor* self, AnyTensor* t,
                 AnyTensor* src1, AnyTensor* src2) {
   same_gpu(s, {self, t, src1, src2});
+  if (self != t && self->storage && (self->storage == src1->storage || self->storage == src2->storage)) {
+    tensor_resize_as(s, self, t, dt);
+    copy_tensor(s, dt, self, t, false);
+    THC_ARG_CHECK(tensor_numel(self) == tensor_numel(src1), 1, "sizes do not match");
+    THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), 3, "sizes do not match");
+    apply_or_throw(s, dt, op, v, self, self, src1, src2);
+    return;
+  }
   if (self != t)
     tensor_resize_as(s, self, t, dt);
   else

@@ -67,6 +67,16 @@ void w_binary(THCState* s, DType dt, PointOp op, MathFn fn, Scalar v, AnyTensor*
 void w_ternary(THCState* s, DType dt, PointOp op, Scalar v, AnyTensor* self, AnyTensor* t,
                AnyTensor* src1, AnyTensor* src2) {
   same_gpu(s, {self, t, src1, src2});
+  // self on the storage of src1 or src2: the reference's copy-then-accumulate order
+  // (generic/THCTensorMathPointwise.cu:586-590) decides what those operands hold
+  if (self != t && self->storage && (self->storage == src1->storage || self->storage == src2->storage)) {
+    tensor_resize_as(s, self, t, dt);
+    copy_tensor(s, dt, self, t, false);
+    THC_ARG_CHECK(tensor_numel(self) == tensor_numel(src1), 1, "sizes do not match");
+    THC_ARG_CHECK(tensor_numel(src1) == tensor_numel(src2), 3, "sizes do not match");
+    run(s, dt, dt, op, 0, v, Scalar{0, 0}, self, self, src1, src2);
+    return;
+  }
   if (self != t)
     tensor_resize_as(s, self, t, dt);
   else

@@ -448,3 +448,34 @@ def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band):
                                                 contiguous_geometry((7, 401, 130))], rng) == "tiled-shift"
     finally:
         thc.set_tuning("apply.tiled.group_p", 8)
+
+
+@pytest.mark.parametrize("kind", ["float", "int"])
+def test_addcmul_when_self_is_a_factor(thc, oracle, kind):
+    """addcmul(self, t, v, src1, src2) with self being src1 (or src2) and not t:
+    the reference first copies t into self and then accumulates in place
+    (generic/THCTensorMathPointwise.cu:586-590), so the factor that is self
+    already holds t's values: self = t + v * t * src2."""
+    rng = np.random.default_rng(17)
+    dtype = np.float32 if kind == "float" else np.int32
+    t = rng.integers(-6, 7, (33, 65)).astype(dtype)
+    a = rng.integers(-6, 7, (33, 65)).astype(dtype)
+    b = rng.integers(-6, 7, (33, 65)).astype(dtype)
+    for which in ("src1", "src2"):
+        dt, da, db = thc.Tensor.from_numpy(t), thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
+        if which == "src1":
+            da.addcmul(dt, 2, da, db)
+            got, want = da.numpy(), t + 2 * t * b
+        else:
+            db.addcmul(dt, 2, da, db)
+            got, want = db.numpy(), t + 2 * a * t
+        assert_bit_equal(got, want.astype(dtype), which)
+        # a view on self's storage counts as well (here: self transposed twice)
+        dt, da, db = thc.Tensor.from_numpy(t), thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
+        alias = da.t().t()
+        da.addcdiv(dt, 3, alias, thc.Tensor.from_numpy(np.ones_like(t)))
+        assert_bit_equal(da.numpy(), (t + 3 * t).astype(dtype), "aliasing view")
+    # self == t stays the one-pass in-place form
+    dt, da, db = thc.Tensor.from_numpy(t), thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
+    dt.addcmul(dt, 2, da, db)
+    assert_bit_equal(dt.numpy(), (t + 2 * a * b).astype(dtype), "in place on t")
