@@ -290,7 +290,7 @@ def build_configs(thc, hip, which, only=None):
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
-                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd")
+                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -367,6 +367,37 @@ def build_configs(thc, hip, which, only=None):
                 "N-add-t-odd": ("c = a:t() + b, 8191x8193 fp32 (no 16-byte aligned rows)", 12 * nodd, nodd,
                                 lambda i: oddO.cadd(oddT, 1.0, oddB)),
             })
+        if set(nx) & {"N-int-add-t", "N-lt-t"}:
+            # transposed operands of ops that have no LDS-tiled kernel of their own (slab-wise densify)
+            it_a = T.from_numpy(rng.integers(-1000, 1000, (8192, 8192)).astype(np.int32)).t()
+            it_b = T.from_numpy(rng.integers(-1000, 1000, (8192, 8192)).astype(np.int32))
+            it_c = T("int").resize((8192, 8192))
+            lt_m = T("byte").resize((8192, 8192))
+            table.update({
+                "N-int-add-t": ("c = a:t() + b, 8192x8192 int32", 12 * 8192 * 8192, 8192 * 8192,
+                                lambda i: it_c.cadd(it_a, 1, it_b)),
+                "N-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 fp32", 9 * 8192 * 8192, 8192 * 8192,
+                           lambda i: lt_m.compare_tensor("lt", sq_t, db)),
+            })
+        if set(nx) & {"N-add-2p25", "N-add-2p26"}:
+            # c = a + b as in C1 at two and four times the size (rotating sets): kernel time against
+            # bytes gives the fixed cost of a launch (t = t0 + bytes / BW)
+            for lg, nset in ((25, 3), (26, 3)):
+                m = 1 << lg
+                ss = [(T.from_numpy(rng.uniform(-1, 1, m).astype(np.float32)),
+                       T.from_numpy(rng.uniform(-1, 1, m).astype(np.float32)), T("float").resize((m,)))
+                      for _ in range(nset)]
+                table["N-add-2p%d" % lg] = ("c = a + b, 2^%d fp32 contiguous, %d rotating sets" % (lg, nset), 12 * m, m,
+                                            (lambda q, k: lambda i: q[i % k][2].cadd(q[i % k][0], 1.0, q[i % k][1]))(ss, nset))
+        if set(nx) & {"CEIL-copy-rot", "CEIL-3r1w-rot"}:
+            # What flat kernels reach on the same stream shapes (the ceilings the strided configurations are
+            # judged against): a 1-read-1-write stream and the 3-read-1-write stream of C2 without the
+            # transposition, outputs rotating so that no write is absorbed by the memory-side cache.
+            cr_out = [T("float").resize((ne,)) for _ in range(4)]
+            table["CEIL-copy-rot"] = ("out = src + 0, 2^26 fp32 contiguous, 4 rotating outputs", 8 * ne, ne,
+                                      lambda i: cr_out[i % 4].add(e_src, 0.0))
+            table["CEIL-3r1w-rot"] = ("out = a*b + d, 8192x8192 fp32, all contiguous, out and d rotate over 3 sets",
+                                      16 * n2 * n2, n2 * n2, lambda i: out2[i % 3].addcmul(dd[i % 3], 1.0, da, db))
         if "N-fill" in nx and xa.numel() != big:
             table["N-fill"] = ("fill of 2^26 fp32", 4 * ne, ne, lambda i: e_dst.fill(0.5))
         for n in nx:
@@ -398,6 +429,10 @@ def build_configs(thc, hip, which, only=None):
     cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
                        12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5), c5_check))
     cfgs[-1].note = "parity on 4 of the 2048 output planes"
+    if which == "all" or (only and "CEIL-2r1w-26GB" in only):
+        a5flat = a5.view_as_strided(0, (2048, 2048, 520), (2048 * 520, 520, 1))
+        cfgs.append(Config("CEIL-2r1w-26GB", "c = a + b on the same 3 x 8.7 GB buffers, all contiguous (flat ceiling of C5)",
+                           12 * n5, n5, 1, lambda i: c5.cadd(a5flat, 1.0, b5)))
     return [c for c in cfgs if c is cfgs[0] or want(c.name)], host
 
 
@@ -499,7 +534,7 @@ def main():
         cfgs = [cfgs[0]] + [c for c in cfgs[1:] if c.name in only]
     results = []
     for cfg in cfgs:
-        steps = args.steps if cfg.name != "C5" else max(3, args.steps // 5)
+        steps = args.steps if cfg.name not in ("C5", "CEIL-2r1w-26GB") else max(3, args.steps // 5)
         wall, region_ms, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
         ok = None if (args.no_check or cfg.check is None) else bool(cfg.check())
         mean_ms = region_ms / steps
