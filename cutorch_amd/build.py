@@ -20,7 +20,7 @@ SOURCES = ["general.cpp", "tensor.cpp", "math.cpp", "math_wide.cpp", "caching_al
            "apply_f32_2.hip", "apply_f16_0.hip", "apply_f16_1.hip", "apply_f16_2.hip", "apply_raw.hip",
            "reduce.hip", "reduce_f32.hip", "reduce_f16.hip", "reduce_w_u8.hip", "reduce_w_i8.hip",
            "reduce_w_i16.hip", "reduce_w_i32.hip", "reduce_w_i64.hip", "reduce_w_f64.hip", "scan.hip", "no_alloc.hip", "convert.hip", "apply_cmp_f.hip", "apply_w_u8.hip",
-           "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip"]
+           "apply_rawmath_u32u64.hip", "apply_rawmath_f64.hip", "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip"]
 HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", "apply_plan.hpp", "apply_impl.hpp", "apply_wide.hpp", "reduce_plan.hpp", "reduce_impl.hpp",
            os.path.join("..", "..", "include", "THC.h")]
 
@@ -48,7 +48,9 @@ def _stale(target, deps):
 # headers only some sources include (touching one rebuilds only those)
 EXTRA_DEPS = {"caching_allocator.cpp": ["caching_pool.hpp", "stream_guard.hpp"],
               "general.cpp": ["stream_guard.hpp"], "tensor.cpp": ["stream_guard.hpp"],
-              "apply.hip": ["stream_guard.hpp"], "reduce.hip": ["stream_guard.hpp"],
+              "apply.hip": ["stream_guard.hpp", "apply_rawmath.hpp"],
+              "apply_rawmath_u32u64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"],
+              "apply_rawmath_f64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"], "reduce.hip": ["stream_guard.hpp"],
               "scan.hip": ["stream_guard.hpp"], "convert.hip": ["stream_guard.hpp"]}
 
 

@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include "apply_plan.hpp"
+#include "apply_rawmath.hpp"
 #include "common.hpp"
 #include "stream_guard.hpp"
 #include "device_util.hpp"
@@ -80,7 +81,8 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
   const bool offTiled = d.op != PointOp::Copy &&
                         (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor ||
                          d.op == PointOp::Math2 || (d.op == PointOp::Math1 && d.dt == DType::F16) ||
-                         !(d.dt == DType::F32 || d.dt == DType::F16));
+                         !(d.dt == DType::F32 || d.dt == DType::F16)) &&
+                        !(d.outDt == d.dt && rawmath_serves(d.dt, d.op));
   // The output's fastest-running dim (smallest stride among dims longer than 1).
   int po = -1;
   for (int dd = out->nDimension - 1; dd >= 0; --dd)
@@ -149,6 +151,11 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     else for_wide_type(dt, [&](auto tag) { apply_cmp<decltype(tag)>(s, pl, sameShape, d); });
   } else if (d.outDt != dt) {
     raise_error("pointwise op cannot change the element type");
+  } else if (rawmath_serves(dt, d.op)) {
+    // plain functors on the element's width (double: on double): all kernels, tiled ones included
+    if (dt == DType::F64) apply_rawmath<double>(s, pl, sameShape, d.op, d.v);
+    else if (dt == DType::I32) apply_rawmath<uint32_t>(s, pl, sameShape, d.op, d.v);
+    else apply_rawmath<uint64_t>(s, pl, sameShape, d.op, d.v);
   } else if ((dt == DType::F32 || dt == DType::F16) && floatFamilyFn) {
     const int g = op_group(d.op);
     const float value = (float)d.v.f, value2 = (float)d.w.f;

@@ -669,18 +669,32 @@ def test_gpu_renorm_of_dense_rows_is_one_pass(thc, oracle, kind):
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["int", "byte", "double"])
 def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
-    """The wider types have no LDS-tiled arithmetic kernels: a transposed input
-    is brought into the output's order by the (tiled) same-type copy first."""
+    """add / sub / mul / cadd of int, long and double run on plain functors with
+    every kernel of the engine, the LDS-tiled ones included; everything else of
+    the wider types (and all comparisons) has no tiled kernels: a transposed
+    input is brought into the output's order by the (tiled) same-type copy first."""
     rng = np.random.default_rng(111)
     dt = np_of(oracle, kind)
     a = rand_storage(rng, kind, 200 * 136, oracle).reshape(200, 136)
     b = rand_storage(rng, kind, 200 * 136, oracle).reshape(136, 200)
     da, db = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
     out = thc.Tensor(kind).cadd(da.t(), 1, db)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == ("contig" if kind == "byte" else "tiled")
     ra = oracle.View(a.reshape(-1).copy(), 0, (136, 200), (1, 136))
     want = oracle.typed_pointwise("add", oracle.View.empty((136, 200), dt), ra, oracle.View.of(b))
     assert_bit_equal(out.numpy(), want.numpy())
+    for name, op, value in (("cmul", "mul", 0), ("csub", "cadd", 3), ("cadd", "cadd", -7)):
+        out = thc.Tensor(kind)
+        if name == "cmul":
+            out.cmul(da.t(), db)
+        else:
+            getattr(out, name)(da.t(), value, db)
+        assert thc.last_kernel() == ("contig" if kind == "byte" else "tiled"), (name, thc.last_kernel())
+        v = -value if name == "csub" else value
+        want = oracle.typed_pointwise(op, oracle.View.empty((136, 200), dt), ra, oracle.View.of(b), value=v)
+        assert_bit_equal(out.numpy(), want.numpy(), name)
+    out = thc.Tensor(kind).cdiv(da.t(), thc.Tensor.from_numpy(np.where(b == 0, 1, b).astype(dt)))
+    assert thc.last_kernel() == ("tiled" if kind == "double" else "contig")   # integer division stays code-dispatched
     m = thc.Tensor("byte").compare_tensor("lt", da.t(), db)
     assert thc.last_kernel() == "contig"
     wm = oracle.typed_compare("lt", oracle.View.empty((136, 200), np.uint8), ra, oracle.View.of(b))
@@ -703,8 +717,11 @@ def test_gpu_transposed_output_and_math_family_are_densified(thc, oracle):
     da, db = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
     base = thc.Tensor.from_numpy(np.zeros((200, 136), np.int32))
     base.t().cadd(da, 3, db)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel().startswith("tiled")     # plain int arithmetic owns tiled kernels
     assert_bit_equal(base.numpy(), (a + 3 * b).T)
+    base.t().cdiv(da, thc.Tensor.from_numpy(np.where(b == 0, 1, b).astype(np.int32)))
+    assert thc.last_kernel() == "contig"             # the code-dispatched family does not: densified
+    assert_bit_equal(base.numpy(), (a.astype(np.int64) / np.where(b == 0, 1, b)).astype(np.int64).astype(np.int32).T)
 
     x = rng.standard_normal((136, 200)).astype(np.float32)
     y = rng.standard_normal((200, 136)).astype(np.float32)
