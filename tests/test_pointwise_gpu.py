@@ -479,3 +479,42 @@ def test_addcmul_when_self_is_a_factor(thc, oracle, kind):
     dt, da, db = thc.Tensor.from_numpy(t), thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
     dt.addcmul(dt, 2, da, db)
     assert_bit_equal(dt.numpy(), (t + 2 * a * b).astype(dtype), "in place on t")
+
+
+def test_streaming_store_variants_give_the_same_bits(thc, oracle):
+    """Outputs of 64 MiB and more are stored with the streaming hint; the knobs
+    force that policy onto small shapes so that every kernel's streaming-store
+    form (flat, strided, flat + gathered, tiled, shifted-window, scans) is
+    compared with the oracle as well."""
+    rng = np.random.default_rng(31)
+    knobs = ("apply.contig.nt_store", "apply.indexed.nt_store", "apply.tiled.nt_store", "scan.nt_store")
+    for k in knobs:
+        thc.set_tuning(k, 1)
+    try:
+        g = contiguous_geometry((100003,))
+        assert run_binary(thc, oracle, "cadd", [g, g, g], rng) == "contig"
+        gp = (64 * 200, 0, (64, 192), (200, 1))                      # padded rows, pack aligned
+        assert run_binary(thc, oracle, "cmul", [gp, gp, contiguous_geometry((64, 192))], rng) == "strided"
+        ga = (130 * 96, 0, (96, 130), (1, 96))                       # a:t(): rows not pack aligned everywhere
+        assert run_binary(thc, oracle, "cadd1", [contiguous_geometry((96, 130)), ga, contiguous_geometry((96, 130))],
+                          rng).startswith("tiled")
+        ga = (128 * 256, 0, (256, 128), (1, 256))
+        assert run_binary(thc, oracle, "cdiv", [contiguous_geometry((256, 128)), ga, contiguous_geometry((256, 128))],
+                          rng) == "tiled"
+        go = (333 * 515 + 1, 1, (333, 515), (1, 333))
+        assert run_binary(thc, oracle, "cadd", [contiguous_geometry((333, 515)), go, contiguous_geometry((333, 515))],
+                          rng) == "tiled-shift"
+        x = rng.integers(-8, 9, (333, 515)).astype(np.float32)
+        bias = rng.integers(-8, 9, 515).astype(np.float32)
+        db = thc.Tensor.from_numpy(bias).view_as_strided(0, (333, 515), (0, 1))
+        out = thc.Tensor("float").cadd(thc.Tensor.from_numpy(x), 1.0, db)
+        assert thc.last_kernel() == "flat-gather"
+        assert_bit_equal(out.numpy(), x + bias)
+        for shape, dim, kernel in (((1200, 3000), 1, "scan-rows"), ((64, 40, 512), 1, "scan-cols")):
+            xi = rng.integers(-9, 10, shape).astype(np.float32)
+            got = thc.Tensor("float").cumsum(thc.Tensor.from_numpy(xi), dim)
+            assert thc.last_kernel() == kernel, thc.last_kernel()
+            assert_bit_equal(got.numpy(), np.cumsum(xi.astype(np.int64), axis=dim).astype(np.float32))
+    finally:
+        for k in knobs:
+            thc.set_tuning(k, -1)
