@@ -585,3 +585,62 @@ def test_long_narrow_slices_reduce_in_chunks(thc, oracle, kind):
     assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
     dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((300, 5000, 3)), kind, "ints")
     assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
+
+
+def test_reductions_beyond_2pow31_elements(thc):
+    """More than 2^31 elements in one tensor: the 64-bit index kernels of the
+    row, column and whole-tensor reductions at their real size (8.6 GB), not
+    forced. The data repeats a block of small integers, so every sum is exact
+    in any order and can be predicted on the host; the extreme values are
+    planted beyond offset 2^31 with a tie, whose lower index must be returned."""
+    from tests.util import device_fill_from_block
+    rng = np.random.default_rng(2 ** 31 % 1000)
+    L = (1 << 20) + 17                                   # block length, coprime to the shapes used
+    block = ((rng.integers(0, 8, L) == 0) * rng.integers(-2, 3, L)).astype(np.float32)
+    n = (1 << 31) + 4099 * 4
+    x = device_fill_from_block(thc, (n,), block)
+    reps, rest = divmod(n, L)
+    want_total = float(block.astype(np.int64).sum() * reps + block[:rest].astype(np.int64).sum())
+    assert abs(want_total) < 2 ** 24
+    assert x.sumall() == want_total
+    # 1-D max / min with index: a long single row, split over workgroups and folded
+    hi = (1 << 31) + 1234
+    for pos in (hi, hi + 4096 + 3):
+        x.narrow(0, pos, 1).fill(7.0)
+        x.narrow(0, pos + 1, 1).fill(-7.0)
+    v, i = thc.Tensor("float"), thc.Tensor("long")
+    v.max(i, x, 0)
+    assert v.numpy().tolist() == [7.0] and i.numpy().tolist() == [hi + 1]          # 1-based, first of the tie
+    v.min(i, x, 0)
+    assert v.numpy().tolist() == [-7.0] and i.numpy().tolist() == [hi + 2]
+    assert x.maxall() == 7.0 and x.minall() == -7.0
+    # 2-D views of the same storage: rows (reduced dim innermost) and columns (reduced dim strided)
+    rows, cols = 4096, (1 << 19) + 4                      # 4096 x 524292 = 2^31 + 16384 elements (within the storage)
+    assert rows * cols <= n
+    m = x.view_as_strided(0, (rows, cols), (cols, 1))
+    s = thc.Tensor("float").sum(m, 1)
+    assert thc.last_kernel().startswith("rows")
+    got = s.numpy().reshape(-1)
+    cs = np.concatenate([[0], np.cumsum(np.tile(block.astype(np.int64), 2))])
+    starts = (np.arange(rows, dtype=np.int64) * cols) % L
+    full, part = divmod(cols, L)
+    want = block.astype(np.int64).sum() * full + (cs[starts + part] - cs[starts])
+    # the planted +7 / -7 pairs cancel in their rows except where a pair straddles a row end
+    patched = np.zeros(rows, np.int64)
+    for pos in (hi, hi + 4096 + 3):
+        for q, val in ((pos, 7), (pos + 1, -7)):
+            patched[q // cols] += val - int(block[q % L])
+    assert np.array_equal(got.astype(np.int64), want + patched)
+    c = thc.Tensor("float").sum(m, 0)
+    assert thc.last_kernel().startswith("cols")
+    assert c.shape == (1, cols)
+    sample = np.array([0, 1, 5, 4099, 262144, cols - 2, cols - 1])
+    offs = (np.arange(rows, dtype=np.int64)[:, None] * cols + sample[None, :])
+    colwant = block[offs % L].astype(np.int64)
+    for pos in (hi, hi + 4096 + 3):
+        for q, val in ((pos, 7), (pos + 1, -7)):
+            r, cc = divmod(q, cols)
+            hit = np.flatnonzero(sample == cc)
+            if hit.size:
+                colwant[r, hit[0]] = val
+    assert np.array_equal(c.numpy().reshape(-1)[sample].astype(np.int64), colwant.sum(axis=0))
