@@ -77,6 +77,75 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
   // would read a transposed input with one useful element per sector. Such an input is first brought into the output's memory order by
   // the same-type copy, which does own a tiled kernel for every element size:
   // two extra coalesced passes instead of one uncoalesced one.
+  // Plans the operands as they are and launches; false only when `decline` is set and the
+  // per-type code refused a plan that would read a transposed operand uncoalesced.
+  auto launch = [&](bool decline) -> bool {
+    Plan pl{};
+    pl.nops = nops;
+    pl.numel = n;
+    bool sameShape = true;
+    for (int k = 0; k < nops; ++k) {
+      pl.ptr[k] = tensor_data(t[k], k == 0 ? d.outDt : d.dt);
+      pl.lay[k] = tensor_layout(t[k]);
+      if (!pl.ptr[k]) raise_error("pointwise apply on a tensor without storage");
+      if (k > 0) {
+        sameShape = sameShape && pl.lay[k].dims == pl.lay[0].dims;
+        for (int d2 = 0; sameShape && d2 < pl.lay[0].dims; ++d2)
+          sameShape = pl.lay[k].size[d2] == pl.lay[0].size[d2];
+      }
+    }
+    const DType dt = d.dt;
+    const bool floatFamilyFn =
+        (d.op != PointOp::Math1 && d.op != PointOp::Math2) || d.fn <= (int)MathFn::SqDiff ||
+        d.fn == (int)MathFn::RenormFactor || d.fn == (int)MathFn::LShiftValue ||
+        d.fn == (int)MathFn::RShiftValue || d.fn == (int)MathFn::CLShift || d.fn == (int)MathFn::CRShift;
+    bool launched = true;
+    if (d.op == PointOp::Copy) {
+      switch (dtype_size(dt)) {
+        case 1: apply_copy<uint8_t>(s, pl, sameShape); break;
+        case 2: apply_copy<uint16_t>(s, pl, sameShape); break;
+        case 4: apply_copy<uint32_t>(s, pl, sameShape); break;
+        default: apply_copy<uint64_t>(s, pl, sameShape); break;
+      }
+    } else if (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor) {
+      if (d.outDt != dt && d.outDt != DType::U8) raise_error("comparison output must be Byte or the input type");
+      if (dt == DType::F32) launched = apply_cmp<float>(s, pl, sameShape, d, decline);
+      else if (dt == DType::F16) launched = apply_cmp<__half>(s, pl, sameShape, d, decline);
+      else for_wide_type(dt, [&](auto tag) { launched = apply_cmp<decltype(tag)>(s, pl, sameShape, d, decline); });
+    } else if (d.outDt != dt) {
+      raise_error("pointwise op cannot change the element type");
+    } else if (rawmath_serves(dt, d.op)) {
+      // plain functors on the element's width (double: on double): all kernels, tiled ones included
+      if (dt == DType::F64) apply_rawmath<double>(s, pl, sameShape, d.op, d.v);
+      else if (dt == DType::I32) apply_rawmath<uint32_t>(s, pl, sameShape, d.op, d.v);
+      else apply_rawmath<uint64_t>(s, pl, sameShape, d.op, d.v);
+    } else if ((dt == DType::F32 || dt == DType::F16) && floatFamilyFn) {
+      const int g = op_group(d.op);
+      const float value = (float)d.v.f, value2 = (float)d.w.f;
+      const MathFn fn = (MathFn)d.fn;
+      if (dt == DType::F32) {
+        if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, d.op, value, fn, value2);
+        else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, d.op, value, fn, value2);
+        else apply_dispatch_group<float, 2>(s, pl, sameShape, d.op, value, fn, value2);
+      } else {
+        if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, d.op, value, fn, value2);
+        else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, d.op, value, fn, value2);
+        else apply_dispatch_group<__half, 2>(s, pl, sameShape, d.op, value, fn, value2);
+      }
+    } else if (dt == DType::F32 || dt == DType::F16) {
+      raise_error("pointwise op not available for this element type");
+    } else {
+      for_wide_type(dt, [&](auto tag) { apply_wide<decltype(tag)>(s, pl, sameShape, d); });
+    }
+    if (launched) THC_CHECK(hipGetLastError());
+    return launched;
+  };
+  // Comparisons of float into a Byte tensor own the pack variant of the tiled kernel: try the
+  // operands as they are first; a declined plan takes the densify route below.
+  if ((d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor) && d.dt == DType::F32 && d.outDt == DType::U8 &&
+      launch(true))
+    return true;
+
   TensorRef dense[kMaxOps] = {{s, nullptr}, {s, nullptr}, {s, nullptr}, {s, nullptr}};
   const bool offTiled = d.op != PointOp::Copy &&
                         (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor ||
@@ -118,63 +187,7 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     }
   }
 
-  Plan pl{};
-  pl.nops = nops;
-  pl.numel = n;
-  bool sameShape = true;
-  for (int k = 0; k < nops; ++k) {
-    pl.ptr[k] = tensor_data(t[k], k == 0 ? d.outDt : d.dt);
-    pl.lay[k] = tensor_layout(t[k]);
-    if (!pl.ptr[k]) raise_error("pointwise apply on a tensor without storage");
-    if (k > 0) {
-      sameShape = sameShape && pl.lay[k].dims == pl.lay[0].dims;
-      for (int d2 = 0; sameShape && d2 < pl.lay[0].dims; ++d2)
-        sameShape = pl.lay[k].size[d2] == pl.lay[0].size[d2];
-    }
-  }
-  const DType dt = d.dt;
-  const bool floatFamilyFn =
-      (d.op != PointOp::Math1 && d.op != PointOp::Math2) || d.fn <= (int)MathFn::SqDiff ||
-      d.fn == (int)MathFn::RenormFactor || d.fn == (int)MathFn::LShiftValue ||
-      d.fn == (int)MathFn::RShiftValue || d.fn == (int)MathFn::CLShift || d.fn == (int)MathFn::CRShift;
-  if (d.op == PointOp::Copy) {
-    switch (dtype_size(dt)) {
-      case 1: apply_copy<uint8_t>(s, pl, sameShape); break;
-      case 2: apply_copy<uint16_t>(s, pl, sameShape); break;
-      case 4: apply_copy<uint32_t>(s, pl, sameShape); break;
-      default: apply_copy<uint64_t>(s, pl, sameShape); break;
-    }
-  } else if (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor) {
-    if (d.outDt != dt && d.outDt != DType::U8) raise_error("comparison output must be Byte or the input type");
-    if (dt == DType::F32) apply_cmp<float>(s, pl, sameShape, d);
-    else if (dt == DType::F16) apply_cmp<__half>(s, pl, sameShape, d);
-    else for_wide_type(dt, [&](auto tag) { apply_cmp<decltype(tag)>(s, pl, sameShape, d); });
-  } else if (d.outDt != dt) {
-    raise_error("pointwise op cannot change the element type");
-  } else if (rawmath_serves(dt, d.op)) {
-    // plain functors on the element's width (double: on double): all kernels, tiled ones included
-    if (dt == DType::F64) apply_rawmath<double>(s, pl, sameShape, d.op, d.v);
-    else if (dt == DType::I32) apply_rawmath<uint32_t>(s, pl, sameShape, d.op, d.v);
-    else apply_rawmath<uint64_t>(s, pl, sameShape, d.op, d.v);
-  } else if ((dt == DType::F32 || dt == DType::F16) && floatFamilyFn) {
-    const int g = op_group(d.op);
-    const float value = (float)d.v.f, value2 = (float)d.w.f;
-    const MathFn fn = (MathFn)d.fn;
-    if (dt == DType::F32) {
-      if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, d.op, value, fn, value2);
-      else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, d.op, value, fn, value2);
-      else apply_dispatch_group<float, 2>(s, pl, sameShape, d.op, value, fn, value2);
-    } else {
-      if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, d.op, value, fn, value2);
-      else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, d.op, value, fn, value2);
-      else apply_dispatch_group<__half, 2>(s, pl, sameShape, d.op, value, fn, value2);
-    }
-  } else if (dt == DType::F32 || dt == DType::F16) {
-    raise_error("pointwise op not available for this element type");
-  } else {
-    for_wide_type(dt, [&](auto tag) { apply_wide<decltype(tag)>(s, pl, sameShape, d); });
-  }
-  THC_CHECK(hipGetLastError());
+  launch(false);
   return true;
 }
 

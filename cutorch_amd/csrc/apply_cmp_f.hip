@@ -2,6 +2,6 @@
 #include "apply_wide.hpp"
 
 namespace thc {
-template void apply_cmp<float>(THCState*, Plan&, bool, const ApplyDesc&);
-template void apply_cmp<__half>(THCState*, Plan&, bool, const ApplyDesc&);
+template bool apply_cmp<float>(THCState*, Plan&, bool, const ApplyDesc&, bool);
+template bool apply_cmp<__half>(THCState*, Plan&, bool, const ApplyDesc&, bool);
 }

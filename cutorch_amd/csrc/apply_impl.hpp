@@ -473,8 +473,10 @@ struct TiledArgs {
 // faster while the rows a tile writes stay within a few MiB of each other;
 // when they are spread over hundreds of MiB (a permuted 3-D operand) the
 // streaming hint wins by ~10%.
-template <typename T, typename Op, typename I, int VEC, int LXP, int LXQ, int MASK, bool NTS>
-__global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in0, const T* in1,
+// TOut differs from T for comparisons into a Byte tensor: the output pack then
+// holds VEC elements of TOut (4 bytes for fp32 inputs).
+template <typename T, typename Op, typename I, int VEC, int LXP, int LXQ, int MASK, bool NTS, typename TOut = T>
+__global__ __launch_bounds__(kBlock) void apply_tiled_kernel(TOut* out, const T* in0, const T* in1,
                                                              const T* in2, TiledArgs<I> args,
                                                              Op op) {
   constexpr int NOPS = Op::NIN + 1;
@@ -483,10 +485,11 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
   constexpr int ROWS_Q = kBlock / LXQ, PASSES_Q = TP / ROWS_Q;  // lanes along q: rows are p
   constexpr int PITCH = TP + 1;  // odd pitch: transposed reads spread over the banks
   using P = Pack<T, VEC>;
+  using PO = Pack<TOut, VEC>;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
 
-  const T* ptr[kMaxOps] = {out, in0, in1, in2};
+  const T* ptr[kMaxOps] = {nullptr, in0, in1, in2};  // the output is addressed through `out` (its own element type)
   const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
   const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
   bool staged[kMaxOps];
@@ -537,9 +540,11 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
     const uint32_t p0 = tp * TP, q0 = tq * TQ;
     const uint32_t pn = min((uint32_t)TP, args.sizeP - p0);  // valid extent
     const uint32_t qn = min((uint32_t)TQ, args.sizeQ - q0);
-    const T* tbase[kMaxOps];  // uniform pointer to the tile origin of operand k
+    const T* tbase[kMaxOps];  // uniform pointer to the tile origin of input k
+    TOut* obase = out + (base[0] + (I)p0 * args.strideP[0] + (I)q0 * args.strideQ[0]);
+    tbase[0] = nullptr;
 #pragma unroll
-    for (int k = 0; k < NOPS; ++k) {
+    for (int k = 1; k < NOPS; ++k) {
       I o = base[k] + (I)p0 * args.strideP[k];
       if (!(staged[k] && fused)) o += (I)q0 * args.strideQ[k];
       tbase[k] = ptr[k] + o;
@@ -621,11 +626,10 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(T* out, const T* in
               in[k - 1] = din[k - 1][r];
             }
           }
-          P res;
+          PO res;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) res.v[e] = op(in[0].v[e], in[1].v[e], in[2].v[e]);
-          store_pack<NTS>(reinterpret_cast<P*>(const_cast<T*>(tbase[0]) + r * rowStep[0] + vo[0]),
-                          res);
+          store_pack<NTS>(reinterpret_cast<PO*>(obase + r * rowStep[0] + vo[0]), res);
         }
       }
     };
@@ -973,11 +977,15 @@ inline bool tile_plan(const Plan& pl, int& p, int& q, int staged[kMaxOps]) {
   return true;
 }
 
-template <typename T, typename Op, typename I>
+// TOut != T (comparisons into a Byte tensor): only the pack variant exists;
+// other layouts are declined (false).
+template <typename T, typename Op, typename I, typename TOut = T>
 bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   int p, q, staged[kMaxOps] = {0, 0, 0, 0};
   if (!tile_plan(pl, p, q, staged)) return false;
   constexpr int VEC = 16 / sizeof(T);
+  constexpr bool kSameType = std::is_same<T, TOut>::value;
+  if (!kSameType) vecOnly = true;
   // vector variant: 64 x 128 elements for 4-byte types (LDS 33 KiB per staged
   // operand); scalar variant: 64 x 64.
   constexpr int LXP = 64 / VEC > 16 ? 16 : (64 / VEC < 8 ? 8 : 64 / VEC);
@@ -991,7 +999,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   bool vec = pl.lay[0].size[p] % VEC == 0 && pl.lay[0].size[q] % VEC == 0;
   for (int k = 0; k < pl.nops && vec; ++k) {
     const int fast = staged[k] ? p : q;
-    vec = aligned16<T>(pl.ptr[k]) && pl.lay[k].stride[fast] == 1;
+    vec = pack_aligned<T, TOut>(pl, k) && pl.lay[k].stride[fast] == 1;
     for (int d = 0; d < nd && vec; ++d)
       if (d != fast) vec = pl.lay[k].stride[d] % VEC == 0;
   }
@@ -1076,10 +1084,10 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   if (total >= kIndex32Limit) return false;  // tile bookkeeping is 32-bit
   args.totalTiles = (uint32_t)total;
   // distance covered by the output rows of one tile
-  const int64_t outSpan = (int64_t)tileP * pl.lay[0].stride[p] * (int64_t)sizeof(T);
+  const int64_t outSpan = (int64_t)tileP * pl.lay[0].stride[p] * (int64_t)sizeof(TOut);
   const int64_t ntKnob = tuning("apply.tiled.nt_store", -1);
   const bool nts = ntKnob >= 0 ? ntKnob != 0
-                               : (outSpan >= (int64_t(32) << 20) || pl.numel * (int64_t)sizeof(T) >= (int64_t(64) << 20));
+                               : (outSpan >= (int64_t(32) << 20) || pl.numel * (int64_t)sizeof(TOut) >= (int64_t(64) << 20));
   args.ntStore = nts ? 1u : 0u;
   bool lineAligned = true;  // every row of every operand starts on a 128-byte line
   for (int k = 0; k < pl.nops; ++k) {
@@ -1100,7 +1108,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
     args.xcdPer = (uint32_t)((total + 7) / 8);
   const int64_t slots = args.xcdPer ? (int64_t)args.xcdPer * 8 : total;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(slots, tuning("apply.tiled.max_grid", 1 << 22)));
-  T* out = (T*)pl.ptr[0];
+  TOut* out = (TOut*)pl.ptr[0];
   const T* i0 = (const T*)pl.ptr[1];
   const T* i1 = (const T*)pl.ptr[2];
   const T* i2 = (const T*)pl.ptr[3];
@@ -1113,18 +1121,20 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   case M:                                                                                         \
     if ((M) < (1 << Op::NIN)) {                                                                   \
       constexpr int MM = (M) < (1 << Op::NIN) ? (M) : 1;                                          \
-      if (shift)                                                                                  \
-        hipLaunchKernelGGL((apply_tiled_shift_kernel<T, Op, I, VEC, LXP, LXQ, MM>), dim3(grid),   \
-                           dim3(kBlock), ldsH, st, out, i0, i1, i2, args, op);                    \
-      else if (!vec)                                                                              \
-        hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, 1, 64, 64, MM, false>), dim3(grid),      \
-                           dim3(kBlock), ldsS, st, out, i0, i1, i2, args, op);                    \
-      else if (nts)                                                                               \
-        hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, VEC, LXP, LXQ, MM, true>), dim3(grid),   \
-                           dim3(kBlock), ldsV, st, out, i0, i1, i2, args, op);                    \
-      else                                                                                        \
-        hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, VEC, LXP, LXQ, MM, false>), dim3(grid),  \
-                           dim3(kBlock), ldsV, st, out, i0, i1, i2, args, op);                    \
+      if constexpr (kSameType) {                                                                  \
+        if (shift)                                                                                \
+          hipLaunchKernelGGL((apply_tiled_shift_kernel<T, Op, I, VEC, LXP, LXQ, MM>), dim3(grid), \
+                             dim3(kBlock), ldsH, st, out, i0, i1, i2, args, op);                  \
+        else if (!vec)                                                                            \
+          hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, 1, 64, 64, MM, false>), dim3(grid),    \
+                             dim3(kBlock), ldsS, st, out, i0, i1, i2, args, op);                  \
+      }                                                                                           \
+      if (vec && nts)                                                                             \
+        hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, VEC, LXP, LXQ, MM, true, TOut>),         \
+                           dim3(grid), dim3(kBlock), ldsV, st, out, i0, i1, i2, args, op);        \
+      else if (vec)                                                                               \
+        hipLaunchKernelGGL((apply_tiled_kernel<T, Op, I, VEC, LXP, LXQ, MM, false, TOut>),        \
+                           dim3(grid), dim3(kBlock), ldsV, st, out, i0, i1, i2, args, op);        \
     }                                                                                             \
     break;
   switch (mask) {
@@ -1197,8 +1207,11 @@ bool launch_flatmix(THCState* s, const Plan& pl, Op op) {
 // TILED = false keeps an op off the LDS-tiled kernels (transposed operands then
 // go through the strided kernel); LEAN trims launch variants. Both exist to
 // bound the number of kernels built for element types off the hot path.
+// With `decline` set, a plan that has a transposed operand but does not fit
+// the pack variant of the tiled kernel is not launched at all (false): the
+// caller densifies that operand first instead of reading it uncoalesced.
 template <typename T, typename Op, typename TOut = T, bool TILED = true, bool LEAN = false>
-void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
+bool run_plan(THCState* s, Plan& pl, bool sameShape, Op op, bool decline = false) {
   bool wide = force_64bit_index();
   for (int k = 0; k < pl.nops; ++k) {
     wide = wide || !fits_32bit(pl.lay[k]);
@@ -1209,7 +1222,7 @@ void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
     for (int k = 0; k < pl.nops && flat; ++k) flat = pl.lay[k].stride[0] == 1;
     if (flat) {
       launch_contig<T, Op, TOut, LEAN>(s, pl, op);
-      return;
+      return true;
     }
     // (plain functors of the float and half slices only: instantiating it for the
     // code-dispatched families and the six wider types doubled the build time)
@@ -1218,29 +1231,34 @@ void run_plan(THCState* s, Plan& pl, bool sameShape, Op op) {
       if constexpr (TILED && std::is_same<T, TOut>::value) {
         if (tuning("apply.tiled.enable", 1) &&
             (wide ? launch_tiled<T, Op, uint64_t>(s, pl, op, true) : launch_tiled<T, Op, uint32_t>(s, pl, op, true)))
-          return;
+          return true;
       }
       if (!indexed_can_pack<T, TOut>(pl) &&
           (wide ? launch_flatmix<T, Op, uint64_t, TOut>(s, pl, op) : launch_flatmix<T, Op, uint32_t, TOut>(s, pl, op)))
-        return;
+        return true;
     }
-    if constexpr (TILED && std::is_same<T, TOut>::value) {
+    if constexpr (TILED) {
       if (tuning("apply.tiled.enable", 1)) {
-        if (wide ? launch_tiled<T, Op, uint64_t>(s, pl, op) : launch_tiled<T, Op, uint32_t>(s, pl, op))
-          return;
+        if (wide ? launch_tiled<T, Op, uint64_t, TOut>(s, pl, op) : launch_tiled<T, Op, uint32_t, TOut>(s, pl, op))
+          return true;
       }
+    }
+    if (decline) {
+      int p, q, staged[kMaxOps] = {0, 0, 0, 0};
+      if (tile_plan(pl, p, q, staged)) return false;  // a transposed operand that no tiled kernel took
     }
     if (wide)
       launch_indexed<T, Op, uint64_t, true, TOut>(s, pl, op);
     else
       launch_indexed<T, Op, uint32_t, true, TOut>(s, pl, op);
-    return;
+    return true;
   }
   for (int k = 0; k < pl.nops; ++k) collapse(pl.lay[k]);
   if (wide)
     launch_indexed<T, Op, uint64_t, false, TOut>(s, pl, op);
   else
     launch_indexed<T, Op, uint32_t, false, TOut>(s, pl, op);
+  return true;
 }
 
 

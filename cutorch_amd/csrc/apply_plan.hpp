@@ -29,7 +29,8 @@ void apply_copy(THCState* s, Plan& pl, bool sameShape);
 // (apply_w_*.hip) and the comparison ops of every type.
 template <typename T>
 void apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d);
+// false = declined (see apply_wide.hpp): the caller densifies and calls again with decline = false
 template <typename T>
-void apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d);
+bool apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool decline);
 
 }  // namespace thc

@@ -3,5 +3,5 @@
 
 namespace thc {
 template void apply_wide<double>(THCState*, Plan&, bool, const ApplyDesc&);
-template void apply_cmp<double>(THCState*, Plan&, bool, const ApplyDesc&);
+template bool apply_cmp<double>(THCState*, Plan&, bool, const ApplyDesc&, bool);
 }

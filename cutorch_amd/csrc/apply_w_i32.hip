@@ -3,5 +3,5 @@
 
 namespace thc {
 template void apply_wide<int32_t>(THCState*, Plan&, bool, const ApplyDesc&);
-template void apply_cmp<int32_t>(THCState*, Plan&, bool, const ApplyDesc&);
+template bool apply_cmp<int32_t>(THCState*, Plan&, bool, const ApplyDesc&, bool);
 }

@@ -369,22 +369,24 @@ struct CmpOp {
   }
 };
 
+// Returns false (nothing launched) when `decline` is set and a transposed
+// operand would have to be read uncoalesced: comparisons of float into a Byte
+// tensor own the pack variant of the LDS-tiled kernel, everything else is
+// densified by the caller first.
 template <typename T>
-void apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d) {
+bool apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool decline) {
   using C = typename Num<T>::C;
   const C v = Num<T>::scalar(d.v);
   const bool byteOut = d.outDt == DType::U8 && !std::is_same<T, uint8_t>::value;
+  constexpr bool kTiled = std::is_same<T, float>::value;
   if (d.op == PointOp::CmpValue) {
     if (byteOut)
-      run_plan<T, CmpOp<T, uint8_t, 1>, uint8_t, false, true>(s, pl, sameShape, CmpOp<T, uint8_t, 1>{d.fn, v});
-    else
-      run_plan<T, CmpOp<T, T, 1>, T, false, true>(s, pl, sameShape, CmpOp<T, T, 1>{d.fn, v});
-  } else {
-    if (byteOut)
-      run_plan<T, CmpOp<T, uint8_t, 2>, uint8_t, false, true>(s, pl, sameShape, CmpOp<T, uint8_t, 2>{d.fn, v});
-    else
-      run_plan<T, CmpOp<T, T, 2>, T, false, true>(s, pl, sameShape, CmpOp<T, T, 2>{d.fn, v});
+      return run_plan<T, CmpOp<T, uint8_t, 1>, uint8_t, kTiled, true>(s, pl, sameShape, CmpOp<T, uint8_t, 1>{d.fn, v}, decline);
+    return run_plan<T, CmpOp<T, T, 1>, T, false, true>(s, pl, sameShape, CmpOp<T, T, 1>{d.fn, v}, decline);
   }
+  if (byteOut)
+    return run_plan<T, CmpOp<T, uint8_t, 2>, uint8_t, kTiled, true>(s, pl, sameShape, CmpOp<T, uint8_t, 2>{d.fn, v}, decline);
+  return run_plan<T, CmpOp<T, T, 2>, T, false, true>(s, pl, sameShape, CmpOp<T, T, 2>{d.fn, v}, decline);
 }
 
 // Every arithmetic op of an element type that has no dedicated slices.

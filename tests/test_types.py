@@ -701,9 +701,34 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
     assert_bit_equal(m.numpy(), wm.numpy())
     f = thc.Tensor.from_numpy(rng.standard_normal((200, 136)).astype(np.float32))
     g = thc.Tensor.from_numpy(rng.standard_normal((136, 200)).astype(np.float32))
+    # float into Byte owns the pack variant of the tiled kernel (4-byte output packs) ...
     m = thc.Tensor("byte").compare_tensor("ge", f.t(), g)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "tiled"
     assert_bit_equal(m.numpy(), (f.numpy().T >= g.numpy()).astype(np.uint8))
+    m = thc.Tensor("byte").compare_value("lt", f.t(), 0.25)
+    assert thc.last_kernel() == "tiled"
+    assert_bit_equal(m.numpy(), (f.numpy().T < np.float32(0.25)).astype(np.uint8))
+    thc.force_64bit_index(True)
+    try:
+        m = thc.Tensor("byte").compare_tensor("ne", g, f.t())
+        assert thc.last_kernel() == "tiled"
+    finally:
+        thc.force_64bit_index(False)
+    assert_bit_equal(m.numpy(), (g.numpy() != f.numpy().T).astype(np.uint8))
+    # ... and only that one: shapes whose rows are not whole aligned packs are declined and densified,
+    # as is a comparison whose output has the input's type
+    f2 = thc.Tensor.from_numpy(rng.standard_normal((201, 137)).astype(np.float32))
+    g2 = thc.Tensor.from_numpy(rng.standard_normal((137, 201)).astype(np.float32))
+    m = thc.Tensor("byte").compare_tensor("le", f2.t(), g2)
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(m.numpy(), (f2.numpy().T <= g2.numpy()).astype(np.uint8))
+    mt = thc.Tensor("float").compare_tensor("gt", f.t(), g, same_type=True)
+    assert thc.last_kernel() == "contig"
+    assert_bit_equal(mt.numpy(), (f.numpy().T > g.numpy()).astype(np.float32))
+    # a transposed Byte OUTPUT of a float comparison (its memory order decides): 4-byte output packs along its rows
+    mb = thc.Tensor.from_numpy(np.zeros((200, 136), np.uint8))
+    mb.t().compare_tensor("lt", g, f.t())
+    assert_bit_equal(mb.numpy().T, (g.numpy() < f.numpy().T).astype(np.uint8))
 
 
 @pytest.mark.gpu
