@@ -37,6 +37,8 @@
 // the lower index on equal values at every level, so the first occurrence wins
 // as in a sequential scan; the first NaN wins over everything.
 #pragma once
+#include <time.h>
+
 #include <cmath>
 #include <limits>
 #include <type_traits>
@@ -2319,6 +2321,43 @@ bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in_, voi
 }
 
 // ------------------------------------------------------------------- all --
+// The scalar of a whole-tensor reduction arrives in a pinned host slot that the
+// last kernel writes. hipStreamSynchronize takes about 10 us to notice that a
+// stream has drained; watching the slot itself takes 1-2. The slot is armed
+// with a bit pattern no reduction is likely to produce (a NaN with an odd
+// payload) before the launch and polled until it changes; if it has not
+// changed after 20 ms (a long queue in front of the kernel, a failed launch, or
+// a result that happens to equal the pattern) the stream is waited for in the
+// ordinary way, so correctness never rests on the pattern.
+constexpr uint64_t kHostSlotArmed = 0x7ff8dead7fc0deadull;
+inline void arm_host_slot(const StreamScratch& sc) {
+  *reinterpret_cast<volatile uint64_t*>(sc.hostResult) = kHostSlotArmed;
+  __atomic_thread_fence(__ATOMIC_SEQ_CST);
+}
+template <typename A>
+A wait_host_slot(THCState* s, const StreamScratch& sc) {
+  static_assert(sizeof(A) == 4 || sizeof(A) == 8, "accumulator width");
+  auto changed = [&]() {
+    if (sizeof(A) == 8) return *reinterpret_cast<const volatile uint64_t*>(sc.hostResult) != kHostSlotArmed;
+    return *reinterpret_cast<const volatile uint32_t*>(sc.hostResult) != (uint32_t)kHostSlotArmed;
+  };
+  bool seen = false;
+  if (tuning("reduce.all.poll", 1)) {
+    timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (uint32_t n = 0; !(seen = changed()); ++n) {
+      __builtin_ia32_pause();
+      if ((n & 1023u) == 1023u) {
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        if ((t1.tv_sec - t0.tv_sec) * 1000000000ll + (t1.tv_nsec - t0.tv_nsec) > 20000000ll) break;
+      }
+    }
+  }
+  if (!seen) THC_CHECK(hipStreamSynchronize(current_stream(s)));
+  __atomic_thread_fence(__ATOMIC_SEQ_CST);
+  return *reinterpret_cast<const volatile A*>(sc.hostResult);
+}
+
 template <typename A>
 constexpr DType acc_dtype() {
   return std::is_same<A, float>::value ? DType::F32
@@ -2368,6 +2407,7 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, const void* src
   }
   // Workgroups of 256 lanes stream chunks that are multiples of one full
   // batch (256 lanes x 8 packs); a few workgroups per CU.
+  arm_host_slot(sc);
   auto stage2 = [&](auto srcTag, auto f, auto idxTag) {
     using TI = decltype(srcTag);
     using F2 = decltype(f);
@@ -2424,8 +2464,7 @@ void reduce_all_with(THCState* s, ReduceGeom g, const void* src, const void* src
   // The one place the caller blocks on the device (THCReduceAll.cuh:333-335):
   // the kernel has stored the scalar into pinned host memory, so waiting for
   // the stream is all that is left of the reference's synchronous D2H copy.
-  THC_CHECK(hipStreamSynchronize(current_stream(s)));
-  const A r = *reinterpret_cast<const volatile A*>(sc.hostResult);
+  const A r = wait_host_slot<A>(s, sc);
   result->f = (double)r;
   result->i = (int64_t)r;
 }
@@ -2488,6 +2527,7 @@ void reduce_all_moments_type(THCState* s, int64_t n, const void* src, Scalar* re
     blocks = (n + chunk - 1) / chunk;
     hipStream_t st = current_stream(s);
     A* part = (A*)sc.partials;
+    arm_host_slot(sc);
     auto go = [&](auto idxTag) {
       using I = decltype(idxTag);
       if (aligned16(src))
@@ -2503,8 +2543,7 @@ void reduce_all_moments_type(THCState* s, int64_t n, const void* src, Scalar* re
                        devOut, hostDev);
     note_kernel("all-moments");
     THC_CHECK(hipGetLastError());
-    THC_CHECK(hipStreamSynchronize(st));
-    const A r = *reinterpret_cast<const volatile A*>(sc.hostResult);
+    const A r = wait_host_slot<A>(s, sc);
     result->f = (double)r;
     result->i = (int64_t)r;
   }
