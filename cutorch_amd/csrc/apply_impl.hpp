@@ -235,6 +235,38 @@ __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T
   // The whole streaming loop sits inside the code dispatch: every code gets its
   // own loop, in which the loads of a batch are scheduled ahead of the math.
   with_fixed_code(op, [&](auto f) {
+    if constexpr (NT && sizeof(P) == 16 && sizeof(PO) == 16) {
+      // Streaming form on buffer instructions: the workgroup's piece of every operand is a
+      // buffer of its own (uniform base in scalar registers, 32-bit lane offsets), whose
+      // bounds check makes the last piece safe without a predicate on any load or store
+      // (out-of-range loads return zero, out-of-range stores are dropped). About 1.5 %
+      // faster than the predicated global form on 2^24 .. 2^26-element adds.
+      constexpr uint32_t kPiecePacks = kBlock * UNROLL;
+      for (uint64_t first = (uint64_t)blockIdx.x * kPiecePacks; first < npack; first += step) {
+        const uint32_t bytes = (uint32_t)min((uint64_t)kPiecePacks, npack - first) * 16u;
+        const BufferRsrc ro = make_rsrc(out + first * VEC, bytes);
+        const BufferRsrc r0 = make_rsrc(Op::NIN > 0 ? in0 + first * VEC : nullptr, Op::NIN > 0 ? bytes : 0u);
+        const BufferRsrc r1 = make_rsrc(Op::NIN > 1 ? in1 + first * VEC : nullptr, Op::NIN > 1 ? bytes : 0u);
+        const BufferRsrc r2 = make_rsrc(Op::NIN > 2 ? in2 + first * VEC : nullptr, Op::NIN > 2 ? bytes : 0u);
+        P a[UNROLL], b[UNROLL], c[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const uint32_t off = (threadIdx.x + (uint32_t)u * kBlock) * 16u;
+          if (Op::NIN > 0) a[u] = buffer_load_pack<P>(r0, off);
+          if (Op::NIN > 1) b[u] = buffer_load_pack<P>(r1, off);
+          if (Op::NIN > 2) c[u] = buffer_load_pack<P>(r2, off);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const uint32_t off = (threadIdx.x + (uint32_t)u * kBlock) * 16u;
+          PO r;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) r.v[e] = f(a[u].v[e], b[u].v[e], c[u].v[e]);
+          buffer_store_pack<NTS>(r, ro, off);
+        }
+      }
+      return;
+    }
     for (uint64_t base = (uint64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x; base < npack;
          base += step) {
       P a[UNROLL], b[UNROLL], c[UNROLL];

@@ -68,6 +68,33 @@ __device__ __forceinline__ void store_pack(P* p, const P& v) {
   }
 }
 
+// Buffer-instruction access to a run of `bytes` bytes at `p`: loads beyond the
+// run return zero and stores beyond it are dropped by the hardware's bounds
+// check, so a kernel needs no predicate for the ragged end of its data.
+// (Word 3 of the descriptor: 32-bit data format, raw addressing.)
+using BufferRsrc = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ BufferRsrc make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+// 16-byte packs, nontemporal hint on the load; the store takes it on request.
+template <typename P>
+__device__ __forceinline__ P buffer_load_pack(BufferRsrc r, uint32_t byteOffset) {
+  static_assert(sizeof(P) == 16, "16-byte packs");
+  typedef unsigned raw __attribute__((ext_vector_type(4)));
+  const raw v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byteOffset, 0, /*nt*/ 2);
+  P out;
+  __builtin_memcpy(&out, &v, 16);
+  return out;
+}
+template <bool NT, typename P>
+__device__ __forceinline__ void buffer_store_pack(const P& v, BufferRsrc r, uint32_t byteOffset) {
+  static_assert(sizeof(P) == 16, "16-byte packs");
+  typedef unsigned raw __attribute__((ext_vector_type(4)));
+  raw x;
+  __builtin_memcpy(&x, &v, 16);
+  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byteOffset, 0, NT ? 2 : 0);
+}
+
 template <typename T>
 struct Cvt {
   static __device__ __forceinline__ float up(T x) { return (float)x; }
