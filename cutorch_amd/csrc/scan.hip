@@ -18,6 +18,7 @@
 // Accumulation is fp32 for float and half (rounded per output element), double
 // for double, wrapping 64-bit for the integer types.
 #include <algorithm>
+#include <cmath>
 #include <type_traits>
 
 #include "common.hpp"
@@ -170,13 +171,20 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
   }
 }
 
+// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits
+// for every global load and store of the wave, which would drain the packs
+// requested ahead for the next segment and the stores of the previous one.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Scan along a strided dim of a dense [outer][R][inner] block. A workgroup
 // owns one `outer` index and TX*VEC adjacent columns and walks R in segments
 // of TY*U rows: thread row ty holds U consecutive rows of the segment in
 // registers, scans them locally, the thread rows exchange their totals
 // through LDS, and a per-column carry links the segments. The input is read
 // once and the output written once.
-template <typename T, typename Op, int VEC>
+template <typename T, typename Op, int VEC, bool PF>
 __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t outer, uint64_t R,
@@ -189,29 +197,38 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
   const uint32_t TY = kBlock / TX;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const uint64_t blocks = outer * colTiles;
+  const uint64_t segRows = (uint64_t)TY * U;
   for (uint64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
     const uint64_t o = b / colTiles, ct = b - o * colTiles;
     const uint64_t col = (ct * TX + tx) * VEC;
     const bool live = col < inner;  // inner % VEC == 0 for VEC > 1
-    const T* src = in + o * R * inner + col;
+    // Loads carry no predicate: rows past the end re-read the last row and idle
+    // lanes read column 0 (both discarded), so the compiler can count exactly
+    // which loads a wait has to cover.
+    const T* src = in + o * R * inner + (live ? col : 0);
     T* dst = out + o * R * inner + col;
     A carry[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) carry[e] = Op::id();
-    uint32_t flip = 0;
-    for (uint64_t seg = 0; seg < R; seg += (uint64_t)TY * U, flip ^= 1) {
+    auto fetch = [&](uint64_t r0, P (&v)[U]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint64_t r = r0 + u < R ? r0 + u : R - 1;
+        v[u] = load_pack<true>(reinterpret_cast<const P*>(src + r * inner));
+      }
+    };
+    // One segment: `cur` holds its packs (PF: requested during the previous
+    // segment; the packs of the following one are requested into `nxt` first).
+    auto step = [&](uint64_t seg, uint32_t flip, P (&cur)[U], P (&nxt)[U]) {
       const uint64_t r0 = seg + (uint64_t)ty * U;
+      if (PF) fetch(r0 + segRows, nxt);
+      else fetch(r0, cur);
       A x[U][VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (live && r0 + u < R) {
-          const P v = load_pack<true>(reinterpret_cast<const P*>(src + (r0 + u) * inner));
+        const bool have = live && r0 + u < R;
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) x[u][e] = scan_up<A>(v.v[e]);
-        } else {
-#pragma unroll
-          for (int e = 0; e < VEC; ++e) x[u][e] = Op::id();
-        }
+        for (int e = 0; e < VEC; ++e) x[u][e] = have ? scan_up<A>(cur[u].v[e]) : Op::id();
       }
 #pragma unroll
       for (int u = 1; u < U; ++u) {
@@ -220,7 +237,7 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
       }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) totals[flip][(ty * TX + tx) * VEC + e] = x[U - 1][e];
-      __syncthreads();  // the other buffer is free again after the next barrier
+      lds_barrier();  // the other buffer is free again after the next barrier
       A offset[VEC], running[VEC];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
@@ -248,8 +265,14 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
       }
 #pragma unroll
       for (int e = 0; e < VEC; ++e) carry[e] = Op::op(carry[e], running[e]);
+    };
+    P bufA[U], bufB[U];
+    if (PF) fetch((uint64_t)ty * U, bufA);
+    for (uint64_t seg = 0; seg < R; seg += 2 * segRows) {
+      step(seg, 0, bufA, bufB);
+      if (seg + segRows < R) step(seg + segRows, 1, bufB, bufA);
     }
-    __syncthreads();  // both LDS buffers are idle before the next tile
+    lds_barrier();  // both LDS buffers are idle before the next tile
   }
 }
 
@@ -499,17 +522,43 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t packs = (inner + pack - 1) / pack;
     // 16..64 lanes along the unit-stride dim: narrower tiles when that is what
     // gives every CU a workgroup
-    uint32_t TX = std::max<uint32_t>(16, pow2_at_least((uint64_t)packs));
-    const int64_t want = 2 * (int64_t)num_compute_units(s);
-    while (TX > 16 && outer * ((packs + TX - 1) / TX) < want) TX >>= 1;
+    // Lanes along the unit-stride dim (the strip a workgroup owns is TX packs wide). Measured on 1 GiB
+    // fp32 scans: with two to three workgroups per CU 512-byte strips run at 0.76-0.77 of peak, 1 KiB
+    // strips at 0.72 (4 thread rows make short segments), 256-byte strips at 0.63, 128-byte ones at 0.54;
+    // one workgroup per CU costs 8 % (with the next segment requested ahead; 17 % without), idle CUs cost
+    // in proportion, four and more workgroups per CU cost about 12 %. The width with the best product
+    // wins; requesting ahead is used below two workgroups per CU (it doubles the registers and is
+    // neutral to slightly slower above).
+    const uint32_t minTX = (uint32_t)std::max<int64_t>(1, tuning("scan.cols.min_tx", 8));
+    const uint32_t maxTX = (uint32_t)std::max<int64_t>(minTX, std::min<int64_t>(64, tuning("scan.cols.max_tx", 64)));
+    const double cus = (double)num_compute_units(s);
+    uint32_t TX = minTX;
+    double bestScore = -1, bestPerCU = 0;
+    for (uint32_t tx = maxTX; tx >= minTX; tx >>= 1) {
+      const double tiles = (double)((packs + tx - 1) / tx), perCU = (double)outer * tiles / cus;
+      const double width = tx >= 64 ? 0.94 : tx == 32 ? 1.0 : tx == 16 ? 0.83 : tx == 8 ? 0.70 : 0.37;
+      const double lanes = (double)packs / (tiles * tx);
+      const double fill = perCU < 1 ? 0.92 * perCU : perCU < 2 ? 0.92 : perCU <= 3 ? 1.0 : 0.88;
+      const double score = width * lanes * fill;
+      if (score > bestScore * 1.001) {
+        bestScore = score;
+        bestPerCU = perCU;
+        TX = tx;
+      }
+      if (tx == 1) break;
+    }
     const int64_t colTiles = (packs + TX - 1) / TX;
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * colTiles, 1 << 30));
-    if (vec)
-      hipLaunchKernelGGL((scan_cols_kernel<T, Op, VECC>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts);
-    else
-      hipLaunchKernelGGL((scan_cols_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts);
+    const int64_t pfKnob = tuning("scan.cols.prefetch", -1);
+    const bool pf = pfKnob >= 0 ? pfKnob != 0 : bestPerCU < 2;
+#define THC_SCAN_COLS(V, F)                                                                              \
+  hipLaunchKernelGGL((scan_cols_kernel<T, Op, V, F>), dim3(grid), dim3(kBlock), 0, st, out, in,          \
+                     (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts)
+    if (vec && pf) THC_SCAN_COLS(VECC, true);
+    else if (vec) THC_SCAN_COLS(VECC, false);
+    else if (pf) THC_SCAN_COLS(1, true);
+    else THC_SCAN_COLS(1, false);
+#undef THC_SCAN_COLS
     note_kernel("scan-cols");
   }
 }

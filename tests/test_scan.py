@@ -141,3 +141,36 @@ def _gpu_scan_cases(thc, oracle, kind):
     assert_bit_equal(t.numpy(), np.cumsum(xi.astype(np.int64), axis=1).astype(np.float32))
     with pytest.raises(thc.THCError, match="out of range"):
         thc.Tensor("float").cumsum(thc.Tensor.from_numpy(xi), 2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double"])
+def test_gpu_scan_over_a_strided_dim_in_every_strip_width(thc, oracle, kind):
+    """The scan over a non-innermost dim picks a strip width (8-64 lanes) and whether the next
+    segment's packs are requested ahead from the shape and the chip; here each is forced in turn.
+    Small integers: exact whatever the split; row counts off the segment size; an odd inner size
+    takes the element-wise variant."""
+    rng = np.random.default_rng(23)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64}[kind]
+    thc.set_tuning("scan.chunked", 0)       # (few long slices would otherwise be cut into chunks of rows,
+    thc.set_tuning("scan.slab", 0)          #  small ones scanned in LDS)
+    try:
+        for shape in ((3, 300, 520), (2, 129, 1024), (1, 64, 96), (2, 1000, 136), (1, 77, 515), (5, 1, 8192), (4, 9, 4100)):
+            sparse = (rng.integers(0, 12, shape) == 0) * rng.integers(-2, 3, shape)
+            x = thc.Tensor.from_numpy(sparse.astype(dtype))
+            want = np.cumsum(sparse, axis=1)
+            assert np.abs(want).max() < 2048
+            for pf in (0, 1):
+                for tx in (8, 16, 32, 64):
+                    thc.set_tuning("scan.cols.prefetch", pf)
+                    thc.set_tuning("scan.cols.min_tx", tx)
+                    thc.set_tuning("scan.cols.max_tx", tx)
+                    got = thc.Tensor(kind).cumsum(x, 1)
+                    assert thc.last_kernel() == "scan-cols", (shape, thc.last_kernel())
+                    assert_bit_equal(got.numpy(), want.astype(dtype), "%s %s pf=%d tx=%d" % (kind, shape, pf, tx))
+    finally:
+        thc.set_tuning("scan.chunked", 1)
+        thc.set_tuning("scan.slab", 1)
+        thc.set_tuning("scan.cols.prefetch", -1)
+        thc.set_tuning("scan.cols.min_tx", 8)
+        thc.set_tuning("scan.cols.max_tx", 64)
