@@ -489,6 +489,7 @@ struct TiledArgs {
   // share cache lines run back to back; 1 = q fastest throughout.
   uint32_t groupP;
   uint32_t ntStore;  // shifted-window variant: whole packs of the output go out with the streaming hint
+  uint32_t ntLoad;   // shifted-window variant: inputs are read with the streaming hint
 };
 
 // A tile spans TP = LXP*VEC elements of dim p and TQ = LXQ*VEC of dim q.
@@ -560,8 +561,19 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(TOut* out, const T*
     const uint32_t tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
     if (tile >= args.totalTiles) continue;  // uniform over the workgroup
     uint32_t rest, tq, tp;
-    args.tilesQ.divmod(tile, rest, tq);
-    args.tilesP.divmod(rest, rest, tp);
+    if (args.groupP > 1) {
+      const uint32_t perBatch = args.tilesP.d * args.tilesQ.d;
+      rest = tile / perBatch;
+      const uint32_t t = tile - rest * perBatch;
+      const uint32_t band = t / (args.groupP * args.tilesQ.d);
+      const uint32_t r = t - band * (args.groupP * args.tilesQ.d);
+      const uint32_t gp = min(args.groupP, args.tilesP.d - band * args.groupP);  // ragged last band
+      tq = r / gp;
+      tp = band * args.groupP + (r - tq * gp);
+    } else {
+      args.tilesQ.divmod(tile, rest, tq);
+      args.tilesP.divmod(rest, rest, tp);
+    }
     I base[kMaxOps] = {0, 0, 0, 0};
     for (int j = 0; j < args.nbatch; ++j) {
       uint32_t r;
@@ -590,11 +602,7 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(TOut* out, const T*
       const bool okP = FULL || lxp * VEC < pn;
       const bool okQ = FULL || lxq * VEC < qn;
       // phase 1: staged inputs, lanes along p, into lds[slot][q][p]
-#pragma unroll
-      for (int k = 1; k < NOPS; ++k) {
-        if (!staged[k]) continue;
-        T* slab = lds + slot[k] * (TQ * PITCH);
-        P v[PASSES_P];
+      auto issue_staged = [&](int k, P (&v)[PASSES_P]) {
         if (!fused) {
 #pragma unroll
           for (int r = 0; r < PASSES_P; ++r) {
@@ -618,6 +626,9 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(TOut* out, const T*
             }
           }
         }
+      };
+      auto write_staged = [&](int k, const P (&v)[PASSES_P]) {
+        T* slab = lds + slot[k] * (TQ * PITCH);
 #pragma unroll
         for (int r = 0; r < PASSES_P; ++r) {
           const uint32_t qi = lyp + r * ROWS_P;
@@ -626,23 +637,50 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_kernel(TOut* out, const T*
             for (int e = 0; e < VEC; ++e) slab[qi * PITCH + lxp * VEC + e] = v[r].v[e];
           }
         }
+      };
+      P din[3][PASSES_Q];
+      auto issue_direct = [&]() {
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k) {
+          if (staged[k]) continue;
+#pragma unroll
+          for (int r = 0; r < PASSES_Q; ++r) {
+            const uint32_t pi = lyq + r * ROWS_Q;
+            if (FULL || (okQ && pi < pn))
+              din[k - 1][r] =
+                  load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
+          }
+        }
+      };
+      // Interior tiles of ops with at most two inputs request the direct operand's packs right
+      // behind the staged ones, so both are in flight while the staged packs go into LDS; the
+      // barrier then orders LDS only. (With three inputs the extra live packs cost a resident
+      // workgroup per CU, and that kernel already runs at the rate of the flat stream.)
+      constexpr bool EARLY = FULL && Op::NIN <= 2;
+      if constexpr (EARLY) {
+        P v[2][PASSES_P];
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k)
+          if (staged[k]) issue_staged(k, v[k - 1]);
+        issue_direct();
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k)
+          if (staged[k]) write_staged(k, v[k - 1]);
+        lds_barrier();
+      } else {
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k) {
+          if (!staged[k]) continue;
+          P v[PASSES_P];
+          issue_staged(k, v);
+          write_staged(k, v);
+        }
+        __syncthreads();
+        issue_direct();
       }
-      __syncthreads();
 
       // phase 2: compute with lanes along q
       const uint32_t qi = lxq * VEC;
-      P din[3][PASSES_Q];
-#pragma unroll
-      for (int k = 1; k < NOPS; ++k) {
-        if (staged[k]) continue;
-#pragma unroll
-        for (int r = 0; r < PASSES_Q; ++r) {
-          const uint32_t pi = lyq + r * ROWS_Q;
-          if (FULL || (okQ && pi < pn))
-            din[k - 1][r] =
-                load_pack<true>(reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k]));
-        }
-      }
 #pragma unroll
       for (int r = 0; r < PASSES_Q; ++r) {
         const uint32_t pi = lyq + r * ROWS_Q;
@@ -773,7 +811,9 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
         const int qi = (int)lyp + r * ROWS_P;
         const T* row = tbase[k] + r * rowStep[k] + vo[k];
         first[r] = (int)(lxp * VEC) - misalignment(row);
-        if (qi < qn && first[r] < pn) v[r] = load_pack<true>(reinterpret_cast<const P*>(row + first[r]));
+        if (qi < qn && first[r] < pn)
+          v[r] = args.ntLoad ? load_pack<true>(reinterpret_cast<const P*>(row + first[r]))
+                             : load_pack<false>(reinterpret_cast<const P*>(row + first[r]));
       }
 #pragma unroll
       for (int r = 0; r < PASSES_P; ++r) {
@@ -803,9 +843,10 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
       if (staged[k]) continue;
 #pragma unroll
       for (int r = 0; r < PASSES_Q; ++r) {
-        if (first[r] < qn)
-          din[k - 1][r] = load_pack<true>(
-              reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k] + first[r]));
+        if (first[r] < qn) {
+          const P* src = reinterpret_cast<const P*>(tbase[k] + r * rowStep[k] + vo[k] + first[r]);
+          din[k - 1][r] = args.ntLoad ? load_pack<true>(src) : load_pack<false>(src);
+        }
       }
     }
 #pragma unroll
@@ -1121,6 +1162,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   const bool nts = ntKnob >= 0 ? ntKnob != 0
                                : (outSpan >= (int64_t(32) << 20) || pl.numel * (int64_t)sizeof(TOut) >= (int64_t(64) << 20));
   args.ntStore = nts ? 1u : 0u;
+  args.ntLoad = tuning("apply.tiled.shift_nt_load", 1) ? 1u : 0u;
   bool lineAligned = true;  // every row of every operand starts on a 128-byte line
   for (int k = 0; k < pl.nops; ++k) {
     lineAligned = lineAligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % 128 == 0;
@@ -1131,7 +1173,11 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   // bands of 8 tiles along p: the staged windows of neighbours in p share cache
   // lines (8191 x 8193: add 4.5 -> 4.7 TB/s, copy 5.1 -> 5.6); only where a
   // band is a small part of p, since p-fastest order as a whole is the slow one
-  args.groupP = shift ? (uint32_t)std::max<int64_t>(1, tuning("apply.tiled.group_p", 8)) : 1;
+  // (the aligned kernel: bands of 16 lift a transposed copy of 8192 x 8192 from 0.65 to 0.70 of
+  // peak -- its only read stream is the staged one; with a direct operand beside it they cost 1-3 %)
+  int64_t bandVec = tuning("apply.tiled.group_p_vec", -1);
+  if (bandVec < 0) bandVec = Op::NIN == 1 ? 16 : 1;
+  args.groupP = (uint32_t)std::max<int64_t>(1, shift ? tuning("apply.tiled.group_p", 8) : bandVec);
   if ((int64_t)args.groupP * 2 > tp) args.groupP = 1;
   const int64_t swz = tuning("apply.tiled.xcd_swizzle", 1);
   // (not with fused q: there the direct operands are one long aligned run and

@@ -189,4 +189,11 @@ __device__ __forceinline__ void write_run_from_lds(T* dst, const T* run, uint32_
   }
 }
 
+// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits
+// for every global load and store of the wave, which would drain packs that
+// were requested ahead and stores that nobody in the workgroup reads back.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 }  // namespace thc

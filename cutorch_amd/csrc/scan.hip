@@ -171,13 +171,6 @@ __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
   }
 }
 
-// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits
-// for every global load and store of the wave, which would drain the packs
-// requested ahead for the next segment and the stores of the previous one.
-__device__ __forceinline__ void lds_barrier() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
 // Scan along a strided dim of a dense [outer][R][inner] block. A workgroup
 // owns one `outer` index and TX*VEC adjacent columns and walks R in segments
 // of TY*U rows: thread row ty holds U consecutive rows of the segment in

@@ -450,6 +450,31 @@ def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band):
         thc.set_tuning("apply.tiled.group_p", 8)
 
 
+@pytest.mark.parametrize("band", [1, 2, 3, 16])
+def test_aligned_tiles_in_bands_along_p(thc, oracle, band):
+    """The pack variant of the tiled kernel can walk its tiles in bands along p too (the default
+    for single-input ops): whole bands, a ragged last band, a batch dim in front, fused q."""
+    rng = np.random.default_rng(92)
+    thc.set_tuning("apply.tiled.group_p_vec", band)
+    try:
+        for rows, cols in ((320, 512), (448, 132), (1000, 64), (2304, 128)):
+            ga = (rows * cols, 0, (rows, cols), (1, rows))               # a:t()
+            gc = contiguous_geometry((rows, cols))
+            assert run_binary(thc, oracle, "cadd", [gc, ga, gc], rng) == "tiled"
+            src = thc.Tensor.from_numpy(rng.integers(-99, 100, (cols, rows)).astype(np.float32))
+            out = thc.Tensor("float").resize((rows, cols)).copy(src.t())
+            assert thc.last_kernel() == "tiled"
+            assert_bit_equal(out.numpy(), src.numpy().T)
+        g3 = (5 * 128 * 400, 0, (5, 400, 128), (128 * 400, 1, 400))      # batch dim in front, p = 400
+        assert run_binary(thc, oracle, "cmul", [contiguous_geometry((5, 400, 128)), g3,
+                                                contiguous_geometry((5, 400, 128))], rng) == "tiled"
+        gp = (40 * 24 * 520, 0, (520, 24, 40), (1, 520, 520 * 24))       # permute(3,2,1): q fuses two dims
+        assert run_binary(thc, oracle, "cadd", [contiguous_geometry((520, 24, 40)), gp,
+                                                contiguous_geometry((520, 24, 40))], rng) == "tiled-fused"
+    finally:
+        thc.set_tuning("apply.tiled.group_p_vec", -1)
+
+
 @pytest.mark.parametrize("kind", ["float", "int"])
 def test_addcmul_when_self_is_a_factor(thc, oracle, kind):
     """addcmul(self, t, v, src1, src2) with self being src1 (or src2) and not t:
