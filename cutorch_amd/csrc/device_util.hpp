@@ -164,6 +164,35 @@ __device__ __forceinline__ uint32_t stage_rows_to_lds(const TIn* first, uint32_t
 }
 
 
+// stage_rows_to_lds in two steps, for runs of at most 8 packs per lane
+// (32 KiB, the neighbours' elements in the first and last pack included):
+// request() asks for the run's packs and keeps them in registers, commit()
+// puts them into LDS. In between, the workgroup can work on the previous run.
+// The loads carry no predicate (lanes past the run's end re-read its last
+// pack), so the compiler can tell exactly which loads a later wait covers.
+template <typename TIn>
+struct RunPrefetch {
+  static constexpr int VEC = 16 / sizeof(TIn);
+  static constexpr int U = 8;
+  using P = Pack<TIn, VEC>;
+  P v[U];
+  uint32_t mis, npacks;
+  __device__ __forceinline__ void request(const TIn* first, uint32_t count) {
+    mis = (uint32_t)((reinterpret_cast<uintptr_t>(first) / sizeof(TIn)) & (uintptr_t)(VEC - 1));
+    const P* src = reinterpret_cast<const P*>(first - mis);
+    npacks = (mis + count + VEC - 1) / VEC;
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = load_pack<true>(src + min(threadIdx.x + u * kBlock, npacks - 1));
+  }
+  // Returns m such that element i of the run is lds[m + i]; the caller synchronises.
+  __device__ __forceinline__ uint32_t commit(TIn* lds) const {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (threadIdx.x + u * kBlock < npacks) reinterpret_cast<P*>(lds)[threadIdx.x + u * kBlock] = v[u];
+    return mis;
+  }
+};
+
 // The way back: `count` elements held in LDS (element i at run[i], any
 // alignment) go to `dst` as 16-byte packs aligned on dst; the packs that
 // straddle the run's ends are stored element by element, so nothing outside

@@ -314,12 +314,24 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const TIn* __restri
           }
         }
       }
-      for (; i < end; i += step) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
+      // a partial last batch: all of its loads in flight at once as well (the missing packs
+      // re-read the lane's first pack of the batch and are not used)
+      if (i < end) {
+        P v[U];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const A x = acc_up<A>(v.v[e]);
-          acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
+        for (int u = 0; u < U; ++u) {
+          const I at = i + u * step < end ? i + u * step : i;
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + at * es));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (i + u * step < end) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const A x = acc_up<A>(v[u].v[e]);
+              acc[e] = f.combine(acc[e], FIRST ? f.modify(x, c) : x);
+            }
+          }
         }
       }
     }
@@ -370,29 +382,35 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(
       const I es = VEC == 1 ? sR : (I)1;
       constexpr int U = 8;
       const I step = (I)G * VEC;
-      I i = begin + lane * VEC;
-      for (; i + (U - 1) * step < end; i += U * step) {
+      // A batch of U packs per lane. The batch's extreme value first (one three-input
+      // instruction per two elements, NaN propagating), then, only in lanes whose batch
+      // beats their running best, the first slot that holds it. A compare-select chain
+      // over every element costs about six instructions per element and made this kernel
+      // issue bound. The last batch of a lane may be partial: its missing packs re-read the
+      // lane's first pack of the batch and count as the start value.
+      auto batch = [&](I i, auto partialTag) {
+        constexpr bool PARTIAL = decltype(partialTag)::value;
         P v[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + (i + u * step) * es));
-        // The batch's extreme value first (one three-input instruction per two
-        // elements, NaN propagating), then, only in lanes whose batch beats
-        // their running best, the first slot that holds it. A compare-select
-        // chain over every element costs about six instructions per element
-        // and made this kernel issue bound.
+        for (int u = 0; u < U; ++u) {
+          const I at = !PARTIAL || i + u * step < end ? i + u * step : i;
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(src + at * es));
+        }
+        A a[U][VEC];
         A m = O::worst();
 #pragma unroll
         for (int u = 0; u < U; ++u) {
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) m = O::extreme(m, acc_up<A>(v[u].v[e]));
+          for (int e = 0; e < VEC; ++e) {
+            a[u][e] = !PARTIAL || i + u * step < end ? acc_up<A>(v[u].v[e]) : O::worst();
+            m = O::extreme(m, a[u][e]);
+          }
         }
         if (O::plain(m)) {
           if (O::better_later(m, bv)) {
             uint32_t slot = 0;
 #pragma unroll
-            for (int q = U * VEC - 1; q >= 0; --q)
-              slot = acc_up<A>(v[q / VEC].v[q % VEC]) == m ? (uint32_t)q : slot;
+            for (int q = U * VEC - 1; q >= 0; --q) slot = a[q / VEC][q % VEC] == m ? (uint32_t)q : slot;
             bv = m;
             bi = i + (I)(slot / VEC) * step + (I)(slot % VEC);
           }
@@ -403,26 +421,17 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_kernel(
           for (int u = 0; u < U; ++u) {
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
-              const A x = acc_up<A>(v[u].v[e]);
-              if (O::better_later(x, bv)) {
-                bv = x;
+              if ((!PARTIAL || i + u * step < end) && O::better_later(a[u][e], bv)) {
+                bv = a[u][e];
                 bi = i + u * step + e;
               }
             }
           }
         }
-      }
-      for (; i < end; i += step) {
-        const P v = load_pack<true>(reinterpret_cast<const P*>(src + i * es));
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-          const A x = acc_up<A>(v.v[e]);
-          if (O::better_later(x, bv)) {
-            bv = x;
-            bi = i + e;
-          }
-        }
-      }
+      };
+      I i = begin + lane * VEC;
+      for (; i + (U - 1) * step < end; i += U * step) batch(i, std::false_type{});
+      if (i < end) batch(i, std::true_type{});
     }
     for (uint32_t o = G >> 1; o > 0; o >>= 1) {
       const A ov = shfl_xor_any(bv, o);
@@ -514,6 +523,9 @@ __global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T
 // address at or below the run's first element, so it and the last pack may
 // hold a few elements of the neighbouring runs) and the lane groups reduce
 // out of LDS, where alignment is free (stage_rows_to_lds, device_util.hpp).
+// A workgroup walks its runs with a stride of the grid: the packs of the next
+// run are requested (RunPrefetch, into registers) before the current one is
+// reduced, and the barriers order LDS only, so those loads stay in flight.
 template <typename TIn, typename TOut, typename F, typename I>
 __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __restrict__ in,
                                                                  TOut* __restrict__ out,
@@ -525,11 +537,18 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
   TIn* lds = reinterpret_cast<TIn*>(lds_raw);
   const uint32_t lane = threadIdx.x % G, grp = threadIdx.x / G, groups = kBlock / G;
   const I numBlocks = (numRows + rowsPerBlock - 1) / rowsPerBlock;
+  RunPrefetch<TIn> next;
+  auto request = [&](I blk) {
+    const I row0 = blk * rowsPerBlock;
+    next.request(in + row0 * R, (uint32_t)min((I)rowsPerBlock, numRows - row0) * (uint32_t)R);
+  };
+  if ((I)blockIdx.x < numBlocks) request(blockIdx.x);
   for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
     const I row0 = blk * rowsPerBlock;
     const uint32_t nrows = (uint32_t)min((I)rowsPerBlock, numRows - row0);
-    const uint32_t mis = stage_rows_to_lds<TIn, 8>(in + row0 * R, nrows * (uint32_t)R, lds);
-    __syncthreads();
+    const uint32_t mis = next.commit(lds);
+    lds_barrier();
+    if (blk + gridDim.x < numBlocks) request(blk + gridDim.x);
     // lanes of one group share r, so they leave the loop together
     for (uint32_t r = grp; r < nrows; r += groups) {
       const TIn* row = lds + mis + r * (uint32_t)R;
@@ -538,11 +557,20 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
       A c = (A)0;
       if constexpr (F::kCentred) c = acc_up<A>(out[outOff]);
       A acc = f.init();
-      for (uint32_t j = lane; j < (uint32_t)R; j += G) acc = f.combine(acc, f.modify(acc_up<A>(row[j]), c));
+      // batches of 8 LDS reads (past the row's end: its last element, not used), then the
+      // dependent chain: one LDS latency per batch instead of one per element
+      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+        TIn x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (j + u * G < (uint32_t)R) acc = f.combine(acc, f.modify(acc_up<A>(x[u]), c));
+      }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) acc = f.combine(acc, shfl_xor_any(acc, o));
       if (lane == 0) out[outOff] = epi.template finish<TOut>(acc);
     }
-    __syncthreads();  // the buffer is refilled by the next run
+    lds_barrier();  // the buffer is refilled by the next run
   }
 }
 
@@ -556,39 +584,54 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
   T* lds = reinterpret_cast<T*>(lds_raw);
   const uint32_t lane = threadIdx.x % G, grp = threadIdx.x / G, groups = kBlock / G;
   const I numBlocks = (numRows + rowsPerBlock - 1) / rowsPerBlock;
+  RunPrefetch<T> next;  // as in reduce_rows_lds_kernel
+  auto request = [&](I blk) {
+    const I row0 = blk * rowsPerBlock;
+    next.request(in + row0 * R, (uint32_t)min((I)rowsPerBlock, numRows - row0) * (uint32_t)R);
+  };
+  if ((I)blockIdx.x < numBlocks) request(blockIdx.x);
   for (I blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
     const I row0 = blk * rowsPerBlock;
     const uint32_t nrows = (uint32_t)min((I)rowsPerBlock, numRows - row0);
-    const uint32_t mis = stage_rows_to_lds<T, 8>(in + row0 * R, nrows * (uint32_t)R, lds);
-    __syncthreads();
+    const uint32_t mis = next.commit(lds);
+    lds_barrier();
+    if (blk + gridDim.x < numBlocks) request(blk + gridDim.x);
     for (uint32_t r = grp; r < nrows; r += groups) {
       const T* row = lds + mis + r * (uint32_t)R;
-      // two independent candidate chains per lane (elements j and j + G of
-      // each step), merged with the lowest-index rule
-      A bv = O::worst(), bv1 = O::worst();
-      uint32_t bi = ~0u, bi1 = ~0u;
-      uint32_t j = lane;
-      for (; j + G < (uint32_t)R; j += 2 * G) {
-        const A x = acc_up<A>(row[j]), x1 = acc_up<A>(row[j + G]);
-        if (O::better_later(x, bv)) {
-          bv = x;
-          bi = j;
+      // Batches of 8 LDS reads (past the row's end: its last element, replaced by the start
+      // value), one LDS latency per batch. As in reduce_rows_index_kernel the batch's extreme
+      // comes first and the slot that holds it is searched only where it beats the running
+      // best; a NaN or a zero as the extreme takes the element-wise path.
+      A bv = O::worst();
+      uint32_t bi = ~0u;
+      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+        A a[8];
+        A m = O::worst();
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          a[u] = j + u * G < (uint32_t)R ? acc_up<A>(x[u]) : O::worst();
+          m = O::extreme(m, a[u]);
         }
-        if (O::better_later(x1, bv1)) {
-          bv1 = x1;
-          bi1 = j + G;
+        if (O::plain(m)) {
+          if (O::better_later(m, bv)) {
+            uint32_t slot = 0;
+#pragma unroll
+            for (int q = 7; q >= 0; --q) slot = a[q] == m ? (uint32_t)q : slot;
+            bv = m;
+            bi = j + slot * G;
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (j + u * G < (uint32_t)R && O::better_later(a[u], bv)) {
+              bv = a[u];
+              bi = j + u * G;
+            }
+          }
         }
-      }
-      if (j < (uint32_t)R) {
-        const A x = acc_up<A>(row[j]);
-        if (O::better_later(x, bv)) {
-          bv = x;
-          bi = j;
-        }
-      }
-      if (O::better(bv1, bi1, bv, bi)) {
-        bv = bv1;
-        bi = bi1;
       }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) {
         const A ov = shfl_xor_any(bv, o);
@@ -607,7 +650,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
         outI[idxOff] = (long)bi + 1;
       }
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -1703,16 +1746,26 @@ bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPer
   // about four runs per CU, each between 4 and 32 KiB (32 KiB = one batch of
   // eight 16-byte loads per lane)
   int64_t chunk = g.outElems * rowBytes / ((int64_t)num_compute_units(s) * 4);
-  chunk = std::min<int64_t>(32768, std::max<int64_t>(4096, chunk));
+  // (a run plus the neighbours' elements in its first and last pack must fit RunPrefetch)
+  chunk = std::min<int64_t>(32768 - 32, std::max<int64_t>(4096, chunk));
   rowsPerBlock = (uint32_t)std::max<int64_t>(1, chunk / rowBytes);
-  // about 16 elements per lane: the group's shuffle tree and the per-row
-  // bookkeeping are a dependent chain, so wide groups on short rows are
-  // latency bound (33-element fp32 rows summed at 0.9 TB/s with a lane per
-  // element, 3.0 with 2 elements per lane, 5.7 with 16; 64 and more lose again)
-  const uint64_t perLane = (uint64_t)tuning("reduce.rows.lds_elems_per_lane", 16);
-  G = pow2_ceil((uint64_t)g.R / perLane + 1);
-  if (G > 1 && (uint64_t)G * perLane > (uint64_t)g.R) G >>= 1;
+  // Lanes per row. The group's shuffle tree and the per-row bookkeeping are a dependent chain, so
+  // wide groups on short rows are latency bound: 33-element fp32 rows are summed at 0.3 of peak with
+  // 2 elements per lane, 0.65 with 8, 0.71 with 16 and 0.77-0.82 with a lane per row; from about 120
+  // elements on, 16 per lane is best (127: 0.80 against 0.69 with 32). Rows whose pitch shares a
+  // power of two with the 32 LDS banks put the lanes of a step on few banks (32-element rows, a
+  // lane per row: 0.27), so such rows get up to gcd(pitch in words, 32) lanes (8 at most) as long as
+  // a lane keeps 8 elements (fewer is slower than the conflicts: 8-element rows 0.17 against 0.65).
+  int64_t perLane = tuning("reduce.rows.lds_elems_per_lane", 0);
+  if (perLane <= 0) perLane = g.R <= 112 ? 32 : 16;
+  G = pow2_ceil((uint64_t)g.R / (uint64_t)perLane + 1);
+  if (G > 1 && (uint64_t)G * (uint64_t)perLane > (uint64_t)g.R) G >>= 1;
   G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
+  if (tuning("reduce.rows.lds_spread_banks", 1) && rowBytes % 4 == 0) {
+    uint32_t shared = 1;
+    while (shared < 8 && (rowBytes / 4) % (shared * 2) == 0) shared *= 2;
+    while (G < shared && (uint64_t)G * 2 * 8 <= (uint64_t)g.R) G <<= 1;  // (a lane keeps a full batch of 8)
+  }
   ldsBytes = (((size_t)rowsPerBlock * (size_t)g.R + 2 * (16 / sizeof(T))) * sizeof(T) + 15) & ~size_t(15);
   return true;
 }
@@ -1746,7 +1799,7 @@ void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typenam
   size_t ldsBytes = 0;
   if (S == 1 && plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
     const int64_t blocks = (rows + ldsRows - 1) / ldsRows;
-    const int grid = capped_grid(s, blocks, "reduce.rows.blocks_per_cu", 64);
+    const int grid = capped_grid(s, blocks, "reduce.rows.lds_blocks_per_cu", 64);
     hipLaunchKernelGGL((reduce_rows_lds_kernel<T, T, F, I>), dim3(grid), dim3(kBlock), ldsBytes,
                        current_stream(s), in, out, oa, (I)rows, (I)g.R, ldsRows, ldsG, epi, f);
     note_kernel("rows-lds");
@@ -2068,7 +2121,7 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
       uint32_t ldsRows = 0, ldsG = 0;
       size_t ldsBytes = 0;
       if (plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
-        const int grid = capped_grid(s, (rows + ldsRows - 1) / ldsRows, "reduce.rows.blocks_per_cu", 64);
+        const int grid = capped_grid(s, (rows + ldsRows - 1) / ldsRows, "reduce.rows.lds_blocks_per_cu", 64);
         hipLaunchKernelGGL((reduce_rows_index_lds_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock),
                            ldsBytes, st, in, outV, outI, oa, oaIdx, (I)rows, (I)g.R, ldsRows, ldsG);
         note_kernel("rows-index-lds");
