@@ -731,7 +731,16 @@ __global__ __launch_bounds__(kBlock) void reduce_slab_kernel(const TIn* __restri
       if constexpr (F::kCentred) ctr = acc_up<A>(out[outOff]);
       const TIn* col = lds + mis + o * slice + c;
       A acc = f.init();
-      for (uint32_t r = first; r < R; r += step) acc = f.combine(acc, f.modify(acc_up<A>(col[r * C]), ctr));
+      // batches of 8 LDS reads (past the column's end: its last element, not used), then
+      // the dependent chain: one LDS latency per batch instead of one per element
+      for (uint32_t r = first; r < R; r += 8 * step) {
+        TIn x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = col[min(r + u * step, R - 1) * C];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (r + u * step < R) acc = f.combine(acc, f.modify(acc_up<A>(x[u]), ctr));
+      }
       return acc;
     };
     if (P == 1) {
@@ -783,11 +792,34 @@ __global__ __launch_bounds__(kBlock) void reduce_slab_index_kernel(const T* __re
       const T* col = lds + mis + o * slice + c;
       bv = O::worst();
       bi = ~0u;
-      for (uint32_t r = first; r < R; r += step) {
-        const A x = acc_up<A>(col[r * C]);
-        if (O::better_later(x, bv)) {
-          bv = x;
-          bi = r;
+      // batches of 8 LDS reads, the batch's extreme first (as in reduce_rows_index_lds_kernel)
+      for (uint32_t r = first; r < R; r += 8 * step) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = col[min(r + u * step, R - 1) * C];
+        A v[8];
+        A m = O::worst();
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          v[u] = r + u * step < R ? acc_up<A>(x[u]) : O::worst();
+          m = O::extreme(m, v[u]);
+        }
+        if (O::plain(m)) {
+          if (O::better_later(m, bv)) {
+            uint32_t slot = 0;
+#pragma unroll
+            for (int q = 7; q >= 0; --q) slot = v[q] == m ? (uint32_t)q : slot;
+            bv = m;
+            bi = r + slot * step;
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (r + u * step < R && O::better_later(v[u], bv)) {
+              bv = v[u];
+              bi = r + u * step;
+            }
+          }
         }
       }
     };
