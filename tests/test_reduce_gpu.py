@@ -644,3 +644,40 @@ def test_reductions_beyond_2pow31_elements(thc):
             if hit.size:
                 colwant[r, hit[0]] = val
     assert np.array_equal(c.numpy().reshape(-1)[sample].astype(np.int64), colwant.sum(axis=0))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double", "int"])
+def test_every_row_length_up_to_300_and_some_beyond(thc, kind):
+    """Row reductions pick lanes per row, batch sizes and a partial last batch from the row length:
+    every length from 1 to 300 and a few longer ones, rows back to back. Small integers, so sums
+    are exact; max/min see ties (lowest index wins), and for the floating types one row with a
+    NaN (first NaN wins) and one with zeros of both signs as the extreme (the first keeps its sign)."""
+    rng = np.random.default_rng(77)
+    dtype = {"float": np.float32, "half": np.float16, "double": np.float64, "int": np.int32}[kind]
+    floating = kind in ("float", "half", "double")
+    for R in list(range(1, 301)) + [383, 384, 500, 511, 512, 777, 1000, 1536, 2047, 4100]:
+        rows = max(3, min(700, 40000 // R))
+        x = rng.integers(-6, 7, (rows, R)).astype(dtype)
+        if floating and R >= 3:
+            x[1, R // 2] = np.nan
+            x[1, R - 1] = np.nan
+            x[2] = np.minimum(x[2], 0)
+            x[2, R // 3] = -0.0
+            x[2, R - 1] = 0.0
+        dev = thc.Tensor.from_numpy(x)
+        got = thc.Tensor(kind).sum(dev, 1).numpy().reshape(rows)
+        want = x.astype(np.float64).sum(axis=1).astype(dtype) if floating else x.sum(axis=1, dtype=np.int64).astype(dtype)
+        assert_bit_equal(got, want, "%s sum R=%d [%s]" % (kind, R, thc.last_kernel()))
+        for which in ("max", "min"):
+            v, i = thc.Tensor(kind), thc.Tensor("long")
+            getattr(v, which)(i, dev, 1)
+            gv, gi = v.numpy().reshape(rows), i.numpy().reshape(rows) - 1
+            xf = x.astype(np.float64)
+            wi = np.empty(rows, np.int64)
+            for r in range(rows):
+                nan = np.flatnonzero(np.isnan(xf[r]))
+                wi[r] = nan[0] if nan.size else (np.argmax(xf[r]) if which == "max" else np.argmin(xf[r]))
+            where = "%s %s R=%d [%s]" % (kind, which, R, thc.last_kernel())
+            assert (gi == wi).all(), (where, np.flatnonzero(gi != wi)[:5])
+            assert_bit_equal(gv, x[np.arange(rows), wi], where)
