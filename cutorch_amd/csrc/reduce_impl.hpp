@@ -557,15 +557,43 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
       A c = (A)0;
       if constexpr (F::kCentred) c = acc_up<A>(out[outOff]);
       A acc = f.init();
-      // batches of 8 LDS reads (past the row's end: its last element, not used), then the
-      // dependent chain: one LDS latency per batch instead of one per element
-      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
-        TIn x[8];
+      if constexpr (sizeof(TIn) == 2) {
+        // 2-byte elements are read from LDS two at a time: the row's pairs start at its first
+        // even element index; a leading and a trailing single element go to lane 0
+        const uint32_t start = mis + r * (uint32_t)R, head = start & 1u;
+        const uint32_t npairs = ((uint32_t)R - head) >> 1;
+        const uint32_t* words = reinterpret_cast<const uint32_t*>(lds) + ((start + head) >> 1);
+        auto take = [&](uint32_t bits) {
+          const uint16_t h = (uint16_t)bits;
+          TIn x;
+          __builtin_memcpy(&x, &h, 2);
+          acc = f.combine(acc, f.modify(acc_up<A>(x), c));
+        };
+        if (head && lane == 0) acc = f.combine(acc, f.modify(acc_up<A>(row[0]), c));
+        for (uint32_t q = lane; q < npairs; q += 8 * G) {
+          uint32_t w[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+          for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, npairs - 1)];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (j + u * G < (uint32_t)R) acc = f.combine(acc, f.modify(acc_up<A>(x[u]), c));
+          for (int u = 0; u < 8; ++u) {
+            if (q + u * G < npairs) {
+              take(w[u]);
+              take(w[u] >> 16);
+            }
+          }
+        }
+        if (head + 2 * npairs < (uint32_t)R && lane == 0) acc = f.combine(acc, f.modify(acc_up<A>(row[(uint32_t)R - 1]), c));
+      } else {
+        // batches of 8 LDS reads (past the row's end: its last element, not used), then the
+        // dependent chain: one LDS latency per batch instead of one per element
+        for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+          TIn x[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (j + u * G < (uint32_t)R) acc = f.combine(acc, f.modify(acc_up<A>(x[u]), c));
+        }
       }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) acc = f.combine(acc, shfl_xor_any(acc, o));
       if (lane == 0) out[outOff] = epi.template finish<TOut>(acc);
@@ -604,34 +632,78 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
       // best; a NaN or a zero as the extreme takes the element-wise path.
       A bv = O::worst();
       uint32_t bi = ~0u;
-      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
-        T x[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
-        A a[8];
+      // one candidate after the running best, in index order
+      auto offer = [&](A x, uint32_t j) {
+        if (O::better_later(x, bv)) {
+          bv = x;
+          bi = j;
+        }
+      };
+      // a batch of N values a[] at row indices idx(s), ascending in s; `live` = slots that exist
+      auto offer_batch = [&](auto& a, auto idx, uint32_t live, auto nTag) {
+        constexpr int N = decltype(nTag)::value;
         A m = O::worst();
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          a[u] = j + u * G < (uint32_t)R ? acc_up<A>(x[u]) : O::worst();
-          m = O::extreme(m, a[u]);
-        }
+        for (int s2 = 0; s2 < N; ++s2) m = O::extreme(m, a[s2]);
         if (O::plain(m)) {
           if (O::better_later(m, bv)) {
             uint32_t slot = 0;
 #pragma unroll
-            for (int q = 7; q >= 0; --q) slot = a[q] == m ? (uint32_t)q : slot;
+            for (int q = N - 1; q >= 0; --q) slot = a[q] == m ? (uint32_t)q : slot;
             bv = m;
-            bi = j + slot * G;
+            bi = idx(slot);
           }
         } else {
 #pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            if (j + u * G < (uint32_t)R && O::better_later(a[u], bv)) {
-              bv = a[u];
-              bi = j + u * G;
-            }
-          }
+          for (int s2 = 0; s2 < N; ++s2)
+            if ((uint32_t)s2 < live) offer(a[s2], idx((uint32_t)s2));
         }
+      };
+      auto by_element = [&]() {
+        for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+          T x[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+          A a[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) a[u] = j + u * G < (uint32_t)R ? acc_up<A>(x[u]) : O::worst();
+          const uint32_t live = min(8u, ((uint32_t)R - j + G - 1) / G);
+          offer_batch(a, [&](uint32_t s2) { return j + s2 * G; }, live, std::integral_constant<int, 8>{});
+        }
+      };
+      if constexpr (sizeof(T) != 2) {
+        by_element();
+      } else if ((uint32_t)R < 16) {  // (most of a 16-slot batch would idle)
+        by_element();
+      } else {
+        // 2-byte elements are read from LDS two at a time (see reduce_rows_lds_kernel); a lane's
+        // candidates still come in index order: the leading single element, its pairs, the trailing one
+        const uint32_t start = mis + r * (uint32_t)R, head = start & 1u;
+        const uint32_t npairs = ((uint32_t)R - head) >> 1;
+        const uint32_t* words = reinterpret_cast<const uint32_t*>(lds) + ((start + head) >> 1);
+        auto half_of = [](uint32_t bits) {
+          const uint16_t h = (uint16_t)bits;
+          T x;
+          __builtin_memcpy(&x, &h, 2);
+          return acc_up<A>(x);
+        };
+        if (head && lane == 0) offer(acc_up<A>(row[0]), 0u);
+        for (uint32_t q = lane; q < npairs; q += 8 * G) {
+          uint32_t w[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, npairs - 1)];
+          A a[16];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            const bool have = q + u * G < npairs;
+            a[2 * u] = have ? half_of(w[u]) : O::worst();
+            a[2 * u + 1] = have ? half_of(w[u] >> 16) : O::worst();
+          }
+          const uint32_t live = 2 * min(8u, (npairs - q + G - 1) / G);
+          offer_batch(a, [&](uint32_t s2) { return head + 2 * (q + (s2 >> 1) * G) + (s2 & 1u); }, live,
+                      std::integral_constant<int, 16>{});
+        }
+        if (head + 2 * npairs < (uint32_t)R && lane == 0) offer(acc_up<A>(row[(uint32_t)R - 1]), (uint32_t)R - 1);
       }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) {
         const A ov = shfl_xor_any(bv, o);
@@ -1788,15 +1860,17 @@ bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPer
   // power of two with the 32 LDS banks put the lanes of a step on few banks (32-element rows, a
   // lane per row: 0.27), so such rows get up to gcd(pitch in words, 32) lanes (8 at most) as long as
   // a lane keeps 8 elements (fewer is slower than the conflicts: 8-element rows 0.17 against 0.65).
+  // (2-byte elements are read from LDS in pairs: the unit below is one LDS read)
+  const uint64_t reads = sizeof(T) == 2 ? ((uint64_t)g.R + 1) / 2 : (uint64_t)g.R;
   int64_t perLane = tuning("reduce.rows.lds_elems_per_lane", 0);
-  if (perLane <= 0) perLane = g.R <= 112 ? 32 : 16;
-  G = pow2_ceil((uint64_t)g.R / (uint64_t)perLane + 1);
-  if (G > 1 && (uint64_t)G * (uint64_t)perLane > (uint64_t)g.R) G >>= 1;
+  if (perLane <= 0) perLane = reads <= 112 ? 32 : 16;
+  G = pow2_ceil(reads / (uint64_t)perLane + 1);
+  if (G > 1 && (uint64_t)G * (uint64_t)perLane > reads) G >>= 1;
   G = std::min<uint32_t>(64, std::max<uint32_t>(1, G));
   if (tuning("reduce.rows.lds_spread_banks", 1) && rowBytes % 4 == 0) {
     uint32_t shared = 1;
     while (shared < 8 && (rowBytes / 4) % (shared * 2) == 0) shared *= 2;
-    while (G < shared && (uint64_t)G * 2 * 8 <= (uint64_t)g.R) G <<= 1;  // (a lane keeps a full batch of 8)
+    while (G < shared && (uint64_t)G * 2 * 8 <= reads) G <<= 1;  // (a lane keeps a full batch of 8)
   }
   ldsBytes = (((size_t)rowsPerBlock * (size_t)g.R + 2 * (16 / sizeof(T))) * sizeof(T) + 15) & ~size_t(15);
   return true;
