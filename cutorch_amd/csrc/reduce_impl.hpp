@@ -1846,7 +1846,7 @@ bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPer
     if (g.R % (VEC * (int64_t)lanes) != 0) vec = false;
   }
   const int64_t limit = vec ? tuning("reduce.rows.lds_max_vec_bytes", 511) : tuning("reduce.rows.lds_max_bytes", 8192);
-  if (rowBytes > limit) return false;
+  if (rowBytes > limit || rowBytes > 32768 - 32) return false;  // (a run of at least one row must fit RunPrefetch)
   // about four runs per CU, each between 4 and 32 KiB (32 KiB = one batch of
   // eight 16-byte loads per lane)
   int64_t chunk = g.outElems * rowBytes / ((int64_t)num_compute_units(s) * 4);
