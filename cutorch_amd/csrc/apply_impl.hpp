@@ -887,6 +887,188 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
   }
 }
 
+// The tiled kernel for 4-byte elements whose rows start anywhere in a cache
+// line (odd sizes, views at odd offsets). Where the shifted-window variant cuts
+// every row at the same logical columns, so that each 496-byte row piece of a
+// tile touches five 128-byte lines and shares its first and last one with the
+// neighbouring tiles (fetched and, worse, partially written twice), this one
+// cuts every row of the output and of the direct operands at ITS OWN line
+// boundaries: tile tq owns, of row p, the four lines [128 tq - o(p), 128 tq -
+// o(p) + 128) with o(p) = elements between the line boundary at or below the
+// row's start and the row's start. All those accesses are whole aligned
+// lines that no other tile touches (except a row's first and last line,
+// which it shares with the rows before and after it in memory). The price is
+// on the staged side: the q range of a tile now shifts from row to row by up
+// to 31 columns, so 159 instead of 128 rows of a staged operand go into LDS
+// (read with 16-byte loads at element alignment: a staged row piece is 256
+// bytes at whatever offset the operand's own pitch gives it).
+// The host guarantees unit stride along every operand's fast dim and direct
+// operands that share the output's misalignment modulo the pack width.
+constexpr int kRaggedLine = 32;  // 128-byte lines (64-byte cut points: less re-fetch of staged rows, 1.07 x, but 4 % more written bytes and 0.60 instead of 0.65 of peak)
+template <typename T, typename Op, typename I, int MASK>
+__global__ __launch_bounds__(kBlock) void apply_tiled_ragged_kernel(T* out, const T* in0, const T* in1,
+                                                                    const T* in2, TiledArgs<I> args, Op op) {
+  static_assert(sizeof(T) == 4, "4-byte elements");
+  constexpr int NOPS = Op::NIN + 1;
+  constexpr int VEC = 4, LXP = 16, LXQ = 32;
+  constexpr int TP = LXP * VEC, TQ = LXQ * VEC;  // 64 x 128
+  constexpr int LINE = kRaggedLine;              // elements between two cut points of a row
+  constexpr int SPAN = TQ + LINE - 1;            // columns a tile may touch
+  constexpr int ROWS_P = kBlock / LXP, PASSES_P = (SPAN + ROWS_P - 1) / ROWS_P;
+  constexpr int ROWS_Q = kBlock / LXQ, PASSES_Q = TP / ROWS_Q;
+  constexpr int PITCH = TP + 1;
+  using P = Pack<T, VEC>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  const T* ptr[kMaxOps] = {out, in0, in1, in2};
+  const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
+  const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  bool staged[kMaxOps];
+  int slot[kMaxOps];
+  {
+    int s = 0;
+    staged[0] = false;
+    slot[0] = -1;
+#pragma unroll
+    for (int k = 1; k < NOPS; ++k) {
+      staged[k] = ((MASK >> (k - 1)) & 1) != 0;
+      slot[k] = staged[k] ? s++ : -1;
+    }
+  }
+  const uint32_t slots = args.xcdPer ? args.xcdPer * 8 : args.totalTiles;
+  for (uint32_t b = blockIdx.x; b < slots; b += gridDim.x) {
+    const uint32_t tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
+    if (tile >= args.totalTiles) continue;  // uniform over the workgroup
+    uint32_t rest, tq, tp;
+    if (args.groupP > 1) {
+      const uint32_t perBatch = args.tilesP.d * args.tilesQ.d;
+      rest = tile / perBatch;
+      const uint32_t t = tile - rest * perBatch;
+      const uint32_t band = t / (args.groupP * args.tilesQ.d);
+      const uint32_t r = t - band * (args.groupP * args.tilesQ.d);
+      const uint32_t gp = min(args.groupP, args.tilesP.d - band * args.groupP);  // ragged last band
+      tq = r / gp;
+      tp = band * args.groupP + (r - tq * gp);
+    } else {
+      args.tilesQ.divmod(tile, rest, tq);
+      args.tilesP.divmod(rest, rest, tp);
+    }
+    I base[kMaxOps] = {0, 0, 0, 0};
+    for (int j = 0; j < args.nbatch; ++j) {
+      uint32_t r;
+      args.bsize[j].divmod(rest, rest, r);
+#pragma unroll
+      for (int k = 0; k < NOPS; ++k) base[k] += (I)r * args.bstride[k][j];
+    }
+    const uint32_t p0 = tp * TP;
+    const int pn = (int)min((uint32_t)TP, args.sizeP - p0);
+    const int sizeQ = (int)args.sizeQ;
+    const int qL = (int)(tq * TQ) - (LINE - 1);  // the first column any row of this tile may hold
+    const bool interior = pn == TP && qL >= 0 && qL + SPAN <= sizeQ;
+
+    auto body = [&](auto fullTag) {
+      constexpr bool FULL = decltype(fullTag)::value;
+      // phase 1: staged inputs, lanes along p, LDS row cq holds column qL + cq
+#pragma unroll
+      for (int k = 1; k < NOPS; ++k) {
+        if (!staged[k]) continue;
+        T* slab = lds + slot[k] * (SPAN * PITCH);
+        const T* origin = ptr[k] + (base[k] + (I)p0 * args.strideP[k]) + lxp * VEC;  // unit stride along p
+        P v[PASSES_P];
+#pragma unroll
+        for (int r = 0; r < PASSES_P; ++r) {
+          const int cq = (int)lyp + r * ROWS_P, q = qL + cq;
+          const bool row = cq < SPAN && (FULL || (q >= 0 && q < sizeQ));
+          const int have = FULL ? VEC : pn - (int)(lxp * VEC);
+          if (row && have >= VEC) {
+            const T* at = origin + (I)q * args.strideQ[k];
+            v[r] = args.ntLoad ? load_loose_pack<true, P>(at) : load_loose_pack<false, P>(at);
+          } else if (row) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+              if (e < have) v[r].v[e] = origin[(I)q * args.strideQ[k] + e];
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < PASSES_P; ++r) {
+          const int cq = (int)lyp + r * ROWS_P;
+          if (cq < SPAN) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) slab[cq * PITCH + lxp * VEC + e] = v[r].v[e];
+          }
+        }
+      }
+      lds_barrier();
+
+      // phase 2: lanes along q; row pi owns the four lines that start o(p) elements before
+      // column tq * TQ
+      int q1[PASSES_Q];  // column of the lane's pack, element 0
+      bool whole[PASSES_Q], any[PASSES_Q];
+#pragma unroll
+      for (int r = 0; r < PASSES_Q; ++r) {
+        const int pi = (int)lyq + r * ROWS_Q;
+        const T* orow = ptr[0] + (base[0] + (I)(p0 + pi) * args.strideP[0]);
+        const int o = (int)((reinterpret_cast<uintptr_t>(orow) / sizeof(T)) & (uintptr_t)(LINE - 1));
+        q1[r] = (int)(tq * TQ) - o + (int)(lxq * VEC);
+        whole[r] = FULL || (pi < pn && q1[r] >= 0 && q1[r] + VEC <= sizeQ);
+        any[r] = FULL || (pi < pn && q1[r] + VEC > 0 && q1[r] < sizeQ);
+      }
+      P din[3][PASSES_Q];
+#pragma unroll
+      for (int k = 1; k < NOPS; ++k) {
+        if (staged[k]) continue;
+#pragma unroll
+        for (int r = 0; r < PASSES_Q; ++r) {
+          const int pi = (int)lyq + r * ROWS_Q;
+          const T* row = ptr[k] + (base[k] + (I)(p0 + pi) * args.strideP[k]);
+          if (whole[r]) {
+            din[k - 1][r] = load_pack<true>(reinterpret_cast<const P*>(row + q1[r]));
+          } else if (any[r]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+              if (q1[r] + e >= 0 && q1[r] + e < sizeQ) din[k - 1][r].v[e] = row[q1[r] + e];
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < PASSES_Q; ++r) {
+        if (!any[r]) continue;
+        const int pi = (int)lyq + r * ROWS_Q;
+        const int cq = q1[r] - qL;  // in [0, SPAN - VEC]
+        P in[3] = {};
+#pragma unroll
+        for (int k = 1; k < NOPS; ++k) {
+          if (staged[k]) {
+            const T* slab = lds + slot[k] * (SPAN * PITCH);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) in[k - 1].v[e] = slab[(cq + e) * PITCH + pi];
+          } else {
+            in[k - 1] = din[k - 1][r];
+          }
+        }
+        P res;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) res.v[e] = op(in[0].v[e], in[1].v[e], in[2].v[e]);
+        T* orow = out + (base[0] + (I)(p0 + pi) * args.strideP[0]);
+        if (whole[r]) {
+          if (args.ntStore) store_pack<true>(reinterpret_cast<P*>(orow + q1[r]), res);
+          else store_pack<false>(reinterpret_cast<P*>(orow + q1[r]), res);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            if (q1[r] + e >= 0 && q1[r] + e < sizeQ) orow[q1[r] + e] = res.v[e];
+        }
+      }
+    };
+    if (interior)
+      body(std::true_type{});
+    else
+      body(std::false_type{});
+    lds_barrier();  // the slabs are reused by the next tile
+  }
+}
+
 // ------------------------------------------------------------------------
 // Host side: launch
 // ------------------------------------------------------------------------
@@ -1106,9 +1288,16 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
         if (d != q) shift = mod(pl.lay[k].stride[d]) == mod(pl.lay[0].stride[d]);
     }
   }
+  // 4-byte elements: tiles cut along every row's own cache lines (apply_tiled_ragged_kernel)
+  bool ragged = false;
+  size_t ldsR = 0;
+  if constexpr (kSameType && sizeof(T) == 4) {
+    ldsR = (size_t)nstaged * (128 + kRaggedLine - 1) * 65 * sizeof(T);
+    ragged = shift && ldsR <= 96 * 1024 && tuning("apply.tiled.ragged", 1);
+  }
   if (!vec && !shift && ldsS > 64 * 1024) return false;
-  const int64_t tileP = vec ? tpV : (shift ? tpV - VEC : tS);
-  const int64_t tileQ = vec ? tqV : (shift ? tqV - VEC : tS);
+  const int64_t tileP = vec ? tpV : (ragged ? 64 : (shift ? tpV - VEC : tS));
+  const int64_t tileQ = vec ? tqV : (ragged ? 128 : (shift ? tqV - VEC : tS));
 
   TiledArgs<I> args{};
   for (int k = 0; k < pl.nops; ++k) {
@@ -1150,7 +1339,8 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
     batch *= pl.lay[0].size[d];
   }
   const int64_t tp = (pl.lay[0].size[p] + tileP - 1) / tileP;
-  const int64_t tq = (sizeQ + tileQ - 1) / tileQ;
+  // (ragged tiles: a row's first line may start up to 31 columns before the row does)
+  const int64_t tq = (sizeQ + (ragged ? kRaggedLine - 1 : 0) + tileQ - 1) / tileQ;
   args.tilesP.set((uint64_t)tp);
   args.tilesQ.set((uint64_t)tq);
   const int64_t total = batch * tp * tq;
@@ -1177,7 +1367,10 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   // peak -- its only read stream is the staged one; with a direct operand beside it they cost 1-3 %)
   int64_t bandVec = tuning("apply.tiled.group_p_vec", -1);
   if (bandVec < 0) bandVec = Op::NIN == 1 ? 16 : 1;
-  args.groupP = (uint32_t)std::max<int64_t>(1, shift ? tuning("apply.tiled.group_p", 8) : bandVec);
+  // (the ragged variant: 8191 x 8193 transposed add 0.63 of peak with bands of 8, 0.65 with 16, 0.675 with 32,
+  // 0.66 with 64)
+  args.groupP = (uint32_t)std::max<int64_t>(
+      1, ragged ? tuning("apply.tiled.group_p_ragged", 32) : (shift ? tuning("apply.tiled.group_p", 8) : bandVec));
   if ((int64_t)args.groupP * 2 > tp) args.groupP = 1;
   const int64_t swz = tuning("apply.tiled.xcd_swizzle", 1);
   // (not with fused q: there the direct operands are one long aligned run and
@@ -1199,8 +1392,14 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   case M:                                                                                         \
     if ((M) < (1 << Op::NIN)) {                                                                   \
       constexpr int MM = (M) < (1 << Op::NIN) ? (M) : 1;                                          \
+      if constexpr (kSameType && sizeof(T) == 4) {                                                \
+        if (ragged)                                                                               \
+          hipLaunchKernelGGL((apply_tiled_ragged_kernel<T, Op, I, MM>), dim3(grid), dim3(kBlock), \
+                             ldsR, st, out, i0, i1, i2, args, op);                                \
+      }                                                                                           \
       if constexpr (kSameType) {                                                                  \
-        if (shift)                                                                                \
+        if (ragged) {                                                                             \
+        } else if (shift)                                                                         \
           hipLaunchKernelGGL((apply_tiled_shift_kernel<T, Op, I, VEC, LXP, LXQ, MM>), dim3(grid), \
                              dim3(kBlock), ldsH, st, out, i0, i1, i2, args, op);                  \
         else if (!vec)                                                                            \
@@ -1221,7 +1420,8 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
     default: return false;
   }
 #undef THC_TILED_CASE
-  note_kernel(vec ? (args.nq > 1 ? "tiled-fused" : "tiled") : (shift ? "tiled-shift" : "tiled-scalar"));
+  note_kernel(vec ? (args.nq > 1 ? "tiled-fused" : "tiled")
+                  : (ragged ? "tiled-ragged" : (shift ? "tiled-shift" : "tiled-scalar")));
   return true;
 }
 

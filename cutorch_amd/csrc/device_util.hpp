@@ -68,6 +68,19 @@ __device__ __forceinline__ void store_pack(P* p, const P& v) {
   }
 }
 
+// A pack of 4-byte elements at an address that is aligned for the element
+// only: still one 16-byte instruction, which global memory serves at any 4-byte
+// alignment (a lane's 16 bytes may then straddle two sectors).
+template <bool NT, typename P, typename T>
+__device__ __forceinline__ P load_loose_pack(const T* p) {
+  static_assert(sizeof(P) == 16 && sizeof(T) == 4, "16-byte packs of 4-byte elements");
+  typedef uint32_t R __attribute__((ext_vector_type(4), aligned(4)));
+  const R r = NT ? __builtin_nontemporal_load(reinterpret_cast<const R*>(p)) : *reinterpret_cast<const R*>(p);
+  P out;
+  __builtin_memcpy(&out, &r, sizeof(P));
+  return out;
+}
+
 // Buffer-instruction access to a run of `bytes` bytes at `p`: loads beyond the
 // run return zero and stores beyond it are dropped by the hardware's bounds
 // check, so a kernel needs no predicate for the ragged end of its data.

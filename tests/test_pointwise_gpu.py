@@ -81,17 +81,19 @@ def test_random_strided_geometries(thc, oracle, seed):
     run_binary(thc, oracle, name, geoms, rng, inplace=(seed % 5 == 0))
 
 
-@pytest.mark.parametrize("shift", [1, 0])
+@pytest.mark.parametrize("shift", [2, 1, 0])
 @pytest.mark.parametrize("force64", [False, True])
 @pytest.mark.parametrize("shape", [(64, 64), (70, 131), (257, 33), (8, 8), (5, 300, 7), (3, 40, 50),
                                    (128, 4, 96), (1, 200, 200), (2, 3, 65, 67)])
 def test_transposed_operand_uses_tiles(thc, oracle, shape, force64, shift):
     """One operand's unit-stride dim is the first logical dim (a:t(), or a
     permute(3,2,1) view); out and b are contiguous. Rows that are not 16-byte
-    aligned run on the shifted-window variant, or, with it switched off, on
-    the element-wise one."""
+    aligned run on the line-aligned ragged variant (shift = 2), with it
+    switched off on the shifted-window variant, and with that switched off
+    too on the element-wise one."""
     rng = np.random.default_rng(sum(shape))
-    thc.set_tuning("apply.tiled.shift", shift)
+    thc.set_tuning("apply.tiled.ragged", 1 if shift == 2 else 0)
+    thc.set_tuning("apply.tiled.shift", 1 if shift else 0)
     nd = len(shape)
     st, run = [0] * nd, 1
     for d in range(nd):            # dim 0 innermost in memory
@@ -107,17 +109,83 @@ def test_transposed_operand_uses_tiles(thc, oracle, shape, force64, shift):
     finally:
         thc.force_64bit_index(False)
         thc.set_tuning("apply.tiled.shift", 1)
+        thc.set_tuning("apply.tiled.ragged", 1)
     dims = [s for s in shape if s != 1]
     if dims[0] >= 8 and dims[-1] >= 8:      # tiny tile dims fall back to the strided kernel
         assert k.startswith("tiled") and k2.startswith("tiled") and k3.startswith("tiled"), (k, k2, k3)
         if dims[0] % 4 or dims[-1] % 4:
-            assert k == ("tiled-shift" if shift else "tiled-scalar"), k
+            assert k == ("tiled-ragged", "tiled-shift", "tiled-scalar")[2 - shift], k
     else:
         assert k.startswith("strided"), (k, k2, k3)
 
 
+@pytest.fixture
+def no_ragged_tiles(thc):
+    """Keeps 4-byte element types off the line-aligned ragged variant, so that the shifted-window
+    variant (which otherwise serves the other element sizes only) runs."""
+    thc.set_tuning("apply.tiled.ragged", 0)
+    yield
+    thc.set_tuning("apply.tiled.ragged", 1)
+
+
+def run_exact(thc, name, geoms, rng, kind, inplace=False):
+    """run_binary for any element type, on small integers (exact in every type) against numpy
+    views of the same storages: name = cadd1 (a + b), cadd (a + 3 b) or cmul."""
+    dtype = {"float": np.float32, "double": np.float64, "int": np.int32, "long": np.int64}[kind]
+    sts = [rng.integers(-9, 10, g[0]).astype(dtype) for g in geoms]
+    dev = [thc.Tensor.from_storage(s, g[1], g[2], g[3], kind) for s, g in zip(sts, geoms)]
+    want = [s.copy() for s in sts]
+    item = np.dtype(dtype).itemsize
+    view = [np.lib.stride_tricks.as_strided(w[g[1]:], g[2], tuple(x * item for x in g[3])) for w, g in zip(want, geoms)]
+    if inplace:
+        dev[1], view[1] = dev[0], view[0]
+    if name == "cmul":
+        dev[0].cmul(dev[1], dev[2])
+        view[0][...] = view[1] * view[2]
+    else:
+        value = 1 if name == "cadd1" else 3
+        dev[0].cadd(dev[1], value, dev[2])
+        view[0][...] = view[1] + value * view[2]
+    assert_bit_equal(dev[0].storage_numpy(), want[0], "%s %s" % (kind, name))
+    return thc.last_kernel()
+
+
+@pytest.mark.parametrize("kind", ["float", "int"])
+def test_line_aligned_ragged_tiles(thc, oracle, kind):
+    """4-byte elements, rows that start anywhere in a cache line: tiles that cut every row at its own
+    line boundaries. Sizes around the tile edges (64 x 128, up to 31 columns of slack) and off the
+    pack width, views 1..3 elements into their storage, storages that start rows at every offset
+    within a line (pitches 129, 130, 161, 8193 mod 32), rows with gaps, a batch dim in front, a
+    transposed output, two staged inputs and in-place use. Whole storages are compared, so a store
+    outside the tensor's own elements fails the test."""
+    rng = np.random.default_rng(81)
+    for rows, cols in ((64, 128), (65, 129), (63, 127), (61, 125), (129, 257), (333, 515), (1001, 67), (9, 700),
+                       (70, 97), (200, 161), (130, 130)):
+        for off in (0, 1, 3, 17):
+            ga = (rows * cols + off, off, (rows, cols), (1, rows))          # a:t()
+            gc = (rows * cols + off, off, (rows, cols), (cols, 1))
+            aligned = rows % 4 == 0 and cols % 4 == 0 and off % 4 == 0
+            want = "tiled" if aligned else "tiled-ragged"
+            assert run_exact(thc, "cadd1", [gc, ga, gc], rng, kind) == want, (rows, cols, off)
+            assert run_exact(thc, "cadd", [gc, gc, ga], rng, kind, inplace=True) == want, (rows, cols, off)
+            assert run_exact(thc, "cadd1", [ga, ga, gc], rng, kind) == want, (rows, cols, off)   # transposed output
+            # transposed output, two staged inputs (two aligned 64 x 128 tiles exceed the pack variant's LDS limit)
+            assert run_exact(thc, "cmul", [ga, gc, gc], rng, kind) == "tiled-ragged", (rows, cols, off)
+    # rows with gaps (a narrowed view of a wider matrix), transposed partner at another offset
+    gout = (200 * 131 + 2, 2, (200, 127), (131, 1))
+    ga = (127 * 203 + 1, 1, (200, 127), (1, 203))
+    gb = (200 * 131 + 2, 2, (200, 127), (131, 1))
+    assert run_exact(thc, "cadd", [gout, ga, gb], rng, kind) == "tiled-ragged"
+    # b starts one element later than out: its packs would not be aligned, the element-wise variant runs
+    gb = (200 * 131 + 3, 3, (200, 127), (131, 1))
+    assert run_exact(thc, "cadd", [gout, ga, gb], rng, kind) == "tiled-scalar"
+    g3 = (7 * 130 * 401 + 5, 5, (7, 401, 130), (130 * 401, 1, 401))     # batch dim in front, p = 401
+    gd = (7 * 401 * 130 + 5, 5, (7, 401, 130), (401 * 130, 130, 1))
+    assert run_exact(thc, "cmul", [gd, g3, gd], rng, kind) == "tiled-ragged"
+
+
 @pytest.mark.parametrize("kind", ["float", "half"])
-def test_shifted_window_tiles_at_every_misalignment(thc, oracle, kind):
+def test_shifted_window_tiles_at_every_misalignment(thc, oracle, kind, no_ragged_tiles):
     """Sizes around the window edges (a tile spans 4 elements fewer than its
     window; 8 for half), views that start 1..3 elements into their storage,
     rows with gaps, and operands whose misalignments differ (those fall back
@@ -147,7 +215,7 @@ def test_shifted_window_tiles_at_every_misalignment(thc, oracle, kind):
     assert run_binary(thc, oracle, "cadd", [gout, ga, gb], rng, kind=kind) == "tiled-scalar"
 
 
-def test_shifted_window_tiles_with_two_staged_inputs(thc, oracle):
+def test_shifted_window_tiles_with_two_staged_inputs(thc, oracle, no_ragged_tiles):
     rng = np.random.default_rng(78)
     x = rng.standard_normal((203, 331)).astype(np.float32)
     y = rng.standard_normal((203, 331)).astype(np.float32)
@@ -432,7 +500,7 @@ def test_broadcast_operands_on_rows_that_are_not_pack_aligned(thc, kind):
 
 
 @pytest.mark.parametrize("band", [1, 2, 3, 8])
-def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band):
+def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band, no_ragged_tiles):
     """The shifted-window variant walks its tiles in bands of `band` tiles along
     p (p fastest inside a band): whole bands, a ragged last band, and shapes
     too short in p for banding must all cover every tile exactly once."""
@@ -528,7 +596,7 @@ def test_streaming_store_variants_give_the_same_bits(thc, oracle):
                           rng) == "tiled"
         go = (333 * 515 + 1, 1, (333, 515), (1, 333))
         assert run_binary(thc, oracle, "cadd", [contiguous_geometry((333, 515)), go, contiguous_geometry((333, 515))],
-                          rng) == "tiled-shift"
+                          rng) == "tiled-ragged"
         x = rng.integers(-8, 9, (333, 515)).astype(np.float32)
         bias = rng.integers(-8, 9, 515).astype(np.float32)
         db = thc.Tensor.from_numpy(bias).view_as_strided(0, (333, 515), (0, 1))
