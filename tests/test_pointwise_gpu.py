@@ -184,6 +184,40 @@ def test_line_aligned_ragged_tiles(thc, oracle, kind):
     assert run_exact(thc, "cmul", [gd, g3, gd], rng, kind) == "tiled-ragged"
 
 
+def test_line_aligned_ragged_tiles_with_three_inputs(thc, oracle):
+    """addcmul on odd shapes with one, two and three transposed inputs: one and two staged inputs run
+    on the ragged tiles (41 KiB of LDS each), three exceed their LDS limit; 32- and 64-bit offsets."""
+    rng = np.random.default_rng(83)
+    rows, cols = 331, 203
+    x, y, z = (rng.integers(-5, 6, (cols, rows)).astype(np.float32) for _ in range(3))     # used as x.t()
+    u, v, w = (rng.integers(-5, 6, (rows, cols)).astype(np.float32) for _ in range(3))
+    dev = {n: thc.Tensor.from_numpy(a) for n, a in dict(x=x, y=y, z=z, u=u, v=v, w=w).items()}
+    for force64 in (False, True):
+        thc.force_64bit_index(force64)
+        try:
+            out = thc.Tensor("float").addcmul(dev["u"], 2.0, dev["x"].t(), dev["v"])
+            assert thc.last_kernel() == "tiled-ragged"
+            assert_bit_equal(out.numpy(), u + 2.0 * x.T * v)
+            out = thc.Tensor("float").addcmul(dev["u"], 2.0, dev["v"], dev["x"].t())
+            assert thc.last_kernel() == "tiled-ragged"
+            assert_bit_equal(out.numpy(), u + 2.0 * v * x.T)
+            out = thc.Tensor("float").addcmul(dev["x"].t(), 2.0, dev["u"], dev["v"])
+            assert thc.last_kernel() == "tiled-ragged"
+            assert_bit_equal(out.numpy(), x.T + 2.0 * u * v)
+            out = thc.Tensor("float").addcmul(dev["u"], 2.0, dev["x"].t(), dev["y"].t())
+            assert thc.last_kernel() == "tiled-ragged"
+            assert_bit_equal(out.numpy(), u + 2.0 * x.T * y.T)
+            out = thc.Tensor("float").addcmul(dev["x"].t(), 0.5, dev["y"].t(), dev["z"].t())
+            assert thc.last_kernel().startswith("tiled") or thc.last_kernel().startswith("strided"), thc.last_kernel()
+            assert_bit_equal(out.numpy(), x.T + 0.5 * y.T * z.T)
+            dev["w"].addcmul(dev["w"], 2.0, dev["x"].t(), dev["v"])                          # in place
+            assert thc.last_kernel() == "tiled-ragged"
+            w = w + 2.0 * x.T * v
+            assert_bit_equal(dev["w"].numpy(), w)
+        finally:
+            thc.force_64bit_index(False)
+
+
 @pytest.mark.parametrize("kind", ["float", "half"])
 def test_shifted_window_tiles_at_every_misalignment(thc, oracle, kind, no_ragged_tiles):
     """Sizes around the window edges (a tile spans 4 elements fewer than its
