@@ -887,8 +887,8 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
   }
 }
 
-// The tiled kernel for 4-byte elements whose rows start anywhere in a cache
-// line (odd sizes, views at odd offsets). Where the shifted-window variant cuts
+// The tiled kernel for 4- and 8-byte elements whose rows start anywhere in a
+// cache line (odd sizes, views at odd offsets). Where the shifted-window variant cuts
 // every row at the same logical columns, so that each 496-byte row piece of a
 // tile touches five 128-byte lines and shares its first and last one with the
 // neighbouring tiles (fetched and, worse, partially written twice), this one
@@ -904,15 +904,17 @@ __global__ __launch_bounds__(kBlock) void apply_tiled_shift_kernel(T* out, const
 // bytes at whatever offset the operand's own pitch gives it).
 // The host guarantees unit stride along every operand's fast dim and direct
 // operands that share the output's misalignment modulo the pack width.
-constexpr int kRaggedLine = 32;  // 128-byte lines (64-byte cut points: less re-fetch of staged rows, 1.07 x, but 4 % more written bytes and 0.60 instead of 0.65 of peak)
+// 128-byte lines (64-byte cut points: less re-fetch of staged rows, 1.07 x, but 4 % more written bytes and 0.60
+// instead of 0.65 of peak)
+constexpr int kRaggedLineBytes = 128;
 template <typename T, typename Op, typename I, int MASK>
 __global__ __launch_bounds__(kBlock) void apply_tiled_ragged_kernel(T* out, const T* in0, const T* in1,
                                                                     const T* in2, TiledArgs<I> args, Op op) {
-  static_assert(sizeof(T) == 4, "4-byte elements");
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "4- or 8-byte elements");
   constexpr int NOPS = Op::NIN + 1;
-  constexpr int VEC = 4, LXP = 16, LXQ = 32;
-  constexpr int TP = LXP * VEC, TQ = LXQ * VEC;  // 64 x 128
-  constexpr int LINE = kRaggedLine;              // elements between two cut points of a row
+  constexpr int VEC = 16 / sizeof(T), LXP = 16, LXQ = 32;
+  constexpr int TP = LXP * VEC, TQ = LXQ * VEC;  // 64 x 128 (32 x 64 for 8-byte elements)
+  constexpr int LINE = kRaggedLineBytes / sizeof(T);  // elements between two cut points of a row
   constexpr int SPAN = TQ + LINE - 1;            // columns a tile may touch
   constexpr int ROWS_P = kBlock / LXP, PASSES_P = (SPAN + ROWS_P - 1) / ROWS_P;
   constexpr int ROWS_Q = kBlock / LXQ, PASSES_Q = TP / ROWS_Q;
@@ -1291,13 +1293,14 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   // 4-byte elements: tiles cut along every row's own cache lines (apply_tiled_ragged_kernel)
   bool ragged = false;
   size_t ldsR = 0;
-  if constexpr (kSameType && sizeof(T) == 4) {
-    ldsR = (size_t)nstaged * (128 + kRaggedLine - 1) * 65 * sizeof(T);
+  constexpr int64_t kRaggedSlack = kRaggedLineBytes / sizeof(T) - 1;  // columns a row's first line may start early
+  if constexpr (kSameType && (sizeof(T) == 4 || sizeof(T) == 8)) {
+    ldsR = (size_t)nstaged * (tqV + kRaggedSlack) * (tpV + 1) * sizeof(T);
     ragged = shift && ldsR <= 96 * 1024 && tuning("apply.tiled.ragged", 1);
   }
   if (!vec && !shift && ldsS > 64 * 1024) return false;
-  const int64_t tileP = vec ? tpV : (ragged ? 64 : (shift ? tpV - VEC : tS));
-  const int64_t tileQ = vec ? tqV : (ragged ? 128 : (shift ? tqV - VEC : tS));
+  const int64_t tileP = vec || ragged ? tpV : (shift ? tpV - VEC : tS);
+  const int64_t tileQ = vec || ragged ? tqV : (shift ? tqV - VEC : tS);
 
   TiledArgs<I> args{};
   for (int k = 0; k < pl.nops; ++k) {
@@ -1340,7 +1343,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   }
   const int64_t tp = (pl.lay[0].size[p] + tileP - 1) / tileP;
   // (ragged tiles: a row's first line may start up to 31 columns before the row does)
-  const int64_t tq = (sizeQ + (ragged ? kRaggedLine - 1 : 0) + tileQ - 1) / tileQ;
+  const int64_t tq = (sizeQ + (ragged ? kRaggedSlack : 0) + tileQ - 1) / tileQ;
   args.tilesP.set((uint64_t)tp);
   args.tilesQ.set((uint64_t)tq);
   const int64_t total = batch * tp * tq;
@@ -1392,7 +1395,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   case M:                                                                                         \
     if ((M) < (1 << Op::NIN)) {                                                                   \
       constexpr int MM = (M) < (1 << Op::NIN) ? (M) : 1;                                          \
-      if constexpr (kSameType && sizeof(T) == 4) {                                                \
+      if constexpr (kSameType && (sizeof(T) == 4 || sizeof(T) == 8)) {                            \
         if (ragged)                                                                               \
           hipLaunchKernelGGL((apply_tiled_ragged_kernel<T, Op, I, MM>), dim3(grid), dim3(kBlock), \
                              ldsR, st, out, i0, i1, i2, args, op);                                \

@@ -68,12 +68,12 @@ __device__ __forceinline__ void store_pack(P* p, const P& v) {
   }
 }
 
-// A pack of 4-byte elements at an address that is aligned for the element
-// only: still one 16-byte instruction, which global memory serves at any 4-byte
-// alignment (a lane's 16 bytes may then straddle two sectors).
+// A pack of 4- or 8-byte elements at an address that is aligned for the
+// element only: still one 16-byte instruction, which global memory serves at
+// any 4-byte alignment (a lane's 16 bytes may then straddle two sectors).
 template <bool NT, typename P, typename T>
 __device__ __forceinline__ P load_loose_pack(const T* p) {
-  static_assert(sizeof(P) == 16 && sizeof(T) == 4, "16-byte packs of 4-byte elements");
+  static_assert(sizeof(P) == 16 && (sizeof(T) == 4 || sizeof(T) == 8), "16-byte packs of 4- or 8-byte elements");
   typedef uint32_t R __attribute__((ext_vector_type(4), aligned(4)));
   const R r = NT ? __builtin_nontemporal_load(reinterpret_cast<const R*>(p)) : *reinterpret_cast<const R*>(p);
   P out;

@@ -150,10 +150,11 @@ def run_exact(thc, name, geoms, rng, kind, inplace=False):
     return thc.last_kernel()
 
 
-@pytest.mark.parametrize("kind", ["float", "int"])
+@pytest.mark.parametrize("kind", ["float", "int", "double", "long"])
 def test_line_aligned_ragged_tiles(thc, oracle, kind):
-    """4-byte elements, rows that start anywhere in a cache line: tiles that cut every row at its own
-    line boundaries. Sizes around the tile edges (64 x 128, up to 31 columns of slack) and off the
+    """4- and 8-byte elements, rows that start anywhere in a cache line: tiles that cut every row at its
+    own line boundaries. Sizes around the tile edges (64 x 128, up to 31 columns of slack; 32 x 64 and 15
+    for 8-byte elements) and off the
     pack width, views 1..3 elements into their storage, storages that start rows at every offset
     within a line (pitches 129, 130, 161, 8193 mod 32), rows with gaps, a batch dim in front, a
     transposed output, two staged inputs and in-place use. Whole storages are compared, so a store
@@ -164,13 +165,15 @@ def test_line_aligned_ragged_tiles(thc, oracle, kind):
         for off in (0, 1, 3, 17):
             ga = (rows * cols + off, off, (rows, cols), (1, rows))          # a:t()
             gc = (rows * cols + off, off, (rows, cols), (cols, 1))
-            aligned = rows % 4 == 0 and cols % 4 == 0 and off % 4 == 0
+            vec = 2 if kind in ("double", "long") else 4
+            aligned = rows % vec == 0 and cols % vec == 0 and off % vec == 0
             want = "tiled" if aligned else "tiled-ragged"
             assert run_exact(thc, "cadd1", [gc, ga, gc], rng, kind) == want, (rows, cols, off)
             assert run_exact(thc, "cadd", [gc, gc, ga], rng, kind, inplace=True) == want, (rows, cols, off)
             assert run_exact(thc, "cadd1", [ga, ga, gc], rng, kind) == want, (rows, cols, off)   # transposed output
-            # transposed output, two staged inputs (two aligned 64 x 128 tiles exceed the pack variant's LDS limit)
-            assert run_exact(thc, "cmul", [ga, gc, gc], rng, kind) == "tiled-ragged", (rows, cols, off)
+            # transposed output, two staged inputs (of 4-byte elements: two aligned 64 x 128 tiles exceed the
+            # pack variant's LDS limit)
+            assert run_exact(thc, "cmul", [ga, gc, gc], rng, kind) == ("tiled" if aligned and vec == 2 else "tiled-ragged")
     # rows with gaps (a narrowed view of a wider matrix), transposed partner at another offset
     gout = (200 * 131 + 2, 2, (200, 127), (131, 1))
     ga = (127 * 203 + 1, 1, (200, 127), (1, 203))
@@ -179,6 +182,7 @@ def test_line_aligned_ragged_tiles(thc, oracle, kind):
     # b starts one element later than out: its packs would not be aligned, the element-wise variant runs
     gb = (200 * 131 + 3, 3, (200, 127), (131, 1))
     assert run_exact(thc, "cadd", [gout, ga, gb], rng, kind) == "tiled-scalar"
+    # (for 8-byte elements out at offset 2 is pack-aligned and b at offset 3 is not: the same case)
     g3 = (7 * 130 * 401 + 5, 5, (7, 401, 130), (130 * 401, 1, 401))     # batch dim in front, p = 401
     gd = (7 * 401 * 130 + 5, 5, (7, 401, 130), (401 * 130, 130, 1))
     assert run_exact(thc, "cmul", [gd, g3, gd], rng, kind) == "tiled-ragged"
