@@ -1269,7 +1269,9 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   const size_t ldsV = nstaged * tqV * (tpV + 1) * sizeof(T);
   const size_t ldsS = nstaged * tS * (tS + 1) * sizeof(T);
   const size_t ldsH = nstaged * (tqV - VEC) * ((tpV - VEC) | 1) * sizeof(T);
-  if (vec && ldsV > 64 * 1024) vec = false;
+  // (a workgroup may ask for up to 160 KiB of LDS here; 80 KiB admits two staged operands of 4-byte
+  // elements, 66.5 KiB, two workgroups per CU)
+  if (vec && ldsV > (size_t)tuning("apply.tiled.max_lds", 80 * 1024)) vec = false;
   if (vecOnly && !vec) return false;
   // Misaligned rows: the shifted-window variant keeps 16-byte accesses when
   // every operand has unit stride along its fast dim and the direct operands
@@ -1296,7 +1298,9 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   constexpr int64_t kRaggedSlack = kRaggedLineBytes / sizeof(T) - 1;  // columns a row's first line may start early
   if constexpr (kSameType && (sizeof(T) == 4 || sizeof(T) == 8)) {
     ldsR = (size_t)nstaged * (tqV + kRaggedSlack) * (tpV + 1) * sizeof(T);
-    ragged = shift && ldsR <= 96 * 1024 && tuning("apply.tiled.ragged", 1);
+    // (48 KiB: one staged operand of 4-byte elements; two of them leave one workgroup per CU, and
+    // x:t() * y:t() on 8191 x 8193 then ran at 0.47-0.51 of peak against 0.57 with the shifted windows)
+    ragged = shift && ldsR <= 48 * 1024 && tuning("apply.tiled.ragged", 1);
   }
   if (!vec && !shift && ldsS > 64 * 1024) return false;
   const int64_t tileP = vec || ragged ? tpV : (shift ? tpV - VEC : tS);

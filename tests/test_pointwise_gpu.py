@@ -171,9 +171,10 @@ def test_line_aligned_ragged_tiles(thc, oracle, kind):
             assert run_exact(thc, "cadd1", [gc, ga, gc], rng, kind) == want, (rows, cols, off)
             assert run_exact(thc, "cadd", [gc, gc, ga], rng, kind, inplace=True) == want, (rows, cols, off)
             assert run_exact(thc, "cadd1", [ga, ga, gc], rng, kind) == want, (rows, cols, off)   # transposed output
-            # transposed output, two staged inputs (of 4-byte elements: two aligned 64 x 128 tiles exceed the
-            # pack variant's LDS limit)
-            assert run_exact(thc, "cmul", [ga, gc, gc], rng, kind) == ("tiled" if aligned and vec == 2 else "tiled-ragged")
+            # transposed output, two staged inputs: of 4-byte elements they would leave the ragged tiles one
+            # workgroup per CU, so odd shapes take the shifted windows there
+            k = run_exact(thc, "cmul", [ga, gc, gc], rng, kind)
+            assert k == ("tiled" if aligned else ("tiled-ragged" if vec == 2 else "tiled-shift")), (rows, cols, off, k)
     # rows with gaps (a narrowed view of a wider matrix), transposed partner at another offset
     gout = (200 * 131 + 2, 2, (200, 127), (131, 1))
     ga = (127 * 203 + 1, 1, (200, 127), (1, 203))
@@ -189,8 +190,8 @@ def test_line_aligned_ragged_tiles(thc, oracle, kind):
 
 
 def test_line_aligned_ragged_tiles_with_three_inputs(thc, oracle):
-    """addcmul on odd shapes with one, two and three transposed inputs: one and two staged inputs run
-    on the ragged tiles (41 KiB of LDS each), three exceed their LDS limit; 32- and 64-bit offsets."""
+    """addcmul on odd shapes with one, two and three transposed inputs: one staged input runs on the
+    ragged tiles (41 KiB of LDS), two on the shifted windows, three on neither; 32- and 64-bit offsets."""
     rng = np.random.default_rng(83)
     rows, cols = 331, 203
     x, y, z = (rng.integers(-5, 6, (cols, rows)).astype(np.float32) for _ in range(3))     # used as x.t()
@@ -209,7 +210,7 @@ def test_line_aligned_ragged_tiles_with_three_inputs(thc, oracle):
             assert thc.last_kernel() == "tiled-ragged"
             assert_bit_equal(out.numpy(), x.T + 2.0 * u * v)
             out = thc.Tensor("float").addcmul(dev["u"], 2.0, dev["x"].t(), dev["y"].t())
-            assert thc.last_kernel() == "tiled-ragged"
+            assert thc.last_kernel() == "tiled-shift"                                        # two staged inputs
             assert_bit_equal(out.numpy(), u + 2.0 * x.T * y.T)
             out = thc.Tensor("float").addcmul(dev["x"].t(), 0.5, dev["y"].t(), dev["z"].t())
             assert thc.last_kernel().startswith("tiled") or thc.last_kernel().startswith("strided"), thc.last_kernel()
