@@ -557,6 +557,33 @@ def test_shifted_window_tiles_in_bands_along_p(thc, oracle, band, no_ragged_tile
         thc.set_tuning("apply.tiled.group_p", 8)
 
 
+@pytest.mark.parametrize("cap", [1, 7, 64])
+def test_tiled_variants_with_several_tiles_per_workgroup(thc, oracle, cap):
+    """With the grid capped below the number of tiles a workgroup walks several tiles and reuses its
+    LDS slabs: every tiled variant (pack, fused q, ragged, shifted windows, element-wise) must still
+    cover every tile exactly once."""
+    rng = np.random.default_rng(93)
+    thc.set_tuning("apply.tiled.max_grid", cap)
+    try:
+        gc = contiguous_geometry((320, 512))
+        assert run_binary(thc, oracle, "cadd", [gc, (320 * 512, 0, (320, 512), (1, 320)), gc], rng) == "tiled"
+        gp = (40 * 24 * 520, 0, (520, 24, 40), (1, 520, 520 * 24))
+        assert run_binary(thc, oracle, "cadd", [contiguous_geometry((520, 24, 40)), gp,
+                                                contiguous_geometry((520, 24, 40))], rng) == "tiled-fused"
+        go = contiguous_geometry((333, 515))
+        ga = (333 * 515 + 1, 1, (333, 515), (1, 333))
+        assert run_binary(thc, oracle, "cadd", [go, ga, go], rng) == "tiled-ragged"
+        assert run_binary(thc, oracle, "cadd", [go, ga, go], rng, kind="half") == "tiled-shift"
+        thc.set_tuning("apply.tiled.ragged", 0)
+        assert run_binary(thc, oracle, "cadd", [go, ga, go], rng) == "tiled-shift"
+        thc.set_tuning("apply.tiled.shift", 0)
+        assert run_binary(thc, oracle, "cadd", [go, ga, go], rng) == "tiled-scalar"
+    finally:
+        thc.set_tuning("apply.tiled.max_grid", 1 << 22)
+        thc.set_tuning("apply.tiled.ragged", 1)
+        thc.set_tuning("apply.tiled.shift", 1)
+
+
 @pytest.mark.parametrize("band", [1, 2, 3, 16])
 def test_aligned_tiles_in_bands_along_p(thc, oracle, band):
     """The pack variant of the tiled kernel can walk its tiles in bands along p too (the default
