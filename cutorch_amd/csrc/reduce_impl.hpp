@@ -972,19 +972,39 @@ __global__ __launch_bounds__(kBlock) void renorm_rows_kernel(const T* __restrict
       const A x = abs_any(acc_up<A>(v));
       return PK == 1 ? x : (PK == 2 ? x * x : pow_abs(x, p));
     };
+    // LDS is read in batches of 8 (past the row's end: its last element, not used): one LDS
+    // latency per batch instead of one per element
+    auto power_sum = [&](const T* row, uint32_t first, uint32_t step) {
+      A acc = (A)0;
+      for (uint32_t j = first; j < (uint32_t)R; j += 8 * step) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * step, (uint32_t)R - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (j + u * step < (uint32_t)R) acc += power(x[u]);
+      }
+      return acc;
+    };
     auto scale = [&](T* row, A sum, uint32_t first, uint32_t step) {
       const A norm = PK == 1 ? sum : (PK == 2 ? sqrt_any(sum) : pow_any(sum, (A)1 / p));
       if (norm > maxnorm) {
         const A factor = acc_up<A>(acc_down<T>(maxnorm / (norm + (A)1e-7)));
-        for (uint32_t j = first; j < (uint32_t)R; j += step) row[j] = acc_down<T>(acc_up<A>(row[j]) * factor);
+        for (uint32_t j = first; j < (uint32_t)R; j += 8 * step) {
+          T x[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * step, (uint32_t)R - 1)];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (j + u * step < (uint32_t)R) row[j + u * step] = acc_down<T>(acc_up<A>(x[u]) * factor);
+        }
       }
     };
     if (rowsPerBlock < kBlock / 64) {
       // long rows, fewer than one per wave: the whole workgroup takes each row
       for (uint32_t r = 0; r < nrows; ++r) {
         T* row = lds + mis + r * (uint32_t)R;
-        A acc = (A)0;
-        for (uint32_t j = threadIdx.x; j < (uint32_t)R; j += kBlock) acc += power(row[j]);
+        A acc = power_sum(row, threadIdx.x, kBlock);
         for (uint32_t o = 32; o > 0; o >>= 1) acc += shfl_xor_any(acc, o);
         if ((threadIdx.x & 63) == 0) waveSum[threadIdx.x >> 6] = acc;
         __syncthreads();
@@ -996,8 +1016,7 @@ __global__ __launch_bounds__(kBlock) void renorm_rows_kernel(const T* __restrict
     } else {
       for (uint32_t r = grp; r < nrows; r += groups) {  // lanes of a group share r
         T* row = lds + mis + r * (uint32_t)R;
-        A acc = (A)0;
-        for (uint32_t j = lane; j < (uint32_t)R; j += G) acc += power(row[j]);
+        A acc = power_sum(row, lane, G);
         for (uint32_t o = G >> 1; o > 0; o >>= 1) acc += shfl_xor_any(acc, o);
         scale(row, acc, lane, G);
       }
@@ -1028,14 +1047,30 @@ __global__ __launch_bounds__(kBlock) void var_rows_lds_kernel(const T* __restric
     __syncthreads();
     for (uint32_t r = grp; r < nrows; r += groups) {
       const T* row = lds + mis + r * (uint32_t)R;
+      // both sweeps read LDS in batches of 8 (past the row's end: its last element, not used)
       A sum = (A)0;
-      for (uint32_t j = lane; j < (uint32_t)R; j += G) sum += acc_up<A>(row[j]);
+      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (j + u * G < (uint32_t)R) sum += acc_up<A>(x[u]);
+      }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) sum += shfl_xor_any(sum, o);
       const A mean = sum / (A)R;
       A ss = (A)0;
-      for (uint32_t j = lane; j < (uint32_t)R; j += G) {
-        const A d = acc_up<A>(row[j]) - mean;
-        ss += d * d;
+      for (uint32_t j = lane; j < (uint32_t)R; j += 8 * G) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = row[min(j + u * G, (uint32_t)R - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (j + u * G < (uint32_t)R) {
+            const A d = acc_up<A>(x[u]) - mean;
+            ss += d * d;
+          }
+        }
       }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) ss += shfl_xor_any(ss, o);
       if (lane == 0) {
@@ -1066,13 +1101,29 @@ __global__ __launch_bounds__(kBlock) void var_slab_kernel(const T* __restrict__ 
       uint32_t o, c;
       a.cdiv.divmod(t, o, c);
       const T* col = lds + mis + o * slice + c;
+      // both sweeps read LDS in batches of 8 (past the column's end: its last element, not used)
       A sum = (A)0;
-      for (uint32_t r = 0; r < R; ++r) sum += acc_up<A>(col[r * C]);
+      for (uint32_t r = 0; r < R; r += 8) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = col[min(r + u, R - 1) * C];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (r + u < R) sum += acc_up<A>(x[u]);
+      }
       const A mean = sum / (A)R;
       A ss = (A)0;
-      for (uint32_t r = 0; r < R; ++r) {
-        const A d = acc_up<A>(col[r * C]) - mean;
-        ss += d * d;
+      for (uint32_t r = 0; r < R; r += 8) {
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = col[min(r + u, R - 1) * C];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (r + u < R) {
+            const A d = acc_up<A>(x[u]) - mean;
+            ss += d * d;
+          }
+        }
       }
       I inOff, outOff;
       a.oa.offsets(o0 + o, inOff, outOff);
