@@ -406,7 +406,14 @@ __global__ __launch_bounds__(kBlock) void scan_chunk_totals_kernel(
     if (P == 1) {
       for (uint32_t c = threadIdx.x; c < inner; c += kBlock) {
         A acc = Op::id();
-        for (uint32_t r = 0; r < rows; ++r) acc = Op::op(acc, scan_up<A>(lds[mis + r * inner + c]));
+        for (uint32_t r = 0; r < rows; r += 8) {  // LDS reads in batches of 8 (past the end: the last row, not used)
+          T x[8];
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u) x[u] = lds[mis + min(r + u, rows - 1) * inner + c];
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u)
+            if (r + u < rows) acc = Op::op(acc, scan_up<A>(x[u]));
+        }
         totals[blk * inner + c] = acc;
       }
     } else {
@@ -415,7 +422,14 @@ __global__ __launch_bounds__(kBlock) void scan_chunk_totals_kernel(
         // a contiguous band of rows per thread keeps the combine order that of the scan
         const uint32_t band = (rows + P - 1) / P, rb = p * band, re = min(rows, rb + band);
         A acc = Op::id();
-        for (uint32_t r = rb; r < re; ++r) acc = Op::op(acc, scan_up<A>(lds[mis + r * inner + c]));
+        for (uint32_t r = rb; r < re; r += 8) {
+          T x[8];
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u) x[u] = lds[mis + min(r + u, re - 1) * inner + c];
+#pragma unroll
+          for (uint32_t u = 0; u < 8; ++u)
+            if (r + u < re) acc = Op::op(acc, scan_up<A>(x[u]));
+        }
         part[p * inner + c] = acc;
       }
       __syncthreads();
