@@ -4,14 +4,16 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs all|primary] [--no-cpu]
 
 A "step" is one pass of the hot path over one batch of synthetic input that is
-already resident in HBM. The headline line is quoted on the strided apply3
-configuration (out = a:t() * b + d on 8192 x 8192 fp32, a viewed transposed,
-out and d rotating over three buffer sets so that the Infinity Cache cannot
-absorb the rewrites of one output buffer); every other benchmark configuration
-is measured in the same run and reported, compactly, under "roofline.configs"
-(fraction of peak, microseconds per launch, parity flag), with a plain
+already resident in HBM. The headline line is quoted on the largest
+configuration that fits one GPU: c = a + b on 2048 x 2048 x 520 fp32 (26 GB),
+a viewed through permute(3,2,1), 64-bit indices. Every other benchmark
+configuration is measured in the same run and reported under
+"roofline.configs" (fraction of peak, microseconds per launch, parity flag)
+and, as flat scalars that survive a parser which keeps scalars only, as
+"roofline.frac_<config>" / "roofline.parity_<config>", with a plain
 1-read-1-write calibration stream ("CAL-copy") that tells a slow box from a
-regression. Prints ONE JSON line.
+regression, and host-side call latencies of three small calls ("latency").
+Prints ONE JSON line.
 
   value               algorithmic bytes * steps / wall time of the timed region
   roofline.achieved   algorithmic bytes / average launch duration, from two
@@ -23,10 +25,13 @@ regression. Prints ONE JSON line.
                       copy of the inputs (bit-exact for add/mul/addcmul and
                       max+argmax, 1e-5 / 2e-3 relative for sums and norms)
   cpu_baseline        the CPU restatement (oracle/) timed on this box's host
-                      cores: the headline workload single-threaded is the
-                      value; all-core figures and the reduction path (row sums
-                      of 65536 x 1024, middle-dim sums of 64 x 4096 x 512) are
-                      reported beside it under "configs"
+                      cores: a 1/16 sample of the headline workload (the same
+                      strides, 32 of the 520 planes) single-threaded is the
+                      value; all-core figures, the strided apply3 (C2) and the
+                      reduction path (row sums of 65536 x 1024, middle-dim sums
+                      of 64 x 4096 x 512) are reported beside it under
+                      "configs" and as flat "<config>_single_gbps" /
+                      "<config>_all_cores_gbps" scalars
   --configs all       adds the neighbours of the hot path (N-* lines) and the
                       full per-configuration detail under "all_configs"
 """
@@ -133,7 +138,41 @@ def build_configs(thc, hip, which, only=None):
     def want(*names):
         return not only or any(n in only for n in names)
 
-    # C2: out = a:t() * b + d. Headline = out and d rotating over three buffer sets.
+    # C5 (the headline): 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path. The 8.7 GB
+    # operands repeat a 2^24-element block of normal(0,1) values (the element at storage offset o is
+    # block[o % 2^24]).
+    if want('C5', 'CEIL-2r1w-26GB'):
+        nb = 1 << 24
+        block = rng.standard_normal(nb, dtype=np.float32)
+        rblock = block[::-1].copy()
+        a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
+        b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), rblock)
+        c5 = T("float").resize((2048, 2048, 520))
+        a5v = a5.view_as_strided(0, (2048, 2048, 520), (1, 2048, 2048 * 2048))
+        n5 = 2048 * 2048 * 520
+        planes = sorted(set(range(0, 2048, 31)) | {1, 1023, 1024, 2047})     # 70 of the 2048 [j][k] planes
+
+        def c5_check():
+            ok = True
+            j, k = np.arange(2048, dtype=np.int64)[:, None], np.arange(520, dtype=np.int64)[None, :]
+            for i in planes:
+                got = c5.select(0, i).numpy()
+                wa = block[(i + 2048 * j + 2048 * 2048 * k) % nb]
+                wb = rblock[((i * 2048 + j) * 520 + k) % nb]
+                ok = ok and bit_equal(got, wa + wb)
+            return ok
+        cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
+                           12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5), c5_check))
+        cfgs[-1].note = "parity on %d of the 2048 output planes, first to last" % len(planes)
+        host["C5"] = (block, rblock)
+        if which == "all" or (only and "CEIL-2r1w-26GB" in only):
+            a5flat = a5.view_as_strided(0, (2048, 2048, 520), (2048 * 520, 520, 1))
+            cfgs.append(Config("CEIL-2r1w-26GB", "c = a + b on the same 3 x 8.7 GB buffers, all contiguous (flat ceiling of C5)",
+                               12 * n5, n5, 1, lambda i: c5.cadd(a5flat, 1.0, b5)))
+        if which == "primary":
+            return [c for c in cfgs if want(c.name)], host
+
+    # C2: out = a:t() * b + d, out and d rotating over three buffer sets.
     n2 = 8192
     a2 = rng.standard_normal((n2, n2), dtype=np.float32)
     b2 = rng.standard_normal((n2, n2), dtype=np.float32)
@@ -159,8 +198,6 @@ def build_configs(thc, hip, which, only=None):
     cfgs.append(Config("C2", desc2 + ", out and d rotate over 3 buffer sets", 16 * n2 * n2, n2 * n2, 3,
                        lambda i: out2[i % 3].addcmul(dd[i % 3], 1.0, at, db), c2_check(2)))
     host["C2"] = (a2, b2, d2[0])
-    if which == "primary":
-        return cfgs, host
     cfgs.append(Config("C2-fixed", desc2 + ", one buffer set (the output is rewritten in place every step)",
                        16 * n2 * n2, n2 * n2, 1, lambda i: out2[0].addcmul(dd[0], 1.0, at, db), c2_check(0)))
 
@@ -290,7 +327,9 @@ def build_configs(thc, hip, which, only=None):
     nx = [n for n in ("N-copy-t", "N-fill", "N-exp", "N-var-rows", "N-std-cols", "N-cumsum-rows",
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
-                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot")
+                      "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
+                      "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
+                      "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -302,6 +341,7 @@ def build_configs(thc, hip, which, only=None):
         s3 = T("float").resize((r3, n3))
         s4o = T("float").resize(s4)
         big = 1 << 28
+        nodd_ = 8191 * 8193
         table = {
             "N-copy-t": ("out:copy(a:t()), 8192x8192 fp32", 8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.copy(sq_t)),
             "N-fill": ("fill of 2^28 fp32", 4 * big, big, lambda i: xa.fill(0.5) if xa.numel() == big else e_dst.fill(0.5)),
@@ -379,6 +419,51 @@ def build_configs(thc, hip, which, only=None):
                 "N-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 fp32", 9 * 8192 * 8192, 8192 * 8192,
                            lambda i: lt_m.compare_tensor("lt", sq_t, db)),
             })
+        if set(nx) & {"N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
+                      "N-cvt-half-t"}:
+            # transposed operands of the op families beyond plain float arithmetic: one-input math on half,
+            # narrow integer arithmetic, two-input float math, integer division, integer comparison into Byte,
+            # type-converting copy
+            m = 8192
+            hx = T.from_numpy(rng.uniform(-2, 2, (m, m)).astype(np.float16)).t()
+            ho = T("half").resize((m, m))
+            hxo = T.from_numpy(rng.uniform(-2, 2, (8193, 8191)).astype(np.float16)).t()
+            hoo = T("half").resize((8191, 8193))
+            sa = T.from_numpy(rng.integers(-1000, 1000, (m, m)).astype(np.int16)).t()
+            sb = T.from_numpy(rng.integers(-1000, 1000, (m, m)).astype(np.int16))
+            sc = T("short").resize((m, m))
+            ja = T.from_numpy(rng.integers(-100000, 100000, (m, m)).astype(np.int32)).t()
+            jb = T.from_numpy(rng.integers(1, 1000, (m, m)).astype(np.int32))
+            jc = T("int").resize((m, m))
+            jm = T("byte").resize((m, m))
+            fo = T("float").resize((m, m))
+            hc = T("half").resize((m, m))
+            table.update({
+                "N-half-exp-t": ("out = exp(a:t()), 8192x8192 fp16", 4 * m * m, m * m, lambda i: ho.unary("exp", hx)),
+                "N-half-exp-t-odd": ("out = exp(a:t()), 8191x8193 fp16 (no 16-byte aligned rows)", 4 * nodd_,
+                                     nodd_, lambda i: hoo.unary("exp", hxo)),
+                "N-short-add-t": ("c = a:t() + b, 8192x8192 int16", 6 * m * m, m * m, lambda i: sc.cadd(sa, 1, sb)),
+                "N-cmax-t": ("c = cmax(a:t(), b), 8192x8192 fp32", 12 * m * m, m * m,
+                             lambda i: fo.binary("cmax", sq_t, db)),
+                "N-int-div-t": ("c = a:t() / b, 8192x8192 int32 (truncating division)", 12 * m * m, m * m,
+                                lambda i: jc.cdiv(ja, jb)),
+                "N-int-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 int32", 9 * m * m, m * m,
+                               lambda i: jm.compare_tensor("lt", ja, jb)),
+                "N-cvt-half-t": ("half <- float converting copy of a:t(), 8192x8192", 6 * m * m, m * m,
+                                 lambda i: hc.copy_from(sq_t)),
+            })
+        if "N-equal" in nx:
+            eq_b = e_src.clone()
+            table["N-equal"] = ("equal(a, b) over 2^26 fp32 (both equal: no early exit possible)", 8 * ne, ne,
+                                lambda i: e_src.equal(eq_b))
+        for tag, lg in (("64M", 24), ("256M", 26), ("1G", 28)):
+            if "N-copy-contig-" + tag in nx:
+                m = 1 << lg
+                cc_src = T.from_numpy(rng.uniform(-1, 1, m).astype(np.float32))
+                cc_dst = [T("float").resize((m,)) for _ in range(3)]
+                table["N-copy-contig-" + tag] = (
+                    "dst:copy(src), 2^%d fp32 contiguous, 3 rotating destinations" % lg, 8 * m, m,
+                    (lambda q, src_: lambda i: q[i % 3].copy(src_))(cc_dst, cc_src))
         if set(nx) & {"N-add-2p25", "N-add-2p26"}:
             # c = a + b as in C1 at two and four times the size (rotating sets): kernel time against
             # bytes gives the fixed cost of a launch (t = t0 + bytes / BW)
@@ -404,36 +489,7 @@ def build_configs(thc, hip, which, only=None):
             d, nb, el, fn = table[n]
             cfgs.append(Config(n, d, nb, el, 1, fn))
 
-    # C5: 2048 x 2048 x 520 with a = permute(3,2,1) view, 64-bit index path. The 8.7 GB operands repeat
-    # a 2^24-element block of normal(0,1) values (the element at storage offset o is block[o % 2^24]).
-    if not want('C5'):
-        return [c for c in cfgs if c is cfgs[0] or want(c.name)], host
-    nb = 1 << 24
-    block = rng.standard_normal(nb, dtype=np.float32)
-    rblock = block[::-1].copy()
-    a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
-    b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), rblock)
-    c5 = T("float").resize((2048, 2048, 520))
-    a5v = a5.view_as_strided(0, (2048, 2048, 520), (1, 2048, 2048 * 2048))
-    n5 = 2048 * 2048 * 520
-
-    def c5_check():
-        ok = True
-        j, k = np.arange(2048, dtype=np.int64)[:, None], np.arange(520, dtype=np.int64)[None, :]
-        for i in (0, 1, 1023, 2047):             # whole [j][k] planes of the output, first to last
-            got = c5.select(0, i).numpy()
-            wa = block[(i + 2048 * j + 2048 * 2048 * k) % nb]
-            wb = rblock[((i * 2048 + j) * 520 + k) % nb]
-            ok = ok and bit_equal(got, wa + wb)
-        return ok
-    cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
-                       12 * n5, n5, 1, lambda i: c5.cadd(a5v, 1.0, b5), c5_check))
-    cfgs[-1].note = "parity on 4 of the 2048 output planes"
-    if which == "all" or (only and "CEIL-2r1w-26GB" in only):
-        a5flat = a5.view_as_strided(0, (2048, 2048, 520), (2048 * 520, 520, 1))
-        cfgs.append(Config("CEIL-2r1w-26GB", "c = a + b on the same 3 x 8.7 GB buffers, all contiguous (flat ceiling of C5)",
-                           12 * n5, n5, 1, lambda i: c5.cadd(a5flat, 1.0, b5)))
-    return [c for c in cfgs if c is cfgs[0] or want(c.name)], host
+    return [c for c in cfgs if want(c.name)], host
 
 
 def time_config(hip, thc, cfg, steps, warmup, stream):
@@ -468,28 +524,40 @@ def time_config(hip, thc, cfg, steps, warmup, stream):
 
 def cpu_baseline(host, cfg_bytes, budget_s=24.0):
     """Times the CPU restatement on this box's host cores, single thread and all
-    cores: the headline workload out = a:t()*b + d on the full 8192x8192
-    operands (TH_TENSOR_APPLY path) and, for the reduction path, the row sums
-    of 65536x1024 and the middle-dim sums of 64x4096x512. Every figure is the
+    cores: a 1/16 sample of the headline workload (c = a + b with a seen through
+    permute(3,2,1): 2048 x 2048 x 32 of the 520 planes, the same strides), the
+    strided apply3 out = a:t()*b + d on the full 8192x8192 operands
+    (TH_TENSOR_APPLY path) and, for the reduction path, the row sums of
+    65536x1024 and the middle-dim sums of 64x4096x512. Every figure is the
     median of the runs after the first, GB/s on the algorithmic bytes."""
     from oracle import th_oracle as oracle
     cores = len(os.sched_getaffinity(0))
     jobs = []
+    nbytes = dict(cfg_bytes)
+    if "C5" in host and "C5" in cfg_bytes:
+        block, rblock = host["C5"]
+        k5 = 32
+        n5 = 2048 * 2048 * k5
+        ha, hb = np.resize(block, n5), np.resize(rblock, n5)
+        va = oracle.View(ha, 0, (2048, 2048, k5), (1, 2048, 2048 * 2048))
+        vb, vc = oracle.View(hb, 0, (2048, 2048, k5)), oracle.View.empty((2048, 2048, k5))
+        jobs.append(("C5", 0.3, lambda: oracle.pointwise("cadd", vc, va, vb, value=1.0)))
+        nbytes["C5"] = 12 * n5
     if "C2" in host and "C2" in cfg_bytes:
         a, b, d = host["C2"]
         n = a.shape[0]
-        va = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
-        vb, vd = oracle.View(b.reshape(-1), 0, (n, n)), oracle.View(d.reshape(-1), 0, (n, n))
-        out = oracle.View.empty((n, n))
-        jobs.append(("C2", 0.5, lambda: oracle.pointwise("addcmul", out, vd, va, vb, value=1.0)))
+        va2 = oracle.View(a.reshape(-1), 0, (n, n), (1, n))
+        vb2, vd2 = oracle.View(b.reshape(-1), 0, (n, n)), oracle.View(d.reshape(-1), 0, (n, n))
+        out2 = oracle.View.empty((n, n))
+        jobs.append(("C2", 0.3, lambda: oracle.pointwise("addcmul", out2, vd2, va2, vb2, value=1.0)))
     if host.get("C3a-sum") is not None and "C3a-sum" in cfg_bytes:
         x = host["C3a-sum"]
         vx, o3 = oracle.View(x.reshape(-1), 0, x.shape), oracle.View.empty((x.shape[0], 1))
-        jobs.append(("C3a-sum", 0.2, lambda: oracle.reduce_dim("sum", vx, 1, out=o3)))
+        jobs.append(("C3a-sum", 0.15, lambda: oracle.reduce_dim("sum", vx, 1, out=o3)))
     if host.get("C4-sum-f32") is not None and host["C4-sum-f32"].size > 64 and "C4-sum-f32" in cfg_bytes:
         x4 = host["C4-sum-f32"]
         v4, o4 = oracle.View(x4.reshape(-1), 0, x4.shape), oracle.View.empty((x4.shape[0], 1, x4.shape[2]))
-        jobs.append(("C4-sum-f32", 0.3, lambda: oracle.reduce_dim("sum", v4, 1, out=o4)))
+        jobs.append(("C4-sum-f32", 0.25, lambda: oracle.reduce_dim("sum", v4, 1, out=o4)))
     res = {}
     for name, share, fn in jobs:
         res[name] = {}
@@ -500,22 +568,68 @@ def cpu_baseline(host, cfg_bytes, budget_s=24.0):
                 t0 = time.perf_counter()
                 fn()
                 times.append(time.perf_counter() - t0)
-            res[name][label] = (cfg_bytes[name] / float(np.median(times[1:])) / 1e9, threads, len(times) - 1)
+            res[name][label] = (nbytes[name] / float(np.median(times[1:])) / 1e9, threads, len(times) - 1)
     oracle.set_num_threads(1)
     return res
+
+
+def call_latency(thc, hip, calls=2000):
+    """Host-side cost of small calls (entry point, planning, launch): microseconds per call with the
+    queue left to fill (calls back to back, one wait at the end) and with the stream drained after every
+    call (launch + completion). "ctypes_us" is what the Python binding itself costs per call (an entry
+    point that does nothing), to be subtracted."""
+    T = thc.Tensor
+    rng = np.random.default_rng(7)
+    a = T.from_numpy(rng.standard_normal(1024).astype(np.float32))
+    b = T.from_numpy(rng.standard_normal(1024).astype(np.float32))
+    c = T("float").resize((1024,))
+    m = T.from_numpy(rng.standard_normal((64, 64)).astype(np.float32))
+    o, ix = T("float").resize((64, 1)), T("long").resize((64, 1))
+    st = thc.state()
+    noop = thc.lib().THCState_getCurrentStream
+    cases = {"cadd_1k": lambda: c.cadd(a, 1.0, b), "sum_64x64": lambda: o.sum(m, 1), "max_64x64": lambda: o.max(ix, m, 1)}
+    out = {}
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        noop(st)
+    out["ctypes_us"] = round((time.perf_counter() - t0) / calls * 1e6, 2)
+    for name, fn in cases.items():
+        for _ in range(50):
+            fn()
+        hip.sync()
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            fn()
+        t_issue = time.perf_counter() - t0
+        hip.sync()
+        t_all = time.perf_counter() - t0
+        t1 = time.perf_counter()
+        for _ in range(calls // 4):
+            fn()
+            hip.sync()
+        t_drained = time.perf_counter() - t1
+        out[name + "_queued_us"] = round(t_issue / calls * 1e6, 2)
+        out[name + "_queued_incl_drain_us"] = round(t_all / calls * 1e6, 2)
+        out[name + "_drained_us"] = round(t_drained / (calls // 4) * 1e6, 2)
+    return out
+
+
+def flat_key(name):
+    return name.replace("-", "_")
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--configs", default="bar", choices=["bar", "all", "primary"],
                     help="bar: the benchmark configurations + calibration stream (default); all: also the "
                          "neighbouring ops (N-*) and full detail; primary: the headline only")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-check", action="store_true", help="skip the per-configuration parity checks")
-    ap.add_argument("--only", default="", help="comma-separated config names to measure")
+    ap.add_argument("--only", default="", help="comma-separated config names to measure (the first one "
+                                               "built becomes the line's headline)")
     ap.add_argument("--tune", action="append", default=[], help="engine tuning knob key=value")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -530,11 +644,11 @@ def main():
         thc.set_tuning(k, int(v))
     only = set(args.only.split(",")) if args.only else None
     cfgs, host = build_configs(thc, hip, args.configs, only)
-    if only:
-        cfgs = [cfgs[0]] + [c for c in cfgs[1:] if c.name in only]
+    if not cfgs:
+        sys.exit("no configuration selected")
     results = []
     for cfg in cfgs:
-        steps = args.steps if cfg.name not in ("C5", "CEIL-2r1w-26GB") else max(3, args.steps // 5)
+        steps = args.steps
         wall, region_ms, ms = time_config(hip, thc, cfg, steps, args.warmup, stream)
         ok = None if (args.no_check or cfg.check is None) else bool(cfg.check())
         mean_ms = region_ms / steps
@@ -555,7 +669,7 @@ def main():
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             measured = json.load(f)
-        traffic = measured.get("C2", {}).get("traffic_bytes")
+        traffic = measured.get(p["name"], {}).get("traffic_bytes")
         traffic_src = "profiles/traffic.json (committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary; not measured in this run)"
         for r in results:
             r["traffic_bytes"] = measured.get(r["name"], {}).get("traffic_bytes")
@@ -569,31 +683,51 @@ def main():
                               "sets": r["rotating_sets"]}
         if r["note"]:
             compact[r["name"]]["note"] = r["note"]
+    roof = {"bound": "hbm", "achieved": p["gbps_mean"], "peak": PEAK_GBPS, "unit": "GB/s",
+            "frac": p["frac_of_peak"], "traffic": traffic, "traffic_source": traffic_src}
+    # the same per configuration as flat scalars (a parser that keeps scalars only still sees them)
+    bar = [r for r in results if r["name"][0] == "C" and r["name"][1].isdigit() and r["name"] != "C2-fixed"]
+    for r in results:
+        roof["frac_" + flat_key(r["name"])] = r["frac_of_peak"]
+        roof["us_" + flat_key(r["name"])] = round(1e3 * r["ms_mean"], 2)
+        if r["parity_ok"] is not None:
+            roof["parity_" + flat_key(r["name"])] = r["parity_ok"]
+    if bar:
+        worst = min(bar, key=lambda r: r["frac_of_peak"])
+        roof["frac_min"] = worst["frac_of_peak"]
+        roof["frac_min_config"] = worst["name"]
+        checked = [r["parity_ok"] for r in bar if r["parity_ok"] is not None]
+        roof["parity_all"] = bool(checked) and all(checked)
+    roof["configs"] = compact
     line = {
         "metric": METRIC, "value": p["wall_gbps"], "unit": "GB/s", "n_gpus": 1,
         "steps": p["steps"], "warmup": args.warmup,
         "ms_per_step": round(1e3 * p["algorithmic_bytes"] / (p["wall_gbps"] * 1e9), 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (fixed-seed host generator, copied to HBM before timing)",
-        "config": {"workload": p["desc"], "elements": cfgs[0].elements, "kernel": p["kernel"],
-                   "parity_ok": p["parity_ok"]},
-        "roofline": {"bound": "hbm", "achieved": p["gbps_mean"], "peak": PEAK_GBPS, "unit": "GB/s",
-                     "frac": p["frac_of_peak"], "traffic": traffic, "traffic_source": traffic_src,
-                     "configs": compact},
+        "config": {"workload": p["desc"], "name": p["name"], "elements": cfgs[0].elements, "kernel": p["kernel"],
+                   "parity_ok": p["parity_ok"], "note": p["note"]},
+        "roofline": roof,
     }
+    if args.configs != "primary" and not only:
+        line["latency"] = call_latency(thc, hip)
     if not args.no_cpu:
         cb = cpu_baseline(host, {c.name: c.nbytes for c in cfgs})
         per = {}
+        head = cb.get(p["name"])
+        base = {"value": round(head["single"][0], 2) if head else None, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": ("1/16 of the headline workload: c = a + b on 2048x2048x32 fp32 with a seen through "
+                           "permute(3,2,1) (the same strides, 32 of the 520 planes; 1.6 GB of traffic per run), "
+                           "median of %d runs" % head["single"][2]) if head and p["name"] == "C5" else
+                          ("the %s workload at full size, median of %d runs" % (p["name"], head["single"][2]) if head else None)}
         for name, r in cb.items():
             per[name] = {"single_gbps": round(r["single"][0], 2), "all_cores_gbps": round(r["all"][0], 2),
                          "cores": r["all"][1], "runs": [r["single"][2], r["all"][2]]}
-        head = cb.get("C2")
-        line["cpu_baseline"] = {
-            "value": round(head["single"][0], 2) if head else None, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": "full workload (8192x8192 addcmul with transposed operand), median of %d runs; "
-                      "\"configs\" holds the same for the reduction path (C3a row sums, C4 middle-dim sums), "
-                      "single thread and all cores" % (head["single"][2] if head else 0),
-            "configs": per}
+            base[flat_key(name) + "_single_gbps"] = round(r["single"][0], 2)
+            base[flat_key(name) + "_all_cores_gbps"] = round(r["all"][0], 2)
+            base["all_cores"] = r["all"][1]
+        base["configs"] = per
+        line["cpu_baseline"] = base
     if args.configs == "all":
         line["all_configs"] = results
     print(json.dumps(line))

@@ -20,9 +20,12 @@ SOURCES = ["general.cpp", "tensor.cpp", "math.cpp", "math_wide.cpp", "caching_al
            "apply_f32_2.hip", "apply_f16_0.hip", "apply_f16_1.hip", "apply_f16_2.hip", "apply_raw.hip",
            "reduce.hip", "reduce_f32.hip", "reduce_f16.hip", "reduce_w_u8.hip", "reduce_w_i8.hip",
            "reduce_w_i16.hip", "reduce_w_i32.hip", "reduce_w_i64.hip", "reduce_w_f64.hip", "scan.hip", "no_alloc.hip", "convert.hip", "apply_cmp_f.hip", "apply_w_u8.hip",
-           "apply_rawmath_u32u64.hip", "apply_rawmath_f64.hip", "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip"]
-HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", "apply_plan.hpp", "apply_impl.hpp", "apply_wide.hpp", "reduce_plan.hpp", "reduce_impl.hpp",
-           os.path.join("..", "..", "include", "THC.h")]
+           "apply_rawmath_u32u64.hip", "apply_rawmath_f64.hip", "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip",
+           "apply_cvt_u8.hip", "apply_cvt_i8.hip", "apply_cvt_i16.hip", "apply_cvt_i32.hip", "apply_cvt_i64.hip",
+           "apply_cvt_f16.hip", "apply_cvt_f32.hip", "apply_cvt_f64.hip"]
+HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", os.path.join("..", "..", "include", "THC.h")]   # every source
+APPLY_HEADERS = ["apply_plan.hpp", "apply_impl.hpp", "apply_ldstile.hpp", "apply_wide.hpp"]   # apply*.hip, convert.hip
+REDUCE_HEADERS = ["reduce_plan.hpp", "reduce_impl.hpp"]                                       # reduce*.hip, scan.hip, no_alloc.hip
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -51,12 +54,15 @@ EXTRA_DEPS = {"caching_allocator.cpp": ["caching_pool.hpp", "stream_guard.hpp"],
               "apply.hip": ["stream_guard.hpp", "apply_rawmath.hpp"],
               "apply_rawmath_u32u64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"],
               "apply_rawmath_f64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"], "reduce.hip": ["stream_guard.hpp"],
-              "scan.hip": ["stream_guard.hpp"], "convert.hip": ["stream_guard.hpp"]}
+              "scan.hip": ["stream_guard.hpp"], "no_alloc.hip": ["stream_guard.hpp"], "convert.hip": ["stream_guard.hpp"]}
+EXTRA_DEPS.update({"apply_cvt_%s.hip" % t: ["apply_convert_impl.hpp"] for t in ("u8", "i8", "i16", "i32", "i64", "f16", "f32", "f64")})
 
 
 def _compile(src, force):
     obj = os.path.join(BUILD, src + ".o")
-    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS + EXTRA_DEPS.get(src, [])]
+    group = APPLY_HEADERS if src.startswith(("apply", "convert")) else (
+        REDUCE_HEADERS if src.startswith(("reduce", "scan", "no_alloc")) else [])
+    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS + group + EXTRA_DEPS.get(src, [])]
     if not force and not _stale(obj, deps):
         return obj
     cmd = [_hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS

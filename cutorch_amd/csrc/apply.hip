@@ -72,11 +72,12 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
     return true;
   }
 
-  // Ops that stay off the LDS-tiled kernels (the six wider element types, the
-  // comparisons, the two-input math family and the one-input family on half)
-  // would read a transposed input with one useful element per sector. Such an input is first brought into the output's memory order by
-  // the same-type copy, which does own a tiled kernel for every element size:
-  // two extra coalesced passes instead of one uncoalesced one.
+  // Ops without specialised tiled kernels (the six wider element types, the comparisons, the
+  // two-input math family and the one-input family on half) meet a transposed input in the general
+  // LDS-tile kernel. What that kernel declines too (no unit stride along an operand's fast dim, a
+  // tile spanning 2^31 elements) would be read with one useful element per sector: such an input is
+  // first brought into the output's memory order by the same-type copy, two extra coalesced passes
+  // instead of one uncoalesced one.
   // Plans the operands as they are and launches; false only when `decline` is set and the
   // per-type code refused a plan that would read a transposed operand uncoalesced.
   auto launch = [&](bool decline) -> bool {
@@ -124,34 +125,30 @@ bool pointwise_apply(THCState* s, const ApplyDesc& d, AnyTensor* out, AnyTensor*
       const float value = (float)d.v.f, value2 = (float)d.w.f;
       const MathFn fn = (MathFn)d.fn;
       if (dt == DType::F32) {
-        if (g == 0) apply_dispatch_group<float, 0>(s, pl, sameShape, d.op, value, fn, value2);
-        else if (g == 1) apply_dispatch_group<float, 1>(s, pl, sameShape, d.op, value, fn, value2);
-        else apply_dispatch_group<float, 2>(s, pl, sameShape, d.op, value, fn, value2);
+        if (g == 0) launched = apply_dispatch_group<float, 0>(s, pl, sameShape, d.op, value, fn, value2, decline);
+        else if (g == 1) launched = apply_dispatch_group<float, 1>(s, pl, sameShape, d.op, value, fn, value2, decline);
+        else launched = apply_dispatch_group<float, 2>(s, pl, sameShape, d.op, value, fn, value2, decline);
       } else {
-        if (g == 0) apply_dispatch_group<__half, 0>(s, pl, sameShape, d.op, value, fn, value2);
-        else if (g == 1) apply_dispatch_group<__half, 1>(s, pl, sameShape, d.op, value, fn, value2);
-        else apply_dispatch_group<__half, 2>(s, pl, sameShape, d.op, value, fn, value2);
+        if (g == 0) launched = apply_dispatch_group<__half, 0>(s, pl, sameShape, d.op, value, fn, value2, decline);
+        else if (g == 1) launched = apply_dispatch_group<__half, 1>(s, pl, sameShape, d.op, value, fn, value2, decline);
+        else launched = apply_dispatch_group<__half, 2>(s, pl, sameShape, d.op, value, fn, value2, decline);
       }
     } else if (dt == DType::F32 || dt == DType::F16) {
       raise_error("pointwise op not available for this element type");
     } else {
-      for_wide_type(dt, [&](auto tag) { apply_wide<decltype(tag)>(s, pl, sameShape, d); });
+      for_wide_type(dt, [&](auto tag) { launched = apply_wide<decltype(tag)>(s, pl, sameShape, d, decline); });
     }
     if (launched) THC_CHECK(hipGetLastError());
     return launched;
   };
-  // Comparisons of float into a Byte tensor own the pack variant of the tiled kernel: try the
-  // operands as they are first; a declined plan takes the densify route below.
-  if ((d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor) && d.dt == DType::F32 && d.outDt == DType::U8 &&
-      launch(true))
-    return true;
-
   TensorRef dense[kMaxOps] = {{s, nullptr}, {s, nullptr}, {s, nullptr}, {s, nullptr}};
   const bool offTiled = d.op != PointOp::Copy &&
                         (d.op == PointOp::CmpValue || d.op == PointOp::CmpTensor ||
                          d.op == PointOp::Math2 || (d.op == PointOp::Math1 && d.dt == DType::F16) ||
                          !(d.dt == DType::F32 || d.dt == DType::F16)) &&
                         !(d.outDt == d.dt && rawmath_serves(d.dt, d.op));
+  // Try the operands as they are first; a declined plan takes the densify route below.
+  if (offTiled && launch(true)) return true;
   // The output's fastest-running dim (smallest stride among dims longer than 1).
   int po = -1;
   for (int dd = out->nDimension - 1; dd >= 0; --dd)
@@ -197,7 +194,12 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
   THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
   if (dst->nDimension == 0) return;
   note_stream_use(s, {dst, src});
-  if ((tensor_is_contiguous(dst) && tensor_is_contiguous(src)) || n == 1) {
+  // Dense to dense: the runtime's copy up to 32 MiB; beyond that the engine's own flat stream
+  // (nontemporal loads, streaming stores) is faster (256 MiB and 1 GiB: 0.65-0.67 of peak bandwidth
+  // for hipMemcpyAsync against 0.78 for the kernel).
+  const bool dense = tensor_is_contiguous(dst) && tensor_is_contiguous(src);
+  const int64_t bytes = (int64_t)n * (int64_t)dtype_size(dt);
+  if ((dense && bytes < tuning("copy.kernel_min_bytes", int64_t(32) << 20)) || n == 1) {
     THC_CHECK(hipMemcpyAsync(tensor_data(dst, dt), tensor_data(src, dt), (size_t)n * dtype_size(dt),
                              hipMemcpyDeviceToDevice, current_stream(s)));
     return;

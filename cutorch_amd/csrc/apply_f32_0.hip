@@ -2,6 +2,5 @@
 #include "apply_impl.hpp"
 
 namespace thc {
-template void apply_dispatch_group<float, 0>(THCState*, Plan&, bool, PointOp, float, MathFn,
-                                             float);
+template bool apply_dispatch_group<float, 0>(THCState*, Plan&, bool, PointOp, float, MathFn, float, bool);
 }

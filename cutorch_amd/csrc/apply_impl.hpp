@@ -1080,9 +1080,14 @@ inline bool aligned16(const void* p) {
 }
 // Operand k of a plan whose inputs are T and whose output (k == 0) is TOut:
 // aligned for packs of 16 / sizeof(T) elements.
+// Elements per pack when inputs are T and the output is TOut: the wider of the two fills 16 bytes.
+template <typename T, typename TOut>
+constexpr int pack_elems() {
+  return 16 / (int)(sizeof(T) > sizeof(TOut) ? sizeof(T) : sizeof(TOut));
+}
 template <typename T, typename TOut>
 inline bool pack_aligned(const Plan& pl, int k) {
-  const size_t bytes = (16 / sizeof(T)) * (k == 0 ? sizeof(TOut) : sizeof(T));
+  const size_t bytes = pack_elems<T, TOut>() * (k == 0 ? sizeof(TOut) : sizeof(T));
   return (reinterpret_cast<uintptr_t>(pl.ptr[k]) & (bytes - 1)) == 0;
 }
 
@@ -1109,7 +1114,7 @@ inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* 
 // LEAN: one unroll variant only (element types off the hot path).
 template <typename T, typename Op, typename TOut = T, bool LEAN = false>
 void launch_contig(THCState* s, const Plan& pl, Op op) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = pack_elems<T, TOut>();
   bool vec = true;
   for (int k = 0; k < pl.nops; ++k) vec = vec && pack_aligned<T, TOut>(pl, k);
   TOut* out = (TOut*)pl.ptr[0];
@@ -1160,7 +1165,7 @@ void launch_contig(THCState* s, const Plan& pl, Op op) {
 // Whether the strided kernel can use 16-byte packs on this (joint) plan.
 template <typename T, typename TOut>
 bool indexed_can_pack(const Plan& pl) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = pack_elems<T, TOut>();
   const int nd = pl.lay[0].dims;
   bool vec = pl.lay[0].size[nd - 1] % VEC == 0;
   for (int k = 0; k < pl.nops && vec; ++k) {
@@ -1172,7 +1177,7 @@ bool indexed_can_pack(const Plan& pl) {
 
 template <typename T, typename Op, typename I, bool JOINT, typename TOut = T>
 void launch_indexed(THCState* s, const Plan& pl, Op op) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = pack_elems<T, TOut>();
   IndexedArgs<I> args{};
   const bool vec = JOINT && indexed_can_pack<T, TOut>(pl);
   const int pack = vec ? VEC : 1;
@@ -1432,6 +1437,10 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
   return true;
 }
 
+}  // namespace thc
+#include "apply_ldstile.hpp"
+namespace thc {
+
 // The flat + gathered kernel applies when the output is one dense aligned run
 // in the order of the joint dims and every input either is such a run too or
 // is a broadcast operand: its elements span at most 1 MiB (the per-element
@@ -1440,7 +1449,7 @@ bool launch_tiled(THCState* s, const Plan& pl, Op op, bool vecOnly = false) {
 // kernel can use packs (6.6 TB/s) they go first (`vecOnly` below).
 template <typename T, typename Op, typename I, typename TOut>
 bool launch_flatmix(THCState* s, const Plan& pl, Op op) {
-  constexpr int VEC = 16 / sizeof(T);
+  constexpr int VEC = pack_elems<T, TOut>();
   if (!tuning("apply.flatmix", 1) || pl.nops < 2) return false;
   const int nd = pl.lay[0].dims;
   auto dense = [&](int k) {
@@ -1528,6 +1537,10 @@ bool run_plan(THCState* s, Plan& pl, bool sameShape, Op op, bool decline = false
           return true;
       }
     }
+    // every functor and type pair without specialised tiled kernels: the general LDS-tile kernel
+    if constexpr (!TILED || !std::is_same<T, TOut>::value) {
+      if (launch_ldstile<T, Op, TOut>(s, pl, op)) return true;
+    }
     if (decline) {
       int p, q, staged[kMaxOps] = {0, 0, 0, 0};
       if (tile_plan(pl, p, q, staged)) return false;  // a transposed operand that no tiled kernel took
@@ -1549,22 +1562,20 @@ bool run_plan(THCState* s, Plan& pl, bool sameShape, Op op, bool decline = false
 
 // Operator groups: one translation unit per (element type, group).
 template <typename T, int GROUP>
-void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
-                          float w) {
-  // The code-dispatched families keep the switch inside the LDS-tiled kernels'
-  // unrolled passes (hoisting it there spills far more). That costs little for
-  // the one-input family on float (5.2-5.7 TB/s on a transposed 8192^2 input)
-  // but the half variant (8 elements a pack) ran at 1.5 TB/s and the two-input
-  // family spilled 400 bytes a lane: those stay off the tiled kernels, and the
-  // front end brings a transposed input into the output's order first.
+bool apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
+                          float w, bool decline) {
+  // The one-input family on float keeps its code switch inside the specialised tiled kernel's
+  // unrolled passes (5.2-5.7 TB/s on a transposed 8192^2 input). On half that form ran at 1.5 TB/s
+  // and the two-input family spilled 400 bytes a lane: those take the general LDS-tile kernel,
+  // whose rolled compute loop decodes the code once per tile.
   if (op == PointOp::Math1) {
     if constexpr (GROUP == 0)
-      run_plan<T, OpMath1, T, std::is_same<T, float>::value>(s, pl, sameShape, OpMath1{v, w, (int)fn});
-    return;
+      return run_plan<T, OpMath1, T, std::is_same<T, float>::value>(s, pl, sameShape, OpMath1{v, w, (int)fn}, decline);
+    return true;
   }
   if (op == PointOp::Math2) {
-    if constexpr (GROUP == 1) run_plan<T, OpMath2, T, false>(s, pl, sameShape, OpMath2{(int)fn});
-    return;
+    if constexpr (GROUP == 1) return run_plan<T, OpMath2, T, false>(s, pl, sameShape, OpMath2{(int)fn}, decline);
+    return true;
   }
   switch (op) {
 #define THC_CASE(G, NAME)                                         \
@@ -1579,6 +1590,7 @@ void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, flo
 #undef THC_CASE
     default: raise_error("pointwise op not available for this element type");
   }
+  return true;
 }
 
 template <typename T>

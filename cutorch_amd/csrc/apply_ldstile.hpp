@@ -1,0 +1,340 @@
+// The LDS-tile kernel of the apply engine for every functor and element-type
+// pair (included by apply_impl.hpp).
+//
+// lib/THC/THCApply.cuh:426-640 runs every op of every type through one
+// strided kernel. Here the specialised tiled kernels of apply_impl.hpp keep
+// their direct operands in registers and are instantiated per staging mask,
+// which is affordable for the plain arithmetic of the hot path only. This
+// kernel is the general form for a transposed operand: EVERY input of a
+// TP x TQ tile goes through LDS (inputs whose unit-stride dim is p are
+// written transposed, the others as they are), so that
+//   * the loads of a tile are issued as one batch into registers and, the
+//     kernel being persistent, the NEXT tile's batch is in flight while the
+//     current tile is computed out of LDS;
+//   * the compute loop is rolled and reads LDS only, so a code-dispatched
+//     functor is decoded once per tile around that loop (one copy of every
+//     function per kernel instead of one per unrolled element);
+//   * which inputs are transposed is a run-time flag (no instantiation per
+//     staging mask), the index type is 64-bit for tile origins only, and the
+//     input and output element types may differ (comparisons, conversions).
+// Rows that are not whole aligned packs (odd sizes, views at odd offsets) take
+// the same kernel with ALIGNED = false: every global access is still an aligned
+// pack covering a window that starts at or below the row piece's first
+// element; the element-wise LDS accesses absorb each operand's own shift.
+#pragma once
+
+namespace thc {
+
+struct LdsTileArgs {
+  int staged[kMaxOps];   // input k is read along p and transposed on its way into LDS
+  uint32_t sizeP, sizeQ;
+  int64_t strideP[kMaxOps];  // elements
+  int64_t strideQ[kMaxOps];
+  int nbatch;            // remaining joint dims
+  Divisor<uint32_t> bsize[kMaxDims];
+  int64_t bstride[kMaxOps][kMaxDims];
+  Divisor<uint32_t> tilesP, tilesQ;
+  uint32_t totalTiles;
+  uint32_t xcdPer;   // tiles per XCD when workgroup slot b takes tile (b % 8) * xcdPer + b / 8; 0 = identity
+  uint32_t groupP;   // tiles are walked in bands of groupP tiles along p (p fastest inside a band); 1 = q fastest
+  uint32_t ntStore;  // whole packs of the output go out with the streaming hint
+};
+
+// Geometry shared by the kernel and the host (LDS bytes, tile extents).
+template <typename T, typename TOut, int LXP, int LXQ, bool ALIGNED>
+struct LdsTileShape {
+  static constexpr int W = sizeof(T) > sizeof(TOut) ? sizeof(T) : sizeof(TOut);
+  static constexpr int VEC = 16 / W;
+  static constexpr int WP = LXP * VEC, WQ = LXQ * VEC;  // window: lanes x pack
+  static constexpr int TP = ALIGNED ? WP : WP - VEC, TQ = ALIGNED ? WQ : WQ - VEC;
+  static constexpr int ROWS_P = kBlock / LXP, ROWS_Q = kBlock / LXQ;
+  static constexpr int NP_S = (TQ + ROWS_P - 1) / ROWS_P;  // packs per lane, lanes along p
+  static constexpr int NP_D = (TP + ROWS_Q - 1) / ROWS_Q;  // packs per lane, lanes along q
+  static constexpr int NP = NP_S > NP_D ? NP_S : NP_D;
+  static constexpr int PITCH_S = TP | 1;  // transposed slab [TQ][PITCH_S]: odd pitch spreads the banks
+  static constexpr int PITCH_D = WQ;      // plain slab [TP][PITCH_D]: whole windows, 16-byte accesses
+  static constexpr int SLAB_RAW = TQ * PITCH_S > TP * PITCH_D ? TQ * PITCH_S : TP * PITCH_D;
+  static constexpr int SLAB = (SLAB_RAW + VEC - 1) / VEC * VEC;  // elements of T per input
+  static constexpr size_t lds_bytes(int nin) { return (size_t)nin * SLAB * sizeof(T); }
+};
+
+template <typename T, typename TOut, typename Op, int LXP, int LXQ, bool ALIGNED>
+__global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const T* in0, const T* in1,
+                                                               const T* in2, LdsTileArgs args, Op op) {
+  using S = LdsTileShape<T, TOut, LXP, LXQ, ALIGNED>;
+  constexpr int NIN = Op::NIN;
+  constexpr int VEC = S::VEC, TP = S::TP, TQ = S::TQ, ROWS_P = S::ROWS_P, ROWS_Q = S::ROWS_Q;
+  constexpr int NP = S::NP, NP_S = S::NP_S, NP_D = S::NP_D, PITCH_S = S::PITCH_S, PITCH_D = S::PITCH_D;
+  static_assert(NIN >= 1 && NIN <= 3, "one to three inputs");
+  using PIN = Pack<T, VEC>;
+  using POUT = Pack<TOut, VEC>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  const T* ptr[3] = {in0, in1, in2};
+  const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
+  const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  auto mis_in = [](const T* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(T)) & (uintptr_t)(VEC - 1)); };
+  auto mis_out = [](const TOut* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(TOut)) & (uintptr_t)(VEC - 1)); };
+
+  struct Tile {       // uniform over the workgroup
+    const T* tb[3];   // tile origin of input k
+    TOut* ob;         // tile origin of the output
+    int pn, qn;       // valid extent
+  };
+  const uint32_t slots = args.xcdPer ? args.xcdPer * 8 : args.totalTiles;
+  // First valid tile at or after slot b (b advances by the grid size); false when none is left.
+  auto locate = [&](uint32_t& b, Tile& t) -> bool {
+    uint32_t tile = 0;
+    for (;; b += gridDim.x) {
+      if (b >= slots) return false;
+      tile = args.xcdPer ? (b % 8) * args.xcdPer + b / 8 : b;
+      if (tile < args.totalTiles) break;
+    }
+    uint32_t rest, tq, tp;
+    if (args.groupP > 1) {
+      const uint32_t perBatch = args.tilesP.d * args.tilesQ.d;
+      rest = tile / perBatch;
+      const uint32_t tt = tile - rest * perBatch;
+      const uint32_t band = tt / (args.groupP * args.tilesQ.d);
+      const uint32_t r = tt - band * (args.groupP * args.tilesQ.d);
+      const uint32_t gp = min(args.groupP, args.tilesP.d - band * args.groupP);  // ragged last band
+      tq = r / gp;
+      tp = band * args.groupP + (r - tq * gp);
+    } else {
+      args.tilesQ.divmod(tile, rest, tq);
+      args.tilesP.divmod(rest, rest, tp);
+    }
+    int64_t base[kMaxOps] = {0, 0, 0, 0};
+    for (int j = 0; j < args.nbatch; ++j) {
+      uint32_t r;
+      args.bsize[j].divmod(rest, rest, r);
+#pragma unroll
+      for (int k = 0; k <= NIN; ++k) base[k] += (int64_t)r * args.bstride[k][j];
+    }
+    const uint32_t p0 = tp * TP, q0 = tq * TQ;
+    t.pn = (int)min((uint32_t)TP, args.sizeP - p0);
+    t.qn = (int)min((uint32_t)TQ, args.sizeQ - q0);
+    t.ob = out + (base[0] + (int64_t)p0 * args.strideP[0] + (int64_t)q0 * args.strideQ[0]);
+#pragma unroll
+    for (int k = 0; k < NIN; ++k)
+      t.tb[k] = ptr[k] + (base[k + 1] + (int64_t)p0 * args.strideP[k + 1] + (int64_t)q0 * args.strideQ[k + 1]);
+    return true;
+  };
+
+  // Requests every pack of the tile's inputs. No load carries a predicate: lanes past the
+  // tile's valid extent re-read a pack inside it, so a later wait covers exactly these loads.
+  auto issue = [&](const Tile& t, PIN (&v)[NIN][NP]) {
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) {
+      if (args.staged[k + 1]) {
+        const uint32_t sq = (uint32_t)args.strideQ[k + 1];
+#pragma unroll
+        for (int r = 0; r < NP_S; ++r) {
+          const int qi = min((int)lyp + r * ROWS_P, t.qn - 1);
+          const T* row = t.tb[k] + (uint32_t)qi * sq;
+          int first = (int)(lxp * VEC) - (ALIGNED ? 0 : mis_in(row));
+          if (first >= t.pn) first = ALIGNED ? 0 : -mis_in(row);
+          v[k][r] = load_pack<true>(reinterpret_cast<const PIN*>(row + first));
+        }
+      } else {
+        const uint32_t sp = (uint32_t)args.strideP[k + 1];
+#pragma unroll
+        for (int r = 0; r < NP_D; ++r) {
+          const int pi = min((int)lyq + r * ROWS_Q, t.pn - 1);
+          const T* row = t.tb[k] + (uint32_t)pi * sp;
+          int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_in(row));
+          if (first >= t.qn) first = ALIGNED ? 0 : -mis_in(row);
+          v[k][r] = load_pack<true>(reinterpret_cast<const PIN*>(row + first));
+        }
+      }
+    }
+  };
+
+  // Registers -> LDS. Transposed inputs land element by element at [q][p]; the others keep
+  // their window (pack j of row p at column j * VEC, the row's own shift included).
+  auto commit = [&](const Tile& t, const PIN (&v)[NIN][NP]) {
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) {
+      T* slab = lds + k * S::SLAB;
+      if (args.staged[k + 1]) {
+        const uint32_t sq = (uint32_t)args.strideQ[k + 1];
+#pragma unroll
+        for (int r = 0; r < NP_S; ++r) {
+          const int qi = (int)lyp + r * ROWS_P;
+          int first = (int)(lxp * VEC);
+          if (!ALIGNED) first -= mis_in(t.tb[k] + (uint32_t)min(qi, t.qn - 1) * sq);
+          if (ALIGNED || qi < TQ) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const int pi = first + e;
+              if (ALIGNED || (pi >= 0 && pi < TP)) slab[qi * PITCH_S + pi] = v[k][r].v[e];
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < NP_D; ++r) {
+          const int pi = (int)lyq + r * ROWS_Q;
+          if (ALIGNED || pi < TP) *reinterpret_cast<PIN*>(slab + pi * PITCH_D + lxq * VEC) = v[k][r];
+        }
+      }
+    }
+  };
+
+  // LDS -> functor -> global, lanes along q. Rolled: the functor's code is fixed outside.
+  auto compute = [&](const Tile& t) {
+    with_fixed_code(op, [&](auto f) {
+#pragma unroll 2
+      for (int r = 0; r < NP_D; ++r) {
+        const int pi = (int)lyq + r * ROWS_Q;
+        const int pic = ALIGNED ? pi : min(pi, min(t.pn, TP) - 1);
+        TOut* orow = t.ob + (uint32_t)pic * (uint32_t)args.strideP[0];
+        const int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_out(orow));
+        PIN in[3] = {};
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) {
+          const T* slab = lds + k * S::SLAB;
+          if (args.staged[k + 1]) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              const int j = ALIGNED ? first + e : min(max(first + e, 0), TQ - 1);
+              in[k].v[e] = slab[j * PITCH_S + pic];
+            }
+          } else if (ALIGNED) {
+            in[k] = *reinterpret_cast<const PIN*>(slab + pic * PITCH_D + first);
+          } else {
+            const int m = mis_in(t.tb[k] + (uint32_t)pic * (uint32_t)args.strideP[k + 1]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) in[k].v[e] = slab[pic * PITCH_D + min(max(first + e, 0), TQ - 1) + m];
+          }
+        }
+        POUT res;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) res.v[e] = f(in[0].v[e], in[1].v[e], in[2].v[e]);
+        if (pi < t.pn && first < t.qn) {
+          if (ALIGNED || (first >= 0 && first + VEC <= t.qn)) {
+            if (args.ntStore) store_pack<true>(reinterpret_cast<POUT*>(orow + first), res);
+            else store_pack<false>(reinterpret_cast<POUT*>(orow + first), res);
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+              if (first + e >= 0 && first + e < t.qn) orow[first + e] = res.v[e];
+          }
+        }
+      }
+    });
+  };
+
+  uint32_t b = blockIdx.x;
+  Tile cur, nxt;
+  PIN v[NIN][NP];
+  bool have = locate(b, cur);
+  if (have) issue(cur, v);
+  while (have) {
+    commit(cur, v);
+    lds_barrier();
+    b += gridDim.x;
+    const bool more = locate(b, nxt);
+    if (more) issue(nxt, v);  // in flight while this tile is computed
+    compute(cur);
+    lds_barrier();            // the slabs are rewritten for the next tile
+    cur = nxt;
+    have = more;
+  }
+}
+
+// Plans and launches the LDS-tile kernel; false (nothing launched) when the plan has no
+// transposed operand or does not fit (no unit stride along an operand's fast dim, negative
+// strides, a tile that spans 2^31 elements, more than 2^32 tiles).
+template <typename T, typename Op, typename TOut>
+bool launch_ldstile(THCState* s, const Plan& pl, Op op) {
+  if constexpr (Op::NIN < 1 || Op::NIN > 3) {
+    return false;
+  } else {
+    int p, q, staged[kMaxOps] = {0, 0, 0, 0};
+    if (!tuning("apply.ldstile.enable", 1) || !tile_plan(pl, p, q, staged)) return false;
+    constexpr int W = sizeof(T) > sizeof(TOut) ? sizeof(T) : sizeof(TOut);
+    constexpr int VEC = 16 / W;
+    // 512-byte rows (of the wider type) along q; along p 128 bytes of the input type at least
+    // (64 bytes for 1-byte elements, whose 128 x 512 tile would take 66 KiB of LDS per input)
+    constexpr int LXQ = 32;
+    constexpr int LXP = (sizeof(T) == 1 && VEC == 16) ? 4 : ((128 / (int)sizeof(T)) / VEC < 8 ? 8 : (128 / (int)sizeof(T)) / VEC);
+    const int nd = pl.lay[0].dims;
+    auto elem_size = [](int k) { return k == 0 ? sizeof(TOut) : sizeof(T); };
+    bool aligned = pl.lay[0].size[p] % VEC == 0 && pl.lay[0].size[q] % VEC == 0;
+    for (int k = 0; k < pl.nops; ++k) {
+      const int fast = staged[k] ? p : q;
+      if (pl.lay[k].stride[fast] != 1) return false;
+      if (reinterpret_cast<uintptr_t>(pl.ptr[k]) % elem_size(k) != 0) return false;
+      aligned = aligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % (VEC * elem_size(k)) == 0;
+      for (int d = 0; d < nd; ++d) {
+        if (pl.lay[k].stride[d] < 0) return false;
+        if (d != fast) aligned = aligned && pl.lay[k].stride[d] % VEC == 0;
+      }
+      // lane offsets inside a tile are 32-bit
+      const int64_t span = (int64_t)(LXQ * VEC) * std::max(pl.lay[k].stride[p], pl.lay[k].stride[q]) + 4096;
+      if (span >= (int64_t(1) << 31)) return false;
+    }
+    LdsTileArgs args{};
+    for (int k = 0; k < pl.nops; ++k) {
+      args.staged[k] = staged[k];
+      args.strideP[k] = pl.lay[k].stride[p];
+      args.strideQ[k] = pl.lay[k].stride[q];
+    }
+    if (pl.lay[0].size[p] >= kIndex32Limit || pl.lay[0].size[q] >= kIndex32Limit) return false;
+    args.sizeP = (uint32_t)pl.lay[0].size[p];
+    args.sizeQ = (uint32_t)pl.lay[0].size[q];
+    int64_t batch = 1;
+    for (int d = nd - 1; d >= 0; --d) {
+      if (d == p || d == q) continue;
+      args.bsize[args.nbatch].set((uint64_t)pl.lay[0].size[d]);
+      for (int k = 0; k < pl.nops; ++k) args.bstride[k][args.nbatch] = pl.lay[k].stride[d];
+      ++args.nbatch;
+      batch *= pl.lay[0].size[d];
+    }
+    using SA = LdsTileShape<T, TOut, LXP, LXQ, true>;
+    using SU = LdsTileShape<T, TOut, LXP, LXQ, false>;
+    const int64_t tileP = aligned ? SA::TP : SU::TP, tileQ = aligned ? SA::TQ : SU::TQ;
+    const int64_t tp = (args.sizeP + tileP - 1) / tileP, tq = (args.sizeQ + tileQ - 1) / tileQ;
+    args.tilesP.set((uint64_t)tp);
+    args.tilesQ.set((uint64_t)tq);
+    const int64_t total = batch * tp * tq;
+    if (total >= (int64_t(1) << 31)) return false;
+    args.totalTiles = (uint32_t)total;
+    const int64_t ntKnob = tuning("apply.tiled.nt_store", -1);
+    args.ntStore = (ntKnob >= 0 ? ntKnob != 0 : pl.numel * (int64_t)sizeof(TOut) >= (int64_t(64) << 20)) ? 1u : 0u;
+    // single-input ops: bands along p (their only read stream is the transposed one); unaligned rows: bands
+    // keep the lines that p-neighbours share in L2, and an XCD gets a contiguous range of tiles
+    int64_t band = tuning("apply.ldstile.group_p", -1);
+    if (band < 0) band = Op::NIN == 1 ? 16 : (aligned ? 1 : 8);
+    args.groupP = (uint32_t)std::max<int64_t>(1, band);
+    if ((int64_t)args.groupP * 2 > tp) args.groupP = 1;
+    if (!aligned && tuning("apply.ldstile.xcd_swizzle", 1) && total >= 64 && total < (int64_t(1) << 28))
+      args.xcdPer = (uint32_t)((total + 7) / 8);
+    const size_t ldsBytes = aligned ? SA::lds_bytes(Op::NIN) : SU::lds_bytes(Op::NIN);
+    if (ldsBytes > 160 * 1024) return false;
+    // persistent grid: as many workgroups as the LDS admits per CU (160 KiB), capped by registers at 8
+    const int64_t perCu = std::max<int64_t>(1, std::min<int64_t>(tuning("apply.ldstile.max_per_cu", 8),
+                                                                 (int64_t)(160 * 1024) / (int64_t)ldsBytes));
+    const int64_t slots = args.xcdPer ? (int64_t)args.xcdPer * 8 : total;
+    int64_t gridCap = tuning("apply.ldstile.max_grid", -1);
+    if (gridCap <= 0) gridCap = perCu * num_compute_units(s);
+    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(slots, gridCap));
+    hipStream_t st = current_stream(s);
+    TOut* o = (TOut*)pl.ptr[0];
+    const T* i0 = (const T*)pl.ptr[1];
+    const T* i1 = (const T*)pl.ptr[2];
+    const T* i2 = (const T*)pl.ptr[3];
+    if (aligned)
+      hipLaunchKernelGGL((apply_ldstile_kernel<T, TOut, Op, LXP, LXQ, true>), dim3(grid), dim3(kBlock), ldsBytes, st,
+                         o, i0, i1, i2, args, op);
+    else
+      hipLaunchKernelGGL((apply_ldstile_kernel<T, TOut, Op, LXP, LXQ, false>), dim3(grid), dim3(kBlock), ldsBytes, st,
+                         o, i0, i1, i2, args, op);
+    note_kernel(aligned ? "lds-tile" : "lds-tile-shift");
+    return true;
+  }
+}
+
+}  // namespace thc

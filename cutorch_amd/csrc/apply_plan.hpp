@@ -20,17 +20,25 @@ inline int op_group(PointOp op) {
 }
 
 // Defined (explicitly instantiated) in the slices.
+// false = declined: `decline` was set and a transposed operand would have been read uncoalesced
+// (the caller brings it into the output's order first and calls again with decline = false)
 template <typename T, int GROUP>
-void apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
-                          float w);
+bool apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, float v, MathFn fn,
+                          float w, bool decline);
 template <typename T>
 void apply_copy(THCState* s, Plan& pl, bool sameShape);
 // Code-dispatched functors for the element types without dedicated slices
 // (apply_w_*.hip) and the comparison ops of every type.
 template <typename T>
-void apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d);
+bool apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool decline);
 // false = declined (see apply_wide.hpp): the caller densifies and calls again with decline = false
 template <typename T>
 bool apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool decline);
+
+// out = (D)in0 through the apply engine: strided and transposed operands of a type-converting
+// copy in one pass (lib/THC/THCTensorCopy.cu:26-122 converts inside its apply2, CopyOp<Dst, Src>).
+// Defined in the apply_cvt_*.hip slices, one per source type.
+template <typename D, typename S>
+void apply_convert(THCState* s, Plan& pl, bool sameShape);
 
 }  // namespace thc

@@ -2,6 +2,6 @@
 #include "apply_wide.hpp"
 
 namespace thc {
-template void apply_wide<uint8_t>(THCState*, Plan&, bool, const ApplyDesc&);
+template bool apply_wide<uint8_t>(THCState*, Plan&, bool, const ApplyDesc&, bool);
 template bool apply_cmp<uint8_t>(THCState*, Plan&, bool, const ApplyDesc&, bool);
 }

@@ -391,14 +391,14 @@ bool apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool d
 
 // Every arithmetic op of an element type that has no dedicated slices.
 template <typename T>
-void apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d) {
+bool apply_wide(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool decline) {
   using C = typename Num<T>::C;
   const C v = Num<T>::scalar(d.v), w = Num<T>::scalar(d.w);
   switch (point_op_inputs(d.op)) {
-    case 0: run_plan<T, WideOp<T, 0>, T, false, true>(s, pl, sameShape, WideOp<T, 0>{(int)d.op, d.fn, v, w}); break;
-    case 1: run_plan<T, WideOp<T, 1>, T, false, true>(s, pl, sameShape, WideOp<T, 1>{(int)d.op, d.fn, v, w}); break;
-    case 2: run_plan<T, WideOp<T, 2>, T, false, true>(s, pl, sameShape, WideOp<T, 2>{(int)d.op, d.fn, v, w}); break;
-    default: run_plan<T, WideOp<T, 3>, T, false, true>(s, pl, sameShape, WideOp<T, 3>{(int)d.op, d.fn, v, w}); break;
+    case 0: return run_plan<T, WideOp<T, 0>, T, false, true>(s, pl, sameShape, WideOp<T, 0>{(int)d.op, d.fn, v, w}, decline);
+    case 1: return run_plan<T, WideOp<T, 1>, T, false, true>(s, pl, sameShape, WideOp<T, 1>{(int)d.op, d.fn, v, w}, decline);
+    case 2: return run_plan<T, WideOp<T, 2>, T, false, true>(s, pl, sameShape, WideOp<T, 2>{(int)d.op, d.fn, v, w}, decline);
+    default: return run_plan<T, WideOp<T, 3>, T, false, true>(s, pl, sameShape, WideOp<T, 3>{(int)d.op, d.fn, v, w}, decline);
   }
 }
 

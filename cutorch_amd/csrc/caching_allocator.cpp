@@ -33,6 +33,9 @@ struct HipBackend {
     }
     return true;  // completed (or unusable: nothing more to wait for)
   }
+  static void event_wait(Event ev) {
+    if (hipEventSynchronize(ev) != hipSuccess) (void)hipGetLastError();
+  }
   static void event_destroy(Event ev) { (void)hipEventDestroy(ev); }
   static void stream_wait(Stream s) { (void)hipStreamSynchronize(s); }
 };

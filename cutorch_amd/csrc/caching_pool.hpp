@@ -15,7 +15,9 @@
 //     allocation are merged back, so a large block that was nibbled at comes
 //     back whole;
 //   - when the driver is out of memory every fully free driver allocation is
-//     released and the request retried.
+//     released and the request retried; if that fails too, the blocks still
+//     held back behind events are waited for and released before the last
+//     attempt. A failed request leaves no error state behind in the backend.
 // Sizes: requests up to 1 MiB are rounded to 512 B and carved out of 2 MiB
 // segments; larger ones are rounded to 128 KiB and allocated on their own, and
 // a parked large block is split only when at least 1 MiB would remain.
@@ -71,7 +73,19 @@ class CachingPool {
         Backend::clear_error();
         release_free_segments();
         err = Backend::dev_malloc(&p, seg);
-        if (err != 0) return err;
+        if (err != 0 && !pending_.empty()) {
+          // blocks still held back behind events: wait for them, release what that frees, try again
+          Backend::clear_error();
+          for (Block* pb : pending_)
+            for (Event ev : pb->events) Backend::event_wait(ev);
+          process_pending();
+          release_free_segments();
+          err = Backend::dev_malloc(&p, seg);
+        }
+        if (err != 0) {
+          Backend::clear_error();  // the failure is reported through the return value only
+          return err;
+        }
       }
       b = new Block{(char*)p, seg, stream, nullptr, nullptr, false, false, small, {}, {}};
       blocks_[b->ptr] = b;

@@ -273,7 +273,8 @@ void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor
 // SqDevOut: sum of (x - c)^2 where c is what the output element holds on entry (the slice's
 //           mean: second sweep of var/std along a dim, THCTensorMathReduce.cuh:268-445)
 // All / Any: logical and / or of a Byte tensor (THCTensorMathReduce.cuh:118-130)
-enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev, SqDevOut, All, Any };
+// NotEqual: number-like indicator of a != b over two dense operands (reduce_all_diff only)
+enum class ReduceOp : int { Sum, Prod, Min, Max, Norm0, Norm1, Norm2, NormP, SqDev, SqDevOut, All, Any, NotEqual };
 // DivBy / DivBySqrt take their divisor from the `p` argument of reduce_dim.
 enum class Epilogue : int { None, Sqrt, PowInv, DivN, DivBy, DivBySqrt };
 
@@ -298,7 +299,8 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, float p, AnyTensor* in, floa
 bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Scalar* result);
 // The same reduction over a - b without materialising the difference. Only
 // for dense operands of a floating type; returns false when it does not apply
-// (the caller then subtracts into a temporary).
+// (the caller then subtracts into a temporary). ReduceOp::NotEqual (any element
+// type) yields a non-zero result iff some a[i] != b[i] (NaN differs from NaN).
 // renorm along dim 0 when src and out are contiguous and a slice fits the
 // staging buffer: one read, one write; false otherwise.
 bool renorm_rows(THCState* s, DType dt, AnyTensor* out, AnyTensor* src, double p, double maxnorm);

@@ -2,34 +2,23 @@
 //
 // Role of THC_copyTensor with differing source and destination types
 // (lib/THC/THCTensorCopy.cu:24-205, the copyCuda<Type> entries of
-// generic/THCTensorCopy.h:16-24). The conversion itself is a flat streaming
-// kernel over dense operands; strided operands are densified or scattered by
-// the same-type copy of the apply engine (which owns the transposing kernels),
-// so a strided conversion costs up to two extra passes instead of 64 more
-// instantiations of every strided kernel.
+// generic/THCTensorCopy.h:16-24). Dense operands take the flat streaming
+// kernel below; strided and transposed operands convert in one pass inside the
+// apply engine (apply_convert: strided packs, the LDS-tile kernel for
+// transposes), as the reference converts inside its apply2
+// (lib/THC/THCTensorCopy.cu:26-122). Only a destination that addresses an
+// element twice goes through a dense temporary.
 // Values convert as C casts do (float -> integer truncates toward zero), half
 // goes through float.
 #include <type_traits>
 
+#include "apply_plan.hpp"
 #include "common.hpp"
 #include "stream_guard.hpp"
 #include "device_util.hpp"
 
 namespace thc {
 namespace {
-
-template <typename D, typename S>
-__device__ __forceinline__ D convert_value(S x) {
-  if constexpr (std::is_same<S, __half>::value) {
-    const float f = __half2float(x);
-    if constexpr (std::is_same<D, __half>::value) return x;
-    else return (D)f;
-  } else if constexpr (std::is_same<D, __half>::value) {
-    return __float2half_rn((float)x);
-  } else {
-    return (D)x;
-  }
-}
 
 // N consecutive elements per lane as one load and one store; N is chosen so
 // that the wider of the two packs is 16 bytes. U packs per lane are loaded
@@ -105,6 +94,24 @@ void convert_copy(THCState* s, DType dstT, AnyTensor* dst, DType srcT, AnyTensor
   THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
   if (n == 0) return;
   note_stream_use(s, {dst, src});
+  if (!(tensor_is_contiguous(dst) && tensor_is_contiguous(src)) && !overlapping(tensor_layout(dst)) &&
+      tuning("convert.one_pass", 1)) {
+    Plan pl{};
+    pl.nops = 2;
+    pl.numel = n;
+    pl.ptr[0] = tensor_data(dst, dstT);
+    pl.ptr[1] = tensor_data(src, srcT);
+    pl.lay[0] = tensor_layout(dst);
+    pl.lay[1] = tensor_layout(src);
+    if (!pl.ptr[0] || !pl.ptr[1]) raise_error("converting copy on a tensor without storage");
+    bool sameShape = pl.lay[0].dims == pl.lay[1].dims;
+    for (int d = 0; sameShape && d < pl.lay[0].dims; ++d) sameShape = pl.lay[0].size[d] == pl.lay[1].size[d];
+    with_type(dstT, [&](auto dtag) {
+      with_type(srcT, [&](auto stag) { apply_convert<decltype(dtag), decltype(stag)>(s, pl, sameShape); });
+    });
+    THC_CHECK(hipGetLastError());
+    return;
+  }
   // The flat kernel pairs elements by logical linear index, which is what a
   // dense tensor's memory order is.
   TensorRef cs(s, tensor_new_contiguous(s, src, srcT));

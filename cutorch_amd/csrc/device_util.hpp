@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 namespace thc {
 
@@ -118,6 +119,20 @@ struct Cvt<__half> {
   static __device__ __forceinline__ float up(__half x) { return __half2float(x); }
   static __device__ __forceinline__ __half down(float x) { return __float2half_rn(x); }
 };
+
+// (D)x with C's conversion rules (float -> integer truncates toward zero); half goes through float.
+template <typename D, typename S>
+__device__ __forceinline__ D convert_value(S x) {
+  if constexpr (std::is_same<S, __half>::value) {
+    const float f = __half2float(x);
+    if constexpr (std::is_same<D, __half>::value) return x;
+    else return (D)f;
+  } else if constexpr (std::is_same<D, __half>::value) {
+    return __float2half_rn((float)x);
+  } else {
+    return (D)x;
+  }
+}
 
 // Division by a launch-invariant divisor.
 // 32-bit: round-up multiply-shift (Granlund & Montgomery, "Division by

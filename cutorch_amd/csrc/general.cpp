@@ -123,8 +123,9 @@ const StreamScratch& stream_scratch(THCState* s) {
   // Arrival counters start at zero and every kernel that uses one resets it.
   THC_CHECK(hipMemsetAsync(sc.counters, 0, kScratchTailBytes, st));
   THC_CHECK(hipStreamSynchronize(st));
-  // One pinned, device-mapped slot: *all reductions store their scalar there.
-  THC_CHECK(hipHostMalloc(reinterpret_cast<void**>(&sc.hostResult), 256, hipHostMallocMapped));
+  // One pinned, device-mapped slot: *all reductions store their scalar there. Coherent (fine-grained),
+  // so that a store by a running kernel becomes visible to the host, which polls the slot.
+  THC_CHECK(hipHostMalloc(reinterpret_cast<void**>(&sc.hostResult), 256, hipHostMallocMapped | hipHostMallocCoherent));
   void* dv = nullptr;
   THC_CHECK(hipHostGetDevicePointer(&dv, sc.hostResult, 0));
   sc.hostResultDev = static_cast<float*>(dv);

@@ -114,6 +114,9 @@ int tensors_equal(THCState* s, DType dt, AnyTensor* a, AnyTensor* b) {
   for (int d = 0; d < a->nDimension; ++d)
     if (a->size[d] != b->size[d]) return 0;
   if (a->nDimension == 0) return 1;
+  // dense operands: one fused two-input reduction, 2 reads per element and no temporary
+  Scalar differ{0.0, 0};
+  if (reduce_all_diff(s, dt, ReduceOp::NotEqual, 0.0, a, b, &differ)) return differ.f == 0.0 && differ.i == 0;
   TensorRef flags(s, tensor_new_with_size(s, a->nDimension, a->size, dt));
   if (!pointwise_apply(s, dt, PointOp::Math2, 0.f, flags.t, a, b, nullptr, false, MathFn::Equal))
     raise_arg_error(2, "%s", kDimWarning);

@@ -18,6 +18,7 @@
 #include <mutex>
 
 #include "reduce_impl.hpp"
+#include "stream_guard.hpp"
 
 namespace thc {
 
@@ -67,6 +68,10 @@ void sumall_no_alloc(THCState* s, AnyTensor* self, float* result) {
                 "sumallNoAlloc: %lld elements exceed the limit of %lld that the fixed partials "
                 "array serves",
                 (long long)n, (long long)kNoAllocMaxElements);
+  // the input may be a caching-allocator block of another stream: it must not be handed out
+  // again before these launches have read it (one relaxed load when only one stream is in use;
+  // no device memory is allocated)
+  note_stream_use(s, {self});
   float* part = scratch_for_current_device();
   const float* src = (const float*)tensor_data(self, DType::F32);
   using F = FSum<float>;

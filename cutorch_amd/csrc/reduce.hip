@@ -208,7 +208,7 @@ bool reduce_all(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* in, Sca
 
 bool reduce_all_diff(THCState* s, DType dt, ReduceOp op, double p, AnyTensor* a, AnyTensor* b,
                      Scalar* result) {
-  if (!dtype_is_float(dt) || a->nDimension == 0 || a->nDimension > kMaxDims) return false;
+  if ((!dtype_is_float(dt) && op != ReduceOp::NotEqual) || a->nDimension == 0 || a->nDimension > kMaxDims) return false;
   if (!tensor_is_contiguous(a) || !tensor_is_contiguous(b)) return false;
   const int64_t n = tensor_numel(a);
   if (n != tensor_numel(b)) return false;

@@ -206,6 +206,27 @@ THC_REDUCE_FUNCTOR(FSqDevOut, true, (A)0, (x - c) * (x - c), a + b)
 THC_REDUCE_FUNCTOR(FAll, false, (A)1, (x != (A)0 ? (A)1 : (A)0), (A)((a != (A)0) && (b != (A)0)))
 THC_REDUCE_FUNCTOR(FAny, false, (A)0, (x != (A)0 ? (A)1 : (A)0), (A)((a != (A)0) || (b != (A)0)))
 #undef THC_REDUCE_FUNCTOR
+// Two-operand functors of reduce_all_diff_kernel: pair(a, b) is the term of one element pair.
+// Without it the term is modify(a - b).
+template <typename A_>
+struct FNotEqual {   // 1 if any pair differs (equal: generic/THCTensorMathPairwise.cu:235-258)
+  using A = A_;
+  static constexpr bool kCentred = false;
+  A p;
+  __host__ __device__ __forceinline__ A init() const { return (A)0; }
+  __device__ __forceinline__ A modify(A x, A) const { return x; }
+  __device__ __forceinline__ A pair(A a, A b) const { return a == b ? (A)0 : (A)1; }
+  __device__ __forceinline__ A combine(A a, A b) const { return a > b ? a : b; }
+};
+template <typename F, typename = void>
+struct HasPair : std::false_type {};
+template <typename F>
+struct HasPair<F, std::void_t<decltype(std::declval<const F&>().pair(typename F::A{}, typename F::A{}))>> : std::true_type {};
+template <typename F>
+__device__ __forceinline__ typename F::A pair_term(const F& f, typename F::A a, typename F::A b) {
+  if constexpr (HasPair<F>::value) return f.pair(a, b);
+  else return f.modify(a - b, (typename F::A)0);
+}
 
 // (value, index) pairs. `better(a, b)`: a must replace b.
 template <bool IS_MAX, typename V>
@@ -1774,8 +1795,7 @@ __global__ __launch_bounds__(kBlock) void reduce_all_diff_kernel(
   constexpr int U = 4;
   constexpr I step = (I)kBlock * VEC;
   if (VEC > 1 && blockIdx.x == gridDim.x - 1 && nv + threadIdx.x < n) {
-    const A x = acc_up<A>(a[nv + threadIdx.x]) - acc_up<A>(b[nv + threadIdx.x]);
-    acc[0] = f.combine(acc[0], f.modify(x, (A)0));
+    acc[0] = f.combine(acc[0], pair_term(f, acc_up<A>(a[nv + threadIdx.x]), acc_up<A>(b[nv + threadIdx.x])));
   }
   I i = begin + threadIdx.x * VEC;
   for (; i + (U - 1) * step < end; i += U * step) {
@@ -1788,20 +1808,15 @@ __global__ __launch_bounds__(kBlock) void reduce_all_diff_kernel(
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const A x = acc_up<A>(va[u].v[e]) - acc_up<A>(vb[u].v[e]);
-        acc[e] = f.combine(acc[e], f.modify(x, (A)0));
-      }
+      for (int e = 0; e < VEC; ++e)
+        acc[e] = f.combine(acc[e], pair_term(f, acc_up<A>(va[u].v[e]), acc_up<A>(vb[u].v[e])));
     }
   }
   for (; i < end; i += step) {
     const P va = load_pack<true>(reinterpret_cast<const P*>(a + i));
     const P vb = load_pack<true>(reinterpret_cast<const P*>(b + i));
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-      const A x = acc_up<A>(va.v[e]) - acc_up<A>(vb.v[e]);
-      acc[e] = f.combine(acc[e], f.modify(x, (A)0));
-    }
+    for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], pair_term(f, acc_up<A>(va.v[e]), acc_up<A>(vb.v[e])));
   }
   A r = acc[0];
 #pragma unroll
@@ -2546,6 +2561,15 @@ inline void arm_host_slot(const StreamScratch& sc) {
   *reinterpret_cast<volatile uint64_t*>(sc.hostResult) = kHostSlotArmed;
   __atomic_thread_fence(__ATOMIC_SEQ_CST);
 }
+inline void cpu_relax() {
+#if defined(__x86_64__) || defined(__i386__)
+  __builtin_ia32_pause();
+#elif defined(__aarch64__)
+  asm volatile("yield" ::: "memory");
+#else
+  asm volatile("" ::: "memory");
+#endif
+}
 template <typename A>
 A wait_host_slot(THCState* s, const StreamScratch& sc) {
   static_assert(sizeof(A) == 4 || sizeof(A) == 8, "accumulator width");
@@ -2558,7 +2582,7 @@ A wait_host_slot(THCState* s, const StreamScratch& sc) {
     timespec t0, t1;
     clock_gettime(CLOCK_MONOTONIC, &t0);
     for (uint32_t n = 0; !(seen = changed()); ++n) {
-      __builtin_ia32_pause();
+      cpu_relax();
       if ((n & 1023u) == 1023u) {
         clock_gettime(CLOCK_MONOTONIC, &t1);
         if ((t1.tv_sec - t0.tv_sec) * 1000000000ll + (t1.tv_nsec - t0.tv_nsec) > 20000000ll) break;
@@ -2771,6 +2795,10 @@ void reduce_all_type(THCState* s, ReduceGeom g, const void* src, const void* src
     case ReduceOp::Prod: reduce_all_with<T>(s, g, src, src2, FProd<A>{p}, false, result); return;
     case ReduceOp::Min: reduce_all_with<T>(s, g, src, src2, FMin<A>{p}, false, result); return;
     case ReduceOp::Max: reduce_all_with<T>(s, g, src, src2, FMax<A>{p}, false, result); return;
+    case ReduceOp::NotEqual:
+      if (src2 == nullptr) break;
+      reduce_all_with<T>(s, g, src, src2, FNotEqual<A>{p}, true, result);
+      return;
     default: break;
   }
   if constexpr (!std::is_integral<A>::value) {

@@ -589,12 +589,18 @@ THC_AMD_DECLARE_MATH_API(THCudaHalfTensor, THHalf, float)
 /* No counterpart in the reference. For callers that cannot allocate device
  * memory: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc. The sum of all elements of `self`, as
- * THCudaTensor_sumall computes it (same launches, same bits), except that
+ * THCudaTensor_sumall computes it (up to 2^31 elements: same launches, same
+ * bits; beyond that more workgroups share the work than sumall uses, so the
+ * order of the partial sums, and with it the last bits of a non-integer sum,
+ * may differ), except that
  *   - `self` must be contiguous (or empty) and hold at most 2^32 elements;
  *     anything else is an argument error and nothing is launched;
  *   - the scalar is written to `*result`, a device-accessible pointer the
  *     caller owns (4 bytes), by the second launch on the current stream; the
- *     call does not wait for the stream and returns nothing;
+ *     call does not wait for the stream and returns nothing. `result` is a raw
+ *     pointer: if it lies in a block of the caching allocator that belongs to
+ *     another stream, the caller reports that use itself
+ *     (THCCachingAllocator_recordStream); `self` is reported by the call;
  *   - no device memory is allocated or freed: the per-workgroup partials go
  *     to a fixed 4 KiB array that every GPU the library runs on holds until
  *     the process ends. All calls on one GPU share that array, so calls that

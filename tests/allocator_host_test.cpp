@@ -31,7 +31,7 @@ struct Fake {
   static std::set<int> done;
 
   static int dev_malloc(void** p, size_t n) {
-    if (liveBytes + n > capacity) return 2;  // "out of memory"
+    if (liveBytes + n > capacity) return stickyError = 2;  // "out of memory"
     bump = (bump + (2u << 20) - 1) & ~uintptr_t((2u << 20) - 1);
     *p = reinterpret_cast<void*>(bump);
     bump += n;
@@ -48,7 +48,10 @@ struct Fake {
     ++frees;
     return 0;
   }
-  static void clear_error() {}
+  static int stickyError;                  // what a failed dev_malloc leaves behind until cleared
+  static void clear_error() { stickyError = 0; }
+  static void event_wait(Event ev) { done.insert(ev); ++eventWaits; }
+  static int eventWaits;
   static int event_record(Event* ev, Stream s) {
     *ev = nextEvent++;
     eventStream[*ev] = s;
@@ -69,6 +72,7 @@ struct Fake {
     mallocs = frees = waits = 0;
   }
 };
+int Fake::stickyError = 0, Fake::eventWaits = 0;
 std::map<char*, size_t> Fake::live;
 size_t Fake::liveBytes = 0, Fake::capacity = size_t(1) << 40;
 int Fake::mallocs = 0, Fake::frees = 0, Fake::nextEvent = 1, Fake::waits = 0;
@@ -242,6 +246,24 @@ static void test_out_of_memory_releases_the_cache() {
     CHECK(b != nullptr && Fake::frees == 1 && Fake::liveBytes == 60 * MiB);
     void* c = nullptr;
     CHECK(pool.malloc(&c, 60 * MiB, 1) != 0 && c == nullptr);   // genuinely out of memory
+    CHECK(Fake::stickyError == 0);               // ... and no error state is left behind for the next device call
+    CHECK(pool.free(b) == 0 && pool.empty_cache() == 0 && Fake::liveBytes == 0);
+  }
+}
+
+static void test_out_of_memory_reclaims_blocks_held_behind_events() {
+  Fake::live.clear();
+  Fake::reset(100 * MiB);
+  {
+    Pool pool;
+    void* a = take(pool, 60 * MiB, 1);
+    pool.record_stream(a, 2);                    // also used on stream 2
+    CHECK(pool.free(a) == 0);
+    CHECK(pool.pending_blocks() == 1);           // held back behind an event on stream 2
+    const int waitsBefore = Fake::eventWaits;
+    void* b = take(pool, 60 * MiB, 3);           // only fits once the held-back block is released
+    CHECK(b != nullptr && Fake::eventWaits > waitsBefore && pool.pending_blocks() == 0);
+    CHECK(Fake::liveBytes == 60 * MiB && Fake::stickyError == 0);
     CHECK(pool.free(b) == 0 && pool.empty_cache() == 0 && Fake::liveBytes == 0);
   }
 }
@@ -299,6 +321,7 @@ int main() {
   test_small_blocks_share_segments();
   test_cross_stream_use_is_guarded();
   test_out_of_memory_releases_the_cache();
+  test_out_of_memory_reclaims_blocks_held_behind_events();
   test_random_traffic_never_overlaps();
   std::puts("ok");
   return 0;

@@ -203,3 +203,38 @@ def test_gpu_half_math(thc, oracle):
             assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= np.spacing(np.abs(want)))
         else:
             assert_bit_equal(got, want, name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double", "byte", "char", "short", "int", "long"])
+def test_gpu_equal_is_one_fused_reduction_on_dense_operands(thc, kind):
+    """equal (generic/THCTensorMathPairwise.cu:235-258): same sizes and every element pair equal under
+    the element type's ==, so NaN differs from NaN, -0 equals +0 and inf equals inf. Dense operands take
+    the fused two-input whole-tensor reduction (no flags temporary); strided ones the two-pass form."""
+    dt = {"float": np.float32, "half": np.float16, "double": np.float64, "byte": np.uint8, "char": np.int8,
+          "short": np.int16, "int": np.int32, "long": np.int64}[kind]
+    rng = np.random.default_rng(95)
+    for n in (1, 5, 4099, (1 << 21) + 77):
+        if kind in ("float", "half", "double"):
+            x = rng.uniform(-4, 4, n).astype(dt)
+        else:
+            info = np.iinfo(dt)
+            x = rng.integers(info.min, info.max, n, dtype=np.int64).astype(dt)
+        a, b = thc.Tensor.from_numpy(x), thc.Tensor.from_numpy(x.copy())
+        assert a.equal(b)
+        assert thc.last_kernel() == "all"
+        for pos in {0, n // 2, n - 1}:
+            y = x.copy()
+            y[pos] = dt(0) if x[pos] != 0 else dt(1)
+            assert not a.equal(thc.Tensor.from_numpy(y)), (kind, n, pos)
+    if kind in ("float", "half", "double"):
+        z = np.array([0.0, 1.0, np.inf, -np.inf, 2.0], dt)
+        assert thc.Tensor.from_numpy(z).equal(thc.Tensor.from_numpy(np.array([-0.0, 1.0, np.inf, -np.inf, 2.0], dt)))
+        w = np.array([0.0, np.nan, 1.0], dt)
+        assert not thc.Tensor.from_numpy(w).equal(thc.Tensor.from_numpy(w.copy()))
+        assert not thc.Tensor.from_numpy(z).equal(thc.Tensor.from_numpy(np.array([0.0, 1.0, -np.inf, np.inf, 2.0], dt)))
+    m = rng.integers(0, 100, (40, 30)).astype(dt)
+    a = thc.Tensor.from_numpy(m)
+    assert not a.equal(thc.Tensor.from_numpy(m.reshape(30, 40)))       # shape mismatch
+    assert a.t().equal(thc.Tensor.from_numpy(np.ascontiguousarray(m.T)))   # strided operand: two passes
+    assert not a.t().equal(thc.Tensor.from_numpy(np.ascontiguousarray(m.T) + dt(1)))

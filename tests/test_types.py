@@ -668,18 +668,18 @@ def test_gpu_renorm_of_dense_rows_is_one_pass(thc, oracle, kind):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["int", "byte", "double"])
-def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
+def test_gpu_transposed_input_of_wider_types_runs_on_lds_tiles(thc, oracle, kind):
     """add / sub / mul / cadd of int, long and double run on plain functors with
-    every kernel of the engine, the LDS-tiled ones included; everything else of
-    the wider types (and all comparisons) has no tiled kernels: a transposed
-    input is brought into the output's order by the (tiled) same-type copy first."""
+    every kernel of the engine, the specialised LDS-tiled ones included; everything
+    else of the wider types (and all comparisons) meets a transposed input in the
+    general LDS-tile kernel: one pass, nothing is densified."""
     rng = np.random.default_rng(111)
     dt = np_of(oracle, kind)
     a = rand_storage(rng, kind, 200 * 136, oracle).reshape(200, 136)
     b = rand_storage(rng, kind, 200 * 136, oracle).reshape(136, 200)
     da, db = thc.Tensor.from_numpy(a), thc.Tensor.from_numpy(b)
     out = thc.Tensor(kind).cadd(da.t(), 1, db)
-    assert thc.last_kernel() == ("contig" if kind == "byte" else "tiled")
+    assert thc.last_kernel() == ("lds-tile-shift" if kind == "byte" else "tiled")   # 200 x 136 bytes: not whole 16-element packs
     ra = oracle.View(a.reshape(-1).copy(), 0, (136, 200), (1, 136))
     want = oracle.typed_pointwise("add", oracle.View.empty((136, 200), dt), ra, oracle.View.of(b))
     assert_bit_equal(out.numpy(), want.numpy())
@@ -689,14 +689,14 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
             out.cmul(da.t(), db)
         else:
             getattr(out, name)(da.t(), value, db)
-        assert thc.last_kernel() == ("contig" if kind == "byte" else "tiled"), (name, thc.last_kernel())
+        assert thc.last_kernel() == ("lds-tile-shift" if kind == "byte" else "tiled"), (name, thc.last_kernel())
         v = -value if name == "csub" else value
         want = oracle.typed_pointwise(op, oracle.View.empty((136, 200), dt), ra, oracle.View.of(b), value=v)
         assert_bit_equal(out.numpy(), want.numpy(), name)
     out = thc.Tensor(kind).cdiv(da.t(), thc.Tensor.from_numpy(np.where(b == 0, 1, b).astype(dt)))
-    assert thc.last_kernel() == ("tiled" if kind == "double" else "contig")   # integer division stays code-dispatched
+    assert thc.last_kernel() == {"double": "tiled", "int": "lds-tile", "byte": "lds-tile-shift"}[kind]   # integer division is code-dispatched
     m = thc.Tensor("byte").compare_tensor("lt", da.t(), db)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == ("lds-tile-shift" if kind == "byte" else "lds-tile")
     wm = oracle.typed_compare("lt", oracle.View.empty((136, 200), np.uint8), ra, oracle.View.of(b))
     assert_bit_equal(m.numpy(), wm.numpy())
     f = thc.Tensor.from_numpy(rng.standard_normal((200, 136)).astype(np.float32))
@@ -715,15 +715,15 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
     finally:
         thc.force_64bit_index(False)
     assert_bit_equal(m.numpy(), (g.numpy() != f.numpy().T).astype(np.uint8))
-    # ... and only that one: shapes whose rows are not whole aligned packs are declined and densified,
-    # as is a comparison whose output has the input's type
+    # ... and only that one: shapes whose rows are not whole aligned packs take the general LDS-tile
+    # kernel, as does a comparison whose output has the input's type
     f2 = thc.Tensor.from_numpy(rng.standard_normal((201, 137)).astype(np.float32))
     g2 = thc.Tensor.from_numpy(rng.standard_normal((137, 201)).astype(np.float32))
     m = thc.Tensor("byte").compare_tensor("le", f2.t(), g2)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile-shift"
     assert_bit_equal(m.numpy(), (f2.numpy().T <= g2.numpy()).astype(np.uint8))
     mt = thc.Tensor("float").compare_tensor("gt", f.t(), g, same_type=True)
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile"
     assert_bit_equal(mt.numpy(), (f.numpy().T > g.numpy()).astype(np.float32))
     # a transposed Byte OUTPUT of a float comparison (its memory order decides): 4-byte output packs along its rows
     mb = thc.Tensor.from_numpy(np.zeros((200, 136), np.uint8))
@@ -732,10 +732,11 @@ def test_gpu_transposed_input_of_wider_types_is_densified(thc, oracle, kind):
 
 
 @pytest.mark.gpu
-def test_gpu_transposed_output_and_math_family_are_densified(thc, oracle):
-    """The same route when it is the output that is transposed (its memory
-    order decides), for a wider type and for the code-dispatched float math,
-    which owns no tiled kernels either; 3-D permutations included."""
+def test_gpu_transposed_output_and_math_family_run_on_lds_tiles(thc, oracle):
+    """The same when it is the output that is transposed (its memory order
+    decides), for a wider type and for the code-dispatched float math; 3-D
+    permutations included. With the general kernel switched off the densify
+    route (same-type copy into the output's order, then the op) still serves."""
     rng = np.random.default_rng(112)
     a = rng.integers(-1000, 1000, (136, 200)).astype(np.int32)
     b = rng.integers(-1000, 1000, (136, 200)).astype(np.int32)
@@ -745,8 +746,17 @@ def test_gpu_transposed_output_and_math_family_are_densified(thc, oracle):
     assert thc.last_kernel().startswith("tiled")     # plain int arithmetic owns tiled kernels
     assert_bit_equal(base.numpy(), (a + 3 * b).T)
     base.t().cdiv(da, thc.Tensor.from_numpy(np.where(b == 0, 1, b).astype(np.int32)))
-    assert thc.last_kernel() == "contig"             # the code-dispatched family does not: densified
-    assert_bit_equal(base.numpy(), (a.astype(np.int64) / np.where(b == 0, 1, b)).astype(np.int64).astype(np.int32).T)
+    assert thc.last_kernel() == "lds-tile"           # the code-dispatched family: the general LDS-tile kernel
+    want_div = (a.astype(np.int64) / np.where(b == 0, 1, b)).astype(np.int64).astype(np.int32).T
+    assert_bit_equal(base.numpy(), want_div)
+    thc.set_tuning("apply.ldstile.enable", 0)
+    try:
+        base.fill(0)
+        base.t().cdiv(da, thc.Tensor.from_numpy(np.where(b == 0, 1, b).astype(np.int32)))
+        assert thc.last_kernel() == "contig"         # densified: copy into the output's order, then a flat op
+    finally:
+        thc.set_tuning("apply.ldstile.enable", 1)
+    assert_bit_equal(base.numpy(), want_div)
 
     x = rng.standard_normal((136, 200)).astype(np.float32)
     y = rng.standard_normal((200, 136)).astype(np.float32)
@@ -757,18 +767,18 @@ def test_gpu_transposed_output_and_math_family_are_densified(thc, oracle):
     want = oracle.pointwise("fn:exp", oracle.View.empty((136, 200)), oracle.View.of(x))
     np.testing.assert_allclose(fbase.numpy().T, want.numpy(), rtol=2e-6)
     out = thc.Tensor("float").binary("cmax", dx, dy.t())
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile"
     assert_bit_equal(out.numpy(), np.maximum(x, y.T))
     fbase.t().binary("cmin", dx, dy.t())   # y is already in the output's order
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile"
     assert_bit_equal(fbase.numpy().T, np.minimum(x, y.T))
     hx = x.astype(np.float16)
     hbase = thc.Tensor.from_numpy(np.zeros((200, 136), np.float16))
     hbase.t().unary("abs", thc.Tensor.from_numpy(hx))
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile"
     assert_bit_equal(hbase.numpy().T, np.abs(hx))
     out = thc.Tensor("half").unary("neg", thc.Tensor.from_numpy(hx).t())
-    assert thc.last_kernel() == "contig"
+    assert thc.last_kernel() == "lds-tile"
     assert_bit_equal(out.numpy(), -hx.T)
 
     z = rng.standard_normal((24, 40, 56)).astype(np.float32)
