@@ -328,7 +328,7 @@ def build_configs(thc, hip, which, only=None):
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
-                      "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
+                      "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G")
           if (only and n in only) or (not only and which == "all")]
     if nx:
@@ -419,7 +419,7 @@ def build_configs(thc, hip, which, only=None):
                 "N-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 fp32", 9 * 8192 * 8192, 8192 * 8192,
                            lambda i: lt_m.compare_tensor("lt", sq_t, db)),
             })
-        if set(nx) & {"N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
+        if set(nx) & {"N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t"}:
             # transposed operands of the op families beyond plain float arithmetic: one-input math on half,
             # narrow integer arithmetic, two-input float math, integer division, integer comparison into Byte,
@@ -439,6 +439,9 @@ def build_configs(thc, hip, which, only=None):
             fo = T("float").resize((m, m))
             hc = T("half").resize((m, m))
             table.update({
+                "N-half-exp": ("out = exp(a), 8192x8192 fp16 contiguous (the flat form of N-half-exp-t)", 4 * m * m, m * m,
+                               lambda i: ho.unary("exp", hc)),
+                "N-half-abs-t": ("out = abs(a:t()), 8192x8192 fp16", 4 * m * m, m * m, lambda i: ho.unary("abs", hx)),
                 "N-half-exp-t": ("out = exp(a:t()), 8192x8192 fp16", 4 * m * m, m * m, lambda i: ho.unary("exp", hx)),
                 "N-half-exp-t-odd": ("out = exp(a:t()), 8191x8193 fp16 (no 16-byte aligned rows)", 4 * nodd_,
                                      nodd_, lambda i: hoo.unary("exp", hxo)),

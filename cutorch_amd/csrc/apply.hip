@@ -194,12 +194,13 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
   THC_ARG_CHECK(n == tensor_numel(src), 2, "sizes do not match");  // THCTensorCopy.cu:29-31
   if (dst->nDimension == 0) return;
   note_stream_use(s, {dst, src});
-  // Dense to dense: the runtime's copy up to 32 MiB; beyond that the engine's own flat stream
+  // Dense to dense: the runtime's copy below 128 MiB; from there on the engine's own flat stream
   // (nontemporal loads, streaming stores) is faster (256 MiB and 1 GiB: 0.65-0.67 of peak bandwidth
-  // for hipMemcpyAsync against 0.78 for the kernel).
+  // for hipMemcpyAsync against 0.77-0.79 for the kernel; 64 MiB with destinations that fit the
+  // memory-side cache: 0.86 against 0.74).
   const bool dense = tensor_is_contiguous(dst) && tensor_is_contiguous(src);
   const int64_t bytes = (int64_t)n * (int64_t)dtype_size(dt);
-  if ((dense && bytes < tuning("copy.kernel_min_bytes", int64_t(32) << 20)) || n == 1) {
+  if ((dense && bytes < tuning("copy.kernel_min_bytes", int64_t(128) << 20)) || n == 1) {
     THC_CHECK(hipMemcpyAsync(tensor_data(dst, dt), tensor_data(src, dt), (size_t)n * dtype_size(dt),
                              hipMemcpyDeviceToDevice, current_stream(s)));
     return;

@@ -51,9 +51,24 @@ struct LdsTileShape {
   static constexpr int NP_S = (TQ + ROWS_P - 1) / ROWS_P;  // packs per lane, lanes along p
   static constexpr int NP_D = (TP + ROWS_Q - 1) / ROWS_Q;  // packs per lane, lanes along q
   static constexpr int NP = NP_S > NP_D ? NP_S : NP_D;
-  static constexpr int PITCH_S = TP | 1;  // transposed slab [TQ][PITCH_S]: odd pitch spreads the banks
-  static constexpr int PITCH_D = WQ;      // plain slab [TP][PITCH_D]: whole windows, 16-byte accesses
-  static constexpr int SLAB_RAW = TQ * PITCH_S > TP * PITCH_D ? TQ * PITCH_S : TP * PITCH_D;
+  // ALIGNED: transposed slab [TQ][PITCH_S] (odd pitch spreads the banks), plain slab [TP][PITCH_D].
+  // Otherwise both slabs carry a margin of one pack (MARG) on the sides towards which a row's shift
+  // can move an element, so that no LDS access needs a predicate or a clamp: the transposed slab
+  // holds tile coordinates (q, p) at [q + MARG][p + MARG], the plain slab holds row p's window
+  // (its own shift included) from column MARG on.
+  static constexpr int MARG = ALIGNED ? 0 : VEC;
+  static constexpr int PITCH_S = ALIGNED ? (TP | 1) : ((WP + VEC) | 1);
+  static constexpr int ROWS_S = ALIGNED ? TQ : WQ + VEC;
+  static constexpr int PITCH_D = ALIGNED ? WQ : WQ + 2 * VEC;
+  static constexpr int ROWS_D = ALIGNED ? TP : WP;
+  static_assert(NP_S * ROWS_P <= ROWS_S && NP_D * ROWS_Q <= ROWS_D, "every lane's row lies inside the slab");
+  // Reading the transposed slab, lane lxq takes rows VEC * lxq + e: lanes 8 apart would meet in one
+  // bank (8 * VEC * PITCH_S elements are a multiple of 32 words). Row q therefore starts
+  // skew(q) = (q / (8 * VEC)) * SKEW_UNIT elements late, one bank per group of 8 lanes.
+  static constexpr int SKEW_UNIT = ALIGNED && sizeof(T) <= 4 ? 4 / (int)sizeof(T) : 0;
+  static constexpr int skew(int q) { return SKEW_UNIT ? (q / (8 * VEC)) * SKEW_UNIT : 0; }
+  static constexpr int SLAB_S = ROWS_S * PITCH_S + skew(ROWS_S);
+  static constexpr int SLAB_RAW = SLAB_S > ROWS_D * PITCH_D ? SLAB_S : ROWS_D * PITCH_D;
   static constexpr int SLAB = (SLAB_RAW + VEC - 1) / VEC * VEC;  // elements of T per input
   static constexpr size_t lds_bytes(int nin) { return (size_t)nin * SLAB * sizeof(T); }
 };
@@ -64,7 +79,7 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
   using S = LdsTileShape<T, TOut, LXP, LXQ, ALIGNED>;
   constexpr int NIN = Op::NIN;
   constexpr int VEC = S::VEC, TP = S::TP, TQ = S::TQ, ROWS_P = S::ROWS_P, ROWS_Q = S::ROWS_Q;
-  constexpr int NP = S::NP, NP_S = S::NP_S, NP_D = S::NP_D, PITCH_S = S::PITCH_S, PITCH_D = S::PITCH_D;
+  constexpr int NP = S::NP, NP_S = S::NP_S, NP_D = S::NP_D, PITCH_S = S::PITCH_S, PITCH_D = S::PITCH_D, MARG = S::MARG;
   static_assert(NIN >= 1 && NIN <= 3, "one to three inputs");
   using PIN = Pack<T, VEC>;
   using POUT = Pack<TOut, VEC>;
@@ -151,8 +166,9 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
     }
   };
 
-  // Registers -> LDS. Transposed inputs land element by element at [q][p]; the others keep
-  // their window (pack j of row p at column j * VEC, the row's own shift included).
+  // Registers -> LDS, without predicates (the slabs have room for every lane's pack). Transposed
+  // inputs land element by element at [q][p]; the others keep their window (pack j of row p at
+  // column j * VEC, the row's own shift included).
   auto commit = [&](const Tile& t, const PIN (&v)[NIN][NP]) {
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
@@ -164,19 +180,15 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
           const int qi = (int)lyp + r * ROWS_P;
           int first = (int)(lxp * VEC);
           if (!ALIGNED) first -= mis_in(t.tb[k] + (uint32_t)min(qi, t.qn - 1) * sq);
-          if (ALIGNED || qi < TQ) {
+          T* at = slab + (qi + MARG) * PITCH_S + S::skew(qi) + (first + MARG);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-              const int pi = first + e;
-              if (ALIGNED || (pi >= 0 && pi < TP)) slab[qi * PITCH_S + pi] = v[k][r].v[e];
-            }
-          }
+          for (int e = 0; e < VEC; ++e) at[e] = v[k][r].v[e];
         }
       } else {
 #pragma unroll
         for (int r = 0; r < NP_D; ++r) {
           const int pi = (int)lyq + r * ROWS_Q;
-          if (ALIGNED || pi < TP) *reinterpret_cast<PIN*>(slab + pi * PITCH_D + lxq * VEC) = v[k][r];
+          *reinterpret_cast<PIN*>(slab + pi * PITCH_D + MARG + lxq * VEC) = v[k][r];
         }
       }
     }
@@ -196,17 +208,16 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
         for (int k = 0; k < NIN; ++k) {
           const T* slab = lds + k * S::SLAB;
           if (args.staged[k + 1]) {
+            const T* at = slab + (first + MARG) * PITCH_S + S::skew(first) + (pic + MARG);  // (skew: ALIGNED only)
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-              const int j = ALIGNED ? first + e : min(max(first + e, 0), TQ - 1);
-              in[k].v[e] = slab[j * PITCH_S + pic];
-            }
+            for (int e = 0; e < VEC; ++e) in[k].v[e] = at[e * PITCH_S];
           } else if (ALIGNED) {
             in[k] = *reinterpret_cast<const PIN*>(slab + pic * PITCH_D + first);
           } else {
             const int m = mis_in(t.tb[k] + (uint32_t)pic * (uint32_t)args.strideP[k + 1]);
+            const T* at = slab + pic * PITCH_D + (first + m + MARG);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) in[k].v[e] = slab[pic * PITCH_D + min(max(first + e, 0), TQ - 1) + m];
+            for (int e = 0; e < VEC; ++e) in[k].v[e] = at[e];
           }
         }
         POUT res;

@@ -121,14 +121,23 @@ struct Cvt<__half> {
 };
 
 // (D)x with C's conversion rules (float -> integer truncates toward zero); half goes through float.
+// A floating value becomes a 1- or 2-byte integer in two steps, to int and then truncated: identical
+// for every value the narrow type can hold, and defined for the others too. The one-step form lets the
+// compiler assume the result fits, and it then packs neighbouring elements of a pack into one register
+// without masking; kernels that compute whole packs at a tensor's edges feed elements through here
+// that are not part of the tensor and whose value is arbitrary.
 template <typename D, typename S>
 __device__ __forceinline__ D convert_value(S x) {
+  constexpr bool kNarrowInt = std::is_integral<D>::value && sizeof(D) < 4;
   if constexpr (std::is_same<S, __half>::value) {
     const float f = __half2float(x);
     if constexpr (std::is_same<D, __half>::value) return x;
+    else if constexpr (kNarrowInt) return (D)(int)f;
     else return (D)f;
   } else if constexpr (std::is_same<D, __half>::value) {
     return __float2half_rn((float)x);
+  } else if constexpr (kNarrowInt && std::is_floating_point<S>::value) {
+    return (D)(int)x;
   } else {
     return (D)x;
   }
