@@ -129,7 +129,7 @@ def sums_close(got, ref64, mass, rel):
     return bool(np.all(np.abs(got - ref64) <= rel * np.maximum(np.abs(ref64), mass / 64.0)))
 
 
-def build_configs(thc, hip, which, only=None):
+def build_configs(thc, hip, which, only=None, stagger=0):
     rng = np.random.default_rng(0xC0FFEE)
     cfgs = []
     T = thc.Tensor
@@ -142,8 +142,8 @@ def build_configs(thc, hip, which, only=None):
     # operands repeat a 2^24-element block of normal(0,1) values (the element at storage offset o is
     # block[o % 2^24]).
     if want('C5', 'CEIL-2r1w-26GB'):
-        nb = 1 << 24
-        block = rng.standard_normal(nb, dtype=np.float32)
+        nb5 = 1 << 24
+        block = rng.standard_normal(nb5, dtype=np.float32)
         rblock = block[::-1].copy()
         a5 = device_fill_from_block(hip, thc, (520, 2048, 2048), block)
         b5 = device_fill_from_block(hip, thc, (2048, 2048, 520), rblock)
@@ -157,8 +157,8 @@ def build_configs(thc, hip, which, only=None):
             j, k = np.arange(2048, dtype=np.int64)[:, None], np.arange(520, dtype=np.int64)[None, :]
             for i in planes:
                 got = c5.select(0, i).numpy()
-                wa = block[(i + 2048 * j + 2048 * 2048 * k) % nb]
-                wb = rblock[((i * 2048 + j) * 520 + k) % nb]
+                wa = block[(i + 2048 * j + 2048 * 2048 * k) % nb5]
+                wb = rblock[((i * 2048 + j) * 520 + k) % nb5]
                 ok = ok and bit_equal(got, wa + wb)
             return ok
         cfgs.append(Config("C5", "c = a + b, 2048x2048x520 fp32, a = permute(3,2,1) view, 64-bit indices",
@@ -208,7 +208,13 @@ def build_configs(thc, hip, which, only=None):
         ha, hb = rng.uniform(-1, 1, n1).astype(np.float32), rng.uniform(-1, 1, n1).astype(np.float32)
         if k == 0:
             h1 = (ha, hb)
-        sets1.append((T.from_numpy(ha), T.from_numpy(hb), T("float").resize((n1,))))
+        if stagger:
+            # operands inside larger allocations, b and c starting `stagger` and 2 x `stagger` elements in: shifts
+            # the three streams against each other in the memory channels' interleave (a probe, see --stagger)
+            pad = lambda h, k: T.from_numpy(np.concatenate([np.zeros(k * stagger, np.float32), h])).narrow(0, k * stagger, n1)
+            sets1.append((pad(ha, 0), pad(hb, 1), T("float").resize((n1 + 2 * stagger,)).narrow(0, 2 * stagger, n1)))
+        else:
+            sets1.append((T.from_numpy(ha), T.from_numpy(hb), T("float").resize((n1,))))
 
     def c1_check(op):
         def check():
@@ -328,7 +334,7 @@ def build_configs(thc, hip, which, only=None):
                       "N-cumsum-cols", "N-dist", "N-varall", "N-int-add", "N-lt-byte", "N-cvt-half",
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
-                      "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
+                      "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G")
           if (only and n in only) or (not only and which == "all")]
     if nx:
@@ -419,8 +425,8 @@ def build_configs(thc, hip, which, only=None):
                 "N-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 fp32", 9 * 8192 * 8192, 8192 * 8192,
                            lambda i: lt_m.compare_tensor("lt", sq_t, db)),
             })
-        if set(nx) & {"N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-cmax-t", "N-int-div-t", "N-int-lt-t",
-                      "N-cvt-half-t"}:
+        if set(nx) & {"N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd",
+                      "N-int-div-t", "N-int-lt-t", "N-cvt-half-t"}:
             # transposed operands of the op families beyond plain float arithmetic: one-input math on half,
             # narrow integer arithmetic, two-input float math, integer division, integer comparison into Byte,
             # type-converting copy
@@ -438,6 +444,12 @@ def build_configs(thc, hip, which, only=None):
             jm = T("byte").resize((m, m))
             fo = T("float").resize((m, m))
             hc = T("half").resize((m, m))
+            sa_odd = T.from_numpy(rng.integers(-1000, 1000, (8193, 8191)).astype(np.int16)).t()
+            sb_odd = T.from_numpy(rng.integers(-1000, 1000, (8191, 8193)).astype(np.int16))
+            so_odd = T("short").resize((8191, 8193))
+            fa_odd = T.from_numpy(rng.standard_normal((8193, 8191), dtype=np.float32)).t()
+            fb_odd = T.from_numpy(rng.standard_normal((8191, 8193), dtype=np.float32))
+            fo_odd = T("float").resize((8191, 8193))
             table.update({
                 "N-half-exp": ("out = exp(a), 8192x8192 fp16 contiguous (the flat form of N-half-exp-t)", 4 * m * m, m * m,
                                lambda i: ho.unary("exp", hc)),
@@ -448,6 +460,14 @@ def build_configs(thc, hip, which, only=None):
                 "N-short-add-t": ("c = a:t() + b, 8192x8192 int16", 6 * m * m, m * m, lambda i: sc.cadd(sa, 1, sb)),
                 "N-cmax-t": ("c = cmax(a:t(), b), 8192x8192 fp32", 12 * m * m, m * m,
                              lambda i: fo.binary("cmax", sq_t, db)),
+                "N-short-neg-t": ("out = -a:t(), 8192x8192 int16", 4 * m * m, m * m, lambda i: sc.unary("neg", sa)),
+                "N-int-neg-t": ("out = -a:t(), 8192x8192 int32", 8 * m * m, m * m, lambda i: jc.unary("neg", ja)),
+                "N-cvt-float-t": ("float <- half converting copy of a:t(), 8192x8192", 6 * m * m, m * m,
+                                  lambda i: fo.copy_from(hx)),
+                "N-short-add-t-odd": ("c = a:t() + b, 8191x8193 int16 (no 16-byte aligned rows)", 6 * nodd_, nodd_,
+                                      lambda i: so_odd.cadd(sa_odd, 1, sb_odd)),
+                "N-cmax-t-odd": ("c = cmax(a:t(), b), 8191x8193 fp32 (no 16-byte aligned rows)", 12 * nodd_, nodd_,
+                                 lambda i: fo_odd.binary("cmax", fa_odd, fb_odd)),
                 "N-int-div-t": ("c = a:t() / b, 8192x8192 int32 (truncating division)", 12 * m * m, m * m,
                                 lambda i: jc.cdiv(ja, jb)),
                 "N-int-lt-t": ("mask = a:t() < b into a Byte tensor, 8192x8192 int32", 9 * m * m, m * m,
@@ -634,6 +654,8 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated config names to measure (the first one "
                                                "built becomes the line's headline)")
     ap.add_argument("--tune", action="append", default=[], help="engine tuning knob key=value")
+    ap.add_argument("--stagger", type=int, default=0, help="probe: C1's second input and its output start this many / twice "
+                                                           "this many elements into their allocations (a multiple of 4)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this engine has no multi-GPU path (run with --gpus 1)")
@@ -646,7 +668,7 @@ def main():
         k, v = kv.split("=")
         thc.set_tuning(k, int(v))
     only = set(args.only.split(",")) if args.only else None
-    cfgs, host = build_configs(thc, hip, args.configs, only)
+    cfgs, host = build_configs(thc, hip, args.configs, only, args.stagger)
     if not cfgs:
         sys.exit("no configuration selected")
     results = []

@@ -151,6 +151,8 @@ def _declare(l):
         f(T + "_copy", None, P, TP, TP)
         f(T + "_copyFromHost", None, P, TP, P)
         f(T + "_copyToHost", None, P, P, TP)
+        f(T + "_copyAsyncFromHost", None, P, TP, P, C.c_ssize_t)
+        f(T + "_copyAsyncToHost", None, P, P, C.c_ssize_t, TP)
         f(T + "_isContiguous", C.c_int, P, TP)
         f(T + "_nElement", C.c_ssize_t, P, TP)
         f(T + "_data", P, P, TP)
@@ -340,6 +342,20 @@ class Tensor(object):
             self._fn("copyToHost")(self._st, out.ctypes.data_as(C.c_void_p), self.h)
             _check()
         return out
+
+    def copy_async_from_host(self, host_ptr, n):
+        """Queues host memory (n elements at host_ptr, ideally pinned) -> this contiguous tensor on the
+        current stream; does not wait (copyAsyncCPU, generic/THCTensorCopy.c:104-132)."""
+        self._fn("copyAsyncFromHost")(self._st, self.h, C.c_void_p(host_ptr), n)
+        _check()
+        return self
+
+    def copy_async_to_host(self, host_ptr, n):
+        """Queues this contiguous tensor -> host memory on the current stream; does not wait
+        (copyAsyncCuda, generic/THCTensorCopy.c:134-164)."""
+        self._fn("copyAsyncToHost")(self._st, C.c_void_p(host_ptr), n, self.h)
+        _check()
+        return self
 
     def storage_numpy(self):
         """The whole underlying storage (to check that holes stay untouched)."""

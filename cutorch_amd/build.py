@@ -63,6 +63,9 @@ def _compile(src, force):
     group = APPLY_HEADERS if src.startswith(("apply", "convert")) else (
         REDUCE_HEADERS if src.startswith(("reduce", "scan", "no_alloc")) else [])
     deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS + group + EXTRA_DEPS.get(src, [])]
+    only = os.environ.get("THC_BUILD_ONLY")   # development aid: rebuild just these sources, reuse every other object as it is
+    if only and os.path.exists(obj) and src not in only.split(","):
+        return obj
     if not force and not _stale(obj, deps):
         return obj
     cmd = [_hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + FLAGS

@@ -41,6 +41,22 @@ struct LdsTileArgs {
 };
 
 // Geometry shared by the kernel and the host (LDS bytes, tile extents).
+//
+// ALIGNED: the tile is the window, WP x WQ; the transposed slab is [WQ][PITCH_S], the plain slab
+// [WP][WQ].
+// Otherwise a tile advances by TP = WP - VEC and TQ = WQ - VEC, one pack less than the window, and
+//   * along p (transposed inputs) a row's window starts at the aligned pack at or below the tile's
+//     first element of that row, so window element w is tile coordinate w - m, m < VEC the row's
+//     own misalignment;
+//   * along q every OUTPUT row cuts the tensor at its own pack boundaries: with mo < VEC the
+//     misalignment of the output row at column q0, the tile owns of that row the 31 whole packs
+//     [q0 - mo, q0 - mo + TQ). No pack is split between two tiles, so partial (element-wise) stores
+//     only happen at the two ends of a tensor row. (Cutting every row at q0 left two partial packs
+//     per row and tile; stores narrower than 4 bytes make the memory side read, merge and write a
+//     whole sector each: a transposed half / short operand of odd shape moved 2.3 x its bytes.)
+//     The transposed slab therefore holds tile rows q0 - VEC .. q0 + TQ - 1 (slab row = tile
+//     coordinate + VEC), and a plain input's window starts at the aligned pack at or below ITS
+//     element at column q0 - mo.
 template <typename T, typename TOut, int LXP, int LXQ, bool ALIGNED>
 struct LdsTileShape {
   static constexpr int W = sizeof(T) > sizeof(TOut) ? sizeof(T) : sizeof(TOut);
@@ -48,54 +64,76 @@ struct LdsTileShape {
   static constexpr int WP = LXP * VEC, WQ = LXQ * VEC;  // window: lanes x pack
   static constexpr int TP = ALIGNED ? WP : WP - VEC, TQ = ALIGNED ? WQ : WQ - VEC;
   static constexpr int ROWS_P = kBlock / LXP, ROWS_Q = kBlock / LXQ;
-  static constexpr int NP_S = (TQ + ROWS_P - 1) / ROWS_P;  // packs per lane, lanes along p
+  static constexpr int NP_S = WQ / ROWS_P;                 // packs per lane, lanes along p
   static constexpr int NP_D = (TP + ROWS_Q - 1) / ROWS_Q;  // packs per lane, lanes along q
   static constexpr int NP = NP_S > NP_D ? NP_S : NP_D;
-  // ALIGNED: transposed slab [TQ][PITCH_S] (odd pitch spreads the banks), plain slab [TP][PITCH_D].
-  // Otherwise both slabs carry a margin of one pack (MARG) on the sides towards which a row's shift
-  // can move an element, so that no LDS access needs a predicate or a clamp: the transposed slab
-  // holds tile coordinates (q, p) at [q + MARG][p + MARG], the plain slab holds row p's window
-  // (its own shift included) from column MARG on.
+  static_assert(WQ % ROWS_P == 0, "whole passes over the window's rows");
   static constexpr int MARG = ALIGNED ? 0 : VEC;
-  static constexpr int PITCH_S = ALIGNED ? (TP | 1) : ((WP + VEC) | 1);
-  static constexpr int ROWS_S = ALIGNED ? TQ : WQ + VEC;
-  static constexpr int PITCH_D = ALIGNED ? WQ : WQ + 2 * VEC;
-  static constexpr int ROWS_D = ALIGNED ? TP : WP;
-  static_assert(NP_S * ROWS_P <= ROWS_S && NP_D * ROWS_Q <= ROWS_D, "every lane's row lies inside the slab");
-  // Reading the transposed slab, lane lxq takes rows VEC * lxq + e: lanes 8 apart would meet in one
-  // bank (8 * VEC * PITCH_S elements are a multiple of 32 words). Row q therefore starts
-  // skew(q) = (q / (8 * VEC)) * SKEW_UNIT elements late, one bank per group of 8 lanes.
-  static constexpr int SKEW_UNIT = ALIGNED && sizeof(T) <= 4 ? 4 / (int)sizeof(T) : 0;
-  static constexpr int skew(int q) { return SKEW_UNIT ? (q / (8 * VEC)) * SKEW_UNIT : 0; }
+  // Pitch of the transposed slab: a whole, ODD number of 32-bit words. Whole words keep a lane's
+  // pack of sub-word elements word-aligned in LDS (16-byte LDS writes at 2-byte alignment stall the
+  // LDS pipeline: half and short tiles spent a fifth of their time in such stalls); the odd word
+  // count spreads rows over the banks.
+  static constexpr int EPW = sizeof(T) >= 4 ? 1 : 4 / (int)sizeof(T);   // elements per word
+  // Unaligned rows of sub-word elements: the transposed slab keeps every row's WINDOW as loaded
+  // (pack j at column j * VEC, a word-aligned LDS write) instead of shifting it into place, and
+  // the readers add the row's shift, which they derive from the row number.
+  static constexpr bool WIN = !ALIGNED && sizeof(T) < 4;
+  // (shifted into place, a row occupies columns MARG - (VEC - 1) .. MARG + WP - 1)
+  static constexpr int PITCH_S = (((ALIGNED || WIN ? WP : WP + VEC) + EPW - 1) / EPW | 1) * EPW;
+  static constexpr int ROWS_S = ALIGNED ? WQ : WQ + VEC;   // (lane 31 of an unaligned tile reads past row WQ: never stored)
+  // plain slab: row p's window from column MARG on; readers look up to 2 VEC - 2 columns beyond it
+  static constexpr int PITCH_D = ALIGNED ? WQ : WQ + 3 * VEC;
+  static constexpr int ROWS_D = WP;
+  static_assert(NP_D * ROWS_Q <= ROWS_D, "every lane's row lies inside the slab");
+  // Reading the transposed slab, lane lxq takes rows VEC * lxq + e: VEC rows are VEC * odd words, so
+  // lanes 32 / VEC apart would meet in one bank. Row r therefore starts skew(r) = (r / 32) words late:
+  // one bank further for every such group of lanes. (Unaligned rows: only the window layout, whose
+  // readers compute an offset per element anyway.)
+  static constexpr int SKEW_UNIT = (ALIGNED || WIN) && sizeof(T) <= 4 ? EPW : 0;
+  static constexpr int skew(int r) { return SKEW_UNIT ? (r / 32) * SKEW_UNIT : 0; }
   static constexpr int SLAB_S = ROWS_S * PITCH_S + skew(ROWS_S);
   static constexpr int SLAB_RAW = SLAB_S > ROWS_D * PITCH_D ? SLAB_S : ROWS_D * PITCH_D;
   static constexpr int SLAB = (SLAB_RAW + VEC - 1) / VEC * VEC;  // elements of T per input
   static constexpr size_t lds_bytes(int nin) { return (size_t)nin * SLAB * sizeof(T); }
 };
 
-template <typename T, typename TOut, typename Op, int LXP, int LXQ, bool ALIGNED>
+// NTL: inputs are read with the streaming (nontemporal) hint. A compile-time choice: a run-time one
+// makes the compiler merge the two forms of every load into one plain load.
+template <typename T, typename TOut, typename Op, int LXP, int LXQ, bool ALIGNED, bool NTL = true>
 __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const T* in0, const T* in1,
                                                                const T* in2, LdsTileArgs args, Op op) {
   using S = LdsTileShape<T, TOut, LXP, LXQ, ALIGNED>;
   constexpr int NIN = Op::NIN;
   constexpr int VEC = S::VEC, TP = S::TP, TQ = S::TQ, ROWS_P = S::ROWS_P, ROWS_Q = S::ROWS_Q;
   constexpr int NP = S::NP, NP_S = S::NP_S, NP_D = S::NP_D, PITCH_S = S::PITCH_S, PITCH_D = S::PITCH_D, MARG = S::MARG;
+  constexpr bool WIN = S::WIN;
   static_assert(NIN >= 1 && NIN <= 3, "one to three inputs");
   using PIN = Pack<T, VEC>;
   using POUT = Pack<TOut, VEC>;
+  // Packs travel from global memory to LDS as raw register images: a pack of sub-word elements kept
+  // as a struct across the tile loop ended up in scratch memory (272 bytes a lane for two inputs of
+  // 16-bit elements, which tripled the kernel's memory traffic).
+  using RAW = typename RawBits<sizeof(PIN)>::type;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
 
   const T* ptr[3] = {in0, in1, in2};
   const uint32_t lxp = threadIdx.x % LXP, lyp = threadIdx.x / LXP;
   const uint32_t lxq = threadIdx.x % LXQ, lyq = threadIdx.x / LXQ;
+  const int sizeQ = (int)args.sizeQ;
   auto mis_in = [](const T* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(T)) & (uintptr_t)(VEC - 1)); };
   auto mis_out = [](const TOut* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(TOut)) & (uintptr_t)(VEC - 1)); };
+  auto load = [&](const T* at) -> RAW {
+    if constexpr (NTL) return __builtin_nontemporal_load(reinterpret_cast<const RAW*>(at));
+    else return *reinterpret_cast<const RAW*>(at);
+  };
 
   struct Tile {       // uniform over the workgroup
-    const T* tb[3];   // tile origin of input k
+    const T* tb[3];   // tile origin (p0, q0) of input k
     TOut* ob;         // tile origin of the output
-    int pn, qn;       // valid extent
+    int pn;           // valid extent along p
+    int qn;           // ALIGNED: valid extent along q
+    int q0;           // first column (unaligned tiles reach back to q0 - VEC + 1 and on to q0 + TQ - 1)
   };
   const uint32_t slots = args.xcdPer ? args.xcdPer * 8 : args.totalTiles;
   // First valid tile at or after slot b (b advances by the grid size); false when none is left.
@@ -129,7 +167,8 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
     }
     const uint32_t p0 = tp * TP, q0 = tq * TQ;
     t.pn = (int)min((uint32_t)TP, args.sizeP - p0);
-    t.qn = (int)min((uint32_t)TQ, args.sizeQ - q0);
+    t.qn = (int)min((int64_t)TQ, (int64_t)args.sizeQ - (int64_t)q0);
+    t.q0 = (int)q0;
     t.ob = out + (base[0] + (int64_t)p0 * args.strideP[0] + (int64_t)q0 * args.strideQ[0]);
 #pragma unroll
     for (int k = 0; k < NIN; ++k)
@@ -137,58 +176,78 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
     return true;
   };
 
+  // Row of transposed input k that lane row `qi` of the staging pass loads: tile coordinate
+  // qi (ALIGNED) or qi - VEC, kept inside the tensor.
+  auto staged_row = [&](const Tile& t, int k, int qi) -> const T* {
+    const int sq = (int)args.strideQ[k + 1];
+    if (ALIGNED) return t.tb[k] + (uint32_t)min(qi, t.qn - 1) * (uint32_t)sq;
+    const int j = min(max(qi - VEC, -t.q0), sizeQ - 1 - t.q0);
+    return t.tb[k] + (ptrdiff_t)(j * sq);
+  };
+  // First column (relative to q0) of the run that output row `pi` owns in this tile, kept inside
+  // the tensor: q0 - mo for an unaligned row.
+  auto row_start = [&](const Tile& t, int pi) -> int {
+    if (ALIGNED) return 0;
+    const int mo = mis_out(t.ob + (uint32_t)pi * (uint32_t)args.strideP[0]);
+    return min(max(-mo, -t.q0), sizeQ - 1 - t.q0);
+  };
+
   // Requests every pack of the tile's inputs. No load carries a predicate: lanes past the
   // tile's valid extent re-read a pack inside it, so a later wait covers exactly these loads.
-  auto issue = [&](const Tile& t, PIN (&v)[NIN][NP]) {
+  auto issue = [&](const Tile& t, RAW (&v)[NIN][NP]) {
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
       if (args.staged[k + 1]) {
-        const uint32_t sq = (uint32_t)args.strideQ[k + 1];
 #pragma unroll
         for (int r = 0; r < NP_S; ++r) {
-          const int qi = min((int)lyp + r * ROWS_P, t.qn - 1);
-          const T* row = t.tb[k] + (uint32_t)qi * sq;
+          const T* row = staged_row(t, k, (int)lyp + r * ROWS_P);
           int first = (int)(lxp * VEC) - (ALIGNED ? 0 : mis_in(row));
           if (first >= t.pn) first = ALIGNED ? 0 : -mis_in(row);
-          v[k][r] = load_pack<true>(reinterpret_cast<const PIN*>(row + first));
+          v[k][r] = load(row + first);
         }
       } else {
         const uint32_t sp = (uint32_t)args.strideP[k + 1];
 #pragma unroll
         for (int r = 0; r < NP_D; ++r) {
           const int pi = min((int)lyq + r * ROWS_Q, t.pn - 1);
-          const T* row = t.tb[k] + (uint32_t)pi * sp;
-          int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_in(row));
-          if (first >= t.qn) first = ALIGNED ? 0 : -mis_in(row);
-          v[k][r] = load_pack<true>(reinterpret_cast<const PIN*>(row + first));
+          const int cs = row_start(t, pi);
+          const T* at = t.tb[k] + (uint32_t)pi * sp + (ptrdiff_t)cs;   // this row's element at the run's start
+          int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_in(at));
+          if (ALIGNED ? first >= t.qn : t.q0 + cs + first >= sizeQ) first = ALIGNED ? 0 : -mis_in(at);
+          v[k][r] = load(at + first);
         }
       }
     }
   };
 
   // Registers -> LDS, without predicates (the slabs have room for every lane's pack). Transposed
-  // inputs land element by element at [q][p]; the others keep their window (pack j of row p at
-  // column j * VEC, the row's own shift included).
-  auto commit = [&](const Tile& t, const PIN (&v)[NIN][NP]) {
+  // inputs land at [q][p] (shifted into place element by element, or as the window they were
+  // loaded as); the others keep their window (pack j of row p at column MARG + j * VEC).
+  auto commit = [&](const Tile& t, const RAW (&v)[NIN][NP]) {
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
       T* slab = lds + k * S::SLAB;
       if (args.staged[k + 1]) {
-        const uint32_t sq = (uint32_t)args.strideQ[k + 1];
 #pragma unroll
         for (int r = 0; r < NP_S; ++r) {
           const int qi = (int)lyp + r * ROWS_P;
-          int first = (int)(lxp * VEC);
-          if (!ALIGNED) first -= mis_in(t.tb[k] + (uint32_t)min(qi, t.qn - 1) * sq);
-          T* at = slab + (qi + MARG) * PITCH_S + S::skew(qi) + (first + MARG);
+          if constexpr (WIN) {
+            *reinterpret_cast<RAW*>(slab + qi * PITCH_S + S::skew(qi) + lxp * VEC) = v[k][r];
+          } else {
+            int first = (int)(lxp * VEC);
+            if (!ALIGNED) first -= mis_in(staged_row(t, k, qi));
+            T* at = slab + qi * PITCH_S + S::skew(qi) + (first + MARG);
+            PIN pk;
+            __builtin_memcpy(&pk, &v[k][r], sizeof(PIN));
 #pragma unroll
-          for (int e = 0; e < VEC; ++e) at[e] = v[k][r].v[e];
+            for (int e = 0; e < VEC; ++e) at[e] = pk.v[e];
+          }
         }
       } else {
 #pragma unroll
         for (int r = 0; r < NP_D; ++r) {
           const int pi = (int)lyq + r * ROWS_Q;
-          *reinterpret_cast<PIN*>(slab + pi * PITCH_D + MARG + lxq * VEC) = v[k][r];
+          *reinterpret_cast<RAW*>(slab + pi * PITCH_D + MARG + lxq * VEC) = v[k][r];
         }
       }
     }
@@ -200,37 +259,67 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
 #pragma unroll 2
       for (int r = 0; r < NP_D; ++r) {
         const int pi = (int)lyq + r * ROWS_Q;
-        const int pic = ALIGNED ? pi : min(pi, min(t.pn, TP) - 1);
+        const int pic = ALIGNED ? pi : min(pi, t.pn - 1);
         TOut* orow = t.ob + (uint32_t)pic * (uint32_t)args.strideP[0];
+        // tile coordinate of the lane's first element; its slab row is first + MARG
         const int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_out(orow));
-        PIN in[3] = {};
+        // (elements are gathered and results kept as scalars: packs of sub-word elements that are
+        // filled or read element by element do not stay in registers)
+        T x[3][VEC] = {};
 #pragma unroll
         for (int k = 0; k < NIN; ++k) {
           const T* slab = lds + k * S::SLAB;
-          if (args.staged[k + 1]) {
+          if (args.staged[k + 1] && WIN) {
+            // row j's window starts mis(row j) elements before its first tile element
+            const int sq = (int)((uint32_t)args.strideQ[k + 1] & (uint32_t)(VEC - 1));
+            int m = (mis_in(t.tb[k]) + first * sq) & (VEC - 1);
+            const T* at = slab + (first + MARG) * PITCH_S + pic;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+              x[k][e] = at[e * PITCH_S + m + S::skew(first + MARG + e)];
+              m = (m + sq) & (VEC - 1);
+            }
+          } else if (args.staged[k + 1]) {
             const T* at = slab + (first + MARG) * PITCH_S + S::skew(first) + (pic + MARG);  // (skew: ALIGNED only)
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) in[k].v[e] = at[e * PITCH_S];
+            for (int e = 0; e < VEC; ++e) x[k][e] = at[e * PITCH_S];
           } else if (ALIGNED) {
-            in[k] = *reinterpret_cast<const PIN*>(slab + pic * PITCH_D + first);
-          } else {
-            const int m = mis_in(t.tb[k] + (uint32_t)pic * (uint32_t)args.strideP[k + 1]);
-            const T* at = slab + pic * PITCH_D + (first + m + MARG);
+            const RAW raw = *reinterpret_cast<const RAW*>(slab + pic * PITCH_D + first);
+            PIN pk;
+            __builtin_memcpy(&pk, &raw, sizeof(PIN));
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) in[k].v[e] = at[e];
+            for (int e = 0; e < VEC; ++e) x[k][e] = pk.v[e];
+          } else {
+            // the window of row pic starts mis(element at the run's start) before that element
+            const int cs = row_start(t, pic);
+            const int m = mis_in(t.tb[k] + (uint32_t)pic * (uint32_t)args.strideP[k + 1] + (ptrdiff_t)cs);
+            const T* at = slab + pic * PITCH_D + (first - cs + m + MARG);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[k][e] = at[e];
           }
         }
+        TOut y[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y[e] = f(x[0][e], x[1][e], x[2][e]);
         POUT res;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) res.v[e] = f(in[0].v[e], in[1].v[e], in[2].v[e]);
-        if (pi < t.pn && first < t.qn) {
-          if (ALIGNED || (first >= 0 && first + VEC <= t.qn)) {
+        for (int e = 0; e < VEC; ++e) res.v[e] = y[e];
+        if constexpr (ALIGNED) {
+          if (pi < t.pn && first < t.qn) {
             if (args.ntStore) store_pack<true>(reinterpret_cast<POUT*>(orow + first), res);
             else store_pack<false>(reinterpret_cast<POUT*>(orow + first), res);
-          } else {
+          }
+        } else {
+          const int g = t.q0 + first;   // column of the pack's first element; lanes 0 .. LXQ - 2 own packs
+          if (pi < t.pn && lxq < LXQ - 1 && g + VEC > 0 && g < sizeQ) {
+            if (g >= 0 && g + VEC <= sizeQ) {
+              if (args.ntStore) store_pack<true>(reinterpret_cast<POUT*>(orow + first), res);
+              else store_pack<false>(reinterpret_cast<POUT*>(orow + first), res);
+            } else {   // the two ends of a tensor row
 #pragma unroll
-            for (int e = 0; e < VEC; ++e)
-              if (first + e >= 0 && first + e < t.qn) orow[first + e] = res.v[e];
+              for (int e = 0; e < VEC; ++e)
+                if (g + e >= 0 && g + e < sizeQ) orow[first + e] = y[e];
+            }
           }
         }
       }
@@ -239,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
 
   uint32_t b = blockIdx.x;
   Tile cur, nxt;
-  PIN v[NIN][NP];
+  RAW v[NIN][NP];
   bool have = locate(b, cur);
   if (have) issue(cur, v);
   while (have) {
@@ -307,7 +396,8 @@ bool launch_ldstile(THCState* s, const Plan& pl, Op op) {
     using SA = LdsTileShape<T, TOut, LXP, LXQ, true>;
     using SU = LdsTileShape<T, TOut, LXP, LXQ, false>;
     const int64_t tileP = aligned ? SA::TP : SU::TP, tileQ = aligned ? SA::TQ : SU::TQ;
-    const int64_t tp = (args.sizeP + tileP - 1) / tileP, tq = (args.sizeQ + tileQ - 1) / tileQ;
+    // (an unaligned row's first run starts up to VEC - 1 columns before the row does)
+    const int64_t tp = (args.sizeP + tileP - 1) / tileP, tq = (args.sizeQ + (aligned ? 0 : VEC - 1) + tileQ - 1) / tileQ;
     args.tilesP.set((uint64_t)tp);
     args.tilesQ.set((uint64_t)tq);
     const int64_t total = batch * tp * tq;
@@ -337,12 +427,27 @@ bool launch_ldstile(THCState* s, const Plan& pl, Op op) {
     const T* i0 = (const T*)pl.ptr[1];
     const T* i1 = (const T*)pl.ptr[2];
     const T* i2 = (const T*)pl.ptr[3];
-    if (aligned)
-      hipLaunchKernelGGL((apply_ldstile_kernel<T, TOut, Op, LXP, LXQ, true>), dim3(grid), dim3(kBlock), ldsBytes, st,
-                         o, i0, i1, i2, args, op);
-    else
-      hipLaunchKernelGGL((apply_ldstile_kernel<T, TOut, Op, LXP, LXQ, false>), dim3(grid), dim3(kBlock), ldsBytes, st,
-                         o, i0, i1, i2, args, op);
+    // Load policy. Ops with two or three inputs always read with the streaming hint (plain loads:
+    // 0.75 -> 0.61 of peak on a transposed cmax of 8192 x 8192 floats). With ONE input both forms are
+    // built and the choice is made here.
+    bool ntl = true;
+    if constexpr (Op::NIN == 1) {
+      const int64_t knob = tuning("apply.ldstile.nt_load", -1);
+      ntl = knob >= 0 ? knob != 0 : !(sizeof(T) == sizeof(TOut) && sizeof(T) < 4);
+    }
+    auto go = [&](auto alignedTag, auto ntlTag) {
+      hipLaunchKernelGGL((apply_ldstile_kernel<T, TOut, Op, LXP, LXQ, decltype(alignedTag)::value, decltype(ntlTag)::value>),
+                         dim3(grid), dim3(kBlock), ldsBytes, st, o, i0, i1, i2, args, op);
+    };
+    if constexpr (Op::NIN == 1) {
+      if (aligned && ntl) go(std::true_type{}, std::true_type{});
+      else if (aligned) go(std::true_type{}, std::false_type{});
+      else if (ntl) go(std::false_type{}, std::true_type{});
+      else go(std::false_type{}, std::false_type{});
+    } else {
+      if (aligned) go(std::true_type{}, std::true_type{});
+      else go(std::false_type{}, std::true_type{});
+    }
     note_kernel(aligned ? "lds-tile" : "lds-tile-shift");
     return true;
   }

@@ -285,14 +285,17 @@ __global__ __launch_bounds__(kBlock) void scan_slab_kernel(T* __restrict__ out,
                                                            const typename ScanAcc<T>::type* __restrict__ carryIn,
                                                            uint64_t outer, uint64_t R, uint32_t inner,
                                                            uint32_t slicesPerBlock, uint64_t S,
-                                                           uint32_t chunkRows, uint32_t dataBytes) {
+                                                           uint32_t chunkRows, uint32_t dataBytes, int reverse) {
   using A = typename ScanAcc<T>::type;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   T* lds = reinterpret_cast<T*>(lds_raw);
   A* part = reinterpret_cast<A*>(lds_raw + dataBytes);  // kBlock band totals behind the staged run
   const bool chunked = S > 1;
   const uint64_t numBlocks = chunked ? outer * S : (outer + slicesPerBlock - 1) / slicesPerBlock;
-  for (uint64_t blk = blockIdx.x; blk < numBlocks; blk += gridDim.x) {
+  for (uint64_t b = blockIdx.x; b < numBlocks; b += gridDim.x) {
+    // Chunk mode is the second read of the input: it walks the chunks last to first, so that it begins
+    // with what the totals pass read last and the memory-side cache may still hold.
+    const uint64_t blk = chunked && reverse ? numBlocks - 1 - b : b;
     uint64_t start;  // element offset of the run in the dense block
     uint32_t ns = 1, rows = (uint32_t)R;
     if (chunked) {
@@ -472,7 +475,7 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const size_t lds = (((size_t)(spb * R * inner) + 2 * kFull) * sizeof(T) + 15) & ~size_t(15);
     hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), lds + kBlock * sizeof(typename ScanAcc<T>::type),
                        st, out, in, nullptr, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint32_t)spb, (uint64_t)1, 0u,
-                       (uint32_t)lds);
+                       (uint32_t)lds, 0);
     note_kernel("scan-slab");
     return;
   }
@@ -504,7 +507,7 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
       launch_scan<A, Op>(s, carries, totals, outer, S, inner, scratch + 2 * need, scratchBytes - 2 * need);
       hipLaunchKernelGGL((scan_slab_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsData + kBlock * sizeof(A), st, out, in,
                          carries, (uint64_t)outer, (uint64_t)R, (uint32_t)inner, 1u, (uint64_t)S, (uint32_t)chunkRows,
-                         (uint32_t)ldsData);
+                         (uint32_t)ldsData, (int)tuning("scan.chunk_reverse", 1));
       note_kernel("scan-chunked");
       return;
     }

@@ -323,6 +323,27 @@ static void tensor_copy_to_host(THCState* s, void* dst, AnyTensor* src, DType dt
   THC_CHECK(hipMemcpy(dst, tensor_data(c.t, dt), (size_t)n * dtype_size(dt), hipMemcpyDeviceToHost));
 }
 
+// Asynchronous copies between a contiguous device tensor and host memory of the same element count,
+// queued on the current stream without waiting (generic/THCTensorCopy.c:104-164, copyAsyncCPU /
+// copyAsyncCuda; those take a TH tensor, which must be contiguous too: here the caller passes its
+// data pointer). The host memory should be pinned for the copy to overlap with anything; the caller
+// keeps it alive and untouched until the stream has passed the copy.
+static void tensor_copy_async(THCState* s, AnyTensor* dev, void* host, ptrdiff_t hostElements, DType dt,
+                              bool toDevice) {
+  const ptrdiff_t n = tensor_numel(dev);
+  THC_ARG_CHECK(n == hostElements, 2, "sizes do not match");
+  THC_ARG_CHECK(n == 0 || tensor_is_contiguous(dev), toDevice ? 2 : 3,
+                toDevice ? "Target tensor must be contiguous" : "Source tensor must be contiguous");
+  THC_ARG_CHECK(n == 0 || host != nullptr, toDevice ? 3 : 2, "no host memory");
+  if (n == 0) return;
+  note_stream_use(s, {dev});
+  const size_t bytes = (size_t)n * dtype_size(dt);
+  if (toDevice)
+    THC_CHECK(hipMemcpyAsync(tensor_data(dev, dt), host, bytes, hipMemcpyHostToDevice, current_stream(s)));
+  else
+    THC_CHECK(hipMemcpyAsync(host, tensor_data(dev, dt), bytes, hipMemcpyDeviceToHost, current_stream(s)));
+}
+
 }  // namespace thc
 
 using namespace thc;
@@ -550,6 +571,12 @@ using namespace thc;
   }                                                                                                \
   THC_API void Tensor##_copyToHost(THCState* s, real* dst, Tensor* src) {                          \
     THC_GUARD_VOID(tensor_copy_to_host(s, dst, TN(src), DT))                                       \
+  }                                                                                                \
+  THC_API void Tensor##_copyAsyncFromHost(THCState* s, Tensor* self, const real* src, ptrdiff_t n) { \
+    THC_GUARD_VOID(tensor_copy_async(s, TN(self), const_cast<real*>(src), n, DT, true))            \
+  }                                                                                                \
+  THC_API void Tensor##_copyAsyncToHost(THCState* s, real* dst, ptrdiff_t n, Tensor* src) {        \
+    THC_GUARD_VOID(tensor_copy_async(s, TN(src), dst, n, DT, false))                               \
   }
 
 THC_AMD_DEFINE_TENSOR_API(THCudaStorage, THCudaTensor, float, DType::F32)

@@ -252,7 +252,17 @@ THC_AMD_DECLARE_STRUCTS(THCudaDoubleStorage, THCudaDoubleTensor, double)
                                              Tensor *src);                     \
   THC_API void Tensor##_copyFromHost(THCState *, Tensor *self,                 \
                                      const real *src);                         \
-  THC_API void Tensor##_copyToHost(THCState *, real *dst, Tensor *src);
+  THC_API void Tensor##_copyToHost(THCState *, real *dst, Tensor *src);        \
+  /* generic/THCTensorCopy.h:40-41 (copyAsyncCPU / copyAsyncCuda, whose host  \
+   * operand is a contiguous TH tensor): `n` elements of host memory, queued  \
+   * on the current stream without waiting; the device tensor must be         \
+   * contiguous and hold n elements. Pin the host memory (hipHostMalloc) for  \
+   * the copy to overlap with other work, and keep it until the stream has    \
+   * passed the copy. */                                                       \
+  THC_API void Tensor##_copyAsyncFromHost(THCState *, Tensor *self,            \
+                                          const real *src, ptrdiff_t n);      \
+  THC_API void Tensor##_copyAsyncToHost(THCState *, real *dst, ptrdiff_t n,    \
+                                        Tensor *src);
 
 THC_AMD_DECLARE_TENSOR_API(THCudaStorage, THCudaTensor, float)
 THC_AMD_DECLARE_TENSOR_API(THCudaHalfStorage, THCudaHalfTensor, THHalf)

@@ -76,6 +76,17 @@ def nonblocking_streams(thc):
         hip.hipStreamDestroy(s)
 
 
+def _still_busy(hip, stream):
+    """True while work queued on `stream` has not completed. An assertion about a block being held back
+    is only meaningful while the other stream is still busy: the caller reads the quantity first and
+    asserts only if the stream was still busy afterwards (on a fast GPU or a slow host the queue may
+    have drained, and then nothing needs to be held back any more)."""
+    hip.hipStreamQuery.argtypes = [C.c_void_p]
+    busy = hip.hipStreamQuery(stream) != 0
+    hip.hipGetLastError()                             # "not ready" is not an error to leave behind
+    return busy
+
+
 def _busy(thc, w, launches):
     """Queues `launches` passes over the 1 GiB tensor w on the current stream (a few ms of work)."""
     for _ in range(launches):
@@ -99,10 +110,12 @@ def test_block_used_on_another_stream_is_held_back(thc, nonblocking_streams):
     _busy(thc, w, 40)                                  # stream B is busy for a while ...
     r.copy(x)                                          # ... and only then reads x
     del x                                              # freed while B's copy has not even started
-    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 1
+    pending = lib.THCAmd_cachingAllocatorPendingBlocks()
     lib.THCState_setCurrentStream(st, sa)
     z = thc.Tensor("float").resize((n,))
-    assert z.data_ptr() != px                          # not handed out while B may still read it
+    pz = z.data_ptr()
+    if _still_busy(hip, sb):
+        assert pending == 1 and pz != px               # not handed out while B may still read it
     z.fill(7.0)                                        # runs on A at once, concurrently with B
     assert hip.hipStreamSynchronize(sa) == 0 and hip.hipStreamSynchronize(sb) == 0
     assert np.all(r.numpy() == 1.0)
@@ -128,8 +141,10 @@ def test_record_stream_entry_point_and_resize_on_another_stream(thc, nonblocking
     lib.THCCachingAllocator_recordStream(C.c_void_p(py), sb)
     lib.THCState_setCurrentStream(st, sa)
     del y
-    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 1
-    assert thc.Tensor("float").resize((1 << 22,)).data_ptr() != py
+    pending = lib.THCAmd_cachingAllocatorPendingBlocks()
+    other = thc.Tensor("float").resize((1 << 22,))
+    if _still_busy(hip, sb):
+        assert pending == 1 and other.data_ptr() != py
     assert hip.hipStreamSynchronize(sb) == 0
     assert lib.THCAmd_cachingAllocatorPendingBlocks() == 0
     # resize on a stream other than the block's own: the old block is copied from on B, then freed
@@ -143,10 +158,41 @@ def test_record_stream_entry_point_and_resize_on_another_stream(thc, nonblocking
     assert t.data_ptr() != pt
     lib.THCState_setCurrentStream(st, sa)
     q = thc.Tensor("float").resize((1 << 20,))
-    assert q.data_ptr() != pt                          # the source of B's pending copy is not recycled on A
+    pq = q.data_ptr()
+    if _still_busy(hip, sb):
+        assert pq != pt                                # the source of B's pending copy is not recycled on A
     q.fill(-1.0)
     assert hip.hipStreamSynchronize(sa) == 0 and hip.hipStreamSynchronize(sb) == 0
     assert np.array_equal(t.numpy()[:1 << 20], np.arange(1 << 20, dtype=np.float32))
+
+
+def test_no_alloc_entry_point_reports_its_input(thc, nonblocking_streams):
+    """THCudaTensor_sumallNoAlloc launches on the current stream without waiting: an input allocated
+    under stream A and summed on stream B must be held back when freed, like any other operand."""
+    hip, (sa, sb) = nonblocking_streams
+    lib, st = thc.lib(), thc.state()
+    lib.THCAmd_cachingAllocatorPendingBlocks.restype = C.c_size_t
+    n = (1 << 22) + 77
+    lib.THCState_setCurrentStream(st, sa)
+    x = thc.Tensor("float").resize((n,)).fill(0.5)
+    px = x.data_ptr()
+    assert hip.hipStreamSynchronize(sa) == 0
+    lib.THCState_setCurrentStream(st, sb)
+    w = thc.Tensor("float").resize((1 << 28,)).fill(0.0)
+    res = thc.Tensor("float").resize((1,)).fill(0.0)
+    _busy(thc, w, 30)
+    x.sumall_no_alloc(res)                             # queued on B behind the busy work
+    del x
+    pending = lib.THCAmd_cachingAllocatorPendingBlocks()
+    lib.THCState_setCurrentStream(st, sa)
+    z = thc.Tensor("float").resize((n,))
+    pz = z.data_ptr()
+    if _still_busy(hip, sb):
+        assert pending == 1 and pz != px
+    z.fill(-3.0)                                       # would corrupt the sum if the block had been handed out
+    assert hip.hipStreamSynchronize(sa) == 0 and hip.hipStreamSynchronize(sb) == 0
+    assert res.numpy().tolist() == [0.5 * n]
+    assert lib.THCAmd_cachingAllocatorPendingBlocks() == 0
 
 
 def test_host_copy_waits_for_a_nonblocking_stream(thc, nonblocking_streams):

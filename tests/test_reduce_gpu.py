@@ -603,6 +603,12 @@ def test_reductions_beyond_2pow31_elements(thc):
     want_total = float(block.astype(np.int64).sum() * reps + block[:rest].astype(np.int64).sum())
     assert abs(want_total) < 2 ** 24
     assert x.sumall() == want_total
+    # the entry point that allocates nothing serves up to 2^32 elements (more workgroups than sumall uses
+    # beyond 2^31: another order of the partial sums, which integer-valued data does not notice)
+    res = thc.Tensor("float").resize((1,)).fill(-1.0)
+    x.sumall_no_alloc(res)
+    thc.synchronize()
+    assert res.numpy().tolist() == [want_total]
     # 1-D max / min with index: a long single row, split over workgroups and folded
     hi = (1 << 31) + 1234
     for pos in (hi, hi + 4096 + 3):

@@ -132,3 +132,42 @@ def test_concurrent_host_threads_on_their_own_streams(thc, streams):
     for s in extra:
         hip.hipStreamDestroy(s)
     assert not errors, errors
+
+
+def test_async_copies_between_pinned_host_memory_and_a_stream(thc, streams):
+    """copyAsyncFromHost / copyAsyncToHost (the raw-pointer forms of copyAsyncCPU / copyAsyncCuda,
+    generic/THCTensorCopy.c:104-164): queued on the current stream in order with the kernels around
+    them, no host wait; contiguity and size are argument errors as in the reference."""
+    hip, (s1, _) = streams
+    lib, st = thc.lib(), thc.state()
+    hip.hipHostMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_uint]
+    hip.hipHostFree.argtypes = [C.c_void_p]
+    n = (1 << 20) + 3
+    src, dst = C.c_void_p(), C.c_void_p()
+    assert hip.hipHostMalloc(C.byref(src), 4 * n, 0) == 0 and hip.hipHostMalloc(C.byref(dst), 4 * n, 0) == 0
+    try:
+        hsrc = np.ctypeslib.as_array(C.cast(src, C.POINTER(C.c_float)), (n,))
+        hdst = np.ctypeslib.as_array(C.cast(dst, C.POINTER(C.c_float)), (n,))
+        rng = np.random.default_rng(63)
+        hsrc[:] = rng.standard_normal(n).astype(np.float32)
+        hdst[:] = -1.0
+        lib.THCState_setCurrentStream(st, s1)
+        t = thc.Tensor("float").resize((n,))
+        t.copy_async_from_host(src.value, n)             # H2D, then a kernel, then D2H: one stream, in order
+        t.mul(t, 2.0)
+        t.copy_async_to_host(dst.value, n)
+        assert hip.hipStreamSynchronize(s1) == 0
+        assert_bit_equal(hdst, hsrc * np.float32(2.0))
+        with pytest.raises(thc.THCError, match="sizes do not match"):
+            t.copy_async_from_host(src.value, n - 1)
+        m = thc.Tensor("float").resize((64, 32))
+        with pytest.raises(thc.THCError, match="Target tensor must be contiguous"):
+            m.t().copy_async_from_host(src.value, 64 * 32)
+        with pytest.raises(thc.THCError, match="Source tensor must be contiguous"):
+            m.t().copy_async_to_host(dst.value, 64 * 32)
+        thc.Tensor("float").copy_async_from_host(src.value, 0)      # empty: nothing to do
+    finally:
+        lib.THCState_setCurrentStream(st, None)
+        thc.synchronize()
+        hip.hipHostFree(src)
+        hip.hipHostFree(dst)
