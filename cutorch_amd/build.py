@@ -22,7 +22,7 @@ SOURCES = ["general.cpp", "tensor.cpp", "math.cpp", "math_wide.cpp", "caching_al
            "reduce_w_i16.hip", "reduce_w_i32.hip", "reduce_w_i64.hip", "reduce_w_f64.hip", "scan.hip", "no_alloc.hip", "convert.hip", "apply_cmp_f.hip", "apply_w_u8.hip",
            "apply_rawmath_u32u64.hip", "apply_rawmath_f64.hip", "apply_w_i8.hip", "apply_w_i16.hip", "apply_w_i32.hip", "apply_w_i64.hip", "apply_w_f64.hip",
            "apply_cvt_u8.hip", "apply_cvt_i8.hip", "apply_cvt_i16.hip", "apply_cvt_i32.hip", "apply_cvt_i64.hip",
-           "apply_cvt_f16.hip", "apply_cvt_f32.hip", "apply_cvt_f64.hip"]
+           "apply_cvt_f16.hip", "apply_cvt_f32.hip", "apply_cvt_f64.hip", "apply_policy.hip"]
 HEADERS = ["common.hpp", "layout.hpp", "device_util.hpp", os.path.join("..", "..", "include", "THC.h")]   # every source
 APPLY_HEADERS = ["apply_plan.hpp", "apply_impl.hpp", "apply_ldstile.hpp", "apply_wide.hpp"]   # apply*.hip, convert.hip
 REDUCE_HEADERS = ["reduce_plan.hpp", "reduce_impl.hpp"]                                       # reduce*.hip, scan.hip, no_alloc.hip

@@ -225,7 +225,8 @@ struct OpMath2 {
 // ------------------------------------------------------------------------
 // TOut differs from T only for ops that change the element type (comparisons
 // into a Byte tensor); the output pack then has VEC elements of TOut.
-template <typename T, typename Op, int VEC, int UNROLL, bool NT, typename TOut = T, bool NTS = false>
+// ST: how the output is stored: 0 plain, 1 nontemporal, 2 device scope (buffer_store_pack).
+template <typename T, typename Op, int VEC, int UNROLL, bool NT, typename TOut = T, int ST = 0>
 __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T* in0, const T* in1,
                                                               const T* in2, uint64_t n, Op op) {
   using P = Pack<T, VEC>;
@@ -262,7 +263,7 @@ __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T
           PO r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = f(a[u].v[e], b[u].v[e], c[u].v[e]);
-          buffer_store_pack<NTS>(r, ro, off);
+          buffer_store_pack<ST>(r, ro, off);
         }
       }
       return;
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(kBlock) void apply_contig_kernel(TOut* out, const T
           PO r;
 #pragma unroll
           for (int e = 0; e < VEC; ++e) r.v[e] = f(a[u].v[e], b[u].v[e], c[u].v[e]);
-          store_pack<NTS>(reinterpret_cast<PO*>(out) + i, r);
+          store_pack<ST != 0>(reinterpret_cast<PO*>(out) + i, r);
         }
       }
     }
@@ -1091,20 +1092,6 @@ inline bool pack_aligned(const Plan& pl, int k) {
   return (reinterpret_cast<uintptr_t>(pl.ptr[k]) & (bytes - 1)) == 0;
 }
 
-// Whether an output of `bytes` goes out with the streaming (nontemporal) hint.
-// Plain stores leave the output in the L2s and the 256 MiB memory-side cache,
-// where a consumer launched next finds it; the dirty lines are written back
-// when the kernel ends. Measured with producer -> consumer pairs of flat fp32
-// kernels over rotating buffers: outputs up to 32 MiB are 3-8 % faster with
-// plain stores, 64 MiB is even, from 128 MiB on the streaming hint wins by
-// 6-8 % (and by 9 % on a transposed 256 MiB addcmul). A timing loop that
-// rewrites ONE output buffer that fits the memory-side cache flatters plain
-// stores (the writes never reach HBM).
-inline bool streaming_store(const char* knob, int64_t bytes) {
-  const int64_t k = tuning(knob, -1);
-  return k >= 0 ? k != 0 : bytes >= (int64_t(64) << 20);
-}
-
 inline int grid_for(THCState* s, int64_t work_items, int per_block, const char* key, int default_per_cu) {
   const int64_t blocks = (work_items + per_block - 1) / per_block;
   const int64_t cap = (int64_t)num_compute_units(s) * tuning(key, default_per_cu);
@@ -1130,13 +1117,27 @@ void launch_contig(THCState* s, const Plan& pl, Op op) {
   const bool nt = (int64_t)n * (int64_t)sizeof(T) * pl.nops >= tuning("apply.contig.nt_bytes", 8 << 20);
   // (a pure write stream, fill, is not helped by the hint: 1 GiB 176 us plain, 186 us streaming)
   const bool nts = Op::NIN > 0 && streaming_store("apply.contig.nt_store", (int64_t)n * (int64_t)sizeof(TOut));
+  // streaming stores below 256 MiB carry the device-scope bit, larger ones the nontemporal hint (buffer_store_pack)
+  const int64_t sc1Knob = tuning("apply.contig.sc1_store", -1);
+  const bool sc1 = sc1Knob >= 0 ? sc1Knob != 0 : (int64_t)n * (int64_t)sizeof(TOut) < (int64_t(256) << 20);
   const int64_t unroll = tuning("apply.contig.unroll", 2);
+  if constexpr (std::is_same<T, float>::value && std::is_same<Op, OpAdd>::value && std::is_same<TOut, float>::value) {
+    const int64_t policy = tuning("apply.contig.policy", -1);
+    if (policy >= 0 && vec &&
+        launch_add_policy(st, (int)policy, out, i0, i1, n, (int)unroll, tuning("apply.contig.max_grid", 1 << 20))) {
+      note_kernel("contig-policy");
+      return;
+    }
+  }
   auto launch = [&](auto uTag) {
     constexpr int UU = decltype(uTag)::value;
     const int64_t blk = (packs + kBlock * UU - 1) / (kBlock * UU);
     const int gr = (int)std::max<int64_t>(1, std::min<int64_t>(blk, tuning("apply.contig.max_grid", 1 << 20)));
-    if (vec && nt && nts)
-      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut, true>), dim3(gr), dim3(kBlock),
+    if (vec && nt && nts && sc1)
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut, 2>), dim3(gr), dim3(kBlock),
+                         0, st, out, i0, i1, i2, n, op);
+    else if (vec && nt && nts)
+      hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut, 1>), dim3(gr), dim3(kBlock),
                          0, st, out, i0, i1, i2, n, op);
     else if (vec && nt)
       hipLaunchKernelGGL((apply_contig_kernel<T, Op, VEC, UU, true, TOut>), dim3(gr), dim3(kBlock),

@@ -232,7 +232,20 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
         for (int r = 0; r < NP_S; ++r) {
           const int qi = (int)lyp + r * ROWS_P;
           if constexpr (WIN) {
-            *reinterpret_cast<RAW*>(slab + qi * PITCH_S + S::skew(qi) + lxp * VEC) = v[k][r];
+            // word by word: the row starts at a multiple of 4 bytes, not of 16, and a 16-byte LDS
+            // write there stalls the LDS pipeline (SQ_LDS_UNALIGNED_STALL)
+            T* at = slab + qi * PITCH_S + S::skew(qi) + lxp * VEC;
+            if constexpr (sizeof(RAW) == 16) {
+              // (may_alias: the slab is read back as elements of T)
+              typedef uint32_t __attribute__((may_alias)) Word;
+              Word* w = reinterpret_cast<Word*>(at);
+              w[0] = v[k][r].x;
+              w[1] = v[k][r].y;
+              w[2] = v[k][r].z;
+              w[3] = v[k][r].w;
+            } else {
+              *reinterpret_cast<RAW*>(at) = v[k][r];
+            }
           } else {
             int first = (int)(lxp * VEC);
             if (!ALIGNED) first -= mis_in(staged_row(t, k, qi));

@@ -41,4 +41,9 @@ bool apply_cmp(THCState* s, Plan& pl, bool sameShape, const ApplyDesc& d, bool d
 template <typename D, typename S>
 void apply_convert(THCState* s, Plan& pl, bool sameShape);
 
+// Probe (apply_policy.hip): the contiguous float add with one of the other cache-policy settings of
+// its loads and stores, chosen by the knob "apply.contig.policy". False = no such variant.
+bool launch_add_policy(hipStream_t st, int policy, float* out, const float* a, const float* b, uint64_t n, int unroll,
+                       int64_t maxGrid);
+
 }  // namespace thc

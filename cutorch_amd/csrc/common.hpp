@@ -146,6 +146,20 @@ void note_kernel(const char* name);  // for THCAmd_lastKernel
 // of THCudaTensor_sumallNoAlloc (so that the entry point itself finds it ready).
 void no_alloc_setup();
 long tuning(const char* key, long fallback);
+
+// Whether an output of `bytes` goes out as streaming stores (store_pack<true>, device_util.hpp).
+// Plain stores leave the output in the L2s and the 256 MiB memory-side cache,
+// where a consumer launched next finds it; the dirty lines are written back
+// when the kernel ends. Measured with producer -> consumer pairs of flat fp32
+// kernels over rotating buffers: outputs up to 32 MiB are 3-8 % faster with
+// plain stores, 64 MiB is even, from 128 MiB on streaming stores win by
+// 6-8 % (and by 9 % on a transposed 256 MiB addcmul). A timing loop that
+// rewrites ONE output buffer that fits the memory-side cache flatters plain
+// stores (the writes never reach HBM).
+inline bool streaming_store(const char* knob, int64_t bytes) {
+  const long k = tuning(knob, -1);
+  return k >= 0 ? k != 0 : bytes >= (int64_t(64) << 20);
+}
 bool force_64bit_index();
 
 // --------------------------------------------------------- storage/tensor --

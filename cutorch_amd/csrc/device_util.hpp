@@ -57,6 +57,19 @@ __device__ __forceinline__ P load_pack(const P* p) {
   }
   return *p;
 }
+// Streaming stores. On buffer instructions (buffer_store_pack below) they carry the device-scope bit
+// (sc1) of the cache policy, which makes the L2 write the data through instead of keeping dirty
+// lines: c = a + b on 3 x 64 MiB of fp32 with nontemporal loads runs at 0.79 of the HBM peak with
+// plain stores, 0.80 with nontemporal stores and 0.86 with sc1 stores (sc0 makes no difference, sc1
+// together with nt loses the gain, the same bit on two 8-byte stores per lane fell to 0.53; loads are
+// indifferent to sc0 / sc1). The gain belongs to working sets of about the size of the 256 MiB
+// memory-side cache (3 x 64 MiB operands 0.78 -> 0.86, a 2 x 128 MiB half-precision exp 0.79 -> 0.89);
+// with operands of 256 MiB and more it is within +-2 % of nontemporal stores, which such outputs
+// keep. A stronger scope than a store needs is always allowed. No builtin puts
+// that bit on a 16-byte store through a pointer, and the instruction written out as inline assembly
+// inside the tiled kernels made the compiler give up on address-space inference for the whole kernel
+// (LDS and global accesses turned into flat ones, the argument block went to scratch), so stores
+// through pointers take the nontemporal hint.
 template <bool NT, typename P>
 __device__ __forceinline__ void store_pack(P* p, const P& v) {
   if (NT) {
@@ -90,7 +103,7 @@ using BufferRsrc = __amdgpu_buffer_rsrc_t;
 __device__ __forceinline__ BufferRsrc make_rsrc(const void* p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
 }
-// 16-byte packs, nontemporal hint on the load; the store takes it on request.
+// 16-byte packs, nontemporal hint on the load; the store carries sc1 on request (see store_pack).
 template <typename P>
 __device__ __forceinline__ P buffer_load_pack(BufferRsrc r, uint32_t byteOffset) {
   static_assert(sizeof(P) == 16, "16-byte packs");
@@ -100,13 +113,14 @@ __device__ __forceinline__ P buffer_load_pack(BufferRsrc r, uint32_t byteOffset)
   __builtin_memcpy(&out, &v, 16);
   return out;
 }
-template <bool NT, typename P>
+// ST: 0 plain, 1 nontemporal, 2 device scope (sc1).
+template <int ST, typename P>
 __device__ __forceinline__ void buffer_store_pack(const P& v, BufferRsrc r, uint32_t byteOffset) {
   static_assert(sizeof(P) == 16, "16-byte packs");
   typedef unsigned raw __attribute__((ext_vector_type(4)));
   raw x;
   __builtin_memcpy(&x, &v, 16);
-  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byteOffset, 0, NT ? 2 : 0);
+  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byteOffset, 0, ST == 2 ? /*sc1*/ 16 : (ST == 1 ? /*nt*/ 2 : 0));
 }
 
 template <typename T>
@@ -233,7 +247,8 @@ struct RunPrefetch {
 // The way back: `count` elements held in LDS (element i at run[i], any
 // alignment) go to `dst` as 16-byte packs aligned on dst; the packs that
 // straddle the run's ends are stored element by element, so nothing outside
-// [dst, dst + count) is written.
+// [dst, dst + count) is written. (Plain stores: with the nontemporal hint renorm of 8192 x 8192 fell
+// from 0.76 to 0.72 of peak and the scan of 10-element rows from 0.80 to 0.73.)
 template <typename T>
 __device__ __forceinline__ void write_run_from_lds(T* dst, const T* run, uint32_t count) {
   constexpr int VEC = 16 / sizeof(T);

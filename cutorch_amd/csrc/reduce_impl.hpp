@@ -554,7 +554,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
                                                                  TOut* __restrict__ out,
                                                                  OuterArgs<I> oa, I numRows, I R,
                                                                  uint32_t rowsPerBlock, uint32_t G,
-                                                                 Epi<typename F::A> epi, F f) {
+                                                                 uint32_t quadMin, Epi<typename F::A> epi, F f) {
   using A = typename F::A;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   TIn* lds = reinterpret_cast<TIn*>(lds_raw);
@@ -581,31 +581,50 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
       if constexpr (F::kCentred) c = acc_up<A>(out[outOff]);
       A acc = f.init();
       if constexpr (sizeof(TIn) == 2) {
-        // 2-byte elements are read from LDS two at a time: the row's pairs start at its first
-        // even element index; a leading and a trailing single element go to lane 0
-        const uint32_t start = mis + r * (uint32_t)R, head = start & 1u;
-        const uint32_t npairs = ((uint32_t)R - head) >> 1;
-        const uint32_t* words = reinterpret_cast<const uint32_t*>(lds) + ((start + head) >> 1);
-        auto take = [&](uint32_t bits) {
-          const uint16_t h = (uint16_t)bits;
-          TIn x;
-          __builtin_memcpy(&x, &h, 2);
-          acc = f.combine(acc, f.modify(acc_up<A>(x), c));
-        };
-        if (head && lane == 0) acc = f.combine(acc, f.modify(acc_up<A>(row[0]), c));
-        for (uint32_t q = lane; q < npairs; q += 8 * G) {
-          uint32_t w[8];
+        // 2-byte elements are read from LDS two or four at a time (W, one 4- or 8-byte read): the
+        // row's words start at its first element whose LDS index is a multiple of W; the elements
+        // before the first word and after the last one go to lane 0
+        auto by_words = [&](auto wTag) {
+          constexpr uint32_t W = decltype(wTag)::value;
+          using Word = typename std::conditional<W == 2, uint32_t, uint2>::type;
+          const uint32_t start = mis + r * (uint32_t)R;
+          const uint32_t head = min((W - (start & (W - 1))) & (W - 1), (uint32_t)R);
+          const uint32_t nw = ((uint32_t)R - head) / W;
+          const Word* words = reinterpret_cast<const Word*>(lds + start + head);
+          auto take = [&](uint32_t bits) {
+            const uint16_t h = (uint16_t)bits;
+            TIn x;
+            __builtin_memcpy(&x, &h, 2);
+            acc = f.combine(acc, f.modify(acc_up<A>(x), c));
+          };
+          if (lane == 0)
+            for (uint32_t j = 0; j < head; ++j) acc = f.combine(acc, f.modify(acc_up<A>(row[j]), c));
+          for (uint32_t q = lane; q < nw; q += 8 * G) {
+            Word w[8];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, npairs - 1)];
+            for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, nw - 1)];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            if (q + u * G < npairs) {
-              take(w[u]);
-              take(w[u] >> 16);
+            for (int u = 0; u < 8; ++u) {
+              if (q + u * G < nw) {
+                if constexpr (W == 2) {
+                  take(w[u]);
+                  take(w[u] >> 16);
+                } else {
+                  take(w[u].x);
+                  take(w[u].x >> 16);
+                  take(w[u].y);
+                  take(w[u].y >> 16);
+                }
+              }
             }
           }
-        }
-        if (head + 2 * npairs < (uint32_t)R && lane == 0) acc = f.combine(acc, f.modify(acc_up<A>(row[(uint32_t)R - 1]), c));
+          if (lane == 0)
+            for (uint32_t j = head + W * nw; j < (uint32_t)R; ++j) acc = f.combine(acc, f.modify(acc_up<A>(row[j]), c));
+        };
+        if ((uint32_t)R >= quadMin)
+          by_words(std::integral_constant<uint32_t, 4>{});
+        else
+          by_words(std::integral_constant<uint32_t, 2>{});
       } else {
         // batches of 8 LDS reads (past the row's end: its last element, not used), then the
         // dependent chain: one LDS latency per batch instead of one per element
@@ -628,7 +647,7 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_lds_kernel(const TIn* __re
 template <typename T, typename I, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
     const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI, OuterArgs<I> oa,
-    OuterArgs<I> oaIdx, I numRows, I R, uint32_t rowsPerBlock, uint32_t G) {
+    OuterArgs<I> oaIdx, I numRows, I R, uint32_t rowsPerBlock, uint32_t G, uint32_t quadMin) {
   using A = typename Acc<T>::type;
   using O = PairOrder<IS_MAX, A>;
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -699,34 +718,52 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_index_lds_kernel(
       } else if ((uint32_t)R < 16) {  // (most of a 16-slot batch would idle)
         by_element();
       } else {
-        // 2-byte elements are read from LDS two at a time (see reduce_rows_lds_kernel); a lane's
-        // candidates still come in index order: the leading single element, its pairs, the trailing one
-        const uint32_t start = mis + r * (uint32_t)R, head = start & 1u;
-        const uint32_t npairs = ((uint32_t)R - head) >> 1;
-        const uint32_t* words = reinterpret_cast<const uint32_t*>(lds) + ((start + head) >> 1);
-        auto half_of = [](uint32_t bits) {
-          const uint16_t h = (uint16_t)bits;
-          T x;
-          __builtin_memcpy(&x, &h, 2);
-          return acc_up<A>(x);
-        };
-        if (head && lane == 0) offer(acc_up<A>(row[0]), 0u);
-        for (uint32_t q = lane; q < npairs; q += 8 * G) {
-          uint32_t w[8];
+        // 2-byte elements are read from LDS two or four at a time (see reduce_rows_lds_kernel); a lane's
+        // candidates still come in index order: the elements before its first word, its words, the rest
+        auto by_words = [&](auto wTag) {
+          constexpr uint32_t W = decltype(wTag)::value;
+          using Word = typename std::conditional<W == 2, uint32_t, uint2>::type;
+          const uint32_t start = mis + r * (uint32_t)R;
+          const uint32_t head = min((W - (start & (W - 1))) & (W - 1), (uint32_t)R);
+          const uint32_t nw = ((uint32_t)R - head) / W;
+          const Word* words = reinterpret_cast<const Word*>(lds + start + head);
+          auto half_of = [](uint32_t bits) {
+            const uint16_t h = (uint16_t)bits;
+            T x;
+            __builtin_memcpy(&x, &h, 2);
+            return acc_up<A>(x);
+          };
+          if (lane == 0)
+            for (uint32_t j = 0; j < head; ++j) offer(acc_up<A>(row[j]), j);
+          for (uint32_t q = lane; q < nw; q += 8 * G) {
+            Word w[8];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, npairs - 1)];
-          A a[16];
+            for (int u = 0; u < 8; ++u) w[u] = words[min(q + u * G, nw - 1)];
+            A a[8 * W];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const bool have = q + u * G < npairs;
-            a[2 * u] = have ? half_of(w[u]) : O::worst();
-            a[2 * u + 1] = have ? half_of(w[u] >> 16) : O::worst();
+            for (int u = 0; u < 8; ++u) {
+              const bool have = q + u * G < nw;
+              if constexpr (W == 2) {
+                a[2 * u] = have ? half_of(w[u]) : O::worst();
+                a[2 * u + 1] = have ? half_of(w[u] >> 16) : O::worst();
+              } else {
+                a[4 * u] = have ? half_of(w[u].x) : O::worst();
+                a[4 * u + 1] = have ? half_of(w[u].x >> 16) : O::worst();
+                a[4 * u + 2] = have ? half_of(w[u].y) : O::worst();
+                a[4 * u + 3] = have ? half_of(w[u].y >> 16) : O::worst();
+              }
+            }
+            const uint32_t live = W * min(8u, (nw - q + G - 1) / G);
+            offer_batch(a, [&](uint32_t s2) { return head + W * (q + (s2 / W) * G) + (s2 % W); }, live,
+                        std::integral_constant<int, 8 * (int)W>{});
           }
-          const uint32_t live = 2 * min(8u, (npairs - q + G - 1) / G);
-          offer_batch(a, [&](uint32_t s2) { return head + 2 * (q + (s2 >> 1) * G) + (s2 & 1u); }, live,
-                      std::integral_constant<int, 16>{});
-        }
-        if (head + 2 * npairs < (uint32_t)R && lane == 0) offer(acc_up<A>(row[(uint32_t)R - 1]), (uint32_t)R - 1);
+          if (lane == 0)
+            for (uint32_t j = head + W * nw; j < (uint32_t)R; ++j) offer(acc_up<A>(row[j]), j);
+        };
+        if ((uint32_t)R >= quadMin)
+          by_words(std::integral_constant<uint32_t, 4>{});
+        else
+          by_words(std::integral_constant<uint32_t, 2>{});
       }
       for (uint32_t o = G >> 1; o > 0; o >>= 1) {
         const A ov = shfl_xor_any(bv, o);
@@ -1897,7 +1934,7 @@ void launch_rows_pass(THCState* s, const TIn* in, TOut* out, typename F::A* part
 // fp32 rows, 3.5 against 5.5 on 64-element ones), up to 8 KiB otherwise.
 template <typename T>
 bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPerBlock, uint32_t& G,
-                   size_t& ldsBytes) {
+                   size_t& ldsBytes, uint32_t* quadMin = nullptr, bool quadWholeOnly = false) {
   if (!tuning("reduce.rows.lds", 1) || g.sR != 1 || g.R < 1 || g.outElems < 1) return false;
   int64_t run = g.R;
   for (int d = g.in.dims - 1; d >= 0; --d) {
@@ -1928,8 +1965,15 @@ bool plan_rows_lds(THCState* s, const ReduceGeom& g, bool vec, uint32_t& rowsPer
   // power of two with the 32 LDS banks put the lanes of a step on few banks (32-element rows, a
   // lane per row: 0.27), so such rows get up to gcd(pitch in words, 32) lanes (8 at most) as long as
   // a lane keeps 8 elements (fewer is slower than the conflicts: 8-element rows 0.17 against 0.65).
-  // (2-byte elements are read from LDS in pairs: the unit below is one LDS read)
-  const uint64_t reads = sizeof(T) == 2 ? ((uint64_t)g.R + 1) / 2 : (uint64_t)g.R;
+  // (2-byte elements are read from LDS in pairs, or four at a time from `quadMin` elements on where
+  // the kernel can do that: the unit below is one LDS read)
+  const int64_t qmin = tuning("reduce.rows.lds_quad_min", 32);
+  // (max / min take four at a time only when the rows are whole quads: the elements before the first and
+  // after the last aligned quad are offered one by one, and with them 33-, 127- and 255-element rows lost
+  // 6-18 % where 32..224-element rows that are multiples of 8 gained 15-40 %; sums gain either way)
+  const bool quad = sizeof(T) == 2 && quadMin != nullptr && g.R >= qmin && (!quadWholeOnly || g.R % 4 == 0);
+  if (quadMin) *quadMin = quad ? 0u : 0xffffffffu;   // the kernel compares the row length with it
+  const uint64_t reads = sizeof(T) == 2 ? ((uint64_t)g.R + (quad ? 3 : 1)) / (quad ? 4 : 2) : (uint64_t)g.R;
   int64_t perLane = tuning("reduce.rows.lds_elems_per_lane", 0);
   if (perLane <= 0) perLane = reads <= 112 ? 32 : 16;
   G = pow2_ceil(reads / (uint64_t)perLane + 1);
@@ -1969,13 +2013,13 @@ void run_rows(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi<typenam
     chunk = (chunk + 63) / 64 * 64;  // keeps chunks pack-aligned
     S = (g.R + chunk - 1) / chunk;
   }
-  uint32_t ldsRows = 0, ldsG = 0;
+  uint32_t ldsRows = 0, ldsG = 0, quadMin = 0;
   size_t ldsBytes = 0;
-  if (S == 1 && plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
+  if (S == 1 && plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes, &quadMin)) {
     const int64_t blocks = (rows + ldsRows - 1) / ldsRows;
     const int grid = capped_grid(s, blocks, "reduce.rows.lds_blocks_per_cu", 64);
     hipLaunchKernelGGL((reduce_rows_lds_kernel<T, T, F, I>), dim3(grid), dim3(kBlock), ldsBytes,
-                       current_stream(s), in, out, oa, (I)rows, (I)g.R, ldsRows, ldsG, epi, f);
+                       current_stream(s), in, out, oa, (I)rows, (I)g.R, ldsRows, ldsG, quadMin, epi, f);
     note_kernel("rows-lds");
     return;
   }
@@ -2292,12 +2336,12 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
     OuterArgs<I> oaIdx = make_outer<I>(g.in, g.idx, nd);
     const int64_t rows = g.outElems;
     {
-      uint32_t ldsRows = 0, ldsG = 0;
+      uint32_t ldsRows = 0, ldsG = 0, quadMin = 0;
       size_t ldsBytes = 0;
-      if (plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes)) {
+      if (plan_rows_lds<T>(s, g, vec, ldsRows, ldsG, ldsBytes, &quadMin, true)) {
         const int grid = capped_grid(s, (rows + ldsRows - 1) / ldsRows, "reduce.rows.lds_blocks_per_cu", 64);
         hipLaunchKernelGGL((reduce_rows_index_lds_kernel<T, I, IS_MAX>), dim3(grid), dim3(kBlock),
-                           ldsBytes, st, in, outV, outI, oa, oaIdx, (I)rows, (I)g.R, ldsRows, ldsG);
+                           ldsBytes, st, in, outV, outI, oa, oaIdx, (I)rows, (I)g.R, ldsRows, ldsG, quadMin);
         note_kernel("rows-index-lds");
         return;
       }

@@ -446,6 +446,176 @@ __global__ __launch_bounds__(kBlock) void scan_chunk_totals_kernel(
   }
 }
 
+// Long scans with few columns in ONE read of the input (4-byte accumulators, at most kBlock
+// columns). The chunks of rows are dealt to a grid no larger than what is resident, chunk c to
+// workgroup c % grid, every workgroup taking its chunks in increasing order. A chunk publishes its
+// column totals, looks back over the chunks before it for the carry, publishes its inclusive prefix
+// and scans. What is published is one 64-bit word per chunk and column, (kind << 32) | value bits,
+// kind 1 = the chunk's own total, 2 = the inclusive prefix up to and including the chunk, written
+// and read with relaxed device-scope atomics: kind and value arrive together, so no fence is
+// needed. The carry is folded left to right from the nearest published prefix, a prefix met on the
+// way replacing the running value (it is that value, bit for bit), so the result does not depend on
+// what happened to be published when: same bits on every run.
+// No wait is unbounded: after `spinLimit` polls of a word that is still empty the reader computes
+// that chunk's column total itself from the input, in the owner's order of operations. A grid that
+// is not resident all at once (the GPU shared with other work) therefore still ends.
+constexpr uint32_t kKindTotal = 1, kKindPrefix = 2;
+
+__global__ __launch_bounds__(kBlock) void scan_clear_words_kernel(uint64_t* words, uint64_t n) {
+  for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) words[i] = 0;
+}
+
+template <typename T, typename Op>
+__global__ __launch_bounds__(kBlock) void scan_lookback_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                                               uint64_t* words, uint64_t outer, uint64_t R,
+                                                               uint32_t inner, uint64_t S, uint32_t chunkRows,
+                                                               uint32_t dataBytes, uint32_t spinLimit) {
+  using A = typename ScanAcc<T>::type;
+  static_assert(sizeof(A) == 4, "value and kind share a 64-bit word");
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  __shared__ A carryS[kBlock];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+  A* part = reinterpret_cast<A*>(lds_raw + dataBytes);  // kBlock band totals behind the staged chunk
+  const uint64_t numChunks = outer * S;
+  auto locate = [&](uint64_t blk, uint64_t& start, uint32_t& rows) {
+    const uint64_t o = blk / S, r0 = (blk - o * S) * chunkRows;
+    rows = (uint32_t)min((uint64_t)chunkRows, R - r0);
+    start = (o * R + r0) * inner;
+  };
+  // bands of rows that share a column (as in scan_slab_kernel): P threads per column
+  auto bands = [&](uint32_t rows, uint32_t& P, uint32_t& band) {
+    P = min(rows, kBlock / inner);
+    band = (rows + P - 1) / P;
+  };
+  auto publish = [&](uint64_t blk, uint32_t c, uint32_t kind, A v) {
+    uint32_t bits;
+    __builtin_memcpy(&bits, &v, 4);
+    __hip_atomic_store(words + blk * inner + c, ((uint64_t)kind << 32) | bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  // kind and value of chunk k, column c; a word that stays empty is replaced by the total computed here
+  auto fetch = [&](uint64_t k, uint32_t c, uint32_t& kind) -> A {
+    uint64_t w = 0;
+    for (uint32_t spin = 0; spin <= spinLimit; ++spin) {
+      w = __hip_atomic_load(words + k * inner + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)(w >> 32) != 0) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+    kind = (uint32_t)(w >> 32);
+    A v;
+    if (kind != 0) {
+      const uint32_t bits = (uint32_t)w;
+      __builtin_memcpy(&v, &bits, 4);
+      return v;
+    }
+    uint64_t start;
+    uint32_t rows, P, band;
+    locate(k, start, rows);
+    bands(rows, P, band);
+    v = Op::id();
+    for (uint32_t p = 0; p < P; ++p) {
+      A acc = Op::id();
+      for (uint32_t r = min(rows, p * band), re = min(rows, r + band); r < re; ++r)
+        acc = Op::op(acc, scan_up<A>(in[start + (uint64_t)r * inner + c]));
+      v = p == 0 ? acc : Op::op(v, acc);
+    }
+    kind = kKindTotal;
+    return v;
+  };
+
+  RunPrefetch<T> next;
+  {
+    uint64_t start;
+    uint32_t rows;
+    if ((uint64_t)blockIdx.x < numChunks) {
+      locate(blockIdx.x, start, rows);
+      next.request(in + start, rows * inner);
+    }
+  }
+  for (uint64_t blk = blockIdx.x; blk < numChunks; blk += gridDim.x) {
+    uint64_t start;
+    uint32_t rows, P, band;
+    locate(blk, start, rows);
+    bands(rows, P, band);
+    const uint32_t count = rows * inner;
+    const uint32_t mis = next.commit(lds);
+    lds_barrier();
+    if (blk + gridDim.x < numChunks) {
+      uint64_t nstart;
+      uint32_t nrows;
+      locate(blk + gridDim.x, nstart, nrows);
+      next.request(in + nstart, nrows * inner);  // in flight while this chunk is scanned
+    }
+    const uint32_t p = threadIdx.x / inner, c = threadIdx.x - p * inner;
+    const uint32_t rb = min(rows, p * band), re = min(rows, rb + band);
+    T* col = lds + mis + c;
+    constexpr uint32_t B = 8;
+    if (p < P) {
+      A acc = Op::id();
+      uint32_t r = rb;
+      for (; r + B <= re; r += B) {
+        T x[B];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) acc = Op::op(acc, scan_up<A>(x[u]));
+      }
+      for (; r < re; ++r) acc = Op::op(acc, scan_up<A>(col[r * inner]));
+      part[p * inner + c] = acc;
+    }
+    lds_barrier();
+    if (threadIdx.x < inner) {
+      A total = part[c];
+      for (uint32_t q = 1; q < P; ++q) total = Op::op(total, part[q * inner + c]);
+      const uint64_t lo = blk - blk % S;  // first chunk of this slice
+      A carry = Op::id();
+      if (blk == lo) {
+        publish(blk, c, kKindPrefix, total);
+      } else {
+        publish(blk, c, kKindTotal, total);
+        // back to the nearest chunk with a published prefix (the slice's first chunk at the latest) ...
+        uint64_t j = blk - 1;
+        uint32_t kind;
+        A v = fetch(j, c, kind);
+        while (kind != kKindPrefix && j != lo) {
+          --j;
+          v = fetch(j, c, kind);
+        }
+        // ... and forward again, left to right
+        carry = v;
+        for (uint64_t k = j + 1; k < blk; ++k) {
+          v = fetch(k, c, kind);
+          carry = kind == kKindPrefix ? v : Op::op(carry, v);
+        }
+        publish(blk, c, kKindPrefix, Op::op(carry, total));
+      }
+      carryS[c] = carry;
+    }
+    lds_barrier();
+    if (p < P) {
+      A acc = carryS[c];
+      for (uint32_t q = 0; q < p; ++q) acc = Op::op(acc, part[q * inner + c]);  // bands before this one, in order
+      uint32_t r = rb;
+      for (; r + B <= re; r += B) {
+        T x[B];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) x[u] = col[(r + u) * inner];
+#pragma unroll
+        for (uint32_t u = 0; u < B; ++u) {
+          acc = Op::op(acc, scan_up<A>(x[u]));
+          col[(r + u) * inner] = scan_down<T>(acc);
+        }
+      }
+      for (; r < re; ++r) {
+        acc = Op::op(acc, scan_up<A>(col[r * inner]));
+        col[r * inner] = scan_down<T>(acc);
+      }
+    }
+    lds_barrier();
+    write_run_from_lds<T>(out + start, lds + mis, count);
+    lds_barrier();  // the buffer is refilled by the next chunk
+  }
+}
+
 uint32_t pow2_at_least(uint64_t x) {
   uint32_t p = 1;
   while (p < x && p < 64) p <<= 1;
@@ -464,6 +634,9 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
   constexpr int VECC = (sizeof(typename ScanAcc<T>::type) == 4 || kFull <= 4) ? kFull : 4;  // column kernel
   hipStream_t st = current_stream(s);
   const bool aligned = ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(in)) & 15u) == 0;
+  // large outputs go out as streaming stores (they cannot stay cache resident for a consumer)
+  const int64_t ntsKnob = tuning("scan.nt_store", -1);
+  const int streaming = (ntsKnob >= 0 ? ntsKnob != 0 : outer * R * inner * (int64_t)sizeof(T) >= (int64_t(64) << 20)) ? 1 : 0;
   // small slices: rows below 2 KiB, or R x inner slices up to 16 KiB
   const int64_t sliceBytes = R * inner * (int64_t)sizeof(T);
   if (tuning("scan.slab", 1) && sliceBytes <= (inner == 1 ? 2047 : 16384) && R > 0 && inner > 0) {
@@ -494,8 +667,35 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t plainBlocks = inner == 1 ? (outer + 3) / 4 : outer * ((packsPerRow + 15) / 16);
     if (!scratch) scratch = (char*)scratch_space(s, &scratchBytes);
     const size_t need = (((size_t)(outer * S * inner) * sizeof(A)) + 255) & ~size_t(255);
-    if (tuning("scan.chunked", 1) && rowBytes <= 32768 && S >= 4 && plainBlocks < (int64_t)num_compute_units(s) &&
-        2 * need <= scratchBytes) {
+    const bool longScan = tuning("scan.chunked", 1) && rowBytes <= 32768 && S >= 4 && plainBlocks < (int64_t)num_compute_units(s);
+    if constexpr (sizeof(A) == 4) {
+      // (a chunk and its neighbours' elements in its first and last pack must fit RunPrefetch: 32 KiB)
+      const int64_t chunkRows = std::max<int64_t>(1, std::min<int64_t>(run, 32768 - 32) / rowBytes);
+      const int64_t S = (R + chunkRows - 1) / chunkRows;
+      const size_t wordsBytes = (size_t)(outer * S * inner) * sizeof(uint64_t);
+      // (not in place: a reader that gives up waiting for a chunk's total computes it from the input)
+      if (longScan && tuning("scan.lookback", 0) && inner <= kBlock && rowBytes <= 32768 - 32 &&
+          wordsBytes <= scratchBytes && (const void*)out != (const void*)in) {
+        uint64_t* words = (uint64_t*)scratch;
+        const uint32_t dataElems = (uint32_t)(chunkRows * inner + 2 * kFull);
+        const size_t ldsData = ((size_t)dataElems * sizeof(T) + 15) & ~size_t(15);
+        const size_t ldsBytes = ldsData + kBlock * sizeof(A);
+        // no more workgroups than are resident at once: every chunk's predecessors are then running or done
+        int perCu = 0;
+        THC_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, scan_lookback_kernel<T, Op>, kBlock, ldsBytes));
+        perCu = (int)std::min<int64_t>(std::max(perCu, 1), tuning("scan.lookback_per_cu", 8));
+        const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * S, (int64_t)num_compute_units(s) * perCu));
+        const uint64_t nwords = (uint64_t)(outer * S * inner);
+        hipLaunchKernelGGL(scan_clear_words_kernel, dim3((unsigned)std::min<uint64_t>((nwords + kBlock - 1) / kBlock, 1024)),
+                           dim3(kBlock), 0, st, words, nwords);
+        hipLaunchKernelGGL((scan_lookback_kernel<T, Op>), dim3(grid), dim3(kBlock), ldsBytes, st, out, in, words,
+                           (uint64_t)outer, (uint64_t)R, (uint32_t)inner, (uint64_t)S, (uint32_t)chunkRows,
+                           (uint32_t)ldsData, (uint32_t)tuning("scan.lookback_spin", 4096));
+        note_kernel("scan-lookback");
+        return;
+      }
+    }
+    if (longScan && 2 * need <= scratchBytes) {
       A* totals = (A*)scratch;
       A* carries = (A*)(scratch + need);
       const uint32_t dataElems = (uint32_t)(chunkRows * inner + 2 * kFull);
@@ -512,9 +712,7 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
       return;
     }
   }
-  // large outputs go out with the streaming hint (they cannot stay cache resident for a consumer)
-  const int64_t ntsKnob = tuning("scan.nt_store", -1);
-  const int nts = (ntsKnob >= 0 ? ntsKnob != 0 : outer * R * inner * (int64_t)sizeof(T) >= (int64_t(64) << 20)) ? 1 : 0;
+  const int nts = streaming;
   if (inner == 1) {
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
     const int64_t blocks = (outer + (kBlock / 64) - 1) / (kBlock / 64);

@@ -459,6 +459,31 @@ def test_short_dense_rows_special_cases(thc, oracle):
     assert i[0] == 1 and i[7] == 21 and i[8] == 1 and i[9] == 6
     v = vals.numpy().ravel()
     assert v[0] == -np.inf and np.isnan(v[7]) and v[8] == 2.5 and v[9] == 7.0
+    # half rows, read from LDS four elements at a time (sums; max / min when the row length is a multiple
+    # of four): every residue of the row start modulo four (storage offsets 0..3), ties across the words
+    # of one batch, NaN, signed zeros
+    for R in (70, 72):
+        for off in range(4):
+            h = np.full((200, R), -np.inf, np.float16)
+            h[3, 41] = np.nan
+            h[4, :] = 1.5
+            h[5, 2] = h[5, 3] = h[5, R - 1] = 9.0
+            h[6, :] = -0.0
+            h[6, 17] = 0.0
+            h[7, R - 1] = 3.0
+            flat = thc.Tensor.from_numpy(np.concatenate([np.zeros(off, np.float16), h.ravel()]))
+            view = flat.view_as_strided(off, (200, R), (R, 1))
+            hv, hi = thc.Tensor("half"), thc.Tensor("long")
+            hv.max(hi, view, 1)
+            assert thc.last_kernel() == "rows-index-lds"
+            i = hi.numpy().ravel()
+            v = hv.numpy().ravel()
+            assert i[0] == 1 and i[3] == 42 and i[4] == 1 and i[5] == 3 and i[7] == R, (R, off, i[:8])
+            assert v[0] == -np.inf and np.isnan(v[3]) and v[4] == 1.5 and v[5] == 9.0 and v[7] == 3.0
+            assert i[6] == 1 and np.signbit(v[6]), (R, off, i[6], v[6])   # a zero keeps the sign of its first occurrence
+            ssum = thc.Tensor("half").sum(view, 1)
+            assert thc.last_kernel() == "rows-lds"
+            assert ssum.numpy().ravel()[4] == np.float16(1.5 * R) and ssum.numpy().ravel()[7] == -np.inf
     # rows dense in the input, outputs strided (a column of a wider matrix)
     rng = np.random.default_rng(55)
     y = rng.integers(-9, 9, (500, 21)).astype(np.float32)

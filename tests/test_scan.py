@@ -74,11 +74,28 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
         try:
             got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), dim)
             assert thc.last_kernel() == "scan-chunked", (shape, thc.last_kernel())
+            results = [got]
+            if kind in ("float", "half"):
+                # the one-read form with look-back (off by default: slower), as it is and with readers
+                # that never wait (a word that is still empty is computed by the reader itself)
+                thc.set_tuning("scan.lookback", 1)
+                for spin in (4096, 0):
+                    thc.set_tuning("scan.lookback_spin", spin)
+                    results.append(thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), dim))
+                    assert thc.last_kernel() == "scan-lookback", (shape, thc.last_kernel())
+                # in place: the two-read form (a reader that gives up waiting would need another chunk's input)
+                same = thc.Tensor.from_numpy(x)
+                same.cumsum(same, dim)
+                assert thc.last_kernel() == "scan-chunked"
+                results.append(same)
         finally:
             thc.set_tuning("scan.chunk_bytes", 32768)
+            thc.set_tuning("scan.lookback", 0)
+            thc.set_tuning("scan.lookback_spin", 4096)
         want = np.cumsum(sparse, axis=dim)
         assert np.abs(want).max() < 2048
-        assert_bit_equal(got.numpy(), want.astype(dtype), "%s %s" % (kind, shape))
+        for r in results:
+            assert_bit_equal(r.numpy(), want.astype(dtype), "%s %s" % (kind, shape))
     rows, every = (150000, 1000) if kind == "double" else (40000, 2000)
     ones = np.ones((rows, 2), dtype)
     ones[::every] = 2
