@@ -245,6 +245,31 @@ def test_many_tiles_bands_and_capped_grid(thc, oracle):
             assert_bit_equal(got, want.numpy(), "%s cmin %s cap %d" % (kind, shape, cap))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["short", "half", "int", "float", "double", "byte"])
+def test_streamed_store_form_gives_the_same_bits(thc, oracle, kind):
+    """Large outputs leave the kernel as nontemporal stores; the knob forces that form onto small aligned
+    and odd shapes, with transposed inputs and with a transposed output."""
+    rng = np.random.default_rng(307)
+    thc.set_tuning("apply.tiled.nt_store", 1)
+    try:
+        for (shape, aligned) in (((208, 144), True), ((201, 137), False), ((300, 701), False), ((64, 512), True)):
+            for transposed in ((1,), (0,), (1, 2)):
+                go, ga, gb, _ = operand_geoms(rng, shape, aligned, transposed)
+                da, ra = pair(thc, oracle, storage_of(rng, oracle, kind, ga[0]), ga, kind)
+                db, rb = pair(thc, oracle, storage_of(rng, oracle, kind, gb[0]), gb, kind)
+                do, ro = pair(thc, oracle, storage_of(rng, oracle, kind, go[0]), go, kind)
+                do.binary("cmax", da, db)
+                assert thc.last_kernel().startswith("lds-tile"), thc.last_kernel()
+                if kind in ("float", "half"):
+                    oracle.pointwise("fn:cmax", ro, ra, rb)
+                else:
+                    oracle.typed_pointwise("fn:cmax", ro, ra, rb)
+                assert_bit_equal(do.storage_numpy(), ro.storage, "%s %s t=%s" % (kind, shape, transposed))
+    finally:
+        thc.set_tuning("apply.tiled.nt_store", -1)
+
+
 def conv_values(rng, oracle, src, dst, n):
     """Source values that convert to `dst` without leaving its range (out-of-range float -> integer
     conversions are undefined in C)."""
