@@ -25,6 +25,20 @@
 
 namespace thc {
 
+// fn(integral_constant<int, B>) ... fn(integral_constant<int, E - 1>): a loop whose index is a
+// compile-time constant in every iteration. The packs a lane holds across the tile loop are
+// an array indexed by such loops only; with ordinary unrolled loops the compiler left part of one
+// rolled in the unaligned kernels, indexed the array at run time and therefore kept two of its
+// packs in scratch memory, each stored there right behind its load (a full memory wait in the
+// middle of the requests that are meant to stay in flight while the tile is computed).
+template <int B, int E, typename Fn>
+__device__ __forceinline__ void static_for(Fn&& fn) {
+  if constexpr (B < E) {
+    fn(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(fn);
+  }
+}
+
 struct LdsTileArgs {
   int staged[kMaxOps];   // input k is read along p and transposed on its way into LDS
   uint32_t sizeP, sizeQ;
@@ -84,7 +98,7 @@ struct LdsTileShape {
   // plain slab: row p's window from column MARG on; readers look up to 2 VEC - 2 columns beyond it
   static constexpr int PITCH_D = ALIGNED ? WQ : WQ + 3 * VEC;
   static constexpr int ROWS_D = WP;
-  static_assert(NP_D * ROWS_Q <= ROWS_D, "every lane's row lies inside the slab");
+  static_assert(NP * ROWS_Q <= ROWS_D && NP * ROWS_P <= ROWS_S, "every lane's row lies inside the slab");
   // Reading the transposed slab, lane lxq takes rows VEC * lxq + e: VEC rows are VEC * odd words, so
   // lanes 32 / VEC apart would meet in one bank. Row r therefore starts skew(r) = (r / 32) words late:
   // one bank further for every such group of lanes. (Unaligned rows: only the window layout, whose
@@ -195,41 +209,45 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
   // Requests every pack of the tile's inputs. No load carries a predicate: lanes past the
   // tile's valid extent re-read a pack inside it, so a later wait covers exactly these loads.
   auto issue = [&](const Tile& t, RAW (&v)[NIN][NP]) {
-#pragma unroll
-    for (int k = 0; k < NIN; ++k) {
+    static_for<0, NIN>([&](auto kTag) {
+      constexpr int k = decltype(kTag)::value;
       if (args.staged[k + 1]) {
-#pragma unroll
-        for (int r = 0; r < NP_S; ++r) {
+        static_for<0, NP>([&](auto rTag) {
+          constexpr int r = decltype(rTag)::value;
           const T* row = staged_row(t, k, (int)lyp + r * ROWS_P);
           int first = (int)(lxp * VEC) - (ALIGNED ? 0 : mis_in(row));
           if (first >= t.pn) first = ALIGNED ? 0 : -mis_in(row);
           v[k][r] = load(row + first);
-        }
+        });
       } else {
         const uint32_t sp = (uint32_t)args.strideP[k + 1];
-#pragma unroll
-        for (int r = 0; r < NP_D; ++r) {
+        // (NP, not NP_D, passes: both branches then fill the same registers. With one pass fewer
+        // here the compiler merged the last load of either branch into one block that picks its
+        // destination at run time, which put two packs of the array into scratch memory, each
+        // stored behind a full memory wait. The extra pass re-reads the tile's last row.)
+        static_for<0, NP>([&](auto rTag) {
+          constexpr int r = decltype(rTag)::value;
           const int pi = min((int)lyq + r * ROWS_Q, t.pn - 1);
           const int cs = row_start(t, pi);
           const T* at = t.tb[k] + (uint32_t)pi * sp + (ptrdiff_t)cs;   // this row's element at the run's start
           int first = (int)(lxq * VEC) - (ALIGNED ? 0 : mis_in(at));
           if (ALIGNED ? first >= t.qn : t.q0 + cs + first >= sizeQ) first = ALIGNED ? 0 : -mis_in(at);
           v[k][r] = load(at + first);
-        }
+        });
       }
-    }
+    });
   };
 
   // Registers -> LDS, without predicates (the slabs have room for every lane's pack). Transposed
   // inputs land at [q][p] (shifted into place element by element, or as the window they were
   // loaded as); the others keep their window (pack j of row p at column MARG + j * VEC).
   auto commit = [&](const Tile& t, const RAW (&v)[NIN][NP]) {
-#pragma unroll
-    for (int k = 0; k < NIN; ++k) {
+    static_for<0, NIN>([&](auto kTag) {
+      constexpr int k = decltype(kTag)::value;
       T* slab = lds + k * S::SLAB;
       if (args.staged[k + 1]) {
-#pragma unroll
-        for (int r = 0; r < NP_S; ++r) {
+        static_for<0, NP>([&](auto rTag) {
+          constexpr int r = decltype(rTag)::value;
           const int qi = (int)lyp + r * ROWS_P;
           if constexpr (WIN) {
             // word by word: the row starts at a multiple of 4 bytes, not of 16, and a 16-byte LDS
@@ -255,15 +273,15 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
 #pragma unroll
             for (int e = 0; e < VEC; ++e) at[e] = pk.v[e];
           }
-        }
+        });
       } else {
-#pragma unroll
-        for (int r = 0; r < NP_D; ++r) {
+        static_for<0, NP>([&](auto rTag) {
+          constexpr int r = decltype(rTag)::value;
           const int pi = (int)lyq + r * ROWS_Q;
           *reinterpret_cast<RAW*>(slab + pi * PITCH_D + MARG + lxq * VEC) = v[k][r];
-        }
+        });
       }
-    }
+    });
   };
 
   // LDS -> functor -> global, lanes along q. Rolled: the functor's code is fixed outside.
