@@ -41,6 +41,7 @@ __device__ __forceinline__ void static_for(Fn&& fn) {
 
 struct LdsTileArgs {
   int staged[kMaxOps];   // input k is read along p and transposed on its way into LDS
+  int sameGrid[kMaxOps]; // input k is read along q and its rows share the output rows' 16-byte grid (unaligned rows)
   uint32_t sizeP, sizeQ;
   int64_t strideP[kMaxOps];  // elements
   int64_t strideQ[kMaxOps];
@@ -320,6 +321,14 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
             __builtin_memcpy(&pk, &raw, sizeof(PIN));
 #pragma unroll
             for (int e = 0; e < VEC; ++e) x[k][e] = pk.v[e];
+          } else if (args.sameGrid[k + 1]) {
+            // every row of this input starts as far from a 16-byte boundary as the output's row does
+            // (operands of one shape and pitch): the window's packs are the output row's packs
+            const RAW raw = *reinterpret_cast<const RAW*>(slab + pic * PITCH_D + MARG + lxq * VEC);
+            PIN pk;
+            __builtin_memcpy(&pk, &raw, sizeof(PIN));
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[k][e] = pk.v[e];
           } else {
             // the window of row pic starts mis(element at the run's start) before that element
             const int cs = row_start(t, pic);
@@ -412,6 +421,13 @@ bool launch_ldstile(THCState* s, const Plan& pl, Op op) {
       args.staged[k] = staged[k];
       args.strideP[k] = pl.lay[k].stride[p];
       args.strideQ[k] = pl.lay[k].stride[q];
+      // an input read along q whose rows all start as far from a 16-byte boundary as the output's
+      bool same = k > 0 && !staged[k] && tuning("apply.ldstile.same_grid", 1) &&
+                  (reinterpret_cast<uintptr_t>(pl.ptr[k]) / elem_size(k)) % VEC ==
+                      (reinterpret_cast<uintptr_t>(pl.ptr[0]) / elem_size(0)) % VEC;
+      for (int d = 0; d < nd && same; ++d)
+        if (d != q) same = pl.lay[k].stride[d] % VEC == pl.lay[0].stride[d] % VEC;
+      args.sameGrid[k] = same ? 1 : 0;
     }
     if (pl.lay[0].size[p] >= kIndex32Limit || pl.lay[0].size[q] >= kIndex32Limit) return false;
     args.sizeP = (uint32_t)pl.lay[0].size[p];

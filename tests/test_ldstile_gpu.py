@@ -135,6 +135,44 @@ def test_one_and_three_input_ops_with_transposed_operands(thc, oracle, kind):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ALL_KINDS)
+def test_odd_shapes_with_inputs_on_the_outputs_pack_grid(thc, oracle, kind):
+    """The common case of an odd shape: the output and the inputs that are not transposed are dense
+    tensors of one shape, pitch and base alignment, so their rows start equally far from 16-byte
+    boundaries (the kernel then reads those inputs from LDS pack by pack). Also mixed: a third input
+    of another pitch and offset, a transposed output whose dense input shares its grid, and the same
+    ops with the fast path switched off."""
+    rng = np.random.default_rng(308)
+    fl = kind in ("float", "half")
+    ref = oracle.pointwise if fl else oracle.typed_pointwise
+    for same_grid in (1, 0):
+        thc.set_tuning("apply.ldstile.same_grid", same_grid)
+        try:
+            for shape in ((201, 137), (300, 701), (77, 1003), (9, 8)):
+                for offset in (0, 3):
+                    dense = geometry(shape, [0, 1], [0, 0], offset)
+                    dense_t = geometry(shape, [1, 0], [0, 0], offset)
+                    other = geometry(shape, [0, 1], [5, 0], offset + 1)
+                    for go, ga, gb, gc in ((dense, dense_t, dense, dense), (dense, dense_t, dense, other),
+                                           (dense_t, dense, dense_t, dense_t)):
+                        da, ra = pair(thc, oracle, storage_of(rng, oracle, kind, ga[0]), ga, kind)
+                        db, rb = pair(thc, oracle, storage_of(rng, oracle, kind, gb[0]), gb, kind)
+                        dc, rc = pair(thc, oracle, storage_of(rng, oracle, kind, gc[0]), gc, kind)
+                        do, ro = pair(thc, oracle, storage_of(rng, oracle, kind, go[0]), go, kind)
+                        do.binary("cmax", da, db)
+                        assert thc.last_kernel().startswith("lds-tile"), thc.last_kernel()
+                        ref("fn:cmax", ro, ra, rb)
+                        assert_bit_equal(do.storage_numpy(), ro.storage, "%s cmax %s off %d grid %d" % (kind, shape, offset, same_grid))
+                        if kind not in ("float", "half"):       # (their addcmul runs on the specialised tiled kernels)
+                            do.addcmul(dc, 2, da, db)
+                            assert thc.last_kernel().startswith("lds-tile"), thc.last_kernel()
+                            ref("addcmul", ro, rc, ra, rb, value=2)
+                            assert_bit_equal(do.storage_numpy(), ro.storage, "%s addcmul %s off %d grid %d" % (kind, shape, offset, same_grid))
+        finally:
+            thc.set_tuning("apply.ldstile.same_grid", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ALL_KINDS)
 def test_comparisons_with_transposed_operands(thc, oracle, kind):
     rng = np.random.default_rng(303)
     cmps = ["lt", "gt", "le", "ge", "eq", "ne"]
