@@ -822,6 +822,82 @@ struct FoldOnly {
   __device__ __forceinline__ A combine(A a, A b) const { return f.combine(a, b); }
 };
 
+// Long narrow slices, first level, without LDS staging: a dense [R][C] slice is read as ONE flat
+// run of aligned 16-byte packs. Lane t of a workgroup takes packs wb + t, wb + t + L, wb + t + 2 L, ...
+// where the workgroup's first pack wb and the number of active lanes L are multiples of the period
+// lcm(VEC, C) / VEC after which the packs' column pattern repeats: the VEC elements of every pack a
+// lane reads then fall into the same VEC columns, so a lane keeps VEC accumulators whose columns are
+// fixed, reads straight from global memory, fully coalesced, and the columns only meet at the end,
+// through LDS, in an order the geometry fixes (same bits on every run): accumulators `pattern` apart
+// (pattern = period * VEC) hold the same column, so `folds` threads per pattern slot first add every
+// folds-th repetition, then a thread per column adds the slots of its column (folds == 0: patterns too
+// long for that, one step). The workgroup writes its C column partials to
+// partial[(o * S + s) * C + c]; the existing levels of the chunked reduction fold those.
+template <typename TIn, typename F, typename I>
+__global__ __launch_bounds__(kBlock) void reduce_tall_kernel(const TIn* __restrict__ in,
+                                                             typename F::A* __restrict__ partial, I sliceElems,
+                                                             uint32_t C, uint32_t S, I packsPerWg, uint32_t lanes,
+                                                             uint32_t pattern, uint32_t folds, F f) {
+  using A = typename F::A;
+  constexpr int VEC = 16 / sizeof(TIn);
+  using P = Pack<TIn, VEC>;
+  __shared__ A part[kBlock * VEC];
+  __shared__ A stage[kBlock];
+  const I o = blockIdx.x / S;
+  const uint32_t s = blockIdx.x - (uint32_t)o * S;
+  const TIn* base = in + o * sliceElems;
+  const I npacks = sliceElems / VEC;
+  const I wb = (I)s * packsPerWg, we = min(npacks, wb + packsPerWg);
+  const uint32_t t = threadIdx.x;
+  A acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) acc[e] = f.init();
+  if (t < lanes && wb < we) {
+    constexpr int U = 8;
+    const P* src = reinterpret_cast<const P*>(base);
+    for (I j = wb + t; j < we; j += (I)U * lanes) {
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = load_pack<true>(src + min(j + (I)u * lanes, we - 1));  // (past the end: not used)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (j + (I)u * lanes < we) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = f.combine(acc[e], f.modify(acc_up<A>(v[u].v[e]), (A)0));
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) part[t * VEC + e] = acc[e];
+  __syncthreads();
+  // accumulator i = t * VEC + e of the workgroup holds column i % C (wb * VEC is a multiple of C)
+  const uint32_t accs = lanes * VEC;
+  if (folds) {
+    if (t < folds * pattern) {
+      const uint32_t k = t / pattern, slot = t - k * pattern;
+      A sub = f.init();
+      for (uint32_t i = k * pattern + slot; i < accs; i += folds * pattern) sub = f.combine(sub, part[i]);
+      stage[t] = sub;
+    }
+    __syncthreads();
+  }
+  for (uint32_t c = t; c < C; c += kBlock) {
+    A total = f.init();
+    if (folds) {
+      for (uint32_t i = c; i < pattern; i += C)
+        for (uint32_t k = 0; k < folds; ++k) total = f.combine(total, stage[k * pattern + i]);
+    } else {
+      for (uint32_t i = c; i < accs; i += C) total = f.combine(total, part[i]);
+    }
+    // the elements behind the slice's last whole pack belong to the last workgroup
+    if (s == S - 1)
+      for (I idx = npacks * VEC + ((c + C - (uint32_t)((npacks * VEC) % C)) % C); idx < sliceElems; idx += C)
+        total = f.combine(total, f.modify(acc_up<A>(base[idx]), (A)0));
+    partial[((I)o * S + s) * C + c] = total;
+  }
+}
+
 template <typename TIn, typename TOut, typename F, typename I>
 __global__ __launch_bounds__(kBlock) void reduce_slab_kernel(const TIn* __restrict__ in,
                                                              TOut* __restrict__ out, SlabArgs<I> a,
@@ -2237,9 +2313,45 @@ bool run_slab_chunked(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi
     return a;
   };
   const Epi<A> none{(int)Epilogue::None, (A)0};
-  launch_slab_level<T, A, F, I>(s, in, buf[0], level_args(g.R, rows1, S1, sizeof(T)), O * S1, none, f);
-  const FoldOnly<F> fold{f};
   int64_t R = S1;
+  // First level: the slices as flat runs of aligned packs where their starts are 16-byte aligned
+  // (reduce_tall_kernel), the LDS-staged slab kernel otherwise.
+  bool flat = tuning("reduce.tall", 1) && aligned16(in) && (O == 1 || (g.R * C) % VEC == 0) && g.R * C >= VEC;
+  int64_t period = 0, lanes = 0, packsPerWg = 0, ST = 0, folds = 0;
+  if (flat) {
+    int64_t gcd = C, b = VEC;
+    while (b) {
+      const int64_t r = gcd % b;
+      gcd = b;
+      b = r;
+    }
+    period = C / gcd;                       // packs after which the column pattern repeats
+    flat = period <= kBlock;
+    if (flat) {
+      lanes = (kBlock / period) * period;
+      const int64_t npacks = g.R * C / VEC;
+      // (two-step fold of the lanes' accumulators: about sqrt(repetitions x slots per column) threads per slot)
+      const int64_t pattern = period * VEC, reps = lanes / period;
+      if (pattern <= kBlock) {
+        folds = 1;
+        while ((folds + 1) * (folds + 1) * pattern <= reps * C && (folds + 1) * pattern <= kBlock && folds + 1 <= reps) ++folds;
+      }
+      const int64_t want = std::max<int64_t>(1, (int64_t)num_compute_units(s) * tuning("reduce.tall.blocks_per_cu", 2) / O);
+      packsPerWg = std::max<int64_t>((npacks + want - 1) / want, lanes * 8);
+      packsPerWg = (packsPerWg + period - 1) / period * period;
+      ST = (npacks + packsPerWg - 1) / packsPerWg;
+      flat = O * ST < (int64_t(1) << 31) && (size_t)(O * ST * C) * sizeof(A) <= half;
+    }
+  }
+  if (flat) {
+    hipLaunchKernelGGL((reduce_tall_kernel<T, F, I>), dim3((unsigned)(O * ST)), dim3(kBlock), 0, current_stream(s), in,
+                       buf[0], (I)(g.R * C), (uint32_t)C, (uint32_t)ST, (I)packsPerWg, (uint32_t)lanes,
+                       (uint32_t)(period * VEC), (uint32_t)folds, f);
+    R = ST;
+  } else {
+    launch_slab_level<T, A, F, I>(s, in, buf[0], level_args(g.R, rows1, S1, sizeof(T)), O * S1, none, f);
+  }
+  const FoldOnly<F> fold{f};
   int cur = 0;
   const int64_t rowsA = std::max<int64_t>(1, kRun / (C * (int64_t)sizeof(A)));
   while (R > rowsA) {
@@ -2263,7 +2375,7 @@ bool run_slab_chunked(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi
   a.slicesPerBlock = (uint32_t)spb;
   a.dataElems = (uint32_t)(spb * R * C + 2 * (16 / sizeof(A)));
   launch_slab_level<A, T, FoldOnly<F>, I>(s, buf[cur], out, a, (O + spb - 1) / spb, epi, fold);
-  note_kernel("slab-chunked");
+  note_kernel(flat ? "tall-flat" : "slab-chunked");
   return true;
 }
 

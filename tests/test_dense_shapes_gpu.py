@@ -73,7 +73,7 @@ def test_dense_shapes_against_numpy(thc, seed):
 def test_dense_shape_sweep_reached_every_kernel_family():
     if len(SEEN) == 0:
         pytest.skip("the sweep did not run in this process")
-    want = {"rows", "rows-lds", "rows-index-lds", "slab", "slab-index", "slab-chunked", "cols", "cols-index",
+    want = {"rows", "rows-lds", "rows-index-lds", "slab", "slab-index", "cols", "cols-index",
             "scan-slab", "scan-chunked", "scan-rows", "scan-cols"}
     assert want <= SEEN, sorted(want - SEEN)
 

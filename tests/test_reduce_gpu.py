@@ -577,23 +577,32 @@ def test_long_narrow_slices_reduce_in_chunks(thc, oracle, kind):
     rng = np.random.default_rng(58)
     dtype = np.float32 if kind == "float" else np.float16
     x = ((rng.integers(0, 40, (100003, 3)) == 0) * rng.integers(-2, 3, (100003, 3))).astype(dtype)  # fits half
-    thc.set_tuning("reduce.slab.run_bytes", 512)
-    try:
-        out = thc.Tensor(kind).norm(thc.Tensor.from_numpy(x), 1, 0)
-        assert thc.last_kernel() == "slab-chunked"
-    finally:
-        thc.set_tuning("reduce.slab.run_bytes", 32768)
     want = np.abs(x.astype(np.int64)).sum(axis=0, keepdims=True)
-    if kind == "float":
-        assert_bit_equal(out.numpy(), want.astype(dtype))
-    else:
-        np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=2e-3)
-    for shape, dim in (((700001, 3), 0), ((3, 50001, 7), 1), ((120000, 10), 0), ((2, 9000, 33), 1)):
+    # (first level: slices that start on 16-byte boundaries are read as flat runs of packs, "tall-flat";
+    # switched off, the LDS-staged first level runs, "slab-chunked")
+    for tall, expect in ((1, "tall-flat"), (0, "slab-chunked")):
+        thc.set_tuning("reduce.slab.run_bytes", 512)
+        thc.set_tuning("reduce.tall", tall)
+        try:
+            out = thc.Tensor(kind).norm(thc.Tensor.from_numpy(x), 1, 0)
+            assert thc.last_kernel() == expect
+        finally:
+            thc.set_tuning("reduce.slab.run_bytes", 32768)
+            thc.set_tuning("reduce.tall", 1)
+        if kind == "float":
+            assert_bit_equal(out.numpy(), want.astype(dtype))
+        else:
+            np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=2e-3)
+    for shape, dim in (((700001, 3), 0), ((3, 50001, 7), 1), ((120000, 10), 0), ((2, 9000, 33), 1), ((1, 300007, 5), 1),
+                       ((2, 40000, 50), 1)):
         x = ((rng.integers(0, 40, shape) == 0) * rng.integers(-2, 3, shape)).astype(dtype)   # sums fit half
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        vec = 4 if kind == "float" else 8
+        outer = int(np.prod(shape[:dim]))
+        flat = outer == 1 or (shape[dim] * int(np.prod(shape[dim + 1:]))) % vec == 0
         for name in ("sum", "norm1", "norm2", "mean"):
             k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
-            assert k == "slab-chunked", (shape, name, k)
+            assert k == ("tall-flat" if flat else "slab-chunked"), (shape, name, k)
         out = thc.Tensor(kind).sum(dev, dim)                       # exact: small integers
         want = x.astype(np.int64).sum(axis=dim, keepdims=True)
         if np.abs(want).max() < (2048 if kind == "half" else 1 << 24):
