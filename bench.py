@@ -335,7 +335,8 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-double-sum", "N-renorm", "N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall",
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
-                      "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G")
+                      "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
+                      "N-add-strided", "N-add-strided-u64")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -475,6 +476,25 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                 "N-cvt-half-t": ("half <- float converting copy of a:t(), 8192x8192", 6 * m * m, m * m,
                                  lambda i: hc.copy_from(sq_t)),
             })
+        if set(nx) & {"N-add-strided", "N-add-strided-u64"}:
+            # an operand with no unit-stride dim (every second column of a 8192 x 16384 buffer): the indexed
+            # kernel, one division chain per element; with 32-bit and with 64-bit index arithmetic (the latter
+            # is what operands beyond 2^31 elements take when no tiled kernel fits them)
+            m = 8192
+            st_buf = T.from_numpy(rng.standard_normal((m, 2 * m), dtype=np.float32))
+            st_a = st_buf.view_as_strided(0, (m, m), (2 * m, 2))
+            st_o = T("float").resize((m, m))
+
+            def strided_add(force):
+                def run(i):
+                    thc.force_64bit_index(force)
+                    st_o.cadd(st_a, 1.0, db)
+                    thc.force_64bit_index(False)
+                return run
+            table["N-add-strided"] = ("c = a + b, 8192x8192 fp32, a = every second column of a 8192x16384 buffer "
+                                      "(32-bit offsets; a's lines are half used)", 12 * m * m, m * m, strided_add(False))
+            table["N-add-strided-u64"] = ("the same with 64-bit index arithmetic forced", 12 * m * m, m * m,
+                                          strided_add(True))
         if "N-equal" in nx:
             eq_b = e_src.clone()
             table["N-equal"] = ("equal(a, b) over 2^26 fp32 (both equal: no early exit possible)", 8 * ne, ne,

@@ -210,3 +210,14 @@ void copy_tensor(THCState* s, DType dt, AnyTensor* dst, AnyTensor* src, bool ign
 }
 
 }  // namespace thc
+
+// The kernels' division by a launch-invariant 64-bit divisor, run on the host (tests without a GPU).
+THC_API void THCAmd_divmod64(unsigned long long n, unsigned long long d, unsigned long long* q,
+                             unsigned long long* r) {
+  thc::Divisor<uint64_t> div;
+  div.set(d);
+  uint64_t qq, rr;
+  div.divmod(n, qq, rr);
+  *q = qq;
+  *r = rr;
+}

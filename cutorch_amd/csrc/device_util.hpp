@@ -178,12 +178,52 @@ struct Divisor<uint32_t> {
     r = n - q * d;
   }
 };
+// 64-bit: the same idea with a 65-bit multiplier 2^64 + m and a shift of 65 + L, L = floor(log2 d)
+// (the round-up method in the form that needs no branch on the divisor: t = mulhi(n, m),
+// floor(n / d) = (((n - t) >> 1) + t) >> L for EVERY 64-bit n; a power of two 2^(L+1) takes m = 0,
+// which leaves n >> (L + 1); d = 1 is the one value the form cannot express). A 64-bit division is a
+// software routine of a few hundred instructions on this hardware; this is four 32-bit multiplies.
+__host__ __device__ __forceinline__ uint64_t mulhi64(uint64_t a, uint64_t b) {
+  const uint64_t a0 = (uint32_t)a, a1 = a >> 32, b0 = (uint32_t)b, b1 = b >> 32;
+  const uint64_t lo = a0 * b0, m1 = a1 * b0 + (lo >> 32), m2 = a0 * b1 + (uint32_t)m1;
+  return a1 * b1 + (m1 >> 32) + (m2 >> 32);
+}
 template <>
 struct Divisor<uint64_t> {
-  uint64_t d;
-  __host__ void set(uint64_t div) { d = div; }
-  __device__ __forceinline__ void divmod(uint64_t n, uint64_t& q, uint64_t& r) const {
-    q = n / d;
+  uint64_t d, m;
+  uint32_t s, one;
+  __host__ void set(uint64_t div) {
+    d = div;
+    m = 0;
+    s = 0;
+    one = div <= 1;
+    if (one) return;
+    uint32_t L = 63;
+    while (!((div >> L) & 1)) --L;
+    if ((div & (div - 1)) == 0) {
+      s = L - 1;
+      return;
+    }
+    // q = floor(2^(64+L) / div) < 2^64 and its remainder, by long division over the numerator's bits
+    uint64_t q = 0, r = 0;
+    for (int i = 64 + (int)L; i >= 0; --i) {
+      const bool carry = r >> 63;
+      r = (r << 1) | (i == 64 + (int)L ? 1u : 0u);
+      if (carry || r >= div) {
+        r -= div;
+        q |= uint64_t(1) << i;  // (i < 64 here: the quotient fits)
+      }
+    }
+    // doubled (one more bit of multiplier), rounded up
+    const uint64_t twice = r + r;
+    q += q;
+    if (twice >= div || twice < r) ++q;
+    m = q + 1;
+    s = L;
+  }
+  __host__ __device__ __forceinline__ void divmod(uint64_t n, uint64_t& q, uint64_t& r) const {
+    const uint64_t t = mulhi64(n, m);
+    q = one ? n : (((n - t) >> 1) + t) >> s;
     r = n - q * d;
   }
 };

@@ -109,6 +109,11 @@ THC_API int THCAmd_collapseDims(int nDim, const long *size, const long *stride,
 THC_API int THCAmd_overlappingIndices(int nDim, const long *size, const long *stride);
 THC_API int THCAmd_canUse32BitIndexMath(int nDim, const long *size, const long *stride);
 THC_API long THCAmd_indexToOffset(int nDim, const long *size, const long *stride, long linearId);
+/* The multiply-shift division the 64-bit index kernels use in place of
+ * IndexToOffset's `/` and `%` (THCTensorInfo.cuh:229-278), evaluated on the
+ * host: q = n / d, r = n % d for d >= 1. */
+THC_API void THCAmd_divmod64(unsigned long long n, unsigned long long d,
+                             unsigned long long *q, unsigned long long *r);
 /* Joint collapse of n same-shaped operands (strides laid out operand-major,
  * n*nDim entries). Returns the collapsed rank, or -1 if the shapes cannot be
  * walked jointly. */

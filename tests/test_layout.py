@@ -148,6 +148,36 @@ def test_fp16_conversion_exhaustive():
         assert lib.THC_float2half(float(x)) == int(w), x
 
 
+def test_64bit_multiply_shift_division_is_exact():
+    """The 64-bit index kernels divide by launch-invariant sizes with a 65-bit multiplier and a shift;
+    against Python's integers for the divisors and dividends where such schemes break first: 1, powers
+    of two and their neighbours, divisors just above and below 2^32 and 2^63, dividends that are
+    multiples of the divisor and one less, and the largest values."""
+    lib = cutorch_amd.lib()
+    lib.THCAmd_divmod64.argtypes = [C.c_ulonglong, C.c_ulonglong, C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong)]
+    lib.THCAmd_divmod64.restype = None
+    rng = np.random.default_rng(11)
+    top = (1 << 64) - 1
+    divisors = {1, 2, 3, 5, 6, 7, 10, 520, 2048, 8191, 8193, 641, 6700417, 274177, 67280421310721, top, top - 1}
+    for k in range(1, 64):
+        divisors |= {1 << k, (1 << k) + 1, (1 << k) - 1}
+    divisors |= {int(x) for x in rng.integers(1, 1 << 63, 200, dtype=np.uint64)}
+    divisors |= {int(x) >> int(sh) for x, sh in zip(rng.integers(1 << 62, 1 << 63, 200, dtype=np.uint64),
+                                                 rng.integers(0, 62, 200))}
+    divisors.discard(0)
+    q, r = C.c_ulonglong(), C.c_ulonglong()
+    for d in sorted(divisors):
+        ns = {0, 1, d - 1, d, d + 1, top, top - 1, top - d, (top // d) * d, (top // d) * d - 1, 1 << 63, (1 << 63) - 1,
+              (1 << 32) - 1, 1 << 32}
+        ns |= {int(x) for x in rng.integers(0, 1 << 63, 24, dtype=np.uint64)}
+        ns |= {(int(x) * d) & top for x in rng.integers(0, 1 << 40, 8, dtype=np.uint64)}
+        for n in ns:
+            if not 0 <= n <= top:
+                continue
+            lib.THCAmd_divmod64(n, d, C.byref(q), C.byref(r))
+            assert (q.value, r.value) == (n // d, n % d), (n, d)
+
+
 def test_library_exports_every_declared_symbol():
     """Every function declared in include/THC.h is exported by libTHC.so."""
     header = os.path.join(ROOT, "include", "THC.h")
