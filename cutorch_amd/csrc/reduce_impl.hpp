@@ -1600,6 +1600,161 @@ __global__ __launch_bounds__(kBlock) void var_cols_kernel(const T* __restrict__ 
   }
 }
 
+// var / std of long narrow slices ([O][R][C] dense, a row shorter than a couple of cache lines) in
+// ONE read: reduce_tall_kernel's reading order (the slice as a flat run of aligned packs, lane t
+// on packs wb + t + k L with wb and L multiples of the period of the packs' column pattern, so
+// every lane's VEC accumulators keep their columns) with a running (count, mean, M2) per
+// accumulator, one reciprocal per pack. The lanes' accumulators meet in LDS, in the order the
+// geometry fixes, by the pairwise update; the workgroup's C results go to three planes of
+// partials, partial[{0, 1, 2} * planeElems + (o * S + s) * C + c] = count, mean, M2.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void var_tall_kernel(const T* __restrict__ in,
+                                                          typename Acc<T>::type* __restrict__ partial,
+                                                          I sliceElems, uint32_t C, uint32_t S, I packsPerWg,
+                                                          uint32_t lanes, uint32_t pattern, uint32_t folds,
+                                                          I planeElems) {
+  using A = typename Acc<T>::type;
+  constexpr int VEC = 16 / sizeof(T);
+  using P = Pack<T, VEC>;
+  __shared__ A smean[kBlock * VEC];
+  __shared__ A sm2[kBlock * VEC];
+  __shared__ A scnt[kBlock];
+  __shared__ A stage[3][kBlock];
+  const I o = blockIdx.x / S;
+  const uint32_t s = blockIdx.x - (uint32_t)o * S;
+  const T* base = in + o * sliceElems;
+  const I npacks = sliceElems / VEC;
+  const I wb = (I)s * packsPerWg, we = min(npacks, wb + packsPerWg);
+  const uint32_t t = threadIdx.x;
+  A cnt = (A)0, mean[VEC], m2[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    mean[e] = (A)0;
+    m2[e] = (A)0;
+  }
+  if (t < lanes && wb < we) {
+    constexpr int U = 8;
+    const P* src = reinterpret_cast<const P*>(base);
+    for (I j = wb + t; j < we; j += (I)U * lanes) {
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = load_pack<true>(src + min(j + (I)u * lanes, we - 1));  // (past the end: not used)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (j + (I)u * lanes < we) {
+          cnt += (A)1;
+          const A inv = (A)1 / cnt;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            const A delta = x - mean[e];
+            mean[e] += delta * inv;
+            m2[e] += delta * (x - mean[e]);
+          }
+        }
+      }
+    }
+  }
+  scnt[t] = cnt;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    smean[t * VEC + e] = mean[e];
+    sm2[t * VEC + e] = m2[e];
+  }
+  __syncthreads();
+  // accumulator i = t * VEC + e holds column i % C; accumulators `pattern` apart hold the same column
+  const uint32_t accs = lanes * VEC;
+  if (folds) {
+    if (t < folds * pattern) {
+      const uint32_t k = t / pattern, slot = t - k * pattern;
+      A n = (A)0, mu = (A)0, q = (A)0;
+      for (uint32_t i = k * pattern + slot; i < accs; i += folds * pattern)
+        moments_merge(n, mu, q, scnt[i / VEC], smean[i], sm2[i]);
+      stage[0][t] = n;
+      stage[1][t] = mu;
+      stage[2][t] = q;
+    }
+    __syncthreads();
+  }
+  for (uint32_t c = t; c < C; c += kBlock) {
+    A n = (A)0, mu = (A)0, q = (A)0;
+    if (folds) {
+      for (uint32_t i = c; i < pattern; i += C)
+        for (uint32_t k = 0; k < folds; ++k)
+          moments_merge(n, mu, q, stage[0][k * pattern + i], stage[1][k * pattern + i], stage[2][k * pattern + i]);
+    } else {
+      for (uint32_t i = c; i < accs; i += C) moments_merge(n, mu, q, scnt[i / VEC], smean[i], sm2[i]);
+    }
+    // the elements behind the slice's last whole pack belong to the last workgroup
+    if (s == S - 1)
+      for (I idx = npacks * VEC + ((c + C - (uint32_t)((npacks * VEC) % C)) % C); idx < sliceElems; idx += C)
+        moments_merge(n, mu, q, (A)1, acc_up<A>(base[idx]), (A)0);
+    const I at = ((I)o * S + s) * C + c;
+    partial[at] = n;
+    partial[planeElems + at] = mu;
+    partial[2 * planeElems + at] = q;
+  }
+}
+
+// The S partials of every output of var_tall_kernel, merged: a workgroup per slice and tile of CT
+// columns, G = kBlock / CT threads per column take every G-th partial in order, thread 0 of the column
+// merges the G results.
+template <typename T, typename I>
+__global__ __launch_bounds__(kBlock) void var_tall_fold_kernel(const typename Acc<T>::type* __restrict__ partial,
+                                                               T* __restrict__ out, OuterArgs<I> oa, I outInner,
+                                                               uint32_t C, uint32_t S, uint32_t CT, uint32_t colTiles,
+                                                               I planeElems, typename Acc<T>::type div, bool wantStd) {
+  using A = typename Acc<T>::type;
+  __shared__ A stage[3][kBlock];
+  const I o = blockIdx.x / colTiles;
+  const uint32_t ct = blockIdx.x - (uint32_t)o * colTiles;
+  const uint32_t G = kBlock / CT, t = threadIdx.x;
+  const uint32_t g = t / CT, c = ct * CT + (t - g * CT);
+  if (g < G) {
+    A n = (A)0, mu = (A)0, q = (A)0;
+    if (c < C) {
+      // eight partials requested at a time (a load per merge would put a memory round trip into every step)
+      constexpr uint32_t U = 8;
+      for (uint32_t sp = g; sp < S; sp += U * G) {
+        A pn[U], pm[U], pq[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u) {
+          const I at = (o * S + min(sp + u * G, S - 1)) * C + c;  // (past the end: not used)
+          pn[u] = partial[at];
+          pm[u] = partial[planeElems + at];
+          pq[u] = partial[2 * planeElems + at];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; ++u)
+          if (sp + u * G < S) moments_merge(n, mu, q, pn[u], pm[u], pq[u]);
+      }
+    }
+    stage[0][t] = n;
+    stage[1][t] = mu;
+    stage[2][t] = q;
+  }
+  __syncthreads();
+  // the G results of a column in a fixed tree
+  uint32_t top = 1;
+  while (top < G) top <<= 1;
+  for (uint32_t h = top >> 1; h > 0; h >>= 1) {
+    if (g < h && g + h < G) {
+      const uint32_t j = t + h * CT;
+      A n = stage[0][t];
+      moments_merge(n, stage[1][t], stage[2][t], stage[0][j], stage[1][j], stage[2][j]);
+      stage[0][t] = n;
+    }
+    __syncthreads();
+  }
+  if (t < CT && c < C) {
+    const A q = stage[2][t];
+    I inOff, outOff;
+    oa.offsets(o, inOff, outOff);
+    const A v = q / div;
+    out[outOff + (I)c * outInner] = acc_down<T>(wantStd ? sqrt_any(v) : v);
+  }
+}
+
 template <typename T, typename I, int VEC, bool IS_MAX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_index_kernel(
     const T* __restrict__ in, T* __restrict__ outV, long* __restrict__ outI,
@@ -2676,6 +2831,58 @@ bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in_, voi
         return true;
       };
       if (g.wide ? slab(uint64_t{}) : slab(uint32_t{})) return true;
+    }
+    {
+      // few long narrow slices that start on 16-byte boundaries: flat runs of packs (see var_tall_kernel;
+      // the column kernel below keeps C of its lanes busy on them: 6.7M x 10 along dim 0 0.23 of peak)
+      auto tall = [&](auto idxTag) {
+        using I = decltype(idxTag);
+        if (!tuning("reduce.tall", 1)) return false;
+        const int64_t C = g.in.size[nd - 1];
+        if (g.sR != C || C > kBlock || C * (int64_t)sizeof(T) > tuning("reduce.slab.chunked_max_row_bytes", 512)) return false;
+        int64_t run = g.R * C;
+        for (int d = nd - 2; d >= 0; --d) {
+          if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
+          run *= g.in.size[d];
+        }
+        const int64_t O = g.outElems / C;
+        if (!aligned16(in_) || C % VEC == 0 || O >= (int64_t)num_compute_units(s)) return false;
+        if (!(O == 1 || (g.R * C) % VEC == 0) || g.R * C < (int64_t)VEC * kBlock * 8) return false;
+        int64_t gcd = C, b = VEC;
+        while (b) {
+          const int64_t r = gcd % b;
+          gcd = b;
+          b = r;
+        }
+        const int64_t period = C / gcd;  // packs after which the column pattern repeats
+        if (period > kBlock) return false;
+        const int64_t lanes = (kBlock / period) * period, pattern = period * VEC, reps = lanes / period;
+        int64_t folds = 0;
+        if (pattern <= kBlock) {
+          folds = 1;
+          while ((folds + 1) * (folds + 1) * pattern <= reps * C && (folds + 1) * pattern <= kBlock && folds + 1 <= reps) ++folds;
+        }
+        const int64_t npacks = g.R * C / VEC;
+        const int64_t want = std::max<int64_t>(1, (int64_t)num_compute_units(s) * tuning("reduce.tall.var_blocks_per_cu", 2) / O);
+        int64_t packsPerWg = std::max<int64_t>((npacks + want - 1) / want, lanes * 8);
+        packsPerWg = (packsPerWg + period - 1) / period * period;
+        const int64_t ST = (npacks + packsPerWg - 1) / packsPerWg;
+        size_t scratchBytes = 0;
+        A* partial = (A*)scratch_space(s, &scratchBytes);
+        const int64_t planeElems = O * ST * C;
+        if (O * ST >= (int64_t(1) << 31) || (size_t)(3 * planeElems) * sizeof(A) > scratchBytes) return false;
+        hipStream_t st = current_stream(s);
+        hipLaunchKernelGGL((var_tall_kernel<T, I>), dim3((unsigned)(O * ST)), dim3(kBlock), 0, st, (const T*)in_, partial,
+                           (I)(g.R * C), (uint32_t)C, (uint32_t)ST, (I)packsPerWg, (uint32_t)lanes, (uint32_t)pattern,
+                           (uint32_t)folds, (I)planeElems);
+        const int64_t CT = std::min<int64_t>(C, 16), colTiles = (C + CT - 1) / CT;
+        hipLaunchKernelGGL((var_tall_fold_kernel<T, I>), dim3((unsigned)(O * colTiles)), dim3(kBlock), 0, st,
+                           (const A*)partial, (T*)out_, make_outer<I>(g.in, g.out, nd - 1), (I)g.out.stride[nd - 1],
+                           (uint32_t)C, (uint32_t)ST, (uint32_t)CT, (uint32_t)colTiles, (I)planeElems, (A)div, wantStd);
+        note_kernel("var-tall");
+        return true;
+      };
+      if (g.wide ? tall(uint64_t{}) : tall(uint32_t{})) return true;
     }
     auto go = [&](auto idxTag) {
       using I = decltype(idxTag);

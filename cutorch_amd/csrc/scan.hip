@@ -182,27 +182,36 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
                                                            uint64_t outer, uint64_t R,
                                                            uint64_t inner, uint32_t TX,
-                                                           uint64_t colTiles, int nts) {
+                                                           uint64_t colTiles, int nts, uint64_t S, uint64_t partRows,
+                                                           const typename ScanAcc<T>::type* __restrict__ carryIn) {
   using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   constexpr int U = 8;
   __shared__ A totals[2][kBlock * VEC];
   const uint32_t TY = kBlock / TX;
   const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
-  const uint64_t blocks = outer * colTiles;
+  const uint64_t blocks = outer * S * colTiles;
   const uint64_t segRows = (uint64_t)TY * U;
+  const uint64_t fullR = R;
   for (uint64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
-    const uint64_t o = b / colTiles, ct = b - o * colTiles;
+    // S > 1: the rows are cut into S parts of partRows rows that scan side by side, part s of slice o
+    // starting every column from carryIn[(o * (S - 1) + s - 1) * inner + column], the scanned totals
+    // of the parts before it
+    const uint64_t o = b / (S * colTiles), rem = b - o * (S * colTiles);
+    const uint64_t part = rem / colTiles, ct = rem - part * colTiles;
+    const uint64_t rBeg = part * partRows;
+    const uint64_t R = min(partRows, fullR - rBeg);  // rows of this part
     const uint64_t col = (ct * TX + tx) * VEC;
     const bool live = col < inner;  // inner % VEC == 0 for VEC > 1
     // Loads carry no predicate: rows past the end re-read the last row and idle
     // lanes read column 0 (both discarded), so the compiler can count exactly
     // which loads a wait has to cover.
-    const T* src = in + o * R * inner + (live ? col : 0);
-    T* dst = out + o * R * inner + col;
+    const T* src = in + (o * fullR + rBeg) * inner + (live ? col : 0);
+    T* dst = out + (o * fullR + rBeg) * inner + col;
     A carry[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) carry[e] = Op::id();
+    for (int e = 0; e < VEC; ++e)
+      carry[e] = part > 0 && live ? carryIn[(o * (S - 1) + part - 1) * inner + col + e] : Op::id();
     auto fetch = [&](uint64_t r0, P (&v)[U]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -266,6 +275,61 @@ __global__ __launch_bounds__(kBlock) void scan_cols_kernel(T* __restrict__ out,
       if (seg + segRows < R) step(seg + segRows, 1, bufB, bufA);
     }
     lds_barrier();  // both LDS buffers are idle before the next tile
+  }
+}
+
+// Column totals of the row parts of scan_cols_kernel's split form, all but the last part of every
+// slice (nothing follows it): totals[(o * (S - 1) + s) * inner + column]. The same tiling; thread
+// row ty adds U rows of every TY * U (scans here combine with + or *, so the order within a part is
+// free; it is fixed by the geometry), the thread rows meet in LDS.
+template <typename T, typename Op, int VEC>
+__global__ __launch_bounds__(kBlock) void scan_cols_totals_kernel(typename ScanAcc<T>::type* __restrict__ totals,
+                                                                  const T* __restrict__ in, uint64_t outer,
+                                                                  uint64_t R, uint64_t inner, uint32_t TX,
+                                                                  uint64_t colTiles, uint64_t S, uint64_t partRows) {
+  using P = Pack<T, VEC>;
+  using A = typename ScanAcc<T>::type;
+  constexpr int U = 8;
+  __shared__ A sums[kBlock * VEC];
+  const uint32_t TY = kBlock / TX;
+  const uint32_t tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const uint64_t blocks = outer * (S - 1) * colTiles;
+  for (uint64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
+    const uint64_t o = b / ((S - 1) * colTiles), rem = b - o * ((S - 1) * colTiles);
+    const uint64_t part = rem / colTiles, ct = rem - part * colTiles;
+    const uint64_t col = (ct * TX + tx) * VEC;
+    const bool live = col < inner;
+    const T* src = in + (o * R + part * partRows) * inner + (live ? col : 0);  // (a full part: partRows rows)
+    A acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = Op::id();
+    for (uint64_t r0 = (uint64_t)ty * U; r0 < partRows; r0 += (uint64_t)TY * U) {
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint64_t r = r0 + u < partRows ? r0 + u : partRows - 1;
+        v[u] = load_pack<true>(reinterpret_cast<const P*>(src + r * inner));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (r0 + u < partRows) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) acc[e] = Op::op(acc[e], scan_up<A>(v[u].v[e]));
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sums[(ty * TX + tx) * VEC + e] = acc[e];
+    lds_barrier();
+    if (ty == 0 && live) {
+      for (uint32_t t = 1; t < TY; ++t) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = Op::op(acc[e], sums[(t * TX + tx) * VEC + e]);
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) totals[(o * (S - 1) + part) * inner + col + e] = acc[e];
+    }
+    lds_barrier();  // the sums are read before the next tile overwrites them
   }
 }
 
@@ -657,9 +721,66 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
   // totals of 32 KiB chunks of rows, their scan (this function again, on the
   // accumulator type), then every chunk scans from its carry. The input is
   // read twice, which still is 500x faster.
+  // The column kernel with the rows cut into parts that scan side by side (totals of the parts, their
+  // scan by this function on the accumulator type, then every part from its carry): for long scans over
+  // rows of whole packs of at least `scan.cols.split_min_row_bytes`, whose lanes the column tiling keeps
+  // busy (fp32: 0.41-0.51 of peak on 8 bytes per element against 0.42-0.46 for the chunks of rows below;
+  // rows of single elements ran at 0.10-0.24 this way and stay with the chunks), and for every long scan
+  // whose chunk totals do not fit the scratch buffer (65536 x 1000 along dim 0 ran on 4-8 workgroups:
+  // 0.09 of peak -> 0.41; 524288 x 100 doubles 0.02 -> 0.31). The input is read twice here too.
+  auto split_cols = [&]() -> bool {
+    using A = typename ScanAcc<T>::type;
+    if (inner <= 1 || !tuning("scan.cols.split", 1)) return false;
+    const bool vec = aligned && inner % VECC == 0;
+    const int64_t pack = vec ? VECC : 1;
+    const int64_t packs = (inner + pack - 1) / pack;
+    const uint32_t TX = std::min<uint32_t>(32, pow2_at_least((uint64_t)packs));
+    const int64_t colTiles = (packs + TX - 1) / TX;
+    const int64_t cus = num_compute_units(s);
+    // (only where even the narrowest column tiles, 8 packs wide, leave CUs without a workgroup: the
+    // one-read kernel on narrower tiles wins otherwise)
+    if (outer * ((packs + 7) / 8) >= cus) return false;
+    const int64_t minRows = std::max<int64_t>(64, tuning("scan.cols.split_min_rows", 256));
+    int64_t S = std::min<int64_t>((cus * tuning("scan.cols.split_per_cu", 2) + outer * colTiles - 1) / (outer * colTiles),
+                                  R / minRows);
+    if (!scratch) scratch = (char*)scratch_space(s, &scratchBytes);
+    const auto need_of = [&](int64_t parts) {
+      return (((size_t)(outer * (parts - 1) * inner) * sizeof(A)) + 255) & ~size_t(255);
+    };
+    while (S >= 2 && 2 * need_of(S) > scratchBytes) S /= 2;
+    if (S < 2) return false;
+    const int64_t partRows = (R + S - 1) / S;
+    S = (R + partRows - 1) / partRows;  // (no empty parts)
+    if (S < 2) return false;
+    const size_t need = need_of(S);
+    A* totals = (A*)scratch;
+    A* carries = (A*)(scratch + need);
+    const int64_t blocks = outer * S * colTiles;
+    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(blocks, 1 << 30));
+    const int gridT = (int)std::max<int64_t>(1, std::min<int64_t>(outer * (S - 1) * colTiles, 1 << 30));
+    const bool pf = blocks < 2 * cus;
+#define THC_SCAN_SPLIT(V, F)                                                                                       \
+  do {                                                                                                             \
+    hipLaunchKernelGGL((scan_cols_totals_kernel<T, Op, V>), dim3(gridT), dim3(kBlock), 0, st, totals, in,          \
+                       (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, (uint64_t)S,         \
+                       (uint64_t)partRows);                                                                        \
+    launch_scan<A, Op>(s, carries, totals, outer, S - 1, inner, scratch + 2 * need, scratchBytes - 2 * need);      \
+    hipLaunchKernelGGL((scan_cols_kernel<T, Op, V, F>), dim3(grid), dim3(kBlock), 0, st, out, in, (uint64_t)outer, \
+                       (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, streaming, (uint64_t)S,               \
+                       (uint64_t)partRows, (const A*)carries);                                                     \
+  } while (0)
+    if (vec && pf) THC_SCAN_SPLIT(VECC, true);
+    else if (vec) THC_SCAN_SPLIT(VECC, false);
+    else if (pf) THC_SCAN_SPLIT(1, true);
+    else THC_SCAN_SPLIT(1, false);
+#undef THC_SCAN_SPLIT
+    note_kernel("scan-cols-split");
+    return true;
+  };
   {
     using A = typename ScanAcc<T>::type;
     const int64_t rowBytes = inner * (int64_t)sizeof(T);
+    if (rowBytes >= tuning("scan.cols.split_min_row_bytes", 256) && aligned && inner % VECC == 0 && split_cols()) return;
     const int64_t run = std::min<int64_t>(32768, std::max<int64_t>(256, tuning("scan.chunk_bytes", 32768)));
     const int64_t chunkRows = std::max<int64_t>(1, run / rowBytes);
     const int64_t S = (R + chunkRows - 1) / chunkRows;
@@ -667,7 +788,10 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t plainBlocks = inner == 1 ? (outer + 3) / 4 : outer * ((packsPerRow + 15) / 16);
     if (!scratch) scratch = (char*)scratch_space(s, &scratchBytes);
     const size_t need = (((size_t)(outer * S * inner) * sizeof(A)) + 255) & ~size_t(255);
-    const bool longScan = tuning("scan.chunked", 1) && rowBytes <= 32768 && S >= 4 && plainBlocks < (int64_t)num_compute_units(s);
+    // (chunks of at least 4 rows: with one row per chunk the totals are the input again, and the levels
+    // below would repeat this one until the scratch buffer is used up)
+    const bool longScan = tuning("scan.chunked", 1) && rowBytes <= 32768 && S >= 4 && chunkRows >= 4 &&
+                          plainBlocks < (int64_t)num_compute_units(s);
     if constexpr (sizeof(A) == 4) {
       // (a chunk and its neighbours' elements in its first and last pack must fit RunPrefetch: 32 KiB)
       const int64_t chunkRows = std::max<int64_t>(1, std::min<int64_t>(run, 32768 - 32) / rowBytes);
@@ -712,6 +836,7 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
       return;
     }
   }
+  if (split_cols()) return;  // (long scans that found no room for their chunk totals)
   const int nts = streaming;
   if (inner == 1) {
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
@@ -761,7 +886,8 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const bool pf = pfKnob >= 0 ? pfKnob != 0 : bestPerCU < 2;
 #define THC_SCAN_COLS(V, F)                                                                              \
   hipLaunchKernelGGL((scan_cols_kernel<T, Op, V, F>), dim3(grid), dim3(kBlock), 0, st, out, in,          \
-                     (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts)
+                     (uint64_t)outer, (uint64_t)R, (uint64_t)inner, TX, (uint64_t)colTiles, nts, (uint64_t)1,    \
+                     (uint64_t)R, (const typename ScanAcc<T>::type*)nullptr)
     if (vec && pf) THC_SCAN_COLS(VECC, true);
     else if (vec) THC_SCAN_COLS(VECC, false);
     else if (pf) THC_SCAN_COLS(1, true);

@@ -164,6 +164,50 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["float", "half", "double"])
+def test_gpu_var_of_long_narrow_slices_reads_flat_packs(thc, kind):
+    """Few long slices of narrow rows (batch statistics of a tall matrix) are read as flat runs of
+    aligned packs with a running (count, mean, M2) per lane and column: against float64 numpy, with a
+    common offset of 40 sigma (8 for half), column counts with every period of the pack pattern,
+    slices with elements behind the last whole pack, several slices, and a first row that is an
+    outlier (what a shifted one-pass sum would lose)."""
+    rng = np.random.default_rng(83)
+    dtype = {"float": np.float32, "half": np.float16, "double": np.float64}[kind]
+    tol = {"float": 2e-5, "half": 4e-3, "double": 1e-12}[kind]
+    centre = 4.0 if kind == "half" else 20.0
+    vec = 16 // np.dtype(dtype).itemsize
+    cases = [((200003, 3), 0), ((70001, 10), 0), ((30000, 33), 0), ((2, 40000, 7), 1), ((3, 16000, 5), 1),
+             ((1, 50001, 9), 1), ((90001, 1, 6), 0), ((25000, 50), 0)]
+    for shape, dim in cases:
+        x = (rng.standard_normal(shape) * 0.5 + centre).astype(dtype)
+        x[(0,) * len(shape)] = 60.0 if kind == "half" else 1e4
+        dev = thc.Tensor.from_numpy(x)
+        ref = x.astype(np.float64)
+        inner = int(np.prod(shape[dim + 1:]))
+        outer = int(np.prod(shape[:dim]))
+        flat = inner % vec != 0 and (outer == 1 or (shape[dim] * inner) % vec == 0)
+        for name, fn in (("var", np.var), ("std", np.std)):
+            for biased in (0, 1):
+                out = getattr(thc.Tensor(kind), name)(dev, dim, biased=biased)
+                assert thc.last_kernel() == ("var-tall" if flat else "var-cols-split"), (shape, dim, thc.last_kernel())
+                want = fn(ref, axis=dim, ddof=0 if biased else 1, keepdims=True)
+                np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol,
+                                           err_msg="%s %s %s" % (kind, name, shape))
+    x = (rng.standard_normal((70001, 10)) + centre).astype(dtype)
+    dev = thc.Tensor.from_numpy(x)
+    a = thc.Tensor(kind).var(dev, 0).numpy()
+    thc.set_tuning("reduce.tall", 0)
+    try:
+        b = thc.Tensor(kind).var(dev, 0).numpy()
+        assert thc.last_kernel() == "var-cols-split"
+    finally:
+        thc.set_tuning("reduce.tall", 1)
+    np.testing.assert_allclose(a.astype(np.float64), b.astype(np.float64), rtol=tol)
+    assert_same = thc.Tensor(kind).var(dev, 0).numpy()
+    assert np.array_equal(a, assert_same)        # same bits on every run
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double"])
 def test_gpu_var_of_short_rows_and_small_slices_is_one_read(thc, kind):
     """Dense short rows and small R x C slices are staged in LDS and swept
     there twice (mean, squared deviations): row lengths around the group

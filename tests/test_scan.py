@@ -71,6 +71,7 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
         sparse = (rng.integers(0, 50, shape) == 0) * rng.integers(-2, 3, shape)     # running sums fit half
         x = sparse.astype(dtype)
         thc.set_tuning("scan.chunk_bytes", chunk)
+        thc.set_tuning("scan.cols.split", 0)     # (wide rows would take the split column kernel)
         try:
             got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), dim)
             assert thc.last_kernel() == "scan-chunked", (shape, thc.last_kernel())
@@ -90,6 +91,7 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
                 results.append(same)
         finally:
             thc.set_tuning("scan.chunk_bytes", 32768)
+            thc.set_tuning("scan.cols.split", 1)
             thc.set_tuning("scan.lookback", 0)
             thc.set_tuning("scan.lookback_spin", 4096)
         want = np.cumsum(sparse, axis=dim)
@@ -113,6 +115,65 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
         assert thc.last_kernel() == "scan-rows"
     finally:
         thc.set_tuning("scan.chunked", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double", "byte", "long"])
+def test_gpu_long_scans_over_wide_rows_split_the_rows(thc, oracle, kind):
+    """A long scan over rows wide enough for the column kernel's lanes, but with too few column tiles
+    for the chip, cuts the rows into parts that scan side by side: totals of the parts, their scan,
+    then every part from its carry. Exact on small integers; row counts that leave a short last
+    part, widths that are and are not whole packs, several slices, in place."""
+    rng = np.random.default_rng(23)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64, "byte": np.uint8,
+             "long": np.int64}[kind]
+    for shape, dim, min_rows in (((20000, 1000), 0, 256), ((3, 9001, 136), 1, 256), ((1, 30011, 257), 1, 256),
+                                 ((2, 4099, 64), 1, 64), ((1500, 2000), 0, 64), ((70001, 100), 0, 256)):
+        if kind == "byte":
+            sparse = (rng.integers(0, 400, shape) == 0) * rng.integers(0, 2, shape)
+        else:
+            sparse = (rng.integers(0, 50, shape) == 0) * rng.integers(-2, 3, shape)     # running sums fit half
+        x = sparse.astype(dtype)
+        thc.set_tuning("scan.cols.split_min_rows", min_rows)
+        thc.set_tuning("scan.cols.split_min_row_bytes", 1)      # (narrower rows are scanned in chunks by default,
+        thc.set_tuning("scan.chunked", 0)                       #  and so are rows that are not whole packs)
+        try:
+            got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), dim)
+            assert thc.last_kernel() == "scan-cols-split", (shape, thc.last_kernel())
+            same = thc.Tensor.from_numpy(x)
+            same.cumsum(same, dim)
+            assert thc.last_kernel() == "scan-cols-split"
+        finally:
+            thc.set_tuning("scan.cols.split_min_rows", 256)
+            thc.set_tuning("scan.cols.split_min_row_bytes", 256)
+            thc.set_tuning("scan.chunked", 1)
+        want = np.cumsum(sparse, axis=dim)
+        assert np.abs(want).max() < (256 if kind == "byte" else 2048)
+        assert_bit_equal(got.numpy(), want.astype(dtype), "%s %s" % (kind, shape))
+        assert_bit_equal(same.numpy(), want.astype(dtype), "%s %s in place" % (kind, shape))
+    if kind != "byte":
+        ones = np.ones((9000, 320), dtype)
+        ones[::700] = 2
+        ones[1::1300, ::7] = -1
+        got = thc.Tensor(kind).cumprod(thc.Tensor.from_numpy(ones), 0)
+        assert thc.last_kernel() == "scan-cols-split"
+        assert_bit_equal(got.numpy(), np.cumprod(ones.astype(np.float64), axis=0).astype(dtype))
+    if kind in ("float", "double"):
+        x = rng.standard_normal((50000, 520)).astype(dtype)
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        got = thc.Tensor(kind).cumsum(dev, 0).numpy().astype(np.float64)
+        assert thc.last_kernel() == "scan-cols-split"
+        want = oracle.scan_dim(ref, 0).numpy().astype(np.float64) if kind == "float" else np.cumsum(x, axis=0)
+        mass = np.cumsum(np.abs(x.astype(np.float64)), axis=0)
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(np.abs(want), mass / 64))
+    thc.set_tuning("scan.cols.split", 0)
+    try:
+        x = ((rng.integers(0, 50, (20000, 1000)) == 0) * 1).astype(dtype)
+        got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), 0)
+        assert thc.last_kernel() in ("scan-cols", "scan-chunked")
+        assert_bit_equal(got.numpy(), np.cumsum(x.astype(np.int64), axis=0).astype(dtype))
+    finally:
+        thc.set_tuning("scan.cols.split", 1)
 
 
 @pytest.mark.gpu
@@ -170,7 +231,8 @@ def test_gpu_scan_over_a_strided_dim_in_every_strip_width(thc, oracle, kind):
     rng = np.random.default_rng(23)
     dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64}[kind]
     thc.set_tuning("scan.chunked", 0)       # (few long slices would otherwise be cut into chunks of rows,
-    thc.set_tuning("scan.slab", 0)          #  small ones scanned in LDS)
+    thc.set_tuning("scan.slab", 0)          #  small ones scanned in LDS,
+    thc.set_tuning("scan.cols.split", 0)    #  long ones over wide rows cut into parts of rows)
     try:
         for shape in ((3, 300, 520), (2, 129, 1024), (1, 64, 96), (2, 1000, 136), (1, 77, 515), (5, 1, 8192), (4, 9, 4100)):
             sparse = (rng.integers(0, 12, shape) == 0) * rng.integers(-2, 3, shape)
@@ -188,6 +250,7 @@ def test_gpu_scan_over_a_strided_dim_in_every_strip_width(thc, oracle, kind):
     finally:
         thc.set_tuning("scan.chunked", 1)
         thc.set_tuning("scan.slab", 1)
+        thc.set_tuning("scan.cols.split", 1)
         thc.set_tuning("scan.cols.prefetch", -1)
         thc.set_tuning("scan.cols.min_tx", 8)
         thc.set_tuning("scan.cols.max_tx", 64)
