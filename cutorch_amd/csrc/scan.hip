@@ -105,21 +105,59 @@ struct ScanMul {
 
 // One wave64 per row. A lane owns VEC consecutive elements of each
 // 64*VEC-element chunk; U chunks are loaded before the first is consumed.
-template <typename T, typename Op, int VEC>
+// S > 1: every row is cut into S pieces of L elements (L a multiple of VEC) that scan side by side,
+// a wave per piece, piece s of a row starting from carryIn[row * (S - 1) + s - 1], the scanned
+// totals of the pieces before it. TOTALS: nothing is stored; the wave adds up (or multiplies) its
+// piece and writes totalsOut[row * (S - 1) + s], for all but the last piece of every row.
+template <typename T, typename Op, int VEC, bool TOTALS = false>
 __global__ __launch_bounds__(kBlock) void scan_rows_kernel(T* __restrict__ out,
                                                            const T* __restrict__ in,
-                                                           uint64_t numRows, uint64_t R, int nts) {
+                                                           uint64_t numRows, uint64_t rowLen, int nts, uint64_t S,
+                                                           uint64_t L,
+                                                           const typename ScanAcc<T>::type* __restrict__ carryIn,
+                                                           typename ScanAcc<T>::type* __restrict__ totalsOut) {
   using P = Pack<T, VEC>;
   using A = typename ScanAcc<T>::type;
   constexpr int U = 4;
   constexpr uint64_t kChunk = 64 * VEC;
   const uint32_t lane = threadIdx.x & 63;
   const uint64_t wavesPerGrid = (uint64_t)gridDim.x * (kBlock / 64);
-  for (uint64_t row = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); row < numRows;
-       row += wavesPerGrid) {
-    const T* src = in + row * R;
-    T* dst = out + row * R;
-    A carry = Op::id();
+  const uint64_t per = TOTALS ? S - 1 : S;  // pieces of a row that this launch covers
+  for (uint64_t vr = (uint64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); vr < numRows * per;
+       vr += wavesPerGrid) {
+    const uint64_t row = vr / per, piece = vr - row * per;
+    const uint64_t R = min(L, rowLen - piece * L);  // elements of this piece
+    const T* src = in + row * rowLen + piece * L;
+    T* dst = out + row * rowLen + piece * L;
+    if constexpr (TOTALS) {
+      A acc = Op::id();
+      for (uint64_t base = 0; base < R; base += U * kChunk) {
+        A x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint64_t i0 = base + u * kChunk + (uint64_t)lane * VEC;
+          x[u] = Op::id();
+          if (VEC > 1) {
+            if (i0 < R) {
+              const P v = load_pack<true>(reinterpret_cast<const P*>(src + i0));
+#pragma unroll
+              for (int k = 0; k < VEC; ++k) x[u] = Op::op(x[u], scan_up<A>(v.v[k]));
+            }
+          } else if (i0 < R) {
+            x[u] = scan_up<A>(src[i0]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc = Op::op(acc, x[u]);
+      }
+      // (+ and * commute: the lanes meet in a butterfly, in an order the geometry fixes)
+#pragma unroll
+      for (uint32_t o = 32; o > 0; o >>= 1)
+        acc = Op::op(acc, lane_exchange(acc, [o](uint32_t w) { return __shfl_xor(w, o, 64); }));
+      if (lane == 0) totalsOut[vr] = acc;
+      continue;
+    }
+    A carry = piece > 0 ? carryIn[row * (S - 1) + piece - 1] : Op::id();
     for (uint64_t base = 0; base < R; base += U * kChunk) {
       A x[U][VEC];
 #pragma unroll
@@ -721,6 +759,50 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
   // totals of 32 KiB chunks of rows, their scan (this function again, on the
   // accumulator type), then every chunk scans from its carry. The input is
   // read twice, which still is 500x faster.
+  // Few long rows (a 1-D cumsum above all): a wave per row leaves the chip idle, and the chunks of rows
+  // below hand every thread a contiguous band of its chunk in LDS, 32 elements apart from its
+  // neighbour's, i.e. all lanes in one bank (2^26 elements: 0.12 of peak). Instead every row is cut
+  // into pieces that scan side by side, a wave per piece: totals of the pieces, their scan by this
+  // function on the accumulator type, then every piece from its carry (0.12 -> 0.44 with 8 workgroups of
+  // pieces per CU; 0.39 with 2, 0.42 with 4). The input is read twice.
+  if (inner == 1 && tuning("scan.rows.split", 1)) {
+    using A = typename ScanAcc<T>::type;
+    const bool vec = aligned && R % VEC == 0;
+    const int64_t perIter = 64 * (vec ? VEC : 1) * 4;  // elements a wave takes per iteration
+    const int64_t minPiece = perIter * std::max<int64_t>(1, tuning("scan.rows.split_min_iters", 8));
+    const int64_t waves = (int64_t)num_compute_units(s) * (kBlock / 64) * tuning("scan.rows.split_per_cu", 8);
+    int64_t S = std::min<int64_t>((waves + outer - 1) / outer, R / minPiece);
+    if (!scratch) scratch = (char*)scratch_space(s, &scratchBytes);
+    const auto need_of = [&](int64_t pieces) { return (((size_t)(outer * (pieces - 1)) * sizeof(A)) + 255) & ~size_t(255); };
+    while (S >= 2 && 2 * need_of(S) > scratchBytes) S /= 2;
+    if (outer * 2 <= waves && S >= 2) {
+      int64_t L = (R + S - 1) / S;
+      L = (L + perIter - 1) / perIter * perIter;  // (whole iterations: pieces start on pack boundaries)
+      S = (R + L - 1) / L;
+      if (S >= 2) {
+        const size_t need = need_of(S);
+        A* totals = (A*)scratch;
+        A* carries = (A*)(scratch + need);
+        const int wpb = kBlock / 64;
+        const int gridT = (int)std::max<int64_t>(1, (outer * (S - 1) + wpb - 1) / wpb);
+        const int grid = (int)std::max<int64_t>(1, (outer * S + wpb - 1) / wpb);
+#define THC_SCAN_ROWS_SPLIT(V)                                                                                     \
+  do {                                                                                                             \
+    hipLaunchKernelGGL((scan_rows_kernel<T, Op, V, true>), dim3(gridT), dim3(kBlock), 0, st, out, in,              \
+                       (uint64_t)outer, (uint64_t)R, 0, (uint64_t)S, (uint64_t)L, (const A*)nullptr, totals);      \
+    launch_scan<A, Op>(s, carries, totals, outer, S - 1, 1, scratch + 2 * need, scratchBytes - 2 * need);          \
+    hipLaunchKernelGGL((scan_rows_kernel<T, Op, V, false>), dim3(grid), dim3(kBlock), 0, st, out, in,              \
+                       (uint64_t)outer, (uint64_t)R, streaming, (uint64_t)S, (uint64_t)L, (const A*)carries,       \
+                       (A*)nullptr);                                                                               \
+  } while (0)
+        if (vec) THC_SCAN_ROWS_SPLIT(VEC);
+        else THC_SCAN_ROWS_SPLIT(1);
+#undef THC_SCAN_ROWS_SPLIT
+        note_kernel("scan-rows-split");
+        return;
+      }
+    }
+  }
   // The column kernel with the rows cut into parts that scan side by side (totals of the parts, their
   // scan by this function on the accumulator type, then every part from its carry): for long scans over
   // rows of whole packs of at least `scan.cols.split_min_row_bytes`, whose lanes the column tiling keeps
@@ -842,12 +924,13 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
     const int64_t cap = (int64_t)num_compute_units(s) * 32;
     const int64_t blocks = (outer + (kBlock / 64) - 1) / (kBlock / 64);
     const int grid = (int)std::max<int64_t>(1, std::min(blocks, cap));
+    using A = typename ScanAcc<T>::type;
     if (aligned && R % VEC == 0)
       hipLaunchKernelGGL((scan_rows_kernel<T, Op, VEC>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, nts);
+                         (uint64_t)outer, (uint64_t)R, nts, (uint64_t)1, (uint64_t)R, (const A*)nullptr, (A*)nullptr);
     else
       hipLaunchKernelGGL((scan_rows_kernel<T, Op, 1>), dim3(grid), dim3(kBlock), 0, st, out, in,
-                         (uint64_t)outer, (uint64_t)R, nts);
+                         (uint64_t)outer, (uint64_t)R, nts, (uint64_t)1, (uint64_t)R, (const A*)nullptr, (A*)nullptr);
     note_kernel("scan-rows");
   } else {
     const bool vec = aligned && inner % VECC == 0;

@@ -71,7 +71,8 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
         sparse = (rng.integers(0, 50, shape) == 0) * rng.integers(-2, 3, shape)     # running sums fit half
         x = sparse.astype(dtype)
         thc.set_tuning("scan.chunk_bytes", chunk)
-        thc.set_tuning("scan.cols.split", 0)     # (wide rows would take the split column kernel)
+        thc.set_tuning("scan.cols.split", 0)     # (wide rows would take the split column kernel,
+        thc.set_tuning("scan.rows.split", 0)     #  long rows a wave per piece)
         try:
             got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), dim)
             assert thc.last_kernel() == "scan-chunked", (shape, thc.last_kernel())
@@ -92,6 +93,7 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
         finally:
             thc.set_tuning("scan.chunk_bytes", 32768)
             thc.set_tuning("scan.cols.split", 1)
+            thc.set_tuning("scan.rows.split", 1)
             thc.set_tuning("scan.lookback", 0)
             thc.set_tuning("scan.lookback_spin", 4096)
         want = np.cumsum(sparse, axis=dim)
@@ -109,12 +111,64 @@ def test_gpu_long_scans_with_few_columns_run_in_chunks(thc, oracle, kind):
     else:
         assert_bit_equal(got.numpy(), want.astype(dtype))
     thc.set_tuning("scan.chunked", 0)
+    thc.set_tuning("scan.rows.split", 0)
     try:
         x = rng.integers(-2, 3, (3, 70001)).astype(dtype)
         got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), 1)
         assert thc.last_kernel() == "scan-rows"
     finally:
         thc.set_tuning("scan.chunked", 1)
+        thc.set_tuning("scan.rows.split", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double", "byte", "long"])
+def test_gpu_few_long_rows_scan_in_pieces(thc, oracle, kind):
+    """A 1-D cumsum (or a few long rows) is cut into pieces that scan side by side, a wave per piece:
+    totals of the pieces, their scan, then every piece from its carry. Exact on small integers; row
+    lengths that are and are not whole packs, storage offsets off the 16-byte grid, in place."""
+    rng = np.random.default_rng(29)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64, "byte": np.uint8,
+             "long": np.int64}[kind]
+    for shape, dim, off, iters in (((1 << 20,), 0, 0, 8), ((1000003,), 0, 0, 8), ((3, 300000), 1, 0, 8),
+                                   ((2, 1, 70001), 2, 1, 2), ((5, 40960), 1, 3, 1), ((1, 123457), 1, 0, 1)):
+        n = int(np.prod(shape))
+        if kind == "byte":
+            sparse = (rng.integers(0, 6000, n + off) == 0) * rng.integers(0, 2, n + off)
+        else:
+            sparse = (rng.integers(0, 600, n + off) == 0) * rng.integers(-2, 3, n + off)     # running sums fit half
+        x = sparse.astype(dtype)
+        strides = [1] * len(shape)
+        for d in range(len(shape) - 2, -1, -1):
+            strides[d] = strides[d + 1] * shape[d + 1]
+        thc.set_tuning("scan.rows.split_min_iters", iters)
+        try:
+            dev = thc.Tensor.from_storage(x, off, shape, tuple(strides), kind=kind)
+            got = thc.Tensor(kind).cumsum(dev, dim)
+            assert thc.last_kernel() == "scan-rows-split", (shape, thc.last_kernel())
+            dev.cumsum(dev, dim)
+            assert thc.last_kernel() == "scan-rows-split"
+        finally:
+            thc.set_tuning("scan.rows.split_min_iters", 8)
+        want = np.cumsum(sparse[off:].reshape(shape), axis=dim)
+        assert np.abs(want).max() < (256 if kind == "byte" else 2048)
+        assert_bit_equal(got.numpy(), want.astype(dtype), "%s %s" % (kind, shape))
+        assert_bit_equal(dev.numpy(), want.astype(dtype), "%s %s in place" % (kind, shape))
+        assert_bit_equal(dev.storage_numpy()[:off], x[:off])       # nothing written before the rows
+    if kind != "byte":
+        ones = np.ones((2, 100000), dtype)
+        ones[:, ::9000] = 2
+        ones[1, 5::17000] = -1
+        got = thc.Tensor(kind).cumprod(thc.Tensor.from_numpy(ones), 1)
+        assert thc.last_kernel() == "scan-rows-split"
+        assert_bit_equal(got.numpy(), np.cumprod(ones.astype(np.float64), axis=1).astype(dtype))
+    if kind in ("float", "double"):
+        x = rng.standard_normal(3000001).astype(dtype)
+        got = thc.Tensor(kind).cumsum(thc.Tensor.from_numpy(x), 0).numpy().astype(np.float64)
+        assert thc.last_kernel() == "scan-rows-split"
+        want = np.cumsum(x.astype(np.float64))
+        mass = np.cumsum(np.abs(x.astype(np.float64)))
+        assert np.all(np.abs(got - want) <= 1e-5 * np.maximum(np.abs(want), mass / 64))
 
 
 @pytest.mark.gpu
