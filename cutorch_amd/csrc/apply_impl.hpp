@@ -1594,9 +1594,4 @@ bool apply_dispatch_group(THCState* s, Plan& pl, bool sameShape, PointOp op, flo
   return true;
 }
 
-template <typename T>
-void apply_copy(THCState* s, Plan& pl, bool sameShape) {
-  run_plan<T>(s, pl, sameShape, OpCopy{});
-}
-
 }  // namespace thc

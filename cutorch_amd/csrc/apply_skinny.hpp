@@ -1,0 +1,259 @@
+// Copies between a layout whose two innermost joint dims are one dense run (long x short, the short
+// dim fastest) and one that keeps the long dim at unit stride, the short dim selecting a plane:
+// tall-and-skinny transposes such as (N, 3) <-> (3, N):t() and the NCHW <-> NHWC conversions of
+// images with few channels. The 64 x 128 tiles of the tiled kernels are nearly empty on a short dim
+// of 3..64 elements (a (2^22, 16) transpose ran at 0.09 of peak through them, and the element-wise
+// strided kernel at 0.33-0.38 on 3 or 4 planes). Here a tile is T long-dim positions x all S
+// short-dim positions, about 16 KiB: on the dense side one contiguous run of T * S elements, on the
+// planar side S runs of T elements. Both sides move 16-byte packs where their alignment allows
+// (element-wise otherwise); the tile changes order in LDS, laid out lds[s * pitch + t].
+// (what the reference's one strided apply does for these copies: lib/THC/THCApply.cuh:426-640,
+// called from lib/THC/THCTensorCopy.cu:26-122)
+#pragma once
+#include <algorithm>
+#include <cstdint>
+
+#include "apply_plan.hpp"
+#include "common.hpp"
+#include "device_util.hpp"
+
+namespace thc {
+namespace {
+
+struct SkinnyArgs {
+  uint32_t S;             // extent of the short dim
+  uint32_t T;             // long-dim positions per tile (a multiple of 16)
+  uint32_t pitch;         // LDS elements between planes
+  uint32_t totalTiles;
+  uint64_t longSize;      // extent of the long dim
+  int64_t planeStride;    // planar side: elements between planes
+  int nbatch;             // dims outside the two, innermost first
+  int ntStore;
+  Divisor<uint32_t> sdiv;           // by S
+  Divisor<uint32_t> tilesPerSlice;  // tiles along the long dim
+  Divisor<uint32_t> bsize[kMaxDims];
+  int64_t denseBatchStride[kMaxDims], planarBatchStride[kMaxDims];
+};
+
+// TO_PLANAR: the source is the dense side. VD / VP: packs on the dense / planar side.
+template <typename E, bool TO_PLANAR, bool VD, bool VP>
+__global__ __launch_bounds__(kBlock) void skinny_copy_kernel(E* __restrict__ dst, const E* __restrict__ src,
+                                                             SkinnyArgs a) {
+  constexpr uint32_t VEC = 16 / sizeof(E);
+  using P = Pack<E, VEC>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  E* lds = reinterpret_cast<E*>(lds_raw);
+  const uint32_t S = a.S, pitch = a.pitch;
+  for (uint32_t b = blockIdx.x; b < a.totalTiles; b += gridDim.x) {
+    uint32_t rest, tl;
+    a.tilesPerSlice.divmod(b, rest, tl);
+    int64_t dOff = 0, pOff = 0;
+    for (int j = 0; j < a.nbatch; ++j) {
+      uint32_t r;
+      a.bsize[j].divmod(rest, rest, r);
+      dOff += (int64_t)r * a.denseBatchStride[j];
+      pOff += (int64_t)r * a.planarBatchStride[j];
+    }
+    const uint64_t t0 = (uint64_t)tl * a.T;
+    const uint32_t tn = (uint32_t)min((uint64_t)a.T, a.longSize - t0);  // long-dim positions of this tile
+    const uint32_t n = tn * S;                                            // elements of this tile
+    dOff += (int64_t)(t0 * S);
+    pOff += (int64_t)t0;
+    const E* dsrc = src + dOff;
+    const E* psrc = src + pOff;
+    E* ddst = dst + dOff;
+    E* pdst = dst + pOff;
+    const uint32_t planePacks = VP ? tn / VEC : 0;  // whole packs of a plane's run
+    // ---- into LDS
+    if (TO_PLANAR) {
+      const uint32_t packs = VD ? n / VEC : 0;
+      constexpr int U = 4;
+      for (uint32_t k0 = threadIdx.x; k0 < packs; k0 += U * kBlock) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(dsrc) + min(k0 + u * kBlock, packs - 1));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t k = k0 + u * kBlock;
+          if (k < packs) {
+            uint32_t t, s;
+            a.sdiv.divmod(k * VEC, t, s);
+#pragma unroll
+            for (uint32_t e = 0; e < VEC; ++e) {
+              lds[s * pitch + t] = v[u].v[e];
+              if (++s == S) {
+                s = 0;
+                ++t;
+              }
+            }
+          }
+        }
+      }
+      for (uint32_t m = packs * VEC + threadIdx.x; m < n; m += kBlock) {
+        uint32_t t, s;
+        a.sdiv.divmod(m, t, s);
+        lds[s * pitch + t] = dsrc[m];
+      }
+    } else {
+      const uint32_t packs = planePacks * S;
+      constexpr int U = 4;
+      for (uint32_t k0 = threadIdx.x; k0 < packs; k0 += U * kBlock) {
+        P v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t k = min(k0 + u * kBlock, packs - 1);
+          const uint32_t s = k / planePacks, j = k - s * planePacks;
+          v[u] = load_pack<true>(reinterpret_cast<const P*>(psrc + (int64_t)s * a.planeStride) + j);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t k = k0 + u * kBlock;
+          if (k < packs) {
+            const uint32_t s = k / planePacks, j = k - s * planePacks;
+#pragma unroll
+            for (uint32_t e = 0; e < VEC; ++e) lds[s * pitch + j * VEC + e] = v[u].v[e];
+          }
+        }
+      }
+      // what the packs leave: the end of every plane's run, or all of it
+      const uint32_t left = tn - planePacks * VEC;
+      for (uint32_t m = threadIdx.x; m < left * S; m += kBlock) {
+        const uint32_t s = m / left, t = planePacks * VEC + (m - s * left);
+        lds[s * pitch + t] = psrc[(int64_t)s * a.planeStride + t];
+      }
+    }
+    __syncthreads();
+    // ---- out of LDS
+    if (TO_PLANAR) {
+      const uint32_t packs = planePacks * S;
+      for (uint32_t k = threadIdx.x; k < packs; k += kBlock) {
+        const uint32_t s = k / planePacks, j = k - s * planePacks;
+        P v;
+#pragma unroll
+        for (uint32_t e = 0; e < VEC; ++e) v.v[e] = lds[s * pitch + j * VEC + e];
+        P* at = reinterpret_cast<P*>(pdst + (int64_t)s * a.planeStride) + j;
+        if (a.ntStore) store_pack<true>(at, v);
+        else store_pack<false>(at, v);
+      }
+      const uint32_t left = tn - planePacks * VEC;
+      for (uint32_t m = threadIdx.x; m < left * S; m += kBlock) {
+        const uint32_t s = m / left, t = planePacks * VEC + (m - s * left);
+        pdst[(int64_t)s * a.planeStride + t] = lds[s * pitch + t];
+      }
+    } else {
+      const uint32_t packs = VD ? n / VEC : 0;
+      for (uint32_t k = threadIdx.x; k < packs; k += kBlock) {
+        uint32_t t, s;
+        a.sdiv.divmod(k * VEC, t, s);
+        P v;
+#pragma unroll
+        for (uint32_t e = 0; e < VEC; ++e) {
+          v.v[e] = lds[s * pitch + t];
+          if (++s == S) {
+            s = 0;
+            ++t;
+          }
+        }
+        P* at = reinterpret_cast<P*>(ddst) + k;
+        if (a.ntStore) store_pack<true>(at, v);
+        else store_pack<false>(at, v);
+      }
+      for (uint32_t m = packs * VEC + threadIdx.x; m < n; m += kBlock) {
+        uint32_t t, s;
+        a.sdiv.divmod(m, t, s);
+        ddst[m] = lds[s * pitch + t];
+      }
+    }
+    __syncthreads();  // the tile is refilled by the next round
+  }
+}
+
+// `pl` is the jointly collapsed plan of a copy, dims ordered by the destination's strides
+// (operand 0 = destination, 1 = source). Returns false when the layouts are not of this kind.
+template <typename E>
+bool launch_skinny_copy(THCState* s, const Plan& pl) {
+  constexpr int64_t VEC = 16 / sizeof(E);
+  if (!tuning("apply.skinny", 1) || pl.nops != 2) return false;
+  const int nd = pl.lay[0].dims;
+  if (nd < 2 || pl.numel >= (int64_t(1) << 40)) return false;
+  const Layout& out = pl.lay[0];
+  const Layout& in = pl.lay[1];
+  const int q = nd - 1, p = nd - 2;
+  // which operand is the dense side, and which of the two dims is the short one (small shapes can be
+  // read both ways: the shorter short dim wins)
+  int dense = -1, ds = -1, dl = -1;
+  const int64_t maxShortBytes = tuning("apply.skinny.max_short_bytes", 256);
+  auto consider = [&](int cand, int cs, int cl) {
+    const int64_t S = pl.lay[cand].size[cs], L = pl.lay[cand].size[cl];
+    if (S < 2 || L < 64 || S * (int64_t)sizeof(E) > maxShortBytes) return;
+    if (dense >= 0 && pl.lay[dense].size[ds] <= S) return;
+    dense = cand, ds = cs, dl = cl;
+  };
+  // planes of the source gathered into dense rows of the destination
+  if (out.stride[q] == 1 && out.stride[p] == out.size[q] && in.stride[p] == 1 && in.stride[q] > 0) consider(0, q, p);
+  // dense rows of the source scattered into planes of the destination
+  if (in.stride[p] == 1 && in.stride[q] == in.size[p] && out.stride[q] == 1 && out.stride[p] > 0) consider(1, p, q);
+  if (dense < 0) return false;
+  const Layout& dn = pl.lay[dense];
+  const Layout& pn = pl.lay[1 - dense];
+  const int64_t S = dn.size[ds], L = dn.size[dl];
+  for (int k = 0; k < 2; ++k)
+    for (int d = 0; d < nd; ++d)
+      if (pl.lay[k].stride[d] < 0) return false;
+  SkinnyArgs a{};
+  a.S = (uint32_t)S;
+  a.longSize = (uint64_t)L;
+  a.planeStride = pn.stride[ds];
+  int64_t T = std::max<int64_t>(64, (tuning("apply.skinny.tile_bytes", 16384) / (S * (int64_t)sizeof(E))) / 16 * 16);
+  T = std::min<int64_t>(T, (L + 15) / 16 * 16);
+  a.T = (uint32_t)T;
+  a.pitch = (uint32_t)(T + 16 / sizeof(E) + 1) | 1u;
+  a.sdiv.set((uint64_t)S);
+  const int64_t tiles = (L + T - 1) / T;
+  a.tilesPerSlice.set((uint64_t)tiles);
+  int64_t total = tiles;
+  a.nbatch = 0;
+  for (int d = nd - 3; d >= 0; --d) {
+    a.bsize[a.nbatch].set((uint64_t)dn.size[d]);
+    a.denseBatchStride[a.nbatch] = dn.stride[d];
+    a.planarBatchStride[a.nbatch] = pn.stride[d];
+    ++a.nbatch;
+    total *= dn.size[d];
+  }
+  if (total >= (int64_t(1) << 31)) return false;
+  a.totalTiles = (uint32_t)total;
+  a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(E)) ? 1 : 0;
+  // packs: every tile's run starts on a 16-byte boundary
+  auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  bool vd = aligned(pl.ptr[dense]), vp = aligned(pl.ptr[1 - dense]) && a.planeStride % VEC == 0;
+  for (int j = 0; j < a.nbatch; ++j) {
+    vd = vd && a.denseBatchStride[j] % VEC == 0;
+    vp = vp && a.planarBatchStride[j] % VEC == 0;
+  }
+  const size_t ldsBytes = ((size_t)S * a.pitch * sizeof(E) + 15) & ~size_t(15);
+  if (ldsBytes > 64 * 1024) return false;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, (int64_t)num_compute_units(s) * 64));
+  E* dst = (E*)pl.ptr[0];
+  const E* src = (const E*)pl.ptr[1];
+  hipStream_t st = current_stream(s);
+#define THC_SKINNY(TP, D, Pk) \
+  hipLaunchKernelGGL((skinny_copy_kernel<E, TP, D, Pk>), dim3(grid), dim3(kBlock), ldsBytes, st, dst, src, a)
+  if (dense == 1) {
+    if (vd && vp) THC_SKINNY(true, true, true);
+    else if (vd) THC_SKINNY(true, true, false);
+    else if (vp) THC_SKINNY(true, false, true);
+    else THC_SKINNY(true, false, false);
+  } else {
+    if (vd && vp) THC_SKINNY(false, true, true);
+    else if (vd) THC_SKINNY(false, true, false);
+    else if (vp) THC_SKINNY(false, false, true);
+    else THC_SKINNY(false, false, false);
+  }
+#undef THC_SKINNY
+  note_kernel("skinny");
+  return true;
+}
+
+}  // namespace
+}  // namespace thc

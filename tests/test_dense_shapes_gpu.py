@@ -90,14 +90,20 @@ def test_transposed_copies_of_every_element_size_at_odd_shapes(thc, kind):
             n = rows * cols
             src = rng.integers(0, 100, n + off_in).astype(dtype)
             dst = np.full(n + off_out, 7, dtype)
-            a = thc.Tensor.from_storage(src, off_in, (rows, cols), (1, rows), kind=kind)     # a = b:t()
-            out = thc.Tensor.from_storage(dst, off_out, (rows, cols), (cols, 1), kind=kind)
-            out.copy(a)
-            k = thc.last_kernel()
-            assert k.startswith("tiled"), (kind, rows, cols, k)
             want = dst.copy()
             want[off_out:] = src[off_in:].reshape(cols, rows).T.reshape(-1)
-            assert_bit_equal(out.storage_numpy(), want, "%s %dx%d +%d/+%d %s" % (kind, rows, cols, off_in, off_out, k))
+            # (a dim short enough for the tall-and-skinny copy takes that kernel unless it is switched off)
+            for skinny in (1, 0):
+                a = thc.Tensor.from_storage(src, off_in, (rows, cols), (1, rows), kind=kind)     # a = b:t()
+                out = thc.Tensor.from_storage(dst, off_out, (rows, cols), (cols, 1), kind=kind)
+                thc.set_tuning("apply.skinny", skinny)
+                try:
+                    out.copy(a)
+                finally:
+                    thc.set_tuning("apply.skinny", 1)
+                k = thc.last_kernel()
+                assert k.startswith("tiled") or (skinny and k == "skinny"), (kind, rows, cols, k)
+                assert_bit_equal(out.storage_numpy(), want, "%s %dx%d +%d/+%d %s" % (kind, rows, cols, off_in, off_out, k))
 
 
 def test_reductions_and_scans_are_reproducible_run_to_run(thc):

@@ -613,6 +613,7 @@ def test_aligned_tiles_in_bands_along_p(thc, oracle, band):
     for single-input ops): whole bands, a ragged last band, a batch dim in front, fused q."""
     rng = np.random.default_rng(92)
     thc.set_tuning("apply.tiled.group_p_vec", band)
+    thc.set_tuning("apply.skinny", 0)          # (copies with a dim of at most 256 bytes would leave the tiled kernel)
     try:
         for rows, cols in ((320, 512), (448, 132), (1000, 64), (2304, 128)):
             ga = (rows * cols, 0, (rows, cols), (1, rows))               # a:t()
@@ -630,6 +631,7 @@ def test_aligned_tiles_in_bands_along_p(thc, oracle, band):
                                                 contiguous_geometry((520, 24, 40))], rng) == "tiled-fused"
     finally:
         thc.set_tuning("apply.tiled.group_p_vec", -1)
+        thc.set_tuning("apply.skinny", 1)
 
 
 @pytest.mark.parametrize("kind", ["float", "int"])

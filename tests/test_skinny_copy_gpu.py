@@ -1,0 +1,91 @@
+"""Copies between a dense (long x short) layout and its planar counterpart (the short dim selecting a
+plane, the long dim at unit stride): tall-and-skinny transposes and NCHW <-> NHWC conversions with few
+channels (lib/THC/THCTensorCopy.cu:26-122 runs them through the one strided apply). Bit-exact against
+numpy on every element size, in both directions, with pack-aligned and unaligned sides, ragged last
+tiles, batch dims, and the storage around the destination untouched."""
+import numpy as np
+import pytest
+
+from tests.util import assert_bit_equal
+
+KINDS = {"float": np.float32, "half": np.float16, "byte": np.uint8, "double": np.float64, "short": np.int16,
+         "long": np.int64}
+
+
+def values(rng, n, dtype):
+    if np.dtype(dtype).kind == "f":
+        return rng.integers(-1000, 1000, n).astype(dtype)
+    info = np.iinfo(dtype)
+    return rng.integers(max(info.min, -30000), min(info.max, 30000), n).astype(dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", sorted(KINDS))
+def test_tall_skinny_transposes_both_directions(thc, kind):
+    rng = np.random.default_rng(41)
+    dtype = KINDS[kind]
+    for long_n, short_n in ((100000, 3), (65536, 4), (70001, 5), (4099, 16), (30000, 31), (1000, 2), (64, 7)):
+        if short_n * np.dtype(dtype).itemsize > 256:
+            continue
+        for off in (0, 1):
+            planar = values(rng, short_n * long_n + off, dtype)
+            src = thc.Tensor.from_storage(planar, off, (long_n, short_n), (1, long_n), kind=kind)     # (short, long):t()
+            dst = thc.Tensor(kind).resize((long_n, short_n))
+            dst.copy(src)
+            assert thc.last_kernel() == "skinny", (kind, long_n, short_n, thc.last_kernel())
+            want = planar[off:].reshape(short_n, long_n).T
+            assert_bit_equal(dst.numpy(), np.ascontiguousarray(want), "%s gather %d x %d off %d" % (kind, long_n, short_n, off))
+            # the other direction: dense rows scattered into planes, into the middle of a larger storage
+            dense = values(rng, long_n * short_n + off, dtype)
+            dsrc = thc.Tensor.from_storage(dense, off, (short_n, long_n), (1, short_n), kind=kind)    # (long, short):t()
+            guard = values(rng, short_n * long_n + 2 * 5 + off, dtype)
+            ddst = thc.Tensor.from_storage(guard, 5 + off, (short_n, long_n), (long_n, 1), kind=kind)
+            ddst.copy(dsrc)
+            assert thc.last_kernel() == "skinny", (kind, long_n, short_n, thc.last_kernel())
+            want = dense[off:].reshape(long_n, short_n).T
+            assert_bit_equal(ddst.numpy(), np.ascontiguousarray(want), "%s scatter %d x %d off %d" % (kind, long_n, short_n, off))
+            after = ddst.storage_numpy()
+            assert_bit_equal(after[:5 + off], guard[:5 + off])
+            assert_bit_equal(after[5 + off + short_n * long_n:], guard[5 + off + short_n * long_n:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "byte"])
+def test_image_layout_conversions(thc, kind):
+    """NCHW -> NHWC and back for 3, 4 and 16 channels: (h, w) collapse to one long dim, n stays a batch
+    dim; a padded plane stride on the planar side; round trip returns the input."""
+    rng = np.random.default_rng(42)
+    dtype = KINDS[kind]
+    for n, c, h, w, pad in ((5, 3, 37, 53, 0), (2, 4, 64, 64, 0), (3, 16, 20, 24, 0), (2, 3, 33, 40, 8)):
+        plane = h * w + pad
+        store = values(rng, n * c * plane, dtype)
+        nchw = store.reshape(n, c, plane)[:, :, :h * w].reshape(n, c, h, w)
+        src = thc.Tensor.from_storage(store, 0, (n, h, w, c), (c * plane, w, 1, plane), kind=kind)   # NHWC view of NCHW
+        nhwc = thc.Tensor(kind).resize((n, h, w, c))
+        nhwc.copy(src)
+        assert thc.last_kernel() == "skinny", (kind, c, thc.last_kernel())
+        assert_bit_equal(nhwc.numpy(), np.ascontiguousarray(nchw.transpose(0, 2, 3, 1)))
+        back_view = nhwc.view_as_strided(0, (n, c, h, w), (h * w * c, 1, w * c, c))                    # NCHW view of NHWC
+        back = thc.Tensor(kind).resize((n, c, h, w))
+        back.copy(back_view)
+        assert thc.last_kernel() == "skinny", (kind, c, thc.last_kernel())
+        assert_bit_equal(back.numpy(), np.ascontiguousarray(nchw))
+
+
+@pytest.mark.gpu
+def test_skinny_copy_declines_what_it_does_not_cover(thc):
+    rng = np.random.default_rng(43)
+    x = rng.standard_normal((300, 200)).astype(np.float32)
+    dst = thc.Tensor("float").resize((200, 300))
+    dst.copy(thc.Tensor.from_numpy(x).t())                 # both dims long: the tiled kernel
+    assert thc.last_kernel() != "skinny"
+    assert_bit_equal(dst.numpy(), np.ascontiguousarray(x.T))
+    thc.set_tuning("apply.skinny", 0)
+    try:
+        y = rng.standard_normal((3, 5000)).astype(np.float32)
+        d2 = thc.Tensor("float").resize((5000, 3))
+        d2.copy(thc.Tensor.from_numpy(y).t())
+        assert thc.last_kernel() != "skinny"
+        assert_bit_equal(d2.numpy(), np.ascontiguousarray(y.T))
+    finally:
+        thc.set_tuning("apply.skinny", 1)
