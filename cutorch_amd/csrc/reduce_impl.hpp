@@ -502,12 +502,24 @@ __global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T
        row += wavesPerGrid) {
     A bv = O::worst();
     I bi = ~(I)0;
-    for (I sp = lane; sp < S; sp += 64) {
-      const A v = partV[row * S + sp];
-      const I ix = partI[row * S + sp];
-      if (O::better(v, ix, bv, bi)) {
-        bv = v;
-        bi = ix;
+    // eight partials requested at a time: with a load per comparison the one wave that folds a long
+    // vector's 8192 partials spent 40 us on memory round trips (argmax of 2^26 elements: 85 -> 51 us)
+    constexpr int U = 8;
+    for (I sp = lane; sp < S; sp += 64 * U) {
+      A v[U];
+      I ix[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const I at = row * S + min(sp + (I)(64 * u), S - 1);  // (past the end: not used)
+        v[u] = partV[at];
+        ix[u] = partI[at];
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (sp + (I)(64 * u) < S && O::better(v[u], ix[u], bv, bi)) {
+          bv = v[u];
+          bi = ix[u];
+        }
       }
     }
     for (uint32_t o = 32; o > 0; o >>= 1) {
@@ -2613,8 +2625,9 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
         return;
       }
     }
-    // Few long rows: cut them as run_rows does.
-    const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.waves_per_cu", 32);
+    // Few long rows: cut them as run_rows does, into fewer pieces: one wave folds a row's partials
+    // (argmax of a 2^26-element vector: 32 pieces per CU 0.56 of peak, 16 0.61, 8 0.62, 4 0.69).
+    const int64_t target = (int64_t)num_compute_units(s) * tuning("reduce.rows.index_waves_per_cu", 4);
     const int64_t minChunk = tuning("reduce.rows.min_chunk", 8192);
     int64_t S = 1, chunk = g.R;
     A* partV = nullptr;
