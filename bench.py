@@ -336,7 +336,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
-                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d")
+                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -382,7 +382,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                              8 * 8192 * 8192, 8192 * 8192, lambda i: sq_out.renorm(sq, 2.0, 0, 1.0)),
             })
         if set(nx) & {"N-sum-rows33", "N-max-rows33", "N-sum-slab", "N-sum-tall", "N-cumsum-rows10",
-                      "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-argmax-1d"}:
+                      "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-argmax-1d", "N-argmax-tall"}:
             # shapes off the aligned grid: short / misaligned rows, small slices, tall narrow matrices
             nr = 1 << 26
             flat = e_src
@@ -396,6 +396,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
             swide = T("float").resize((65536, 1000))
             s1d = T("float").resize((nr,))
             omax1, imax1 = T("float").resize((1,)), T("long").resize((1,))
+            omaxt, imaxt = T("float").resize((1, 10)), T("long").resize((1, 10))
             oddT = T.from_numpy(rng.standard_normal((8193, 8191), dtype=np.float32)).t()
             oddB = T.from_numpy(rng.standard_normal((8191, 8193), dtype=np.float32))
             oddO = T("float").resize((8191, 8193))
@@ -418,6 +419,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                                   lambda i: swide.cumsum(vwide, 0)),
                 "N-cumsum-1d": ("cumsum of a 2^26-element fp32 vector (a wave per piece, input read twice, counted once)",
                                 8 * nr, nr, lambda i: s1d.cumsum(flat, 0)),
+                "N-argmax-tall": ("max+argmax over dim 0 of 6710886x10 fp32", 4 * n10, n10, lambda i: omaxt.max(imaxt, v10, 0)),
                 "N-argmax-1d": ("max+argmax of a 2^26-element fp32 vector", 4 * nr, nr, lambda i: omax1.max(imax1, flat, 0)),
                 "N-cumsum-rows10": ("cumsum over last dim of 6710886x10 fp32", 8 * n10, n10, lambda i: s10.cumsum(v10, 1)),
                 "N-cumsum-tall": ("cumsum over dim 0 of 6710886x10 fp32 (input read twice, counted once)", 8 * n10, n10,

@@ -548,6 +548,129 @@ __global__ __launch_bounds__(kBlock) void fold_pairs_kernel(const typename Acc<T
   }
 }
 
+// max/min with index over the long dim of few long narrow slices ([O][R][C] dense, the shapes of
+// reduce_tall_kernel, which is defined further down and whose reading order this is): the slice as a
+// flat run of aligned packs, lane t on packs wb + t + k L with wb and L multiples of the period of
+// the packs' column pattern, so every lane's VEC running (value, row) pairs keep their columns and
+// the rows a lane meets advance by VEC * L / C per step. A lane sees its rows in increasing order
+// (ties never replace, the first NaN stays); lanes and workgroups merge with the index-aware order.
+// Partials go to partV / partI[(o * C + c) * S + s], which fold_pairs_kernel folds per output.
+template <typename T, typename I, bool IS_MAX>
+__global__ __launch_bounds__(kBlock) void reduce_tall_index_kernel(const T* __restrict__ in,
+                                                                   typename Acc<T>::type* __restrict__ partV,
+                                                                   I* __restrict__ partI, I sliceElems, uint32_t C,
+                                                                   uint32_t S, I packsPerWg, uint32_t lanes,
+                                                                   uint32_t pattern, uint32_t folds, Divisor<I> cdiv) {
+  using A = typename Acc<T>::type;
+  using O = PairOrder<IS_MAX, A>;
+  constexpr int VEC = 16 / sizeof(T);
+  using P = Pack<T, VEC>;
+  __shared__ A sv[kBlock * VEC];
+  __shared__ I si[kBlock * VEC];
+  __shared__ A stv[kBlock];
+  __shared__ I sti[kBlock];
+  const I o = blockIdx.x / S;
+  const uint32_t s = blockIdx.x - (uint32_t)o * S;
+  const T* base = in + o * sliceElems;
+  const I npacks = sliceElems / VEC;
+  const I wb = (I)s * packsPerWg, we = min(npacks, wb + packsPerWg);
+  const uint32_t t = threadIdx.x;
+  A bv[VEC];
+  I bi[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    bv[e] = O::worst();
+    bi[e] = ~(I)0;
+  }
+  if (t < lanes && wb < we) {
+    constexpr int U = 8;
+    const P* src = reinterpret_cast<const P*>(base);
+    I row[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      I r;
+      cdiv.divmod((wb + t) * VEC + e, row[e], r);
+    }
+    const I rowStep = (I)lanes * VEC / C;  // (exact: lanes * VEC is a multiple of C)
+    for (I j = wb + t; j < we; j += (I)U * lanes) {
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = load_pack<true>(src + min(j + (I)u * lanes, we - 1));  // (past the end: not used)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (j + (I)u * lanes < we) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            if (O::better_later(x, bv[e])) {
+              bv[e] = x;
+              bi[e] = row[e] + (I)u * rowStep;
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) row[e] += (I)U * rowStep;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    sv[t * VEC + e] = bv[e];
+    si[t * VEC + e] = bi[e];
+  }
+  __syncthreads();
+  // accumulator i = t * VEC + e holds column i % C; accumulators `pattern` apart hold the same column
+  const uint32_t accs = lanes * VEC;
+  if (folds) {
+    if (t < folds * pattern) {
+      const uint32_t k = t / pattern, slot = t - k * pattern;
+      A v = O::worst();
+      I ix = ~(I)0;
+      for (uint32_t i = k * pattern + slot; i < accs; i += folds * pattern) {
+        if (O::better(sv[i], si[i], v, ix)) {
+          v = sv[i];
+          ix = si[i];
+        }
+      }
+      stv[t] = v;
+      sti[t] = ix;
+    }
+    __syncthreads();
+  }
+  for (uint32_t c = t; c < C; c += kBlock) {
+    A v = O::worst();
+    I ix = ~(I)0;
+    if (folds) {
+      for (uint32_t i = c; i < pattern; i += C)
+        for (uint32_t k = 0; k < folds; ++k)
+          if (O::better(stv[k * pattern + i], sti[k * pattern + i], v, ix)) {
+            v = stv[k * pattern + i];
+            ix = sti[k * pattern + i];
+          }
+    } else {
+      for (uint32_t i = c; i < accs; i += C)
+        if (O::better(sv[i], si[i], v, ix)) {
+          v = sv[i];
+          ix = si[i];
+        }
+    }
+    // the elements behind the slice's last whole pack belong to the last workgroup
+    if (s == S - 1)
+      for (I idx = npacks * VEC + ((c + C - (uint32_t)((npacks * VEC) % C)) % C); idx < sliceElems; idx += C) {
+        I rowOf, r;
+        cdiv.divmod(idx, rowOf, r);
+        const A x = acc_up<A>(base[idx]);
+        if (O::better(x, rowOf, v, ix)) {
+          v = x;
+          ix = rowOf;
+        }
+      }
+    const I at = ((I)o * C + c) * S + s;
+    partV[at] = v;
+    partI[at] = ix;
+  }
+}
+
 // Short rows that lie back to back in memory (row r starts at in + r * R).
 // A lane group per row reads 64-byte pieces at the rows' own, mostly
 // misaligned, addresses (100-element fp32 rows summed at 2.8 TB/s, 10-element
@@ -2685,6 +2808,61 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
       note_kernel("slab-index");
       return;
     }
+  }
+  {
+    // few long narrow slices that start on 16-byte boundaries: flat runs of packs (reduce_tall_index_kernel;
+    // the column kernel below keeps C of its lanes busy on them: 6.7M x 10 along dim 0 0.30 of peak)
+    auto tall = [&]() {
+      if (!tuning("reduce.tall", 1)) return false;
+      const int64_t C = g.in.size[nd - 1];
+      if (g.in.stride[nd - 1] != 1 || g.sR != C || C > kBlock ||
+          C * (int64_t)sizeof(T) > tuning("reduce.slab.chunked_max_row_bytes", 512))
+        return false;
+      int64_t run = g.R * C;
+      for (int d = nd - 2; d >= 0; --d) {
+        if (g.in.size[d] != 1 && g.in.stride[d] != run) return false;
+        run *= g.in.size[d];
+      }
+      const int64_t O = g.outElems / C;
+      if (!aligned16(in) || C % VEC == 0 || O >= (int64_t)num_compute_units(s)) return false;
+      if (!(O == 1 || (g.R * C) % VEC == 0) || g.R * C < (int64_t)VEC * kBlock * 8) return false;
+      int64_t gcd = C, b = VEC;
+      while (b) {
+        const int64_t r = gcd % b;
+        gcd = b;
+        b = r;
+      }
+      const int64_t period = C / gcd;  // packs after which the column pattern repeats
+      if (period > kBlock) return false;
+      const int64_t lanes = (kBlock / period) * period, pattern = period * VEC, reps = lanes / period;
+      int64_t folds = 0;
+      if (pattern <= kBlock) {
+        folds = 1;
+        while ((folds + 1) * (folds + 1) * pattern <= reps * C && (folds + 1) * pattern <= kBlock && folds + 1 <= reps) ++folds;
+      }
+      const int64_t npacks = g.R * C / VEC;
+      const int64_t want = std::max<int64_t>(1, (int64_t)num_compute_units(s) * tuning("reduce.tall.index_blocks_per_cu", 2) / O);
+      int64_t packsPerWg = std::max<int64_t>((npacks + want - 1) / want, lanes * 8);
+      packsPerWg = (packsPerWg + period - 1) / period * period;
+      const int64_t ST = (npacks + packsPerWg - 1) / packsPerWg;
+      size_t scratchBytes = 0;
+      char* scratch = (char*)scratch_space(s, &scratchBytes);
+      if (O * ST >= (int64_t(1) << 31) || (size_t)(16 * ST * g.outElems) > scratchBytes) return false;
+      I* partI = (I*)scratch;  // both parts start 8-byte aligned
+      A* partV = (A*)(scratch + 8 * (size_t)ST * (size_t)g.outElems);
+      Divisor<I> cdiv;
+      cdiv.set((uint64_t)C);
+      hipLaunchKernelGGL((reduce_tall_index_kernel<T, I, IS_MAX>), dim3((unsigned)(O * ST)), dim3(kBlock), 0, st, in,
+                         partV, partI, (I)(g.R * C), (uint32_t)C, (uint32_t)ST, (I)packsPerWg, (uint32_t)lanes,
+                         (uint32_t)pattern, (uint32_t)folds, cdiv);
+      const int64_t rows = g.outElems;
+      const int fgrid = capped_grid(s, (rows + kBlock / 64 - 1) / (kBlock / 64), "reduce.rows.blocks_per_cu", 64);
+      hipLaunchKernelGGL((fold_pairs_kernel<T, I, IS_MAX>), dim3(fgrid), dim3(kBlock), 0, st, partV, partI, outV, outI,
+                         make_outer<I>(g.in, g.out, nd), make_outer<I>(g.in, g.idx, nd), (I)rows, (I)ST);
+      note_kernel("tall-index");
+      return true;
+    };
+    if (tall()) return;
   }
   {
     // the (value, index) kernel does several ALU steps per element: two workgroups

@@ -169,6 +169,70 @@ def test_minmax_with_many_ties(thc, oracle, which, kind):
         run_minmax(thc, oracle, which, dev, ref, dim, kind)
 
 
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double", "byte"])
+def test_minmax_of_long_narrow_slices(thc, oracle, kind):
+    """max / min with index along the long dim of few long narrow slices (flat runs of packs, every
+    lane keeping (value, row) pairs per column): tie-heavy data (the first of equal extremes wins at
+    every level), NaN / inf / signed zeros planted at the ends of workgroup pieces and in the
+    elements behind the last whole pack, columns that are all -inf; against the oracle and, for the
+    planted cases, numpy's first-occurrence argmax."""
+    rng = np.random.default_rng(37)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64, "byte": np.uint8}[kind]
+    vec = 16 // np.dtype(dtype).itemsize
+    for shape, dim in (((200003, 3), 0), ((70001, 10), 0), ((30000, 33), 0), ((2, 40000, 7), 1), ((3, 16000, 5), 1),
+                       ((1, 50001, 9), 1), ((25000, 50), 0)):
+        inner = int(np.prod(shape[dim + 1:]))
+        outer = int(np.prod(shape[:dim]))
+        flat = inner % vec != 0 and (outer == 1 or (shape[dim] * inner) % vec == 0)
+        lo, hi = (0, 4) if kind == "byte" else (-3, 4)
+        x = rng.integers(lo, hi, shape).astype(dtype)
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        for which in ("max", "min"):
+            if kind in ("float", "half"):      # (the oracle's restatement is the float one)
+                k = run_minmax(thc, oracle, which, dev, ref, dim, kind)
+                assert k == ("tall-index" if flat else "cols-index-split"), (shape, which, k)
+            vals, idx = thc.Tensor(kind), thc.Tensor("long")
+            getattr(vals, which)(idx, dev, dim)
+            assert thc.last_kernel() == ("tall-index" if flat else "cols-index-split"), (shape, which, thc.last_kernel())
+            want = (np.argmax if which == "max" else np.argmin)(x, axis=dim) + 1
+            assert np.array_equal(idx.numpy().reshape(want.shape), want), (shape, which)
+            wantv = (np.max if which == "max" else np.min)(x, axis=dim)
+            assert_bit_equal(vals.numpy().reshape(wantv.shape), wantv, "%s %s values" % (shape, which))
+    if kind in ("float", "half"):
+        x = rng.integers(-3, 4, (70001, 10)).astype(dtype)
+        x[:, 0] = -np.inf                      # a column without a candidate: index 1
+        x[:, 1] = 0.0
+        x[5, 1], x[600, 1] = -0.0, -0.0        # zeros: the first one (+0 at row 0) stays for max and min
+        x[69999, 2] = np.nan                   # in the last workgroup's piece
+        x[70000, 3] = np.nan                   # behind the last whole pack (70001 * 10 is not a multiple of 4 or 8)
+        x[40000, 4], x[123, 4] = np.nan, np.nan
+        x[33333, 5] = np.inf
+        x[33333, 6] = -np.inf
+        dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
+        for which in ("max", "min"):
+            vals, idx = thc.Tensor(kind), thc.Tensor("long")
+            getattr(vals, which)(idx, dev, 0)
+            assert thc.last_kernel() == "tall-index"
+            rv, ri = oracle.minmax_dim(which, ref, 0)
+            assert np.array_equal(idx.numpy(), ri.numpy()), which
+            g, w = vals.numpy(), rv.numpy()
+            assert np.array_equal(np.isnan(g), np.isnan(w))
+            assert_bit_equal(g[~np.isnan(g)], w[~np.isnan(w)])
+            i = idx.numpy().reshape(-1)
+            assert i[2] == 70000 and i[3] == 70001 and i[4] == 124 and i[1] == 1
+            assert i[0] == (1 if which == "max" else 1)
+            assert not np.signbit(g.reshape(-1)[1])
+    thc.set_tuning("reduce.tall", 0)
+    try:
+        x = rng.integers(0, 4, (70001, 10)).astype(dtype)
+        vals, idx = thc.Tensor(kind), thc.Tensor("long")
+        vals.max(idx, thc.Tensor.from_numpy(x), 0)
+        assert thc.last_kernel().startswith("cols-index"), thc.last_kernel()
+        assert np.array_equal(idx.numpy().reshape(-1), np.argmax(x, axis=0) + 1)
+    finally:
+        thc.set_tuning("reduce.tall", 1)
+
+
 def test_minmax_config3_pattern(thc, oracle):
     """normal(0,1) rows with ~1% of each row overwritten by copies of other
     entries of the same row, the row maximum included (benchmark config 3)."""
@@ -611,8 +675,8 @@ def test_long_narrow_slices_reduce_in_chunks(thc, oracle, kind):
     x = rng.standard_normal((90000, 5)).astype(np.float32)
     x[77777, 2] = np.nan
     vals, idx = thc.Tensor("float"), thc.Tensor("long")
-    vals.max(idx, thc.Tensor.from_numpy(x), 0)                     # the indexed form keeps its own kernel
-    assert thc.last_kernel().startswith("cols-index")
+    vals.max(idx, thc.Tensor.from_numpy(x), 0)                     # the indexed form has its own flat-pack kernel
+    assert thc.last_kernel() == "tall-index"
     assert np.isnan(vals.numpy()[0, 2]) and idx.numpy()[0, 2] == 77778
     # aligned packs, or many slices: the column kernels stay
     dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((3, 50000, 8)), kind, "ints")
