@@ -963,6 +963,14 @@ void launch_scan(THCState* s, T* out, const T* in, int64_t outer, int64_t R, int
       }
       if (tx == 1) break;
     }
+    // A scanned dim shorter than the rows a workgroup takes per step (thread rows x 8) leaves thread rows
+    // without work (8 rows under 4 thread rows: a quarter of the lanes load): wider strips, fewer thread
+    // rows, where the rows are long enough to fill them.
+    if (tuning("scan.cols.short_wide", 1)) {
+      while (TX < kBlock && (int64_t)(kBlock / TX) * 8 > 2 * R && packs >= 2 * (int64_t)TX &&
+             outer * ((packs + 2 * TX - 1) / (2 * TX)) >= 2 * (int64_t)cus)
+        TX *= 2;
+    }
     const int64_t colTiles = (packs + TX - 1) / TX;
     const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(outer * colTiles, 1 << 30));
     const int64_t pfKnob = tuning("scan.cols.prefetch", -1);

@@ -233,6 +233,44 @@ def test_minmax_of_long_narrow_slices(thc, oracle, kind):
         thc.set_tuning("reduce.tall", 1)
 
 
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double"])
+def test_short_reduced_dim_over_long_rows(thc, oracle, kind):
+    """A reduced (or scanned) dim of 2..16 elements over long unit-stride rows: the column kernels widen
+    their segments until no thread row is left without work (one thread row at 8 rows and fewer).
+    sum / max / min / var / cumsum against numpy on small integers, pack-aligned and odd row lengths."""
+    rng = np.random.default_rng(39)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64}[kind]
+    for shape, dim in (((2, 40000), 0), ((3, 70001), 0), ((8, 16384), 0), ((5, 4, 8192), 1), ((16, 9000), 0),
+                       ((7, 2, 33000), 1), ((4, 1 << 18), 0)):
+        x = rng.integers(-3, 4, shape).astype(dtype)
+        dev = thc.Tensor.from_numpy(x)
+        for knob in (1, 0):
+            thc.set_tuning("reduce.cols.short_wide", knob)
+            thc.set_tuning("scan.cols.short_wide", knob)
+            try:
+                got = thc.Tensor(kind).sum(dev, dim)
+                assert thc.last_kernel().startswith("cols"), thc.last_kernel()
+                assert_bit_equal(got.numpy(), x.astype(np.int64).sum(axis=dim, keepdims=True).astype(dtype))
+                for which, arg, ext in (("max", np.argmax, np.max), ("min", np.argmin, np.min)):
+                    vals, idx = thc.Tensor(kind), thc.Tensor("long")
+                    getattr(vals, which)(idx, dev, dim)
+                    assert thc.last_kernel().startswith("cols-index"), thc.last_kernel()
+                    assert np.array_equal(idx.numpy(), np.expand_dims(arg(x, axis=dim), dim) + 1), (shape, which)
+                    assert_bit_equal(vals.numpy(), ext(x, axis=dim, keepdims=True))
+                scan = thc.Tensor(kind).cumsum(dev, dim)
+                assert thc.last_kernel().startswith("scan-cols"), thc.last_kernel()
+                assert_bit_equal(scan.numpy(), np.cumsum(x.astype(np.int64), axis=dim).astype(dtype))
+                if kind != "int":
+                    var = thc.Tensor(kind).var(dev, dim)
+                    assert thc.last_kernel().startswith("var-cols"), thc.last_kernel()
+                    want = np.var(x.astype(np.float64), axis=dim, ddof=1, keepdims=True)
+                    np.testing.assert_allclose(var.numpy().astype(np.float64), want, rtol=2e-3 if kind == "half" else 1e-5,
+                                               atol=1e-6)
+            finally:
+                thc.set_tuning("reduce.cols.short_wide", 1)
+                thc.set_tuning("scan.cols.short_wide", 1)
+
+
 def test_minmax_config3_pattern(thc, oracle):
     """normal(0,1) rows with ~1% of each row overwritten by copies of other
     entries of the same row, the row maximum included (benchmark config 3)."""
