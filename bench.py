@@ -336,7 +336,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
-                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall")
+                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -519,6 +519,12 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                                      lambda i: nhwc.copy(nhwc_view))
             table["N-copy-skinny16"] = ("(2^22, 16) <- (16, 2^22):t() copy, fp32", 8 * (1 << 26), 1 << 26,
                                         lambda i: sk_dst.copy(sk_src))
+        if "N-add-view-odd" in nx:
+            # views whose rows start off the 16-byte grid and have an odd length: x[:, 3:8190] of wider matrices
+            vw = [T.from_numpy(rng.standard_normal((8192, 8200), dtype=np.float32)) for _ in range(3)]
+            va, vb, vc = (w.narrow(1, o, 8187) for w, o in zip(vw, (3, 1, 2)))
+            table["N-add-view-odd"] = ("c = a + b on 8192x8187 fp32 views of 8192x8200 matrices at column offsets 2, 3, 1",
+                                       12 * 8192 * 8187, 8192 * 8187, lambda i: vc.cadd(va, 1.0, vb))
         if "N-equal" in nx:
             eq_b = e_src.clone()
             table["N-equal"] = ("equal(a, b) over 2^26 fp32 (both equal: no early exit possible)", 8 * ne, ne,

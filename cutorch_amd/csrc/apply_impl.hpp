@@ -319,22 +319,27 @@ struct IndexedArgs {
 template <typename T, typename Op, typename I, int VEC, bool JOINT, typename TOut = T>
 __global__ __launch_bounds__(kBlock) void apply_indexed_kernel(TOut* out, const T* in0, const T* in1,
                                                                const T* in2, I total,
-                                                               IndexedArgs<I> args, Op op) {
+                                                               IndexedArgs<I> args, Op op, I innerElems) {
+  // (innerElems, VEC > 1: elements of the innermost dim, whose last pack may be partial)
   using P = Pack<T, VEC>;
   using PO = Pack<TOut, VEC>;
   constexpr int NOPS = Op::NIN + 1;
   const I step = (I)gridDim.x * kBlock;
   for (I lin = (I)blockIdx.x * kBlock + threadIdx.x; lin < total; lin += step) {
     I off[kMaxOps] = {0, 0, 0, 0};
+    I inner = 0;  // JOINT: this pack's index along the innermost dim
     if (JOINT) {
       I rest = lin;
-      for (int d = args.dims[0] - 1; d > 0; --d) {
+      const int last = args.dims[0] - 1;
+      for (int d = last; d > 0; --d) {
         I q, r;
         args.size[0][d].divmod(rest, q, r);
         rest = q;
+        if (VEC > 1 && d == last) inner = r;
 #pragma unroll
         for (int k = 0; k < NOPS; ++k) off[k] += r * args.stride[k][d];
       }
+      if (VEC > 1 && last == 0) inner = rest;
 #pragma unroll
       for (int k = 0; k < NOPS; ++k) off[k] += rest * args.stride[k][0];
     } else {
@@ -350,17 +355,50 @@ __global__ __launch_bounds__(kBlock) void apply_indexed_kernel(TOut* out, const 
         off[k] += rest * args.stride[k][0];
       }
     }
-    P a{}, b{}, c{};
-    if (Op::NIN > 0) a = load_pack<true>(reinterpret_cast<const P*>(in0 + off[1]));
-    if (Op::NIN > 1) b = load_pack<true>(reinterpret_cast<const P*>(in1 + off[2]));
-    if (Op::NIN > 2) c = load_pack<true>(reinterpret_cast<const P*>(in2 + off[3]));
-    with_fixed_code(op, [&](auto f) {
-      PO r;
+    if constexpr (VEC == 1) {
+      P a{}, b{}, c{};
+      if (Op::NIN > 0) a = load_pack<true>(reinterpret_cast<const P*>(in0 + off[1]));
+      if (Op::NIN > 1) b = load_pack<true>(reinterpret_cast<const P*>(in1 + off[2]));
+      if (Op::NIN > 2) c = load_pack<true>(reinterpret_cast<const P*>(in2 + off[3]));
+      with_fixed_code(op, [&](auto f) {
+        PO r;
+        r.v[0] = f(a.v[0], b.v[0], c.v[0]);
+        if (args.ntStore) store_pack<true>(reinterpret_cast<PO*>(out + off[0]), r);
+        else store_pack<false>(reinterpret_cast<PO*>(out + off[0]), r);
+      });
+    } else {
+      // Packs sit at element-aligned addresses (rows need not start on the 16-byte grid), and the last
+      // pack of a row holds what is left of it: its missing elements repeat the pack's first one on the
+      // way in (no lane computes on values that are not the tensor's) and are not stored.
+      const I left = innerElems - inner * (I)VEC;
+      P a{}, b{}, c{};
+      if (left >= (I)VEC) {
+        if (Op::NIN > 0) a = load_pack_unaligned<true, P>(in0 + off[1]);
+        if (Op::NIN > 1) b = load_pack_unaligned<true, P>(in1 + off[2]);
+        if (Op::NIN > 2) c = load_pack_unaligned<true, P>(in2 + off[3]);
+      } else {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) r.v[e] = f(a.v[e], b.v[e], c.v[e]);
-      if (args.ntStore) store_pack<true>(reinterpret_cast<PO*>(out + off[0]), r);
-      else store_pack<false>(reinterpret_cast<PO*>(out + off[0]), r);
-    });
+        for (int e = 0; e < VEC; ++e) {
+          const I ee = (I)e < left ? (I)e : (I)0;
+          if (Op::NIN > 0) a.v[e] = in0[off[1] + ee];
+          if (Op::NIN > 1) b.v[e] = in1[off[2] + ee];
+          if (Op::NIN > 2) c.v[e] = in2[off[3] + ee];
+        }
+      }
+      with_fixed_code(op, [&](auto f) {
+        PO r;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.v[e] = f(a.v[e], b.v[e], c.v[e]);
+        if (left >= (I)VEC) {
+          if (args.ntStore) store_pack_unaligned<true, PO>(out + off[0], r);
+          else store_pack_unaligned<false, PO>(out + off[0], r);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e)
+            if ((I)e < left) out[off[0] + e] = r.v[e];
+        }
+      });
+    }
   }
 }
 
@@ -1176,12 +1214,34 @@ bool indexed_can_pack(const Plan& pl) {
   return vec;
 }
 
+// Whether the strided kernel can run on packs at element-aligned addresses with a partial last pack per
+// row: unit stride along the innermost dim for every operand, rows of at least a few packs, and every
+// pack start 4-byte aligned (always so for 4- and 8-byte elements).
+template <typename T, typename TOut>
+bool indexed_can_pack_unaligned(const Plan& pl) {
+  constexpr int VEC = pack_elems<T, TOut>();
+  if (VEC == 1 || !tuning("apply.indexed.unaligned_packs", 1)) return false;
+  const int nd = pl.lay[0].dims;
+  if (pl.lay[0].size[nd - 1] < 4 * VEC) return false;
+  for (int k = 0; k < pl.nops; ++k) {
+    if (pl.lay[k].stride[nd - 1] != 1) return false;
+    const size_t es = k == 0 ? sizeof(TOut) : sizeof(T);
+    const size_t al = std::min<size_t>(4, VEC * es);
+    if (reinterpret_cast<uintptr_t>(pl.ptr[k]) % al != 0) return false;
+    for (int d = 0; d < nd - 1; ++d)
+      if ((pl.lay[k].stride[d] * (int64_t)es) % (int64_t)al != 0) return false;
+  }
+  return true;
+}
+
 template <typename T, typename Op, typename I, bool JOINT, typename TOut = T>
 void launch_indexed(THCState* s, const Plan& pl, Op op) {
   constexpr int VEC = pack_elems<T, TOut>();
   IndexedArgs<I> args{};
-  const bool vec = JOINT && indexed_can_pack<T, TOut>(pl);
+  const bool aligned = JOINT && indexed_can_pack<T, TOut>(pl);
+  const bool vec = aligned || (JOINT && indexed_can_pack_unaligned<T, TOut>(pl));
   const int pack = vec ? VEC : 1;
+  int64_t total = 1;
   for (int k = 0; k < pl.nops; ++k) {
     const int nd = pl.lay[k].dims;
     args.dims[k] = nd;
@@ -1189,15 +1249,17 @@ void launch_indexed(THCState* s, const Plan& pl, Op op) {
       int64_t sz = pl.lay[k].size[d];
       int64_t sd = pl.lay[k].stride[d];
       if (vec && d == nd - 1) {
-        sz /= pack;
+        sz = (sz + pack - 1) / pack;
         sd *= pack;
       }
       args.size[k][d].set((uint64_t)sz);
       args.stride[k][d] = (I)sd;
+      if (k == 0) total *= sz;
     }
   }
+  const I innerElems = (I)pl.lay[0].size[pl.lay[0].dims - 1];
   args.ntStore = vec && streaming_store("apply.indexed.nt_store", pl.numel * (int64_t)sizeof(TOut)) ? 1 : 0;
-  const int64_t total = pl.numel / pack;
+  if (!JOINT) total = pl.numel;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((total + kBlock - 1) / kBlock,
                                                                tuning("apply.indexed.max_grid", 1 << 22)));
   TOut* out = (TOut*)pl.ptr[0];
@@ -1207,12 +1269,12 @@ void launch_indexed(THCState* s, const Plan& pl, Op op) {
   hipStream_t st = current_stream(s);
   if (vec) {
     hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, VEC, JOINT, TOut>), dim3(grid), dim3(kBlock),
-                       0, st, out, i0, i1, i2, (I)total, args, op);
+                       0, st, out, i0, i1, i2, (I)total, args, op, innerElems);
   } else {
     hipLaunchKernelGGL((apply_indexed_kernel<T, Op, I, 1, JOINT, TOut>), dim3(grid), dim3(kBlock), 0,
-                       st, out, i0, i1, i2, (I)total, args, op);
+                       st, out, i0, i1, i2, (I)total, args, op, innerElems);
   }
-  note_kernel(JOINT ? (vec ? "strided" : "strided-scalar") : "generic");
+  note_kernel(JOINT ? (vec ? (aligned ? "strided" : "strided-unaligned") : "strided-scalar") : "generic");
 }
 
 // Pick (p, q) for the tiled kernel. q = innermost joint dim. An operand is

@@ -57,6 +57,37 @@ __device__ __forceinline__ P load_pack(const P* p) {
   }
   return *p;
 }
+// The same accesses at addresses that are only 4-byte aligned (rows of 4- and 8-byte elements that start
+// off the 16-byte grid): still ONE 16-byte instruction per pack, which the hardware splits where it has to.
+template <int N>
+struct RawBitsU : RawBits<N> {};
+template <>
+struct RawBitsU<16> {
+  typedef unsigned type __attribute__((ext_vector_type(4), aligned(4)));
+};
+template <>
+struct RawBitsU<8> {
+  typedef unsigned type __attribute__((ext_vector_type(2), aligned(4)));
+};
+template <bool NT, typename P>
+__device__ __forceinline__ P load_pack_unaligned(const void* p) {
+  using R = typename RawBitsU<sizeof(P)>::type;
+  R r;
+  if (NT) r = __builtin_nontemporal_load(reinterpret_cast<const R*>(p));
+  else r = *reinterpret_cast<const R*>(p);
+  P out;
+  __builtin_memcpy(&out, &r, sizeof(P));
+  return out;
+}
+template <bool NT, typename P>
+__device__ __forceinline__ void store_pack_unaligned(void* p, const P& v) {
+  using R = typename RawBitsU<sizeof(P)>::type;
+  R r;
+  __builtin_memcpy(&r, &v, sizeof(P));
+  if (NT) __builtin_nontemporal_store(r, reinterpret_cast<R*>(p));
+  else *reinterpret_cast<R*>(p) = r;
+}
+
 // Streaming stores. On buffer instructions (buffer_store_pack below) they carry the device-scope bit
 // (sc1) of the cache policy, which makes the L2 write the data through instead of keeping dirty
 // lines: c = a + b on 3 x 64 MiB of fp32 with nontemporal loads runs at 0.79 of the HBM peak with

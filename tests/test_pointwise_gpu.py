@@ -555,10 +555,75 @@ def test_broadcast_operands_on_rows_that_are_not_pack_aligned(thc, kind):
         bias = rng.integers(-8, 9, 515).astype(dtype)
         db = thc.Tensor.from_numpy(bias).view_as_strided(0, (333, 515), (0, 1))
         out = thc.Tensor(kind).cadd(thc.Tensor.from_numpy(x), 1.0, db)
-        assert thc.last_kernel() == "strided-scalar"
+        assert thc.last_kernel() in ("strided-scalar", "strided-unaligned")     # (packs for 4- and 8-byte elements)
         assert_bit_equal(out.numpy(), (x + bias).astype(dtype))
     finally:
         thc.set_tuning("apply.flatmix", 1)
+
+
+@pytest.mark.parametrize("kind", ["float", "int", "double", "long", "half", "byte"])
+def test_strided_rows_off_the_16_byte_grid(thc, kind):
+    """Views whose rows start off the 16-byte grid and have odd lengths (x[:, 1:-2] of a wider matrix):
+    4- and 8-byte elements move as packs at element-aligned addresses with a partial last pack per row,
+    narrower elements element by element. In place and out of place, one to three inputs, every
+    operand at its own offset; the whole destination storage is compared."""
+    rng = np.random.default_rng(77)
+    dtype = {"float": np.float32, "int": np.int32, "double": np.float64, "long": np.int64, "half": np.float16,
+             "byte": np.uint8}[kind]
+    wide = dtype().itemsize >= 4
+    for rows, cols, pitch, offs in ((37, 101, 128, (1, 3, 2, 5)), (64, 8187, 8200, (3, 1, 1, 2)), (5, 16, 19, (1, 2, 3, 0)),
+                                    (3, 7, 9, (1, 1, 1, 1)), (200, 33, 40, (0, 1, 2, 3)), (6, 700, 4097, (5, 6, 7, 9))):
+        lo, hi = (0, 5) if kind == "byte" else (-4, 5)
+        hosts = [rng.integers(lo, hi, rows * pitch + 16).astype(dtype) for _ in range(4)]
+        def view(i):
+            return thc.Tensor.from_storage(hosts[i], offs[i], (rows, cols), (pitch, 1), kind=kind)
+        def host_view(i):
+            return np.lib.stride_tricks.as_strided(hosts[i][offs[i]:], (rows, cols), (pitch * dtype().itemsize, dtype().itemsize))
+        expect = "strided-unaligned" if wide and cols >= 4 * (16 // dtype().itemsize) else "strided-scalar"
+        # two inputs, out of place
+        out = view(0)
+        out.cadd(view(1), 2, view(2))
+        k = thc.last_kernel()
+        want = hosts[0].copy()
+        np.lib.stride_tricks.as_strided(want[offs[0]:], (rows, cols), (pitch * dtype().itemsize, dtype().itemsize))[...] = \
+            (host_view(1) + dtype(2) * host_view(2)).astype(dtype)
+        assert k in (expect, "strided"), (kind, rows, cols, k)
+        assert_bit_equal(out.storage_numpy(), want, "%s cadd %dx%d %s" % (kind, rows, cols, k))
+        # one input, in place
+        acc = view(3)
+        acc.mul(acc, 3)
+        want3 = hosts[3].copy()
+        np.lib.stride_tricks.as_strided(want3[offs[3]:], (rows, cols), (pitch * dtype().itemsize, dtype().itemsize))[...] = \
+            (host_view(3) * dtype(3)).astype(dtype)
+        assert_bit_equal(acc.storage_numpy(), want3, "%s mul in place %dx%d" % (kind, rows, cols))
+        # copy between views at different offsets, and a fill
+        dst = view(0)
+        dst.copy(view(2))
+        want0 = hosts[0].copy()
+        np.lib.stride_tricks.as_strided(want0[offs[0]:], (rows, cols), (pitch * dtype().itemsize, dtype().itemsize))[...] = host_view(2)
+        assert_bit_equal(dst.storage_numpy(), want0, "%s copy %dx%d %s" % (kind, rows, cols, thc.last_kernel()))
+        f = view(1)
+        f.fill(2)
+        want1 = hosts[1].copy()
+        np.lib.stride_tricks.as_strided(want1[offs[1]:], (rows, cols), (pitch * dtype().itemsize, dtype().itemsize))[...] = dtype(2)
+        assert_bit_equal(f.storage_numpy(), want1, "%s fill %dx%d %s" % (kind, rows, cols, thc.last_kernel()))
+    if kind == "float":
+        # three inputs, and a comparison into a Byte tensor (4 elements per pack on both sides)
+        rows, cols, pitch = 50, 1001, 1024
+        hs = [rng.integers(-4, 5, rows * pitch + 8).astype(np.float32) for _ in range(4)]
+        vs = [thc.Tensor.from_storage(h, o, (rows, cols), (pitch, 1)) for h, o in zip(hs, (1, 2, 3, 1))]
+        hv = [np.lib.stride_tricks.as_strided(h[o:], (rows, cols), (pitch * 4, 4)) for h, o in zip(hs, (1, 2, 3, 1))]
+        vs[0].addcmul(vs[1], 2.0, vs[2], vs[3])
+        assert thc.last_kernel() == "strided-unaligned"
+        want = hs[0].copy()
+        np.lib.stride_tricks.as_strided(want[1:], (rows, cols), (pitch * 4, 4))[...] = hv[1] + np.float32(2) * hv[2] * hv[3]
+        assert_bit_equal(vs[0].storage_numpy(), want)
+        mstore = np.full(rows * pitch + 8, 9, np.uint8)
+        mask = thc.Tensor.from_storage(mstore, 4, (rows, cols), (pitch, 1), kind="byte")
+        mask.compare_tensor("lt", vs[2], vs[3])
+        wantm = mstore.copy()
+        np.lib.stride_tricks.as_strided(wantm[4:], (rows, cols), (pitch, 1))[...] = (hv[2] < hv[3]).astype(np.uint8)
+        assert_bit_equal(mask.storage_numpy(), wantm, "lt into bytes %s" % thc.last_kernel())
 
 
 @pytest.mark.parametrize("band", [1, 2, 3, 8])
