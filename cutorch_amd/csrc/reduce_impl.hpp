@@ -2581,7 +2581,8 @@ bool run_slab_chunked(THCState* s, const ReduceGeom& g, const T* in, T* out, Epi
   // (6.3-6.8 against 5.8-6.0 TB/s on 16..64-column fp32 slices, 6.1 against
   // 3.9 on 4096 slices of 4096 x 3).
   constexpr int64_t VEC = 16 / sizeof(T);
-  if (aligned16(in) && C % VEC == 0) return false;
+  // (2-byte elements: the flat runs of packs win on pack-aligned rows too, 0.39-0.54 -> 0.54-0.61 of peak)
+  if (aligned16(in) && C % VEC == 0 && !tuning("reduce.tall.aligned_sum", sizeof(T) == 2 ? 1 : 0)) return false;
   if (O >= (int64_t)num_compute_units(s)) return false;
   // bytes staged per workgroup (tunable so that tests reach many levels)
   const int64_t kRun = std::min<int64_t>(32768, std::max<int64_t>(256, tuning("reduce.slab.run_bytes", 32768)));
@@ -2815,7 +2816,8 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
   }
   {
     // few long narrow slices that start on 16-byte boundaries: flat runs of packs (reduce_tall_index_kernel;
-    // the column kernel below keeps C of its lanes busy on them: 6.7M x 10 along dim 0 0.30 of peak)
+    // the column kernel below keeps C of its lanes busy on them: 6.7M x 10 along dim 0 0.30 of peak); rows
+    // of whole packs as well (1M x 64 fp32 0.42 -> 0.66, 512K x 100 0.25 -> 0.61, half 0.15-0.30 -> 0.43-0.46)
     auto tall = [&]() {
       if (!tuning("reduce.tall", 1)) return false;
       const int64_t C = g.in.size[nd - 1];
@@ -2828,7 +2830,7 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
         run *= g.in.size[d];
       }
       const int64_t O = g.outElems / C;
-      if (!aligned16(in) || C % VEC == 0 || O >= (int64_t)num_compute_units(s)) return false;
+      if (!aligned16(in) || (C % VEC == 0 && !tuning("reduce.tall.aligned_index", 1)) || O >= (int64_t)num_compute_units(s)) return false;
       if (!(O == 1 || (g.R * C) % VEC == 0) || g.R * C < (int64_t)VEC * kBlock * 8) return false;
       int64_t gcd = C, b = VEC;
       while (b) {
@@ -3041,7 +3043,7 @@ bool reduce_var_cols_type(THCState* s, const ReduceGeom& g, const void* in_, voi
           run *= g.in.size[d];
         }
         const int64_t O = g.outElems / C;
-        if (!aligned16(in_) || C % VEC == 0 || O >= (int64_t)num_compute_units(s)) return false;
+        if (!aligned16(in_) || (C % VEC == 0 && !tuning("reduce.tall.aligned_var", sizeof(T) == 2 ? 1 : 0)) || O >= (int64_t)num_compute_units(s)) return false;
         if (!(O == 1 || (g.R * C) % VEC == 0) || g.R * C < (int64_t)VEC * kBlock * 8) return false;
         int64_t gcd = C, b = VEC;
         while (b) {

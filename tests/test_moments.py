@@ -156,7 +156,8 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
         for name in ("var", "std"):
             for biased in (0, 1):
                 out = getattr(thc.Tensor(kind), name)(dev, dim, biased=biased)
-                assert thc.last_kernel().startswith(expect.replace("-scalar", "")), (shape, thc.last_kernel())
+                k = thc.last_kernel()      # (half: long narrow slices of whole packs take the flat runs as well)
+                assert k.startswith(expect.replace("-scalar", "")) or (kind == "half" and k == "var-tall"), (shape, k)
                 want = oracle.reduce_dim(name + ("_biased" if biased else ""), ref, dim).numpy().astype(np.float64)
                 np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol * (8 if kind == "float" else 1),
                                            atol=0, err_msg="%s %s %s" % (shape, name, kind))

@@ -88,7 +88,7 @@ def test_non_innermost_dim(thc, oracle, name, kind):
                        ((3, 50, 8, 24), 1), ((2, 2000, 3), 1), ((16, 33, 1), 1)):
         dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry(shape), kind, "uniform")
         k = run_reduce(thc, oracle, name, dev, ref, dim, kind)
-        assert k.startswith("cols") or k == "slab" or shape[-1] == 1, k
+        assert k.startswith("cols") or k in ("slab", "tall-flat") or shape[-1] == 1, k
 
 
 def test_split_reduction_is_used_and_correct(thc, oracle):
@@ -180,10 +180,10 @@ def test_minmax_of_long_narrow_slices(thc, oracle, kind):
     dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64, "byte": np.uint8}[kind]
     vec = 16 // np.dtype(dtype).itemsize
     for shape, dim in (((200003, 3), 0), ((70001, 10), 0), ((30000, 33), 0), ((2, 40000, 7), 1), ((3, 16000, 5), 1),
-                       ((1, 50001, 9), 1), ((25000, 50), 0)):
+                       ((1, 50001, 9), 1), ((25000, 50), 0), ((40000, 16), 0), ((3, 9001, 64), 1)):
         inner = int(np.prod(shape[dim + 1:]))
         outer = int(np.prod(shape[:dim]))
-        flat = inner % vec != 0 and (outer == 1 or (shape[dim] * inner) % vec == 0)
+        flat = outer == 1 or (shape[dim] * inner) % vec == 0      # (every slice starts on a 16-byte boundary)
         lo, hi = (0, 4) if kind == "byte" else (-3, 4)
         x = rng.integers(lo, hi, shape).astype(dtype)
         dev, ref = thc.Tensor.from_numpy(x), oracle.View.of(x)
@@ -716,9 +716,10 @@ def test_long_narrow_slices_reduce_in_chunks(thc, oracle, kind):
     vals.max(idx, thc.Tensor.from_numpy(x), 0)                     # the indexed form has its own flat-pack kernel
     assert thc.last_kernel() == "tall-index"
     assert np.isnan(vals.numpy()[0, 2]) and idx.numpy()[0, 2] == 77778
-    # aligned packs, or many slices: the column kernels stay
+    # rows of whole aligned packs (4-byte elements; on half the flat runs win there too), or many slices:
+    # the column kernels stay
     dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((3, 50000, 8)), kind, "ints")
-    assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
+    assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("tall-flat" if kind == "half" else "cols")
     dev, ref = dev_and_ref(thc, oracle, rng, contiguous_geometry((300, 5000, 3)), kind, "ints")
     assert run_reduce(thc, oracle, "sum", dev, ref, 1, kind).startswith("cols")
 
