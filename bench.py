@@ -336,7 +336,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
-                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd")
+                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd", "N-cvt-image")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -508,7 +508,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                                       "(32-bit offsets; a's lines are half used)", 12 * m * m, m * m, strided_add(False))
             table["N-add-strided-u64"] = ("the same with 64-bit index arithmetic forced", 12 * m * m, m * m,
                                           strided_add(True))
-        if set(nx) & {"N-copy-nhwc3", "N-copy-skinny16"}:
+        if set(nx) & {"N-copy-nhwc3", "N-copy-skinny16", "N-cvt-image"}:
             # tall-and-skinny transposes: a short dim of a few elements against a long one
             img = T.from_numpy(rng.standard_normal((64, 3, 512, 512), dtype=np.float32))
             nhwc_view = img.view_as_strided(0, (64, 512, 512, 3), (3 * 262144, 512, 1, 262144))
@@ -517,6 +517,11 @@ def build_configs(thc, hip, which, only=None, stagger=0):
             sk_dst = T("float").resize((1 << 22, 16))
             table["N-copy-nhwc3"] = ("NCHW -> NHWC copy of 64x3x512x512 fp32", 8 * 64 * 3 * 262144, 64 * 3 * 262144,
                                      lambda i: nhwc.copy(nhwc_view))
+            img8 = T.from_numpy(rng.integers(0, 256, (64, 512, 512, 3)).astype(np.uint8))          # NHWC bytes
+            chw_view = img8.view_as_strided(0, (64, 3, 512, 512), (3 * 262144, 1, 1536, 3))
+            chw = T("float").resize((64, 3, 512, 512))
+            table["N-cvt-image"] = ("float NCHW <- byte NHWC converting copy of 64x512x512x3", 5 * 64 * 3 * 262144,
+                                    64 * 3 * 262144, lambda i: chw.copy_from(chw_view))
             table["N-copy-skinny16"] = ("(2^22, 16) <- (16, 2^22):t() copy, fp32", 8 * (1 << 26), 1 << 26,
                                         lambda i: sk_dst.copy(sk_src))
         if "N-add-view-odd" in nx:

@@ -55,7 +55,9 @@ EXTRA_DEPS = {"caching_allocator.cpp": ["caching_pool.hpp", "stream_guard.hpp"],
               "apply_rawmath_u32u64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"],
               "apply_rawmath_f64.hip": ["apply_rawmath.hpp", "apply_rawmath_impl.hpp"], "reduce.hip": ["stream_guard.hpp"],
               "scan.hip": ["stream_guard.hpp"], "no_alloc.hip": ["stream_guard.hpp"], "convert.hip": ["stream_guard.hpp"]}
-EXTRA_DEPS.update({"apply_cvt_%s.hip" % t: ["apply_convert_impl.hpp"] for t in ("u8", "i8", "i16", "i32", "i64", "f16", "f32", "f64")})
+EXTRA_DEPS.update({"apply_cvt_%s.hip" % t: ["apply_convert_impl.hpp", "apply_skinny.hpp"]
+                   for t in ("u8", "i8", "i16", "i32", "i64", "f16", "f32", "f64")})
+EXTRA_DEPS["apply_raw.hip"] = ["apply_skinny.hpp"]
 
 
 def _compile(src, force):

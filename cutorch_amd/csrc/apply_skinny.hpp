@@ -12,6 +12,7 @@
 #pragma once
 #include <algorithm>
 #include <cstdint>
+#include <type_traits>
 
 #include "apply_plan.hpp"
 #include "common.hpp"
@@ -35,14 +36,21 @@ struct SkinnyArgs {
   int64_t denseBatchStride[kMaxDims], planarBatchStride[kMaxDims];
 };
 
-// TO_PLANAR: the source is the dense side. VD / VP: packs on the dense / planar side.
-template <typename E, bool TO_PLANAR, bool VD, bool VP>
-__global__ __launch_bounds__(kBlock) void skinny_copy_kernel(E* __restrict__ dst, const E* __restrict__ src,
+// TO_PLANAR: the source is the dense side. VD / VP: packs on the dense / planar side. ES / ED: source
+// and destination element types (raw unsigned integers of the element size for same-type copies); a
+// converting copy converts on the way into LDS, which holds destination elements.
+template <typename ES, typename ED, bool TO_PLANAR, bool VD, bool VP>
+__global__ __launch_bounds__(kBlock) void skinny_copy_kernel(ED* __restrict__ dst, const ES* __restrict__ src,
                                                              SkinnyArgs a) {
-  constexpr uint32_t VEC = 16 / sizeof(E);
-  using P = Pack<E, VEC>;
+  constexpr uint32_t VS = 16 / sizeof(ES), VT = 16 / sizeof(ED);
+  using PS = Pack<ES, VS>;
+  using PT = Pack<ED, VT>;
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  E* lds = reinterpret_cast<E*>(lds_raw);
+  ED* lds = reinterpret_cast<ED*>(lds_raw);
+  auto cvt = [](ES x) -> ED {
+    if constexpr (std::is_same<ES, ED>::value) return x;
+    else return convert_value<ED, ES>(x);
+  };
   const uint32_t S = a.S, pitch = a.pitch;
   for (uint32_t b = blockIdx.x; b < a.totalTiles; b += gridDim.x) {
     uint32_t rest, tl;
@@ -59,29 +67,25 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(E* __restrict__ dst
     const uint32_t n = tn * S;                                            // elements of this tile
     dOff += (int64_t)(t0 * S);
     pOff += (int64_t)t0;
-    const E* dsrc = src + dOff;
-    const E* psrc = src + pOff;
-    E* ddst = dst + dOff;
-    E* pdst = dst + pOff;
-    const uint32_t planePacks = VP ? tn / VEC : 0;  // whole packs of a plane's run
     // ---- into LDS
     if (TO_PLANAR) {
-      const uint32_t packs = VD ? n / VEC : 0;
+      const ES* dsrc = src + dOff;
+      const uint32_t packs = VD ? n / VS : 0;
       constexpr int U = 4;
       for (uint32_t k0 = threadIdx.x; k0 < packs; k0 += U * kBlock) {
-        P v[U];
+        PS v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          v[u] = load_pack<true>(reinterpret_cast<const P*>(dsrc) + min(k0 + u * kBlock, packs - 1));
+          v[u] = load_pack<true>(reinterpret_cast<const PS*>(dsrc) + min(k0 + u * kBlock, packs - 1));
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t k = k0 + u * kBlock;
           if (k < packs) {
             uint32_t t, s;
-            a.sdiv.divmod(k * VEC, t, s);
+            a.sdiv.divmod(k * VS, t, s);
 #pragma unroll
-            for (uint32_t e = 0; e < VEC; ++e) {
-              lds[s * pitch + t] = v[u].v[e];
+            for (uint32_t e = 0; e < VS; ++e) {
+              lds[s * pitch + t] = cvt(v[u].v[e]);
               if (++s == S) {
                 s = 0;
                 ++t;
@@ -90,76 +94,81 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(E* __restrict__ dst
           }
         }
       }
-      for (uint32_t m = packs * VEC + threadIdx.x; m < n; m += kBlock) {
+      for (uint32_t m = packs * VS + threadIdx.x; m < n; m += kBlock) {
         uint32_t t, s;
         a.sdiv.divmod(m, t, s);
-        lds[s * pitch + t] = dsrc[m];
+        lds[s * pitch + t] = cvt(dsrc[m]);
       }
     } else {
+      const ES* psrc = src + pOff;
+      const uint32_t planePacks = VP ? tn / VS : 0;  // whole packs of a plane's run
       const uint32_t packs = planePacks * S;
       constexpr int U = 4;
-      for (uint32_t k0 = threadIdx.x; k0 < packs; k0 += U * kBlock) {
-        P v[U];
+      for (uint32_t k0 = threadIdx.x; VP && k0 < packs; k0 += U * kBlock) {
+        PS v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t k = min(k0 + u * kBlock, packs - 1);
-          const uint32_t s = k / planePacks, j = k - s * planePacks;
-          v[u] = load_pack<true>(reinterpret_cast<const P*>(psrc + (int64_t)s * a.planeStride) + j);
+          const uint32_t s = k / (VP ? planePacks : 1u), j = k - s * planePacks;
+          v[u] = load_pack<true>(reinterpret_cast<const PS*>(psrc + (int64_t)s * a.planeStride) + j);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t k = k0 + u * kBlock;
           if (k < packs) {
-            const uint32_t s = k / planePacks, j = k - s * planePacks;
+            const uint32_t s = k / (VP ? planePacks : 1u), j = k - s * planePacks;
 #pragma unroll
-            for (uint32_t e = 0; e < VEC; ++e) lds[s * pitch + j * VEC + e] = v[u].v[e];
+            for (uint32_t e = 0; e < VS; ++e) lds[s * pitch + j * VS + e] = cvt(v[u].v[e]);
           }
         }
       }
       // what the packs leave: the end of every plane's run, or all of it
-      const uint32_t left = tn - planePacks * VEC;
+      const uint32_t left = tn - planePacks * VS;
       for (uint32_t m = threadIdx.x; m < left * S; m += kBlock) {
-        const uint32_t s = m / left, t = planePacks * VEC + (m - s * left);
-        lds[s * pitch + t] = psrc[(int64_t)s * a.planeStride + t];
+        const uint32_t s = m / left, t = planePacks * VS + (m - s * left);
+        lds[s * pitch + t] = cvt(psrc[(int64_t)s * a.planeStride + t]);
       }
     }
     __syncthreads();
     // ---- out of LDS
     if (TO_PLANAR) {
+      ED* pdst = dst + pOff;
+      const uint32_t planePacks = VP ? tn / VT : 0;
       const uint32_t packs = planePacks * S;
-      for (uint32_t k = threadIdx.x; k < packs; k += kBlock) {
-        const uint32_t s = k / planePacks, j = k - s * planePacks;
-        P v;
+      for (uint32_t k = threadIdx.x; VP && k < packs; k += kBlock) {
+        const uint32_t s = k / (VP ? planePacks : 1u), j = k - s * planePacks;
+        PT v;
 #pragma unroll
-        for (uint32_t e = 0; e < VEC; ++e) v.v[e] = lds[s * pitch + j * VEC + e];
-        P* at = reinterpret_cast<P*>(pdst + (int64_t)s * a.planeStride) + j;
+        for (uint32_t e = 0; e < VT; ++e) v.v[e] = lds[s * pitch + j * VT + e];
+        PT* at = reinterpret_cast<PT*>(pdst + (int64_t)s * a.planeStride) + j;
         if (a.ntStore) store_pack<true>(at, v);
         else store_pack<false>(at, v);
       }
-      const uint32_t left = tn - planePacks * VEC;
+      const uint32_t left = tn - planePacks * VT;
       for (uint32_t m = threadIdx.x; m < left * S; m += kBlock) {
-        const uint32_t s = m / left, t = planePacks * VEC + (m - s * left);
+        const uint32_t s = m / left, t = planePacks * VT + (m - s * left);
         pdst[(int64_t)s * a.planeStride + t] = lds[s * pitch + t];
       }
     } else {
-      const uint32_t packs = VD ? n / VEC : 0;
+      ED* ddst = dst + dOff;
+      const uint32_t packs = VD ? n / VT : 0;
       for (uint32_t k = threadIdx.x; k < packs; k += kBlock) {
         uint32_t t, s;
-        a.sdiv.divmod(k * VEC, t, s);
-        P v;
+        a.sdiv.divmod(k * VT, t, s);
+        PT v;
 #pragma unroll
-        for (uint32_t e = 0; e < VEC; ++e) {
+        for (uint32_t e = 0; e < VT; ++e) {
           v.v[e] = lds[s * pitch + t];
           if (++s == S) {
             s = 0;
             ++t;
           }
         }
-        P* at = reinterpret_cast<P*>(ddst) + k;
+        PT* at = reinterpret_cast<PT*>(ddst) + k;
         if (a.ntStore) store_pack<true>(at, v);
         else store_pack<false>(at, v);
       }
-      for (uint32_t m = packs * VEC + threadIdx.x; m < n; m += kBlock) {
+      for (uint32_t m = packs * VT + threadIdx.x; m < n; m += kBlock) {
         uint32_t t, s;
         a.sdiv.divmod(m, t, s);
         ddst[m] = lds[s * pitch + t];
@@ -171,9 +180,9 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(E* __restrict__ dst
 
 // `pl` is the jointly collapsed plan of a copy, dims ordered by the destination's strides
 // (operand 0 = destination, 1 = source). Returns false when the layouts are not of this kind.
-template <typename E>
+template <typename ES, typename ED = ES>
 bool launch_skinny_copy(THCState* s, const Plan& pl) {
-  constexpr int64_t VEC = 16 / sizeof(E);
+  using E = typename std::conditional<(sizeof(ES) > sizeof(ED)), ES, ED>::type;  // the wider element sizes the tiles
   if (!tuning("apply.skinny", 1) || pl.nops != 2) return false;
   const int nd = pl.lay[0].dims;
   if (nd < 2 || pl.numel >= (int64_t(1) << 40)) return false;
@@ -208,7 +217,7 @@ bool launch_skinny_copy(THCState* s, const Plan& pl) {
   int64_t T = std::max<int64_t>(64, (tuning("apply.skinny.tile_bytes", 16384) / (S * (int64_t)sizeof(E))) / 16 * 16);
   T = std::min<int64_t>(T, (L + 15) / 16 * 16);
   a.T = (uint32_t)T;
-  a.pitch = (uint32_t)(T + 16 / sizeof(E) + 1) | 1u;
+  a.pitch = (uint32_t)(T + 16 / sizeof(ED) + 1) | 1u;
   a.sdiv.set((uint64_t)S);
   const int64_t tiles = (L + T - 1) / T;
   a.tilesPerSlice.set((uint64_t)tiles);
@@ -223,22 +232,23 @@ bool launch_skinny_copy(THCState* s, const Plan& pl) {
   }
   if (total >= (int64_t(1) << 31)) return false;
   a.totalTiles = (uint32_t)total;
-  a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(E)) ? 1 : 0;
-  // packs: every tile's run starts on a 16-byte boundary
+  a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(ED)) ? 1 : 0;
+  // packs: every tile's run starts on a 16-byte boundary (operand 0 holds ED elements, operand 1 ES)
   auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
-  bool vd = aligned(pl.ptr[dense]), vp = aligned(pl.ptr[1 - dense]) && a.planeStride % VEC == 0;
+  const int64_t denseBytes = dense == 0 ? sizeof(ED) : sizeof(ES), planarBytes = dense == 0 ? sizeof(ES) : sizeof(ED);
+  bool vd = aligned(pl.ptr[dense]), vp = aligned(pl.ptr[1 - dense]) && (a.planeStride * planarBytes) % 16 == 0;
   for (int j = 0; j < a.nbatch; ++j) {
-    vd = vd && a.denseBatchStride[j] % VEC == 0;
-    vp = vp && a.planarBatchStride[j] % VEC == 0;
+    vd = vd && (a.denseBatchStride[j] * denseBytes) % 16 == 0;
+    vp = vp && (a.planarBatchStride[j] * planarBytes) % 16 == 0;
   }
-  const size_t ldsBytes = ((size_t)S * a.pitch * sizeof(E) + 15) & ~size_t(15);
+  const size_t ldsBytes = ((size_t)S * a.pitch * sizeof(ED) + 15) & ~size_t(15);
   if (ldsBytes > 64 * 1024) return false;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, (int64_t)num_compute_units(s) * 64));
-  E* dst = (E*)pl.ptr[0];
-  const E* src = (const E*)pl.ptr[1];
+  ED* dst = (ED*)pl.ptr[0];
+  const ES* src = (const ES*)pl.ptr[1];
   hipStream_t st = current_stream(s);
 #define THC_SKINNY(TP, D, Pk) \
-  hipLaunchKernelGGL((skinny_copy_kernel<E, TP, D, Pk>), dim3(grid), dim3(kBlock), ldsBytes, st, dst, src, a)
+  hipLaunchKernelGGL((skinny_copy_kernel<ES, ED, TP, D, Pk>), dim3(grid), dim3(kBlock), ldsBytes, st, dst, src, a)
   if (dense == 1) {
     if (vd && vp) THC_SKINNY(true, true, true);
     else if (vd) THC_SKINNY(true, true, false);

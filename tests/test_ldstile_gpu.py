@@ -339,8 +339,8 @@ def test_converting_copies_of_transposed_and_strided_operands(thc, oracle, src):
                 dd, rd = pair(thc, oracle, storage_of(rng, oracle, dst, go[0]), go, dst)
                 dd.copy_from(ds)
                 k = thc.last_kernel()
-                if transposed:
-                    assert k.startswith("lds-tile"), (k, src, dst, shape)
+                if transposed:      # (a short dim of at most 256 bytes: the tall-and-skinny copy, for some pairs)
+                    assert k.startswith("lds-tile") or k == "skinny", (k, src, dst, shape)
                 else:
                     assert k.startswith("strided") or k in ("convert", "contig", "contig-scalar"), (k, src, dst, shape)
                 oracle.typed_convert(rd, rs)

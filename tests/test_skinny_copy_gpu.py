@@ -89,3 +89,37 @@ def test_skinny_copy_declines_what_it_does_not_cover(thc):
         assert_bit_equal(d2.numpy(), np.ascontiguousarray(y.T))
     finally:
         thc.set_tuning("apply.skinny", 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("src_kind,dst_kind", [("byte", "float"), ("float", "byte"), ("byte", "half"), ("half", "byte"),
+                                               ("half", "float"), ("float", "half"), ("float", "double"),
+                                               ("double", "float")])
+def test_converting_copies_between_image_layouts(thc, src_kind, dst_kind):
+    """Type-converting copies of the same layouts (lib/THC/THCTensorCopy.cu:26-122 converts inside the
+    apply): a byte HWC image into float CHW planes and back, tall-and-skinny transposes; values that
+    every type involved represents exactly, so numpy's astype is the expected result bit for bit."""
+    rng = np.random.default_rng(44)
+    sdt, ddt = KINDS.get(src_kind, np.float32), KINDS.get(dst_kind, np.float32)
+    for n, c, h, w in ((3, 3, 37, 53), (2, 4, 64, 64), (1, 16, 20, 24)):
+        hwc = rng.integers(0, 200, (n, h, w, c)).astype(sdt)
+        src = thc.Tensor.from_numpy(hwc)
+        chw_view = src.view_as_strided(0, (n, c, h, w), (h * w * c, 1, w * c, c))       # NCHW view of the NHWC data
+        out = thc.Tensor(dst_kind).resize((n, c, h, w))
+        out.copy_from(chw_view)
+        assert thc.last_kernel() == "skinny", (src_kind, dst_kind, thc.last_kernel())
+        assert_bit_equal(out.numpy(), np.ascontiguousarray(hwc.transpose(0, 3, 1, 2)).astype(ddt))
+        chw = rng.integers(0, 200, (n, c, h, w)).astype(sdt)
+        src2 = thc.Tensor.from_numpy(chw)
+        hwc_view = src2.view_as_strided(0, (n, h, w, c), (c * h * w, w, 1, h * w))       # NHWC view of the NCHW data
+        out2 = thc.Tensor(dst_kind).resize((n, h, w, c))
+        out2.copy_from(hwc_view)
+        assert thc.last_kernel() == "skinny", (src_kind, dst_kind, thc.last_kernel())
+        assert_bit_equal(out2.numpy(), np.ascontiguousarray(chw.transpose(0, 2, 3, 1)).astype(ddt))
+    for long_n, short_n, off in ((70001, 3, 1), (4099, 5, 0)):
+        planar = rng.integers(0, 200, short_n * long_n + off).astype(sdt)
+        src = thc.Tensor.from_storage(planar, off, (long_n, short_n), (1, long_n), kind=src_kind)
+        dst = thc.Tensor(dst_kind).resize((long_n, short_n))
+        dst.copy_from(src)
+        assert thc.last_kernel() == "skinny"
+        assert_bit_equal(dst.numpy(), np.ascontiguousarray(planar[off:].reshape(short_n, long_n).T).astype(ddt))
