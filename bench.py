@@ -336,7 +336,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
-                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd", "N-cvt-image")
+                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd", "N-cvt-image", "N-transpose-16x16", "N-sumall-t")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -508,7 +508,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                                       "(32-bit offsets; a's lines are half used)", 12 * m * m, m * m, strided_add(False))
             table["N-add-strided-u64"] = ("the same with 64-bit index arithmetic forced", 12 * m * m, m * m,
                                           strided_add(True))
-        if set(nx) & {"N-copy-nhwc3", "N-copy-skinny16", "N-cvt-image"}:
+        if set(nx) & {"N-copy-nhwc3", "N-copy-skinny16", "N-cvt-image", "N-transpose-16x16"}:
             # tall-and-skinny transposes: a short dim of a few elements against a long one
             img = T.from_numpy(rng.standard_normal((64, 3, 512, 512), dtype=np.float32))
             nhwc_view = img.view_as_strided(0, (64, 512, 512, 3), (3 * 262144, 512, 1, 262144))
@@ -522,6 +522,11 @@ def build_configs(thc, hip, which, only=None, stagger=0):
             chw = T("float").resize((64, 3, 512, 512))
             table["N-cvt-image"] = ("float NCHW <- byte NHWC converting copy of 64x512x512x3", 5 * 64 * 3 * 262144,
                                     64 * 3 * 262144, lambda i: chw.copy_from(chw_view))
+            small = T.from_numpy(rng.standard_normal((1 << 18, 16, 16), dtype=np.float32))
+            small_t = small.view_as_strided(0, (1 << 18, 16, 16), (256, 1, 16))
+            small_o = T("float").resize((1 << 18, 16, 16))
+            table["N-transpose-16x16"] = ("2^18 transposed 16 x 16 fp32 matrices copied", 8 * (1 << 26), 1 << 26,
+                                          lambda i: small_o.copy(small_t))
             table["N-copy-skinny16"] = ("(2^22, 16) <- (16, 2^22):t() copy, fp32", 8 * (1 << 26), 1 << 26,
                                         lambda i: sk_dst.copy(sk_src))
         if "N-add-view-odd" in nx:
@@ -530,6 +535,9 @@ def build_configs(thc, hip, which, only=None, stagger=0):
             va, vb, vc = (w.narrow(1, o, 8187) for w, o in zip(vw, (3, 1, 2)))
             table["N-add-view-odd"] = ("c = a + b on 8192x8187 fp32 views of 8192x8200 matrices at column offsets 2, 3, 1",
                                        12 * 8192 * 8187, 8192 * 8187, lambda i: vc.cadd(va, 1.0, vb))
+        if "N-sumall-t" in nx:
+            table["N-sumall-t"] = ("sumall over the transposed view of 8192x8192 fp32 (blocks on the scalar)", 4 * 8192 * 8192,
+                                   8192 * 8192, lambda i: sq_t.sumall())
         if "N-equal" in nx:
             eq_b = e_src.clone()
             table["N-equal"] = ("equal(a, b) over 2^26 fp32 (both equal: no early exit possible)", 8 * ne, ne,

@@ -6,9 +6,11 @@ namespace thc {
 template <typename T>
 void apply_copy(THCState* s, Plan& pl, bool sameShape) {
   if (sameShape) {
-    // tall-and-skinny transposes (a short dim of a few elements against a long one) have a kernel of their own
+    // tall-and-skinny transposes (a short dim of a few elements against a long one) and batches of small
+    // transposed matrices have kernels of their own
     Plan c = pl;
-    if (joint_collapse(c.nops, c.lay, /*reorder=*/true) && launch_skinny_copy<T>(s, c)) return;
+    if (joint_collapse(c.nops, c.lay, /*reorder=*/true) && (launch_skinny_copy<T>(s, c) || launch_small_transpose<T>(s, c)))
+      return;
   }
   run_plan<T>(s, pl, sameShape, OpCopy{});
 }

@@ -265,5 +265,165 @@ bool launch_skinny_copy(THCState* s, const Plan& pl) {
   return true;
 }
 
+
+// Batches of small dense matrices transposed ((B, P, Q) <- (B, Q, P) with P, Q below 64: per-pixel
+// 3 x 3 or 4 x 4 matrices, 16 x 16 blocks): a 64 x 128 tile of the tiled kernels holds one such matrix
+// and little else (2^18 x 16 x 16 ran at 0.12 of peak, 2^20 x 8 x 8 at 0.035). A tile here is K whole
+// matrices, about 16 KiB, one contiguous run on BOTH sides: packs in, packs out, the order changed in
+// LDS (source rows at a pitch of P + 1 elements).
+struct SmallTransposeArgs {
+  uint32_t P, Q, K;        // out is (.., P, Q), source rows are P long; K matrices per tile
+  uint32_t pitch;          // LDS elements per matrix
+  uint32_t totalTiles;
+  uint64_t batch;          // matrices in the innermost batch dim (contiguous on both sides)
+  int nbatch;              // dims outside that one, innermost first
+  int ntStore;
+  Divisor<uint32_t> pdiv, qdiv, pqdiv, tilesPerRun;
+  Divisor<uint32_t> bsize[kMaxDims];
+  int64_t dstBatchStride[kMaxDims], srcBatchStride[kMaxDims];
+};
+
+template <typename ES, typename ED, bool VIN, bool VOUT>
+__global__ __launch_bounds__(kBlock) void small_transpose_kernel(ED* __restrict__ dst, const ES* __restrict__ src,
+                                                                 SmallTransposeArgs a) {
+  constexpr uint32_t VS = 16 / sizeof(ES), VT = 16 / sizeof(ED);
+  using PS = Pack<ES, VS>;
+  using PT = Pack<ED, VT>;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  ED* lds = reinterpret_cast<ED*>(lds_raw);
+  auto cvt = [](ES x) -> ED {
+    if constexpr (std::is_same<ES, ED>::value) return x;
+    else return convert_value<ED, ES>(x);
+  };
+  const uint32_t P = a.P, PQ = a.P * a.Q, rowPitch = a.P + 1;
+  // source element m of a tile is (k, q, p) = (m / PQ, (m % PQ) / P, m % P); it waits at
+  // lds[k * pitch + q * (P + 1) + p] for destination element (k, p, q)
+  auto src_slot = [&](uint32_t m) {
+    uint32_t k, r, q, pp;
+    a.pqdiv.divmod(m, k, r);
+    a.pdiv.divmod(r, q, pp);
+    return k * a.pitch + q * rowPitch + pp;
+  };
+  auto dst_slot = [&](uint32_t m) {
+    uint32_t k, r, pp, q;
+    a.pqdiv.divmod(m, k, r);
+    a.qdiv.divmod(r, pp, q);
+    return k * a.pitch + q * rowPitch + pp;
+  };
+  for (uint32_t b = blockIdx.x; b < a.totalTiles; b += gridDim.x) {
+    uint32_t rest, tl;
+    a.tilesPerRun.divmod(b, rest, tl);
+    int64_t dOff = 0, sOff = 0;
+    for (int j = 0; j < a.nbatch; ++j) {
+      uint32_t r;
+      a.bsize[j].divmod(rest, rest, r);
+      dOff += (int64_t)r * a.dstBatchStride[j];
+      sOff += (int64_t)r * a.srcBatchStride[j];
+    }
+    const uint64_t k0 = (uint64_t)tl * a.K;
+    const uint32_t kn = (uint32_t)min((uint64_t)a.K, a.batch - k0);
+    const uint32_t n = kn * PQ;
+    const ES* in = src + sOff + (int64_t)(k0 * PQ);
+    ED* out = dst + dOff + (int64_t)(k0 * PQ);
+    const uint32_t packsIn = VIN ? n / VS : 0;
+    constexpr int U = 4;
+    for (uint32_t i0 = threadIdx.x; i0 < packsIn; i0 += U * kBlock) {
+      PS v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const PS*>(in) + min(i0 + u * kBlock, packsIn - 1));
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t i = i0 + u * kBlock;
+        if (i < packsIn) {
+#pragma unroll
+          for (uint32_t e = 0; e < VS; ++e) lds[src_slot(i * VS + e)] = cvt(v[u].v[e]);
+        }
+      }
+    }
+    for (uint32_t m = packsIn * VS + threadIdx.x; m < n; m += kBlock) lds[src_slot(m)] = cvt(in[m]);
+    __syncthreads();
+    const uint32_t packsOut = VOUT ? n / VT : 0;
+    for (uint32_t i = threadIdx.x; i < packsOut; i += kBlock) {
+      PT v;
+#pragma unroll
+      for (uint32_t e = 0; e < VT; ++e) v.v[e] = lds[dst_slot(i * VT + e)];
+      PT* at = reinterpret_cast<PT*>(out) + i;
+      if (a.ntStore) store_pack<true>(at, v);
+      else store_pack<false>(at, v);
+    }
+    for (uint32_t m = packsOut * VT + threadIdx.x; m < n; m += kBlock) out[m] = lds[dst_slot(m)];
+    __syncthreads();  // the tile is refilled by the next round
+  }
+}
+
+// `pl` as for launch_skinny_copy. Returns false when the layouts are not of this kind.
+template <typename ES, typename ED = ES>
+bool launch_small_transpose(THCState* s, const Plan& pl) {
+  using E = typename std::conditional<(sizeof(ES) > sizeof(ED)), ES, ED>::type;
+  if (!tuning("apply.small_transpose", 1) || pl.nops != 2) return false;
+  const int nd = pl.lay[0].dims;
+  if (nd < 3 || pl.numel >= (int64_t(1) << 40)) return false;
+  const Layout& out = pl.lay[0];
+  const Layout& in = pl.lay[1];
+  const int q = nd - 1, p = nd - 2, bd = nd - 3;
+  const int64_t P = out.size[p], Q = out.size[q], PQ = P * Q;
+  if (P < 2 || Q < 2 || P >= 64 || Q >= 64) return false;
+  if (out.stride[q] != 1 || out.stride[p] != Q || in.stride[p] != 1 || in.stride[q] != P) return false;
+  if (out.stride[bd] != PQ || in.stride[bd] != PQ || out.size[bd] < 8) return false;
+  for (int k = 0; k < 2; ++k)
+    for (int d = 0; d < nd; ++d)
+      if (pl.lay[k].stride[d] < 0) return false;
+  SmallTransposeArgs a{};
+  a.P = (uint32_t)P;
+  a.Q = (uint32_t)Q;
+  a.batch = (uint64_t)out.size[bd];
+  // K matrices per tile: about 16 KiB, a whole number of 16-element groups so that tiles start on pack boundaries
+  int64_t K = std::max<int64_t>(1, tuning("apply.skinny.tile_bytes", 16384) / (PQ * (int64_t)sizeof(E)));
+  int64_t unit = 16;
+  for (int64_t g = PQ; g % 2 == 0 && unit > 1; g /= 2) unit /= 2;  // 16 / gcd(PQ, 16)
+  K = std::max<int64_t>(unit, K / unit * unit);
+  K = std::min<int64_t>(K, (out.size[bd] + unit - 1) / unit * unit);
+  a.K = (uint32_t)K;
+  a.pitch = (uint32_t)(Q * (P + 1));
+  a.pdiv.set((uint64_t)P);
+  a.qdiv.set((uint64_t)Q);
+  a.pqdiv.set((uint64_t)PQ);
+  const int64_t tiles = (out.size[bd] + K - 1) / K;
+  a.tilesPerRun.set((uint64_t)tiles);
+  int64_t total = tiles;
+  a.nbatch = 0;
+  for (int d = nd - 4; d >= 0; --d) {
+    a.bsize[a.nbatch].set((uint64_t)out.size[d]);
+    a.dstBatchStride[a.nbatch] = out.stride[d];
+    a.srcBatchStride[a.nbatch] = in.stride[d];
+    ++a.nbatch;
+    total *= out.size[d];
+  }
+  if (total >= (int64_t(1) << 31)) return false;
+  a.totalTiles = (uint32_t)total;
+  a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(ED)) ? 1 : 0;
+  auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
+  bool vout = aligned(pl.ptr[0]), vin = aligned(pl.ptr[1]);
+  for (int j = 0; j < a.nbatch; ++j) {
+    vout = vout && (a.dstBatchStride[j] * (int64_t)sizeof(ED)) % 16 == 0;
+    vin = vin && (a.srcBatchStride[j] * (int64_t)sizeof(ES)) % 16 == 0;
+  }
+  const size_t ldsBytes = ((size_t)K * a.pitch * sizeof(ED) + 15) & ~size_t(15);
+  if (ldsBytes > 64 * 1024) return false;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(total, (int64_t)num_compute_units(s) * 64));
+  ED* dst = (ED*)pl.ptr[0];
+  const ES* src = (const ES*)pl.ptr[1];
+  hipStream_t st = current_stream(s);
+#define THC_SMALLT(VI, VO) \
+  hipLaunchKernelGGL((small_transpose_kernel<ES, ED, VI, VO>), dim3(grid), dim3(kBlock), ldsBytes, st, dst, src, a)
+  if (vin && vout) THC_SMALLT(true, true);
+  else if (vin) THC_SMALLT(true, false);
+  else if (vout) THC_SMALLT(false, true);
+  else THC_SMALLT(false, false);
+#undef THC_SMALLT
+  note_kernel("small-transpose");
+  return true;
+}
+
 }  // namespace
 }  // namespace thc

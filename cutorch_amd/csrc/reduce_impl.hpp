@@ -2847,7 +2847,7 @@ void run_index_typed(THCState* s, const ReduceGeom& g, const T* in, T* outV, lon
         while ((folds + 1) * (folds + 1) * pattern <= reps * C && (folds + 1) * pattern <= kBlock && folds + 1 <= reps) ++folds;
       }
       const int64_t npacks = g.R * C / VEC;
-      const int64_t want = std::max<int64_t>(1, (int64_t)num_compute_units(s) * tuning("reduce.tall.index_blocks_per_cu", 2) / O);
+      const int64_t want = std::max<int64_t>(1, (int64_t)num_compute_units(s) * tuning("reduce.tall.index_blocks_per_cu", 4) / O);
       int64_t packsPerWg = std::max<int64_t>((npacks + want - 1) / want, lanes * 8);
       packsPerWg = (packsPerWg + period - 1) / period * period;
       const int64_t ST = (npacks + packsPerWg - 1) / packsPerWg;

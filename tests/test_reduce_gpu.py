@@ -344,6 +344,36 @@ def test_all_reductions(thc, oracle, kind):
         assert dev.minall() == oracle.reduce_all("min", ref)
 
 
+@pytest.mark.parametrize("kind", ["float", "double", "int"])
+def test_all_reductions_on_permuted_dense_views(thc, kind):
+    """A transposed or permuted view of a dense block is reduced in storage order (no contiguous copy is
+    made first): sums, extremes, products and moments of integer-valued data are exact whatever the order."""
+    rng = np.random.default_rng(47)
+    dtype = {"float": np.float32, "double": np.float64, "int": np.int32}[kind]
+    for shape, perm in (((300, 700), (1, 0)), ((37, 41, 53), (2, 0, 1)), ((5, 6, 7, 8), (3, 1, 0, 2)), ((1, 90000), (1, 0))):
+        x = rng.integers(-3, 4, shape).astype(dtype)
+        view = thc.Tensor.from_numpy(x)
+        strides = [int(s // x.itemsize) for s in x.strides]
+        pv = view.view_as_strided(0, tuple(shape[p] for p in perm), tuple(strides[p] for p in perm))
+        assert not pv.is_contiguous() or 1 in shape
+        for knob in (1, 0):
+            thc.set_tuning("reduce.all.by_stride", knob)
+            try:
+                assert pv.sumall() == x.astype(np.int64).sum()
+                assert pv.maxall() == x.max() and pv.minall() == x.min()
+                if kind != "int":
+                    np.testing.assert_allclose(pv.varall(), np.var(x.astype(np.float64), ddof=1), rtol=1e-5)
+                    np.testing.assert_allclose(pv.normall(2.0), np.sqrt((x.astype(np.float64) ** 2).sum()), rtol=1e-6)
+                    assert pv.meanall() == pytest.approx(x.astype(np.float64).mean(), rel=1e-6, abs=1e-7)
+            finally:
+                thc.set_tuning("reduce.all.by_stride", 1)
+    if kind != "int":
+        ones = np.ones((64, 130), dtype)
+        ones[::7, ::11] = 2
+        pv = thc.Tensor.from_numpy(ones).t()
+        assert pv.prodall() == float(np.prod(ones.astype(np.float64)))      # 2^120
+
+
 def test_all_reductions_on_strided_views(thc, oracle):
     rng = np.random.default_rng(42)
     for shape in ((40, 50), (7, 8, 9), (300,)):

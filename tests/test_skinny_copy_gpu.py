@@ -123,3 +123,45 @@ def test_converting_copies_between_image_layouts(thc, src_kind, dst_kind):
         dst.copy_from(src)
         assert thc.last_kernel() == "skinny"
         assert_bit_equal(dst.numpy(), np.ascontiguousarray(planar[off:].reshape(short_n, long_n).T).astype(ddt))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", sorted(KINDS))
+def test_batches_of_small_transposed_matrices(thc, kind):
+    """(B, P, Q) <- (B, Q, P) transposed per matrix, P and Q below 64: tiles of whole matrices that are one
+    contiguous run on both sides. Square and oblong matrices, batch counts off the tile size, an outer
+    batch dim with padding between its rows, storage offsets off the 16-byte grid, whole destination
+    storage compared."""
+    rng = np.random.default_rng(45)
+    dtype = KINDS[kind]
+    for b, p, q in ((1000, 4, 4), (5003, 3, 3), (777, 8, 8), (300, 16, 16), (129, 32, 32), (65, 5, 7), (40, 63, 2), (2500, 2, 3)):
+        for off_in, off_out in ((0, 0), (1, 3)):
+            src = values(rng, b * p * q + off_in, dtype)
+            dst = values(rng, b * p * q + off_out + 4, dtype)
+            a = thc.Tensor.from_storage(src, off_in, (b, p, q), (p * q, 1, p), kind=kind)        # per-matrix transpose
+            out = thc.Tensor.from_storage(dst, off_out, (b, p, q), (p * q, q, 1), kind=kind)
+            out.copy(a)
+            assert thc.last_kernel() == "small-transpose", (kind, b, p, q, thc.last_kernel())
+            want = dst.copy()
+            want[off_out:off_out + b * p * q] = src[off_in:].reshape(b, q, p).transpose(0, 2, 1).reshape(-1)
+            assert_bit_equal(out.storage_numpy(), want, "%s %dx%dx%d +%d/+%d" % (kind, b, p, q, off_in, off_out))
+    # an outer batch dim whose rows are padded on both sides
+    o, b, p, q, pad_in, pad_out = 3, 50, 6, 5, 16, 32
+    src = values(rng, o * (b * p * q + pad_in), dtype)
+    dst = values(rng, o * (b * p * q + pad_out), dtype)
+    a = thc.Tensor.from_storage(src, 0, (o, b, p, q), (b * p * q + pad_in, p * q, 1, p), kind=kind)
+    out = thc.Tensor.from_storage(dst, 0, (o, b, p, q), (b * p * q + pad_out, p * q, q, 1), kind=kind)
+    out.copy(a)
+    assert thc.last_kernel() == "small-transpose"
+    want = dst.copy().reshape(o, -1)
+    want[:, :b * p * q] = src.reshape(o, -1)[:, :b * p * q].reshape(o, b, q, p).transpose(0, 1, 3, 2).reshape(o, -1)
+    assert_bit_equal(out.storage_numpy(), want.reshape(-1))
+    thc.set_tuning("apply.small_transpose", 0)
+    try:
+        x = values(rng, 200 * 4 * 4, dtype)
+        out = thc.Tensor(kind).resize((200, 4, 4))
+        out.copy(thc.Tensor.from_storage(x, 0, (200, 4, 4), (16, 1, 4), kind=kind))
+        assert thc.last_kernel() != "small-transpose"
+        assert_bit_equal(out.numpy(), x.reshape(200, 4, 4).transpose(0, 2, 1))
+    finally:
+        thc.set_tuning("apply.small_transpose", 1)
