@@ -336,7 +336,7 @@ def build_configs(thc, hip, which, only=None, stagger=0):
                       "N-cumsum-rows10", "N-cumsum-tall", "N-add-t-odd", "N-bias-odd", "N-int-add-t", "N-lt-t", "N-add-2p25", "N-add-2p26", "CEIL-copy-rot", "CEIL-3r1w-rot",
                       "N-half-exp", "N-half-abs-t", "N-half-exp-t", "N-half-exp-t-odd", "N-short-add-t", "N-short-add-t-odd", "N-short-neg-t", "N-int-neg-t", "N-cvt-float-t", "N-cmax-t", "N-cmax-t-odd", "N-int-div-t", "N-int-lt-t",
                       "N-cvt-half-t", "N-equal", "N-copy-contig-64M", "N-copy-contig-256M", "N-copy-contig-1G",
-                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd", "N-cvt-image", "N-transpose-16x16", "N-sumall-t")
+                      "N-add-strided", "N-add-strided-u64", "N-var-tall", "N-cumsum-wide", "N-cumsum-1d", "N-copy-nhwc3", "N-copy-skinny16", "N-argmax-1d", "N-argmax-tall", "N-add-view-odd", "N-cvt-image", "N-transpose-16x16", "N-sumall-t", "N-std-rows8192")
           if (only and n in only) or (not only and which == "all")]
     if nx:
         ne = 1 << 26
@@ -535,6 +535,10 @@ def build_configs(thc, hip, which, only=None, stagger=0):
             va, vb, vc = (w.narrow(1, o, 8187) for w, o in zip(vw, (3, 1, 2)))
             table["N-add-view-odd"] = ("c = a + b on 8192x8187 fp32 views of 8192x8200 matrices at column offsets 2, 3, 1",
                                        12 * 8192 * 8187, 8192 * 8187, lambda i: vc.cadd(va, 1.0, vb))
+        if "N-std-rows8192" in nx:
+            std_o = T("float").resize((8192, 1))
+            table["N-std-rows8192"] = ("std over last dim of 8192x8192 fp32 (rows beyond a lane group's registers, one read)",
+                                       4 * 8192 * 8192 + 4 * 8192, 8192 * 8192, lambda i: std_o.std(sq, 1))
         if "N-sumall-t" in nx:
             table["N-sumall-t"] = ("sumall over the transposed view of 8192x8192 fp32 (blocks on the scalar)", 4 * 8192 * 8192,
                                    8192 * 8192, lambda i: sq_t.sumall())

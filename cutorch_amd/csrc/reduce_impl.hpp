@@ -1468,6 +1468,15 @@ __global__ __launch_bounds__(kBlock) void var_rows_kernel(const T* __restrict__ 
   }
 }
 
+// var / std along a unit-stride dim of rows too long for the registers (layer statistics over 4096 or
+// 8192 features): a wave per row in ONE read, every lane running (count, mean, M2) per pack slot over
+// its packs, 8 requested at a time, then the slots and the lanes merged pairwise (the two-sweep
+// form read such rows twice: 0.40 of peak on 8192 x 8192).
+template <typename T, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void var_rows_long_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                                               OuterArgs<I> oa, I numRows, I R,
+                                                               typename Acc<T>::type div, bool wantStd);
+
 // ------------------------------------------------------------------ cols --
 template <typename I>
 struct ColsArgs {
@@ -1611,6 +1620,62 @@ __device__ __forceinline__ void moments_merge(A& na, A& ma, A& sa, A nb, A mb, A
     sa += sb + delta * delta * na * w;
   }
   na = n;
+}
+
+template <typename T, typename I, int VEC>
+__global__ __launch_bounds__(kBlock) void var_rows_long_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                                               OuterArgs<I> oa, I numRows, I R,
+                                                               typename Acc<T>::type div, bool wantStd) {
+  using P = Pack<T, VEC>;
+  using A = typename Acc<T>::type;
+  constexpr int U = 8;
+  const uint32_t lane = threadIdx.x & 63;
+  const I wavesPerGrid = (I)gridDim.x * (kBlock / 64);
+  const I step = (I)64 * VEC;
+  for (I row = (I)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); row < numRows; row += wavesPerGrid) {
+    I inOff, outOff;
+    oa.offsets(row, inOff, outOff);
+    const T* src = in + inOff;
+    A cnt = (A)0, mean[VEC], m2[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      mean[e] = (A)0;
+      m2[e] = (A)0;
+    }
+    for (I i = (I)lane * VEC; i < R; i += (I)U * step) {
+      P v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const I at = i + (I)u * step < R ? i + (I)u * step : i;  // (past the end: re-read, not used)
+        v[u] = load_pack<true>(reinterpret_cast<const P*>(src + at));
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (i + (I)u * step < R) {
+          cnt += (A)1;
+          const A inv = (A)1 / cnt;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            const A x = acc_up<A>(v[u].v[e]);
+            const A delta = x - mean[e];
+            mean[e] += delta * inv;
+            m2[e] += delta * (x - mean[e]);
+          }
+        }
+      }
+    }
+    A n = cnt, mu = mean[0], q = m2[0];
+#pragma unroll
+    for (int e = 1; e < VEC; ++e) moments_merge(n, mu, q, cnt, mean[e], m2[e]);
+    for (uint32_t o = 32; o > 0; o >>= 1) {
+      const A on = shfl_xor_any(n, o), omu = shfl_xor_any(mu, o), oq = shfl_xor_any(q, o);
+      moments_merge(n, mu, q, on, omu, oq);
+    }
+    if (lane == 0) {
+      const A v = q / div;
+      out[outOff] = acc_down<T>(wantStd ? sqrt_any(v) : v);
+    }
+  }
 }
 
 template <typename T, typename I, int VEC>
@@ -2961,6 +3026,25 @@ bool reduce_var_rows_type(THCState* s, const ReduceGeom& g, const void* in_, voi
     bool inRegisters = g.sR == 1 && aligned16(in) && g.R % VEC == 0 && g.R <= 64 * VEC * U;
     for (int d = 0; d < g.in.dims && inRegisters; ++d)
       inRegisters = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+    bool longRows = g.sR == 1 && aligned16(in) && g.R % VEC == 0 && g.R > 64 * VEC * U && tuning("reduce.var.long_rows", 1) &&
+                    g.outElems >= (int64_t)num_compute_units(s) * 4;
+    for (int d = 0; d < g.in.dims && longRows; ++d) longRows = g.in.stride[d] % VEC == 0 || g.in.size[d] == 1;
+    if (longRows) {
+      const int wpb = kBlock / 64;
+      const int grid = capped_grid(s, (g.outElems + wpb - 1) / wpb, "reduce.rows.blocks_per_cu", 64);
+      hipStream_t st = current_stream(s);
+      if (g.wide) {
+        OuterArgs<uint64_t> oa = make_outer<uint64_t>(g.in, g.out, g.in.dims);
+        hipLaunchKernelGGL((var_rows_long_kernel<T, uint64_t, VEC>), dim3(grid), dim3(kBlock), 0, st, in, out, oa,
+                           (uint64_t)g.outElems, (uint64_t)g.R, (A)div, wantStd);
+      } else {
+        OuterArgs<uint32_t> oa = make_outer<uint32_t>(g.in, g.out, g.in.dims);
+        hipLaunchKernelGGL((var_rows_long_kernel<T, uint32_t, VEC>), dim3(grid), dim3(kBlock), 0, st, in, out, oa,
+                           (uint32_t)g.outElems, (uint32_t)g.R, (A)div, wantStd);
+      }
+      note_kernel("var-rows-long");
+      return true;
+    }
     if (!inRegisters) {
       // rows that cannot be read as aligned packs: short dense ones are staged
       // through LDS (the register kernel, where it applies, is the faster one:

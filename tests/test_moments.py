@@ -165,6 +165,42 @@ def test_gpu_var_along_strided_dim_is_one_read_and_stable(thc, oracle, kind):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["float", "half", "double"])
+def test_gpu_var_of_long_rows_is_one_read(thc, kind):
+    """Rows too long for a lane group's registers (statistics over thousands of features) with enough
+    rows for the chip: a wave per row runs (count, mean, M2) per lane and merges; against float64 numpy
+    with a common offset of 40 sigma (8 for half), row lengths off the batch size, a strided row pitch."""
+    rng = np.random.default_rng(84)
+    dtype = {"float": np.float32, "half": np.float16, "double": np.float64}[kind]
+    tol = {"float": 2e-5, "half": 4e-3, "double": 1e-12}[kind]
+    centre = 4.0 if kind == "half" else 20.0
+    vec = 16 // np.dtype(dtype).itemsize
+    for rows, n, pitch in ((1500, 8192, 8192), (1100, 64 * vec * 8 + vec, 64 * vec * 8 + vec), (1030, 5000 // vec * vec, 6000 // vec * vec),
+                           (2, 1024, 70000 // vec * vec)):
+        store = (rng.standard_normal(rows * pitch) * 0.5 + centre).astype(dtype)
+        dev = thc.Tensor.from_storage(store, 0, (rows, n), (pitch, 1), kind=kind)
+        ref = store.reshape(rows, pitch)[:, :n].astype(np.float64)
+        for name, fn in (("var", np.var), ("std", np.std)):
+            for biased in (0, 1):
+                out = getattr(thc.Tensor(kind), name)(dev, 1, biased=biased)
+                if rows >= 1024:
+                    assert thc.last_kernel() == "var-rows-long", (rows, n, thc.last_kernel())
+                want = fn(ref, axis=1, ddof=0 if biased else 1, keepdims=True)
+                np.testing.assert_allclose(out.numpy().astype(np.float64), want, rtol=tol, err_msg="%s %s %d x %d" % (kind, name, rows, n))
+    x = (rng.standard_normal((1200, 4096)) + centre).astype(dtype)
+    dev = thc.Tensor.from_numpy(x)
+    a = thc.Tensor(kind).var(dev, 1).numpy()
+    assert np.array_equal(a, thc.Tensor(kind).var(dev, 1).numpy())        # same bits on every run
+    thc.set_tuning("reduce.var.long_rows", 0)
+    try:
+        b = thc.Tensor(kind).var(dev, 1).numpy()
+        assert thc.last_kernel() != "var-rows-long"
+    finally:
+        thc.set_tuning("reduce.var.long_rows", 1)
+    np.testing.assert_allclose(a.astype(np.float64), b.astype(np.float64), rtol=tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["float", "half", "double"])
 def test_gpu_var_of_long_narrow_slices_reads_flat_packs(thc, kind):
     """Few long slices of narrow rows (batch statistics of a tall matrix) are read as flat runs of
     aligned packs with a running (count, mean, M2) per lane and column: against float64 numpy, with a
