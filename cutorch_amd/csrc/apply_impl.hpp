@@ -1537,8 +1537,20 @@ bool launch_flatmix(THCState* s, const Plan& pl, Op op) {
       if (pl.lay[k].stride[d] < 0) return false;
       span += (pl.lay[k].size[d] - 1) * pl.lay[k].stride[d];
     }
-    // small AND smaller than the output: a broadcast operand, not a permuted one
-    if (span > limit || span * 8 > pl.numel) return false;
+    // small AND smaller than the output: a broadcast operand, not a permuted one. Under rows of a few
+    // elements ((N, 3) scaled by a column: the strided kernels go element by element there) any operand
+    // that is the output's own order with some dims repeated (stride 0) will do: its gathers run ahead
+    // monotonically, neighbouring lanes on neighbouring addresses.
+    bool repeated = pl.lay[0].size[nd - 1] * (int64_t)sizeof(T) < 64 && tuning("apply.flatmix.repeated", 1);
+    if (repeated) {
+      int64_t run = 1;
+      for (int d = nd - 1; d >= 0 && repeated; --d) {
+        if (pl.lay[k].stride[d] == 0 || pl.lay[k].size[d] == 1) continue;
+        repeated = pl.lay[k].stride[d] == run;
+        run *= pl.lay[k].size[d];
+      }
+    }
+    if (!repeated && (span > limit || span * 8 > pl.numel)) return false;
     ++gathered;
   }
   if (gathered == 0) return false;

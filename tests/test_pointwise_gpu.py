@@ -561,6 +561,38 @@ def test_broadcast_operands_on_rows_that_are_not_pack_aligned(thc, kind):
         thc.set_tuning("apply.flatmix", 1)
 
 
+@pytest.mark.parametrize("kind", ["float", "half", "int", "double"])
+def test_rows_of_a_few_elements_with_a_repeated_operand(thc, kind):
+    """(N, 3) scaled by a column, (N, 2, 5) plus a per-N offset: the output and one input are one dense
+    run, the other input is the output's own order with dims repeated (stride 0) and as large as N; under
+    rows of a few elements it is gathered beside the flat packs instead of going element by element."""
+    rng = np.random.default_rng(78)
+    dtype = {"float": np.float32, "half": np.float16, "int": np.int32, "double": np.float64}[kind]
+    for shape, rep_strides in (((70001, 3), (1, 0)), ((4099, 2, 5), (1, 0, 0)), ((3001, 4, 3), (4, 1, 0)), ((50000, 7), (1, 0))):
+        x = rng.integers(-4, 5, shape).astype(dtype)
+        small_shape = tuple(n if st else 1 for n, st in zip(shape, rep_strides))
+        rep = rng.integers(-3, 4, small_shape).astype(dtype)
+        dx = thc.Tensor.from_numpy(x)
+        drep = thc.Tensor.from_numpy(rep.reshape(-1)).view_as_strided(0, shape, rep_strides)
+        flat = kind in ("float", "half")          # (the other types' functors have no flat + gathered kernel)
+        out = thc.Tensor(kind).cmul(dx, drep)
+        assert not flat or thc.last_kernel() == "flat-gather", (kind, shape, thc.last_kernel())
+        assert_bit_equal(out.numpy(), (x * rep).astype(dtype))
+        acc = thc.Tensor.from_numpy(x.copy())
+        acc.cadd(acc, 2, drep)                                   # in place on the dense operand
+        assert not flat or thc.last_kernel() == "flat-gather"
+        assert_bit_equal(acc.numpy(), (x + dtype(2) * rep).astype(dtype))
+    thc.set_tuning("apply.flatmix.repeated", 0)
+    try:
+        x = rng.integers(-4, 5, (5000, 3)).astype(dtype)
+        col = rng.integers(-3, 4, (5000, 1)).astype(dtype)
+        out = thc.Tensor(kind).cmul(thc.Tensor.from_numpy(x), thc.Tensor.from_numpy(col.reshape(-1)).view_as_strided(0, (5000, 3), (1, 0)))
+        assert thc.last_kernel() != "flat-gather"
+        assert_bit_equal(out.numpy(), (x * col).astype(dtype))
+    finally:
+        thc.set_tuning("apply.flatmix.repeated", 1)
+
+
 @pytest.mark.parametrize("kind", ["float", "int", "double", "long", "half", "byte"])
 def test_strided_rows_off_the_16_byte_grid(thc, kind):
     """Views whose rows start off the 16-byte grid and have odd lengths (x[:, 1:-2] of a wider matrix):
