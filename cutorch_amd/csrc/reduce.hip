@@ -165,7 +165,7 @@ void reduce_dim_index(THCState* s, DType dt, bool isMax, AnyTensor* values, AnyT
 Layout layout_by_stride(const AnyTensor* t) {
   Layout l = tensor_layout(t);
   for (int d = 0; d < l.dims; ++d)
-    if (l.stride[d] < 0) return l;
+    if (l.stride[d] < 0 || (l.stride[d] == 0 && l.size[d] > 1)) return l;  // (repeated dims keep their place)
   int order[kMaxDims];
   for (int d = 0; d < l.dims; ++d) order[d] = d;
   std::stable_sort(order, order + l.dims, [&](int a, int b) {

@@ -367,6 +367,9 @@ def test_all_reductions_on_permuted_dense_views(thc, kind):
                     assert pv.meanall() == pytest.approx(x.astype(np.float64).mean(), rel=1e-6, abs=1e-7)
             finally:
                 thc.set_tuning("reduce.all.by_stride", 1)
+    row = rng.integers(-3, 4, 700).astype(dtype)
+    expanded = thc.Tensor.from_numpy(row).view_as_strided(0, (300, 700), (0, 1))        # a repeated dim stays where it is
+    assert expanded.sumall() == 300 * int(row.astype(np.int64).sum()) and expanded.maxall() == row.max()
     if kind != "int":
         ones = np.ones((64, 130), dtype)
         ones[::7, ::11] = 2
