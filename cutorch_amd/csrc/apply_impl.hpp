@@ -1215,8 +1215,9 @@ bool indexed_can_pack(const Plan& pl) {
 }
 
 // Whether the strided kernel can run on packs at element-aligned addresses with a partial last pack per
-// row: unit stride along the innermost dim for every operand, rows of at least a few packs, and every
-// pack start 4-byte aligned (always so for 4- and 8-byte elements).
+// row: unit stride along the innermost dim for every operand and rows of at least a few packs. Global
+// accesses may sit at any byte address here, so 1- and 2-byte elements at odd element offsets qualify as
+// well (`apply.indexed.pack_align` restores a coarser requirement: 4 = every pack start 4-byte aligned).
 template <typename T, typename TOut>
 bool indexed_can_pack_unaligned(const Plan& pl) {
   constexpr int VEC = pack_elems<T, TOut>();
@@ -1226,7 +1227,7 @@ bool indexed_can_pack_unaligned(const Plan& pl) {
   for (int k = 0; k < pl.nops; ++k) {
     if (pl.lay[k].stride[nd - 1] != 1) return false;
     const size_t es = k == 0 ? sizeof(TOut) : sizeof(T);
-    const size_t al = std::min<size_t>(4, VEC * es);
+    const size_t al = std::min<size_t>((size_t)std::max<int64_t>(1, tuning("apply.indexed.pack_align", 1)), VEC * es);
     if (reinterpret_cast<uintptr_t>(pl.ptr[k]) % al != 0) return false;
     for (int d = 0; d < nd - 1; ++d)
       if ((pl.lay[k].stride[d] * (int64_t)es) % (int64_t)al != 0) return false;

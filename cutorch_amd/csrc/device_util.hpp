@@ -57,17 +57,26 @@ __device__ __forceinline__ P load_pack(const P* p) {
   }
   return *p;
 }
-// The same accesses at addresses that are only 4-byte aligned (rows of 4- and 8-byte elements that start
-// off the 16-byte grid): still ONE 16-byte instruction per pack, which the hardware splits where it has to.
+// The same accesses at addresses that are only element aligned (rows that start off the 16-byte grid):
+// still ONE 16-byte instruction per pack, which the hardware splits where it has to (global memory
+// accesses may sit at any byte address on this target).
 template <int N>
 struct RawBitsU : RawBits<N> {};
 template <>
 struct RawBitsU<16> {
-  typedef unsigned type __attribute__((ext_vector_type(4), aligned(4)));
+  typedef unsigned type __attribute__((ext_vector_type(4), aligned(1)));
 };
 template <>
 struct RawBitsU<8> {
-  typedef unsigned type __attribute__((ext_vector_type(2), aligned(4)));
+  typedef unsigned type __attribute__((ext_vector_type(2), aligned(1)));
+};
+template <>
+struct RawBitsU<4> {
+  typedef uint32_t type __attribute__((aligned(1)));
+};
+template <>
+struct RawBitsU<2> {
+  typedef uint16_t type __attribute__((aligned(1)));
 };
 template <bool NT, typename P>
 __device__ __forceinline__ P load_pack_unaligned(const void* p) {

@@ -596,13 +596,13 @@ def test_rows_of_a_few_elements_with_a_repeated_operand(thc, kind):
 @pytest.mark.parametrize("kind", ["float", "int", "double", "long", "half", "byte"])
 def test_strided_rows_off_the_16_byte_grid(thc, kind):
     """Views whose rows start off the 16-byte grid and have odd lengths (x[:, 1:-2] of a wider matrix):
-    4- and 8-byte elements move as packs at element-aligned addresses with a partial last pack per row,
-    narrower elements element by element. In place and out of place, one to three inputs, every
+    the elements move as packs at element-aligned addresses with a partial last pack per row (rows
+    shorter than four packs element by element). In place and out of place, one to three inputs, every
     operand at its own offset; the whole destination storage is compared."""
     rng = np.random.default_rng(77)
     dtype = {"float": np.float32, "int": np.int32, "double": np.float64, "long": np.int64, "half": np.float16,
              "byte": np.uint8}[kind]
-    wide = dtype().itemsize >= 4
+    wide = True      # (packs at element-aligned addresses for every element size)
     for rows, cols, pitch, offs in ((37, 101, 128, (1, 3, 2, 5)), (64, 8187, 8200, (3, 1, 1, 2)), (5, 16, 19, (1, 2, 3, 0)),
                                     (3, 7, 9, (1, 1, 1, 1)), (200, 33, 40, (0, 1, 2, 3)), (6, 700, 4097, (5, 6, 7, 9))):
         lo, hi = (0, 5) if kind == "byte" else (-4, 5)
