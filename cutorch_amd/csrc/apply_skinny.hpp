@@ -5,8 +5,8 @@
 // of 3..64 elements (a (2^22, 16) transpose ran at 0.09 of peak through them, and the element-wise
 // strided kernel at 0.33-0.38 on 3 or 4 planes). Here a tile is T long-dim positions x all S
 // short-dim positions, about 16 KiB: on the dense side one contiguous run of T * S elements, on the
-// planar side S runs of T elements. Both sides move 16-byte packs where their alignment allows
-// (element-wise otherwise); the tile changes order in LDS, laid out lds[s * pitch + t].
+// planar side S runs of T elements. Both sides move 16-byte packs, at element-aligned addresses where
+// a run starts off the 16-byte grid; the tile changes order in LDS, laid out lds[s * pitch + t].
 // (what the reference's one strided apply does for these copies: lib/THC/THCApply.cuh:426-640,
 // called from lib/THC/THCTensorCopy.cu:26-122)
 #pragma once
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(ED* __restrict__ ds
         PS v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-          v[u] = load_pack<true>(reinterpret_cast<const PS*>(dsrc) + min(k0 + u * kBlock, packs - 1));
+          v[u] = load_pack_unaligned<true, PS>(dsrc + (size_t)min(k0 + u * kBlock, packs - 1) * VS);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const uint32_t k = k0 + u * kBlock;
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(ED* __restrict__ ds
         for (int u = 0; u < U; ++u) {
           const uint32_t k = min(k0 + u * kBlock, packs - 1);
           const uint32_t s = k / (VP ? planePacks : 1u), j = k - s * planePacks;
-          v[u] = load_pack<true>(reinterpret_cast<const PS*>(psrc + (int64_t)s * a.planeStride) + j);
+          v[u] = load_pack_unaligned<true, PS>(psrc + (int64_t)s * a.planeStride + (int64_t)j * VS);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -140,9 +140,9 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(ED* __restrict__ ds
         PT v;
 #pragma unroll
         for (uint32_t e = 0; e < VT; ++e) v.v[e] = lds[s * pitch + j * VT + e];
-        PT* at = reinterpret_cast<PT*>(pdst + (int64_t)s * a.planeStride) + j;
-        if (a.ntStore) store_pack<true>(at, v);
-        else store_pack<false>(at, v);
+        ED* at = pdst + (int64_t)s * a.planeStride + (int64_t)j * VT;
+        if (a.ntStore) store_pack_unaligned<true, PT>(at, v);
+        else store_pack_unaligned<false, PT>(at, v);
       }
       const uint32_t left = tn - planePacks * VT;
       for (uint32_t m = threadIdx.x; m < left * S; m += kBlock) {
@@ -164,9 +164,9 @@ __global__ __launch_bounds__(kBlock) void skinny_copy_kernel(ED* __restrict__ ds
             ++t;
           }
         }
-        PT* at = reinterpret_cast<PT*>(ddst) + k;
-        if (a.ntStore) store_pack<true>(at, v);
-        else store_pack<false>(at, v);
+        ED* at = ddst + (size_t)k * VT;
+        if (a.ntStore) store_pack_unaligned<true, PT>(at, v);
+        else store_pack_unaligned<false, PT>(at, v);
       }
       for (uint32_t m = packs * VT + threadIdx.x; m < n; m += kBlock) {
         uint32_t t, s;
@@ -234,12 +234,18 @@ bool launch_skinny_copy(THCState* s, const Plan& pl) {
   a.totalTiles = (uint32_t)total;
   a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(ED)) ? 1 : 0;
   // packs: every tile's run starts on a 16-byte boundary (operand 0 holds ED elements, operand 1 ES)
+  // (`apply.skinny.aligned_packs_only`: packs only where every tile's run starts on a 16-byte boundary, the
+  // element-wise variants elsewhere; by default packs sit at element-aligned addresses, which this target allows)
   auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
   const int64_t denseBytes = dense == 0 ? sizeof(ED) : sizeof(ES), planarBytes = dense == 0 ? sizeof(ES) : sizeof(ED);
-  bool vd = aligned(pl.ptr[dense]), vp = aligned(pl.ptr[1 - dense]) && (a.planeStride * planarBytes) % 16 == 0;
-  for (int j = 0; j < a.nbatch; ++j) {
-    vd = vd && (a.denseBatchStride[j] * denseBytes) % 16 == 0;
-    vp = vp && (a.planarBatchStride[j] * planarBytes) % 16 == 0;
+  bool vd = true, vp = true;
+  if (tuning("apply.skinny.aligned_packs_only", 0)) {
+    vd = aligned(pl.ptr[dense]);
+    vp = aligned(pl.ptr[1 - dense]) && (a.planeStride * planarBytes) % 16 == 0;
+    for (int j = 0; j < a.nbatch; ++j) {
+      vd = vd && (a.denseBatchStride[j] * denseBytes) % 16 == 0;
+      vp = vp && (a.planarBatchStride[j] * planarBytes) % 16 == 0;
+    }
   }
   const size_t ldsBytes = ((size_t)S * a.pitch * sizeof(ED) + 15) & ~size_t(15);
   if (ldsBytes > 64 * 1024) return false;
@@ -330,7 +336,7 @@ __global__ __launch_bounds__(kBlock) void small_transpose_kernel(ED* __restrict_
     for (uint32_t i0 = threadIdx.x; i0 < packsIn; i0 += U * kBlock) {
       PS v[U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) v[u] = load_pack<true>(reinterpret_cast<const PS*>(in) + min(i0 + u * kBlock, packsIn - 1));
+      for (int u = 0; u < U; ++u) v[u] = load_pack_unaligned<true, PS>(in + (size_t)min(i0 + u * kBlock, packsIn - 1) * VS);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const uint32_t i = i0 + u * kBlock;
@@ -347,9 +353,9 @@ __global__ __launch_bounds__(kBlock) void small_transpose_kernel(ED* __restrict_
       PT v;
 #pragma unroll
       for (uint32_t e = 0; e < VT; ++e) v.v[e] = lds[dst_slot(i * VT + e)];
-      PT* at = reinterpret_cast<PT*>(out) + i;
-      if (a.ntStore) store_pack<true>(at, v);
-      else store_pack<false>(at, v);
+      ED* at = out + (size_t)i * VT;
+      if (a.ntStore) store_pack_unaligned<true, PT>(at, v);
+      else store_pack_unaligned<false, PT>(at, v);
     }
     for (uint32_t m = packsOut * VT + threadIdx.x; m < n; m += kBlock) out[m] = lds[dst_slot(m)];
     __syncthreads();  // the tile is refilled by the next round
@@ -403,10 +409,14 @@ bool launch_small_transpose(THCState* s, const Plan& pl) {
   a.totalTiles = (uint32_t)total;
   a.ntStore = streaming_store("apply.tiled.nt_store", pl.numel * (int64_t)sizeof(ED)) ? 1 : 0;
   auto aligned = [](const void* ptr) { return reinterpret_cast<uintptr_t>(ptr) % 16 == 0; };
-  bool vout = aligned(pl.ptr[0]), vin = aligned(pl.ptr[1]);
-  for (int j = 0; j < a.nbatch; ++j) {
-    vout = vout && (a.dstBatchStride[j] * (int64_t)sizeof(ED)) % 16 == 0;
-    vin = vin && (a.srcBatchStride[j] * (int64_t)sizeof(ES)) % 16 == 0;
+  bool vout = true, vin = true;
+  if (tuning("apply.skinny.aligned_packs_only", 0)) {
+    vout = aligned(pl.ptr[0]);
+    vin = aligned(pl.ptr[1]);
+    for (int j = 0; j < a.nbatch; ++j) {
+      vout = vout && (a.dstBatchStride[j] * (int64_t)sizeof(ED)) % 16 == 0;
+      vin = vin && (a.srcBatchStride[j] * (int64_t)sizeof(ES)) % 16 == 0;
+    }
   }
   const size_t ldsBytes = ((size_t)K * a.pitch * sizeof(ED) + 15) & ~size_t(15);
   if (ldsBytes > 64 * 1024) return false;

@@ -27,6 +27,8 @@ def test_tall_skinny_transposes_both_directions(thc, kind):
     for long_n, short_n in ((100000, 3), (65536, 4), (70001, 5), (4099, 16), (30000, 31), (1000, 2), (64, 7)):
         if short_n * np.dtype(dtype).itemsize > 256:
             continue
+        # (odd storage offsets: packs at element-aligned addresses; with the knob, the element-wise variants)
+        thc.set_tuning("apply.skinny.aligned_packs_only", 1 if long_n in (70001, 4099) else 0)
         for off in (0, 1):
             planar = values(rng, short_n * long_n + off, dtype)
             src = thc.Tensor.from_storage(planar, off, (long_n, short_n), (1, long_n), kind=kind)     # (short, long):t()
@@ -47,6 +49,7 @@ def test_tall_skinny_transposes_both_directions(thc, kind):
             after = ddst.storage_numpy()
             assert_bit_equal(after[:5 + off], guard[:5 + off])
             assert_bit_equal(after[5 + off + short_n * long_n:], guard[5 + off + short_n * long_n:])
+    thc.set_tuning("apply.skinny.aligned_packs_only", 0)
 
 
 @pytest.mark.gpu
@@ -135,6 +138,7 @@ def test_batches_of_small_transposed_matrices(thc, kind):
     rng = np.random.default_rng(45)
     dtype = KINDS[kind]
     for b, p, q in ((1000, 4, 4), (5003, 3, 3), (777, 8, 8), (300, 16, 16), (129, 32, 32), (65, 5, 7), (40, 63, 2), (2500, 2, 3)):
+        thc.set_tuning("apply.skinny.aligned_packs_only", 1 if b in (5003, 300) else 0)
         for off_in, off_out in ((0, 0), (1, 3)):
             src = values(rng, b * p * q + off_in, dtype)
             dst = values(rng, b * p * q + off_out + 4, dtype)
@@ -145,6 +149,7 @@ def test_batches_of_small_transposed_matrices(thc, kind):
             want = dst.copy()
             want[off_out:off_out + b * p * q] = src[off_in:].reshape(b, q, p).transpose(0, 2, 1).reshape(-1)
             assert_bit_equal(out.storage_numpy(), want, "%s %dx%dx%d +%d/+%d" % (kind, b, p, q, off_in, off_out))
+    thc.set_tuning("apply.skinny.aligned_packs_only", 0)
     # an outer batch dim whose rows are padded on both sides
     o, b, p, q, pad_in, pad_out = 3, 50, 6, 5, 16, 32
     src = values(rng, o * (b * p * q + pad_in), dtype)
