@@ -138,12 +138,9 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
   const int sizeQ = (int)args.sizeQ;
   auto mis_in = [](const T* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(T)) & (uintptr_t)(VEC - 1)); };
   auto mis_out = [](const TOut* row) { return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(TOut)) & (uintptr_t)(VEC - 1)); };
-  // (global packs may sit at element-aligned addresses: rows of whole packs that start off the 16-byte grid
-  // run the ALIGNED form too; LDS accesses keep the 16-byte type)
-  using RAWG = typename RawBitsU<sizeof(PIN)>::type;
   auto load = [&](const T* at) -> RAW {
-    if constexpr (NTL) return __builtin_nontemporal_load(reinterpret_cast<const RAWG*>(at));
-    else return *reinterpret_cast<const RAWG*>(at);
+    if constexpr (NTL) return __builtin_nontemporal_load(reinterpret_cast<const RAW*>(at));
+    else return *reinterpret_cast<const RAW*>(at);
   };
 
   struct Tile {       // uniform over the workgroup
@@ -349,8 +346,8 @@ __global__ __launch_bounds__(kBlock) void apply_ldstile_kernel(TOut* out, const 
         for (int e = 0; e < VEC; ++e) res.v[e] = y[e];
         if constexpr (ALIGNED) {
           if (pi < t.pn && first < t.qn) {
-            if (args.ntStore) store_pack_unaligned<true, POUT>(orow + first, res);
-            else store_pack_unaligned<false, POUT>(orow + first, res);
+            if (args.ntStore) store_pack<true>(reinterpret_cast<POUT*>(orow + first), res);
+            else store_pack<false>(reinterpret_cast<POUT*>(orow + first), res);
           }
         } else {
           const int g = t.q0 + first;   // column of the pack's first element; lanes 0 .. LXQ - 2 own packs
@@ -405,56 +402,19 @@ bool launch_ldstile(THCState* s, const Plan& pl, Op op) {
     constexpr int LXP = (sizeof(T) == 1 && VEC == 16) ? 4 : ((128 / (int)sizeof(T)) / VEC < 8 ? 8 : (128 / (int)sizeof(T)) / VEC);
     const int nd = pl.lay[0].dims;
     auto elem_size = [](int k) { return k == 0 ? sizeof(TOut) : sizeof(T); };
-    // The pack form needs whole packs along p and q; where the packs sit is free (element-aligned global
-    // accesses), unless `apply.ldstile.any_address` is switched off: then every pack must start on a
-    // 16-byte boundary and everything else takes the shifted windows.
-    const bool anyAddress = tuning("apply.ldstile.any_address", 1) != 0;
     bool aligned = pl.lay[0].size[p] % VEC == 0 && pl.lay[0].size[q] % VEC == 0;
     for (int k = 0; k < pl.nops; ++k) {
       const int fast = staged[k] ? p : q;
       if (pl.lay[k].stride[fast] != 1) return false;
       if (reinterpret_cast<uintptr_t>(pl.ptr[k]) % elem_size(k) != 0) return false;
-      if (!anyAddress) aligned = aligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % (VEC * elem_size(k)) == 0;
+      aligned = aligned && reinterpret_cast<uintptr_t>(pl.ptr[k]) % (VEC * elem_size(k)) == 0;
       for (int d = 0; d < nd; ++d) {
         if (pl.lay[k].stride[d] < 0) return false;
-        if (d != fast && !anyAddress) aligned = aligned && pl.lay[k].stride[d] % VEC == 0;
+        if (d != fast) aligned = aligned && pl.lay[k].stride[d] % VEC == 0;
       }
       // lane offsets inside a tile are 32-bit
       const int64_t span = (int64_t)(LXQ * VEC) * std::max(pl.lay[k].stride[p], pl.lay[k].stride[q]) + 4096;
       if (span >= (int64_t(1) << 31)) return false;
-    }
-    // Sizes that are not whole packs, behind `apply.ldstile.peel` (off): the block of whole packs runs the
-    // pack form, the strips that are left (fewer than VEC rows or columns) the strided kernel. Measured on
-    // 8191 x 8193 against the shifted windows over everything: half exp 0.43 -> 0.44 of peak, int16 add
-    // 0.53 -> 0.55, fp32 cmax 0.60 -> 0.58: the strips' two launches cost what the block gains.
-    if (!aligned && anyAddress && tuning("apply.ldstile.peel", 0) && pl.lay[0].size[p] >= 8 * VEC &&
-        pl.lay[0].size[q] >= 8 * VEC) {
-      const int64_t P = pl.lay[0].size[p], Q = pl.lay[0].size[q];
-      const int64_t Pm = P / VEC * VEC, Qm = Q / VEC * VEC;
-      auto sub = [&](int64_t p0, int64_t pn, int64_t q0, int64_t qn) {
-        Plan c = pl;
-        for (int k = 0; k < pl.nops; ++k) {
-          c.lay[k].size[p] = pn;
-          c.lay[k].size[q] = qn;
-          c.ptr[k] = (char*)pl.ptr[k] + (p0 * pl.lay[k].stride[p] + q0 * pl.lay[k].stride[q]) * (int64_t)elem_size(k);
-        }
-        c.numel = pl.numel / (P * Q) * (pn * qn);
-        return c;
-      };
-      bool wide = force_64bit_index();
-      for (int k = 0; k < pl.nops; ++k) wide = wide || !fits_32bit(pl.lay[k]);
-      auto strip = [&](const Plan& c) {
-        if (c.numel <= 0) return;
-        if (wide) launch_indexed<T, Op, uint64_t, true, TOut>(s, c, op);
-        else launch_indexed<T, Op, uint32_t, true, TOut>(s, c, op);
-      };
-      const Plan mainBlock = sub(0, Pm, 0, Qm);
-      if (launch_ldstile<T, Op, TOut>(s, mainBlock, op)) {
-        strip(sub(0, P, Qm, Q - Qm));   // the last columns of every row
-        strip(sub(Pm, P - Pm, 0, Qm));  // the last rows, up to those columns
-        note_kernel("lds-tile-peeled");
-        return true;
-      }
     }
     LdsTileArgs args{};
     for (int k = 0; k < pl.nops; ++k) {

@@ -72,27 +72,11 @@ def operand_geoms(rng, shape, aligned, transposed):
     return geoms
 
 
-@pytest.fixture(autouse=True, params=["any-address", "any-address-peel", "aligned-only"])
-def pack_addressing(request, thc):
-    """Every test of this module runs three times: with packs at element-aligned addresses (rows of whole
-    packs take the pack form wherever they start: the default), the same with other sizes peeled into a
-    block of whole packs and two strips, and with packs on 16-byte boundaries only (everything else on
-    the shifted windows)."""
-    thc.set_tuning("apply.ldstile.any_address", 0 if request.param == "aligned-only" else 1)
-    thc.set_tuning("apply.ldstile.peel", 1 if request.param == "any-address-peel" else 0)
-    yield request.param
-    thc.set_tuning("apply.ldstile.any_address", 1)
-    thc.set_tuning("apply.ldstile.peel", 0)
-
-
 def expect_kernel(thc, shape, aligned, kind=None):
     k = thc.last_kernel()
     assert k.startswith("lds-tile") or k.startswith("tiled"), (k, shape, kind)
     if min(shape[0], shape[-1]) >= 8 and not aligned:
-        if thc.lib().THCAmd_getTuning(b"apply.ldstile.any_address"):
-            assert k in ("lds-tile-peeled", "lds-tile", "lds-tile-shift", "tiled-shift", "tiled-ragged", "tiled-scalar"), (k, shape, kind)
-        else:
-            assert k in ("lds-tile-shift", "tiled-shift", "tiled-ragged", "tiled-scalar"), (k, shape, kind)
+        assert k in ("lds-tile-shift", "tiled-shift", "tiled-ragged", "tiled-scalar"), (k, shape, kind)
 
 
 @pytest.mark.gpu
